@@ -1,0 +1,306 @@
+// C ABI of the dfdx ROCm matmul backend: context, storage helpers, GEMM dispatch.
+#include "../../include/dfdx_rocm.h"
+#include "gemm_internal.h"
+
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+using namespace dfdx_rocm;
+
+struct dfdx_rocm_ctx {
+    int device;
+    hipStream_t stream;
+    int compute_units;
+    int clock_mhz;
+    char name[128];
+    std::mutex mu;
+};
+
+namespace {
+
+#define HIP_TRY(expr)                      \
+    do {                                   \
+        hipError_t e__ = (expr);           \
+        if (e__ != hipSuccess) return (int)e__; \
+    } while (0)
+
+int bind(dfdx_rocm_ctx *ctx) {
+    if (!ctx) return DFDX_ROCM_ERR_INVALID_ARG;
+    HIP_TRY(hipSetDevice(ctx->device));
+    return DFDX_ROCM_OK;
+}
+
+// Validates `d` and produces the canonical problem (row-major C whenever the view allows it).
+int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
+    if (!d) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (d->dtype < DFDX_ROCM_F32 || d->dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (d->m < 0 || d->n < 0 || d->k < 0 || d->batch1 < 1 || d->batch2 < 1) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (d->m == 0 || d->n == 0) {
+        out->m = 0;
+        return DFDX_ROCM_OK;
+    }
+    if (!d->c || (d->k > 0 && (!d->a || !d->b))) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (d->c_rs < 0 || d->c_cs < 0 || d->c_b1 < 0 || d->c_b2 < 0) return DFDX_ROCM_ERR_INVALID_ARG;
+    // An output view that maps two logical elements to one address cannot be written without a reduction.
+    if ((d->m > 1 && d->c_rs == 0) || (d->n > 1 && d->c_cs == 0)) return DFDX_ROCM_ERR_ALIASED_OUTPUT;
+    if (!d->reduce_batch && ((d->batch1 > 1 && d->c_b1 == 0) || (d->batch2 > 1 && d->c_b2 == 0)))
+        return DFDX_ROCM_ERR_ALIASED_OUTPUT;
+    GemmProblem p;
+    p.dtype = d->dtype;
+    p.accumulate = d->accumulate != 0;
+    p.reduce = d->reduce_batch != 0 && d->batch1 * d->batch2 > 1;
+    p.bias_mode = d->bias ? BIAS_PER_COL : BIAS_NONE;
+    p.m = d->m; p.n = d->n; p.k = d->k;
+    p.nb1 = d->batch1; p.nb2 = d->batch2;
+    p.a = d->a; p.a_rs = d->a_rs; p.a_cs = d->a_cs; p.a_b1 = d->a_b1; p.a_b2 = d->a_b2;
+    p.b = d->b; p.b_rs = d->b_rs; p.b_cs = d->b_cs; p.b_b1 = d->b_b1; p.b_b2 = d->b_b2;
+    p.c = d->c; p.c_rs = d->c_rs; p.c_cs = d->c_cs;
+    p.c_b1 = p.reduce ? 0 : d->c_b1; p.c_b2 = p.reduce ? 0 : d->c_b2;
+    p.bias = d->bias;
+    // column-major C (a permuted operand's gradient): compute C^T = B^T A^T instead
+    if (p.c_cs != 1 && p.c_rs == 1 && p.n > 1) p = transposed(p);
+    *out = p;
+    return DFDX_ROCM_OK;
+}
+
+struct Plan {
+    int kernel, variant;
+};
+
+int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProblem &p, Plan *plan) {
+    const bool is16 = p.dtype == DT_F16 || p.dtype == DT_BF16;
+    const bool is32 = p.dtype == DT_F32;
+    switch (d->kernel) {
+    case DFDX_ROCM_KERNEL_GENERIC:
+        *plan = {DFDX_ROCM_KERNEL_GENERIC, 0};
+        return DFDX_ROCM_OK;
+    case DFDX_ROCM_KERNEL_GEMV:
+        if (!gemv_supported(p)) return DFDX_ROCM_ERR_UNSUPPORTED;
+        *plan = {DFDX_ROCM_KERNEL_GEMV, 0};
+        return DFDX_ROCM_OK;
+    case DFDX_ROCM_KERNEL_MFMA: {
+        int v = d->variant;
+        if (v == 0) v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units) : 0;
+        const bool ok = is16 ? mfma16_supported(p, v) : is32 ? mfma32_supported(p, v) : false;
+        if (!ok) return DFDX_ROCM_ERR_UNSUPPORTED;
+        *plan = {DFDX_ROCM_KERNEL_MFMA, v};
+        return DFDX_ROCM_OK;
+    }
+    case DFDX_ROCM_KERNEL_AUTO:
+        break;
+    default:
+        return DFDX_ROCM_ERR_INVALID_ARG;
+    }
+    if (gemv_supported(p)) {
+        *plan = {DFDX_ROCM_KERNEL_GEMV, 0};
+        return DFDX_ROCM_OK;
+    }
+    int v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units) : 0;
+    if (v > 0) {
+        *plan = {DFDX_ROCM_KERNEL_MFMA, v};
+        return DFDX_ROCM_OK;
+    }
+    *plan = {DFDX_ROCM_KERNEL_GENERIC, 0};
+    return DFDX_ROCM_OK;
+}
+
+int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &p, const Plan &plan) {
+    hipError_t e;
+    switch (plan.kernel) {
+    case DFDX_ROCM_KERNEL_GENERIC: e = launch_generic(p, ctx->stream); break;
+    case DFDX_ROCM_KERNEL_GEMV: e = launch_gemv(p, ctx->stream); break;
+    case DFDX_ROCM_KERNEL_MFMA:
+        e = (p.dtype == DT_F32) ? launch_mfma32(p, plan.variant, ctx->stream) : launch_mfma16(p, plan.variant, ctx->stream);
+        break;
+    default: return DFDX_ROCM_ERR_INVALID_ARG;
+    }
+    return (int)e;
+}
+
+}  // namespace
+
+extern "C" {
+
+int dfdx_rocm_create(int ordinal, void *stream, dfdx_rocm_ctx **out) {
+    if (!out || ordinal < 0) return DFDX_ROCM_ERR_INVALID_ARG;
+    *out = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || ordinal >= count) return DFDX_ROCM_ERR_NO_DEVICE;
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, ordinal));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) return DFDX_ROCM_ERR_NO_DEVICE;  // code objects are gfx950 only
+    HIP_TRY(hipSetDevice(ordinal));
+    dfdx_rocm_ctx *ctx = new (std::nothrow) dfdx_rocm_ctx();
+    if (!ctx) return (int)hipErrorOutOfMemory;
+    ctx->device = ordinal;
+    ctx->stream = (hipStream_t)stream;
+    ctx->compute_units = prop.multiProcessorCount;
+    ctx->clock_mhz = prop.clockRate / 1000;
+    std::snprintf(ctx->name, sizeof(ctx->name), "%s (%s)", prop.name, prop.gcnArchName);
+    *out = ctx;
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_destroy(dfdx_rocm_ctx *ctx) {
+    if (!ctx) return DFDX_ROCM_OK;
+    delete ctx;
+    return DFDX_ROCM_OK;
+}
+
+const char *dfdx_rocm_strerror(int code) {
+    switch (code) {
+    case DFDX_ROCM_OK: return "ok";
+    case DFDX_ROCM_ERR_INVALID_ARG: return "dfdx_rocm: invalid argument";
+    case DFDX_ROCM_ERR_UNSUPPORTED: return "dfdx_rocm: no kernel for this request";
+    case DFDX_ROCM_ERR_NO_DEVICE: return "dfdx_rocm: no usable gfx950 device";
+    case DFDX_ROCM_ERR_ALIASED_OUTPUT: return "dfdx_rocm: output view aliases itself (zero stride)";
+    default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "dfdx_rocm: unknown error";
+}
+
+int dfdx_rocm_device_info(dfdx_rocm_ctx *ctx, char *name, size_t name_len, int *compute_units, int *clock_mhz) {
+    if (!ctx) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (name && name_len) std::snprintf(name, name_len, "%s", ctx->name);
+    if (compute_units) *compute_units = ctx->compute_units;
+    if (clock_mhz) *clock_mhz = ctx->clock_mhz;
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_alloc(dfdx_rocm_ctx *ctx, size_t bytes, int zeroed, void **out) {
+    if (!out) return DFDX_ROCM_ERR_INVALID_ARG;
+    *out = nullptr;
+    if (int e = bind(ctx)) return e;
+    if (bytes == 0) bytes = 16;
+    void *p = nullptr;
+    HIP_TRY(hipMalloc(&p, bytes));
+    if (zeroed) {
+        hipError_t e = hipMemsetAsync(p, 0, bytes, ctx->stream);
+        if (e != hipSuccess) {
+            (void)hipFree(p);
+            return (int)e;
+        }
+    }
+    *out = p;
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_free(dfdx_rocm_ctx *ctx, void *ptr) {
+    if (int e = bind(ctx)) return e;
+    if (!ptr) return DFDX_ROCM_OK;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));  // pending kernels may still use the buffer
+    HIP_TRY(hipFree(ptr));
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_memset_zero(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes) {
+    if (int e = bind(ctx)) return e;
+    if (!ptr && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (bytes) HIP_TRY(hipMemsetAsync(ptr, 0, bytes, ctx->stream));
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_copy_h2d(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    if (int e = bind(ctx)) return e;
+    if ((!dst || !src) && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (bytes) {
+        HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));  // the host buffer may be reused on return
+    }
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_copy_d2h(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    if (int e = bind(ctx)) return e;
+    if ((!dst || !src) && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (bytes) {
+        HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_copy_d2d(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    if (int e = bind(ctx)) return e;
+    if ((!dst || !src) && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (bytes) HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_synchronize(dfdx_rocm_ctx *ctx) {
+    if (int e = bind(ctx)) return e;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_gemm(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc) {
+    if (int e = bind(ctx)) return e;
+    GemmProblem p;
+    if (int e = make_problem(desc, &p)) return e;
+    if (p.m == 0) return DFDX_ROCM_OK;
+    Plan plan;
+    if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    return run_plan(ctx, p, plan);
+}
+
+int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int *kernel, int *variant, char *name,
+                        size_t name_len) {
+    if (!ctx) return DFDX_ROCM_ERR_INVALID_ARG;
+    GemmProblem p;
+    if (int e = make_problem(desc, &p)) return e;
+    Plan plan = {DFDX_ROCM_KERNEL_GENERIC, 0};
+    if (p.m != 0)
+        if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    if (kernel) *kernel = plan.kernel;
+    if (variant) *variant = plan.variant;
+    if (name && name_len) {
+        if (plan.kernel == DFDX_ROCM_KERNEL_MFMA)
+            std::snprintf(name, name_len, "%s_%s", p.dtype == DT_F32 ? "mfma32" : "mfma16",
+                          p.dtype == DT_F32 ? mfma32_variant_name(plan.variant) : mfma16_variant_name(plan.variant));
+        else
+            std::snprintf(name, name_len, "%s", plan.kernel == DFDX_ROCM_KERNEL_GEMV ? "gemv" : "generic");
+    }
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_mfma_variant_count(int dtype) {
+    if (dtype == DFDX_ROCM_F16 || dtype == DFDX_ROCM_BF16) return mfma16_variant_count();
+    if (dtype == DFDX_ROCM_F32) return mfma32_variant_count();
+    return 0;
+}
+
+int dfdx_rocm_gemm_time(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int warmup, int iters, float *avg_ms) {
+    if (!avg_ms || iters < 1 || warmup < 0) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (int e = bind(ctx)) return e;
+    GemmProblem p;
+    if (int e = make_problem(desc, &p)) return e;
+    if (p.m == 0) {
+        *avg_ms = 0.0f;
+        return DFDX_ROCM_OK;
+    }
+    Plan plan;
+    if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    for (int i = 0; i < warmup; i++)
+        if (int e = run_plan(ctx, p, plan)) return e;
+    hipEvent_t t0, t1;
+    HIP_TRY(hipEventCreate(&t0));
+    HIP_TRY(hipEventCreate(&t1));
+    int rc = DFDX_ROCM_OK;
+    hipError_t he = hipEventRecord(t0, ctx->stream);
+    for (int i = 0; i < iters && rc == DFDX_ROCM_OK && he == hipSuccess; i++) rc = run_plan(ctx, p, plan);
+    if (he == hipSuccess) he = hipEventRecord(t1, ctx->stream);
+    if (he == hipSuccess) he = hipEventSynchronize(t1);
+    float ms = 0.0f;
+    if (he == hipSuccess) he = hipEventElapsedTime(&ms, t0, t1);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    if (rc != DFDX_ROCM_OK) return rc;
+    if (he != hipSuccess) return (int)he;
+    *avg_ms = ms / (float)iters;
+    return DFDX_ROCM_OK;
+}
+
+}  // extern "C"

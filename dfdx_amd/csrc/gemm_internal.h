@@ -1,0 +1,77 @@
+// Internal interfaces between the C ABI (api.cpp) and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dfdx_rocm {
+
+enum { DT_F32 = 0, DT_F16 = 1, DT_BF16 = 2, DT_F64 = 3 };
+enum { BIAS_NONE = 0, BIAS_PER_COL = 1, BIAS_PER_ROW = 2 };
+
+// One strided, batched GEMM:  C[b][i,j] = (accumulate ? C : 0) + bias + sum_k A[b][i,k] * B[b][k,j].
+// Strides are in elements.  With `reduce` set, all nb1*nb2 batches are summed into one C.
+struct GemmProblem {
+    int dtype;
+    int accumulate;
+    int reduce;
+    int bias_mode;
+    int64_t m, n, k;
+    int64_t nb1, nb2;
+    const void *a;
+    int64_t a_rs, a_cs, a_b1, a_b2;
+    const void *b;
+    int64_t b_rs, b_cs, b_b1, b_b2;
+    void *c;
+    int64_t c_rs, c_cs, c_b1, c_b2;
+    const void *bias;
+};
+
+static inline size_t dtype_size(int dt) { return dt == DT_F32 ? 4 : (dt == DT_F64 ? 8 : 2); }
+
+// Swap the roles of the operands: C^T = B^T A^T.  Used to turn a column-major C into a row-major one.
+static inline GemmProblem transposed(const GemmProblem &p) {
+    GemmProblem t = p;
+    t.m = p.n; t.n = p.m;
+    t.a = p.b; t.a_rs = p.b_cs; t.a_cs = p.b_rs; t.a_b1 = p.b_b1; t.a_b2 = p.b_b2;
+    t.b = p.a; t.b_rs = p.a_cs; t.b_cs = p.a_rs; t.b_b1 = p.a_b1; t.b_b2 = p.a_b2;
+    t.c_rs = p.c_cs; t.c_cs = p.c_rs;
+    if (p.bias_mode == BIAS_PER_COL) t.bias_mode = BIAS_PER_ROW;
+    else if (p.bias_mode == BIAS_PER_ROW) t.bias_mode = BIAS_PER_COL;
+    return t;
+}
+
+// ---- generic kernel (gemm_generic.hip): every dtype, every stride pattern ----
+hipError_t launch_generic(const GemmProblem &p, hipStream_t stream);
+
+// ---- MFMA kernels for 16-bit inputs (gemm_mfma16.hip) ----
+// Variants are numbered from 1.  `supported` checks alignment / layout preconditions.
+int mfma16_variant_count();
+const char *mfma16_variant_name(int variant);
+bool mfma16_supported(const GemmProblem &p, int variant);
+int mfma16_pick_variant(const GemmProblem &p, int compute_units);
+hipError_t launch_mfma16(const GemmProblem &p, int variant, hipStream_t stream);
+
+// ---- MFMA kernels for f32 (gemm_mfma32.hip) ----
+int mfma32_variant_count();
+const char *mfma32_variant_name(int variant);
+bool mfma32_supported(const GemmProblem &p, int variant);
+int mfma32_pick_variant(const GemmProblem &p, int compute_units);
+hipError_t launch_mfma32(const GemmProblem &p, int variant, hipStream_t stream);
+
+// ---- bandwidth-bound vector products (gemv.hip) ----
+bool gemv_supported(const GemmProblem &p);
+hipError_t launch_gemv(const GemmProblem &p, hipStream_t stream);
+
+// XCD-aware remap of a linear workgroup id: consecutive ids are dispatched round-robin
+// over the 8 XCDs, so ids that share an XCD (and its L2) are pid, pid+8, pid+16 ...
+// This returns a work index such that each XCD owns one contiguous range of work.
+__device__ __forceinline__ int xcd_remap(int pid, int total) {
+    constexpr int NXCD = 8;
+    if (total < 2 * NXCD) return pid;
+    const int per = (total + NXCD - 1) / NXCD;
+    const int tall = (total % NXCD == 0) ? NXCD : total % NXCD;  // XCDs that own `per` items; the rest own per-1
+    const int xcd = pid % NXCD, local = pid / NXCD;
+    return xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+}
+
+}  // namespace dfdx_rocm

@@ -1,0 +1,444 @@
+// MFMA GEMM for 16-bit inputs (f16 / bf16) with f32 accumulation on gfx950 (CDNA4).
+//
+// One workgroup computes a BM x BN tile of C.  A and B tiles of BK k-values are
+// staged in LDS as [row][k] (k contiguous, rows padded by 16 B so that the 16 B
+// fragment reads of consecutive rows fall into distinct banks), double buffered:
+// while the matrix cores work on buffer `cur`, the global loads for the next k
+// step are in flight into registers and are written to the other buffer after the
+// MFMAs have been issued.  One barrier per k step.
+//
+// Operand layouts are handled in the loaders, with no transpose copy in HBM:
+//   k-contiguous operand (A row-major, or B stored [N][K]): 16 B global loads along k
+//     go straight to LDS.
+//   m/n-contiguous operand (A stored [K][M], or B row-major [K][N]): 16 B global loads
+//     along m/n for KR consecutive k rows, transposed 8xKR in registers with 16-bit
+//     packs, then written to LDS k-contiguous.
+// The MFMA is issued with the operands swapped (D^T = B^T A^T) so that every lane
+// ends up holding 4 consecutive n for one m, i.e. vector stores into row-major C.
+//
+// Preconditions (checked by mfma16_supported): C has unit column stride; each of A, B
+// has one unit stride; pointers, leading strides and batch strides are multiples of
+// 8 elements (16 B) and the contiguous extent is a multiple of 8.
+#include "gemm_internal.h"
+
+namespace dfdx_rocm {
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct Params {
+    const uint16_t *a;
+    const uint16_t *b;
+    uint16_t *c;
+    const uint16_t *bias;
+    int m, n, k;
+    int lda, ldb;  // stride (elements) of the non-unit axis of A / B
+    int64_t ldc;
+    int64_t a_b1, a_b2, b_b1, b_b2, c_b1, c_b2;
+    int nb2;       // inner batch count (batch id -> b1 = id / nb2, b2 = id % nb2)
+    int kbatches;  // batches folded into the k loop (reduce mode), else 1
+    int tiles_m, tiles_n, tiles_per_batch, total_blocks;
+    int accumulate, bias_mode, c_vec;
+    int group_m;
+};
+
+template <typename T> struct Mma;
+template <> struct Mma<_Float16> {
+    static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
+    static __device__ __forceinline__ uint16_t from_f32(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+};
+template <> struct Mma<__bf16> {
+    static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
+    static __device__ __forceinline__ uint16_t from_f32(float v) {
+        uint32_t x = __float_as_uint(v);
+        if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+        return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);  // round to nearest even
+    }
+};
+
+__device__ __forceinline__ u32x4 ldg16(const uint16_t *p, bool pred) {
+    u32x4 z = {0u, 0u, 0u, 0u};
+    return pred ? *(const u32x4 *)p : z;
+}
+
+// Loader of one operand tile: ROWS (m or n extent) x BK, NT threads.
+// KC = operand is k-contiguous in global memory.
+template <int ROWS, int BK, int NT, bool KC> struct Loader {
+    static constexpr int LOADS = ROWS * BK / 8 / NT;  // 16 B loads per thread per k step
+    static_assert(LOADS >= 1 && (ROWS * BK / 8) % NT == 0, "tile does not divide over the threads");
+    // m/n-contiguous: each unit is KR k-rows x 8 columns
+    static constexpr int KR = LOADS >= 8 ? 8 : LOADS;
+    static constexpr int UNITS = LOADS / KR;
+    static constexpr int NKB = BK / KR;
+    static constexpr int CPR = BK / 8;  // 16 B chunks per row (k-contiguous case)
+    static constexpr int LDS_ROW = BK + 8;
+
+    u32x4 regs[LOADS];
+
+    // `g` points at element (row0, k0) of the operand; ld = stride of the non-unit axis.
+    __device__ __forceinline__ void load(const uint16_t *g, int ld, int rows_left, int k_left, int tid) {
+        if constexpr (KC) {
+#pragma unroll
+            for (int i = 0; i < LOADS; i++) {
+                const int cid = i * NT + tid;
+                const int row = cid / CPR, ch = cid % CPR;
+                regs[i] = ldg16(g + row * ld + ch * 8, row < rows_left && ch * 8 < k_left);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) {
+                const int uid = u * NT + tid;
+                const int kb = uid % NKB, mb = uid / NKB;
+#pragma unroll
+                for (int r = 0; r < KR; r++) {
+                    const int kk = kb * KR + r;
+                    regs[u * KR + r] = ldg16(g + kk * ld + mb * 8, mb * 8 < rows_left && kk < k_left);
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void store(uint16_t *lds, int tid) const {
+        if constexpr (KC) {
+#pragma unroll
+            for (int i = 0; i < LOADS; i++) {
+                const int cid = i * NT + tid;
+                const int row = cid / CPR, ch = cid % CPR;
+                *(u32x4 *)(lds + row * LDS_ROW + ch * 8) = regs[i];
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) {
+                const int uid = u * NT + tid;
+                const int kb = uid % NKB, mb = uid / NKB;
+                uint16_t *dst = lds + (mb * 8) * LDS_ROW + kb * KR;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {  // output row j: column mb*8+j of the unit, KR k-values
+                    uint32_t w[KR / 2];
+#pragma unroll
+                    for (int q = 0; q < KR / 2; q++) {
+                        const uint32_t lo = regs[u * KR + 2 * q][j / 2], hi = regs[u * KR + 2 * q + 1][j / 2];
+                        w[q] = (j & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+                    }
+                    if constexpr (KR == 8) {
+                        u32x4 v = {w[0], w[1], w[2], w[3]};
+                        *(u32x4 *)(dst + j * LDS_ROW) = v;
+                    } else if constexpr (KR == 4) {
+                        u32x2 v = {w[0], w[1]};
+                        *(u32x2 *)(dst + j * LDS_ROW) = v;
+                    } else {
+                        *(uint32_t *)(dst + j * LDS_ROW) = w[0];
+                    }
+                }
+            }
+        }
+    }
+};
+
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(const Params p) {
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int LDS_ROW = BK + 8;
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 16 == 0, "bad tile");
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint16_t *As = (uint16_t *)smem;          // [2][BM][LDS_ROW]
+    uint16_t *Bs = As + 2 * BM * LDS_ROW;     // [2][BN][LDS_ROW]
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64, wave = tid / 64;
+    const int wm0 = (wave / WAVES_N) * WTM, wn0 = (wave % WAVES_N) * WTN;
+    const int l32 = lane % 32, lh = lane / 32;
+
+    // ---- which tile -------------------------------------------------------
+    const int work = xcd_remap(blockIdx.x, p.total_blocks);
+    const int batch = work / p.tiles_per_batch;
+    const int tile = work % p.tiles_per_batch;
+    const int gsize = p.group_m * p.tiles_n;
+    const int group = tile / gsize;
+    const int first_m = group * p.group_m;
+    const int gm = min(p.tiles_m - first_m, p.group_m);
+    const int tm_idx = first_m + (tile % gsize) % gm;
+    const int tn_idx = (tile % gsize) / gm;
+    const int bm0 = tm_idx * BM, bn0 = tn_idx * BN;
+
+    const int ktiles = (p.k + BK - 1) / BK;
+    const int iters = ktiles * p.kbatches;
+
+    // uniform pointer to element (bm0, 0) of A / (0, bn0) of B for k-loop step `it`
+    auto a_tile = [&](int it) -> const uint16_t * {
+        const int kb = p.kbatches > 1 ? it / ktiles : batch;
+        const int kt = p.kbatches > 1 ? it % ktiles : it;
+        const uint16_t *base = p.a + (int64_t)(kb / p.nb2) * p.a_b1 + (int64_t)(kb % p.nb2) * p.a_b2;
+        return A_KC ? base + (int64_t)bm0 * p.lda + kt * BK : base + (int64_t)kt * BK * p.lda + bm0;
+    };
+    auto b_tile = [&](int it) -> const uint16_t * {
+        const int kb = p.kbatches > 1 ? it / ktiles : batch;
+        const int kt = p.kbatches > 1 ? it % ktiles : it;
+        const uint16_t *base = p.b + (int64_t)(kb / p.nb2) * p.b_b1 + (int64_t)(kb % p.nb2) * p.b_b2;
+        return B_KC ? base + (int64_t)bn0 * p.ldb + kt * BK : base + (int64_t)kt * BK * p.ldb + bn0;
+    };
+    auto k_left = [&](int it) -> int {
+        const int kt = p.kbatches > 1 ? it % ktiles : it;
+        return p.k - kt * BK;
+    };
+
+    Loader<BM, BK, NT, A_KC> la;
+    Loader<BN, BK, NT, B_KC> lb;
+    const int rows_left = p.m - bm0, cols_left = p.n - bn0;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    if (iters > 0) {
+        la.load(a_tile(0), p.lda, rows_left, k_left(0), tid);
+        lb.load(b_tile(0), p.ldb, cols_left, k_left(0), tid);
+        la.store(As, tid);
+        lb.store(Bs, tid);
+    }
+    __syncthreads();
+
+    const uint16_t *a_frag0 = As + (wm0 + l32) * LDS_ROW + lh * 8;
+    const uint16_t *b_frag0 = Bs + (wn0 + l32) * LDS_ROW + lh * 8;
+
+    for (int it = 0; it < iters; it++) {
+        const int cur = it & 1;
+        const bool more = it + 1 < iters;
+        if (more) {
+            la.load(a_tile(it + 1), p.lda, rows_left, k_left(it + 1), tid);
+            lb.load(b_tile(it + 1), p.ldb, cols_left, k_left(it + 1), tid);
+        }
+        const uint16_t *af_base = a_frag0 + cur * BM * LDS_ROW;
+        const uint16_t *bf_base = b_frag0 + cur * BN * LDS_ROW;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ks++) {
+            u32x4 af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) af[i] = *(const u32x4 *)(af_base + i * 32 * LDS_ROW + ks * 16);
+#pragma unroll
+            for (int j = 0; j < TN; j++) bf[j] = *(const u32x4 *)(bf_base + j * 32 * LDS_ROW + ks * 16);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) acc[i][j] = Mma<T>::mfma(bf[j], af[i], acc[i][j]);
+        }
+        if (more) {
+            la.store(As + (cur ^ 1) * BM * LDS_ROW, tid);
+            lb.store(Bs + (cur ^ 1) * BN * LDS_ROW, tid);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds m = l32 (per tile), n = 8g + 4*lh + 0..3 --------
+    const int cb = p.kbatches > 1 ? 0 : batch;
+    uint16_t *cbase = p.c + (int64_t)(cb / p.nb2) * p.c_b1 + (int64_t)(cb % p.nb2) * p.c_b2;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int gm_row = bm0 + wm0 + i * 32 + l32;
+        if (gm_row >= p.m) continue;
+        uint16_t *crow = cbase + (int64_t)gm_row * p.ldc;
+        const float rbias = (p.bias_mode == BIAS_PER_ROW) ? Mma<T>::to_f32(p.bias[gm_row]) : 0.0f;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int gn = bn0 + wn0 + j * 32 + g * 8 + lh * 4;
+                if (gn >= p.n) continue;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = acc[i][j][g * 4 + e] + rbias;
+                if (p.c_vec) {  // n % 4 == 0 here, so the 4 columns are all in range
+                    if (p.bias_mode == BIAS_PER_COL) {
+                        const u32x2 bv = *(const u32x2 *)(p.bias + gn);
+                        v[0] += Mma<T>::to_f32((uint16_t)(bv[0] & 0xffffu));
+                        v[1] += Mma<T>::to_f32((uint16_t)(bv[0] >> 16));
+                        v[2] += Mma<T>::to_f32((uint16_t)(bv[1] & 0xffffu));
+                        v[3] += Mma<T>::to_f32((uint16_t)(bv[1] >> 16));
+                    }
+                    if (p.accumulate) {
+                        const u32x2 old = *(const u32x2 *)(crow + gn);
+                        v[0] += Mma<T>::to_f32((uint16_t)(old[0] & 0xffffu));
+                        v[1] += Mma<T>::to_f32((uint16_t)(old[0] >> 16));
+                        v[2] += Mma<T>::to_f32((uint16_t)(old[1] & 0xffffu));
+                        v[3] += Mma<T>::to_f32((uint16_t)(old[1] >> 16));
+                    }
+                    u32x2 o;
+                    o[0] = (uint32_t)Mma<T>::from_f32(v[0]) | ((uint32_t)Mma<T>::from_f32(v[1]) << 16);
+                    o[1] = (uint32_t)Mma<T>::from_f32(v[2]) | ((uint32_t)Mma<T>::from_f32(v[3]) << 16);
+                    *(u32x2 *)(crow + gn) = o;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (gn + e >= p.n) break;
+                        float x = v[e];
+                        if (p.bias_mode == BIAS_PER_COL) x += Mma<T>::to_f32(p.bias[gn + e]);
+                        if (p.accumulate) x += Mma<T>::to_f32(crow[gn + e]);
+                        crow[gn + e] = Mma<T>::from_f32(x);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ host side --
+
+struct Variant {
+    const char *name;
+    int bm, bn, bk, waves_m, waves_n;
+};
+
+// Variant ids are 1-based indices into this table.
+constexpr Variant kVariants[] = {
+    {"256x256x64_w2x4", 256, 256, 64, 2, 4},
+    {"256x256x64_w2x2", 256, 256, 64, 2, 2},
+    {"256x128x64_w2x2", 256, 128, 64, 2, 2},
+    {"128x128x64_w2x2", 128, 128, 64, 2, 2},
+    {"128x64x64_w4x1", 128, 64, 64, 4, 1},
+    {"64x64x64_w2x2", 64, 64, 64, 2, 2},
+};
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+
+template <typename T, int BM, int BN, int BK, int WM, int WN>
+hipError_t launch_layout(const Params &p, bool a_kc, bool b_kc, hipStream_t stream) {
+    constexpr int NT = WM * WN * 64;
+    constexpr size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * 2;
+    dim3 grid((unsigned)p.total_blocks), block(NT);
+#define DFDX_LAUNCH(AKC, BKC)                                                                                   \
+    do {                                                                                                        \
+        auto kern = gemm_mfma16_kernel<T, BM, BN, BK, WM, WN, AKC, BKC>;                                        \
+        static bool configured = false;                                                                         \
+        if (!configured) {                                                                                      \
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,   \
+                                               (int)lds);                                                       \
+            if (e != hipSuccess) return e;                                                                      \
+            configured = true;                                                                                  \
+        }                                                                                                       \
+        kern<<<grid, block, lds, stream>>>(p);                                                                  \
+    } while (0)
+    if (a_kc && b_kc) DFDX_LAUNCH(true, true);
+    else if (a_kc && !b_kc) DFDX_LAUNCH(true, false);
+    else if (!a_kc && b_kc) DFDX_LAUNCH(false, true);
+    else DFDX_LAUNCH(false, false);
+#undef DFDX_LAUNCH
+    return hipGetLastError();
+}
+
+template <typename T> hipError_t launch_variant(int variant, const Params &p, bool a_kc, bool b_kc, hipStream_t s) {
+    switch (variant) {
+    case 1: return launch_layout<T, 256, 256, 64, 2, 4>(p, a_kc, b_kc, s);
+    case 2: return launch_layout<T, 256, 256, 64, 2, 2>(p, a_kc, b_kc, s);
+    case 3: return launch_layout<T, 256, 128, 64, 2, 2>(p, a_kc, b_kc, s);
+    case 4: return launch_layout<T, 128, 128, 64, 2, 2>(p, a_kc, b_kc, s);
+    case 5: return launch_layout<T, 128, 64, 64, 4, 1>(p, a_kc, b_kc, s);
+    case 6: return launch_layout<T, 64, 64, 64, 2, 2>(p, a_kc, b_kc, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+// Layout of a (rows x kdim) operand: k-contiguous when the k stride is 1 (or k has one
+// element and rows are 16 B apart), rows-contiguous when the row stride is 1.
+struct OperandLayout {
+    bool ok, kc;
+    int64_t ld;
+};
+inline OperandLayout classify(int64_t rows, int64_t kdim, int64_t row_stride, int64_t k_stride) {
+    OperandLayout r{false, false, 0};
+    if (k_stride == 1 && kdim % 8 == 0 && (rows == 1 || (row_stride % 8 == 0 && row_stride >= kdim))) {
+        r.ok = true; r.kc = true; r.ld = rows == 1 ? kdim : row_stride;
+    } else if (row_stride == 1 && rows % 8 == 0 && (kdim == 1 || (k_stride % 8 == 0 && k_stride >= rows))) {
+        r.ok = true; r.kc = false; r.ld = kdim == 1 ? rows : k_stride;
+    }
+    return r;
+}
+
+}  // namespace
+
+int mfma16_variant_count() { return kNumVariants; }
+const char *mfma16_variant_name(int v) { return (v >= 1 && v <= kNumVariants) ? kVariants[v - 1].name : "?"; }
+
+bool mfma16_supported(const GemmProblem &p, int variant) {
+    if (p.dtype != DT_F16 && p.dtype != DT_BF16) return false;
+    if (variant < 1 || variant > kNumVariants) return false;
+    if (p.m < 1 || p.n < 1 || p.k < 1) return false;
+    if (p.m > (1 << 30) || p.n > (1 << 30) || p.k > (1 << 30)) return false;
+    if (p.c_cs != 1 && p.n != 1) return false;
+    if (p.n > 1 && p.m > 1 && p.c_rs < p.n) return false;
+    const OperandLayout la = classify(p.m, p.k, p.a_rs, p.a_cs);
+    const OperandLayout lb = classify(p.n, p.k, p.b_cs, p.b_rs);
+    if (!la.ok || !lb.ok) return false;
+    const Variant &v = kVariants[variant - 1];
+    // 32-bit offsets inside one tile
+    if (la.ld * (la.kc ? v.bm : v.bk) >= (1ll << 31) || lb.ld * (lb.kc ? v.bn : v.bk) >= (1ll << 31)) return false;
+    if (!aligned16(p.a) || !aligned16(p.b)) return false;
+    if (p.nb1 * p.nb2 > 1) {
+        if (p.a_b1 % 8 || p.a_b2 % 8 || p.b_b1 % 8 || p.b_b2 % 8) return false;
+        if (p.a_b1 < 0 || p.a_b2 < 0 || p.b_b1 < 0 || p.b_b2 < 0) return false;
+    }
+    const int64_t tiles = ((p.m + v.bm - 1) / v.bm) * ((p.n + v.bn - 1) / v.bn);
+    const int64_t blocks = tiles * (p.reduce ? 1 : p.nb1 * p.nb2);
+    if (blocks >= (1ll << 31) || p.nb1 * p.nb2 >= (1ll << 31)) return false;
+    if (p.k * (p.reduce ? p.nb1 * p.nb2 : 1) >= (1ll << 31)) return false;
+    return true;
+}
+
+int mfma16_pick_variant(const GemmProblem &p, int compute_units) {
+    // Largest tile that still gives every compute unit at least one workgroup; ties go to the larger tile.
+    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+    const int order[] = {1, 3, 4, 5, 6};
+    for (int v : order) {
+        const Variant &t = kVariants[v - 1];
+        if (!mfma16_supported(p, v)) continue;
+        if (p.n <= 64 && t.bn > 64) continue;
+        const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
+        if (blocks >= compute_units || v == 6) return v;
+    }
+    return mfma16_supported(p, 6) ? 6 : 0;
+}
+
+hipError_t launch_mfma16(const GemmProblem &g, int variant, hipStream_t stream) {
+    if (!mfma16_supported(g, variant)) return hipErrorInvalidValue;
+    const Variant &v = kVariants[variant - 1];
+    const OperandLayout la = classify(g.m, g.k, g.a_rs, g.a_cs);
+    const OperandLayout lb = classify(g.n, g.k, g.b_cs, g.b_rs);
+    Params p;
+    p.a = (const uint16_t *)g.a; p.b = (const uint16_t *)g.b; p.c = (uint16_t *)g.c; p.bias = (const uint16_t *)g.bias;
+    p.m = (int)g.m; p.n = (int)g.n; p.k = (int)g.k;
+    p.lda = (int)la.ld; p.ldb = (int)lb.ld;
+    p.ldc = g.m == 1 ? g.n : g.c_rs;
+    p.a_b1 = g.a_b1; p.a_b2 = g.a_b2; p.b_b1 = g.b_b1; p.b_b2 = g.b_b2; p.c_b1 = g.c_b1; p.c_b2 = g.c_b2;
+    p.nb2 = (int)g.nb2;
+    const int nbatch = (int)(g.nb1 * g.nb2);
+    p.kbatches = g.reduce ? nbatch : 1;
+    p.tiles_m = (int)((g.m + v.bm - 1) / v.bm);
+    p.tiles_n = (int)((g.n + v.bn - 1) / v.bn);
+    p.tiles_per_batch = p.tiles_m * p.tiles_n;
+    p.total_blocks = p.tiles_per_batch * (g.reduce ? 1 : nbatch);
+    p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
+    p.c_vec = (g.n % 4 == 0) && (p.ldc % 4 == 0) && (((uintptr_t)g.c & 7u) == 0) &&
+              (g.c_b1 % 4 == 0) && (g.c_b2 % 4 == 0) && (!g.bias || ((uintptr_t)g.bias & 7u) == 0);
+    p.group_m = 4;
+    if (g.dtype == DT_F16) return launch_variant<_Float16>(variant, p, la.kc, lb.kc, stream);
+    return launch_variant<__bf16>(variant, p, la.kc, lb.kc, stream);
+}
+
+}  // namespace dfdx_rocm

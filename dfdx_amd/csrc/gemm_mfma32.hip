@@ -1,0 +1,359 @@
+// MFMA GEMM for f32 on gfx950 (CDNA4): v_mfma_f32_32x32x2_f32, f32 accumulate.
+//
+// Same skeleton as the 16-bit kernel: BM x BN tile per workgroup, LDS double buffer,
+// global loads for step k+1 in flight while the matrix cores work on step k, one
+// barrier per step.  An f32 MFMA lane supplies ONE k value per instruction, so no
+// transpose is ever needed: a k-contiguous operand is kept in LDS as [row][k] and
+// read 16 B at a time (4 k values feeding 4 MFMAs), an m/n-contiguous operand is
+// kept as [k][row] and read 4 B at a time.  Which k a lane feeds to which MFMA is
+// the same for both operands (k = 8*s + 4*(lane/32) + e for MFMA e of sub-step s),
+// which is all the instruction needs.
+//
+// Preconditions (mfma32_supported): C unit column stride; A and B each have a unit
+// stride; pointers, leading and batch strides multiples of 4 elements (16 B); the
+// contiguous extent a multiple of 4.
+#include "gemm_internal.h"
+
+namespace dfdx_rocm {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+struct Params {
+    const float *a;
+    const float *b;
+    float *c;
+    const float *bias;
+    int m, n, k;
+    int lda, ldb;
+    int64_t ldc;
+    int64_t a_b1, a_b2, b_b1, b_b2, c_b1, c_b2;
+    int nb2, kbatches;
+    int tiles_m, tiles_n, tiles_per_batch, total_blocks;
+    int accumulate, bias_mode, c_vec;
+    int group_m;
+};
+
+__device__ __forceinline__ f32x4 ldg4(const float *p, bool pred) {
+    f32x4 z = {0.f, 0.f, 0.f, 0.f};
+    return pred ? *(const f32x4 *)p : z;
+}
+
+template <int ROWS, int BK, int NT, bool KC> struct Loader {
+    static constexpr int LOADS = ROWS * BK / 4 / NT;
+    static_assert(LOADS >= 1 && (ROWS * BK / 4) % NT == 0, "tile does not divide over the threads");
+    static constexpr int CPR = KC ? BK / 4 : ROWS / 4;               // 16 B chunks per LDS row
+    static constexpr int LDS_ROW = KC ? BK + 4 : ROWS + 8;            // floats
+    static constexpr int LDS_SIZE = KC ? ROWS * LDS_ROW : BK * LDS_ROW;
+    f32x4 regs[LOADS];
+
+    __device__ __forceinline__ void load(const float *g, int ld, int rows_left, int k_left, int tid) {
+#pragma unroll
+        for (int i = 0; i < LOADS; i++) {
+            const int cid = i * NT + tid;
+            const int r = cid / CPR, ch = cid % CPR;
+            if constexpr (KC) regs[i] = ldg4(g + r * ld + ch * 4, r < rows_left && ch * 4 < k_left);
+            else regs[i] = ldg4(g + r * ld + ch * 4, ch * 4 < rows_left && r < k_left);
+        }
+    }
+    __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < LOADS; i++) {
+            const int cid = i * NT + tid;
+            const int r = cid / CPR, ch = cid % CPR;
+            *(f32x4 *)(lds + r * LDS_ROW + ch * 4) = regs[i];
+        }
+    }
+};
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(const Params p) {
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    using LA = Loader<BM, BK, NT, A_KC>;
+    using LB = Loader<BN, BK, NT, B_KC>;
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 8 == 0, "bad tile");
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    float *As = (float *)smem;             // [2][LA::LDS_SIZE]
+    float *Bs = As + 2 * LA::LDS_SIZE;     // [2][LB::LDS_SIZE]
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64, wave = tid / 64;
+    const int wm0 = (wave / WAVES_N) * WTM, wn0 = (wave % WAVES_N) * WTN;
+    const int l32 = lane % 32, lh = lane / 32;
+
+    const int work = xcd_remap(blockIdx.x, p.total_blocks);
+    const int batch = work / p.tiles_per_batch;
+    const int tile = work % p.tiles_per_batch;
+    const int gsize = p.group_m * p.tiles_n;
+    const int group = tile / gsize;
+    const int first_m = group * p.group_m;
+    const int gm = min(p.tiles_m - first_m, p.group_m);
+    const int tm_idx = first_m + (tile % gsize) % gm;
+    const int tn_idx = (tile % gsize) / gm;
+    const int bm0 = tm_idx * BM, bn0 = tn_idx * BN;
+
+    const int ktiles = (p.k + BK - 1) / BK;
+    const int iters = ktiles * p.kbatches;
+
+    auto a_tile = [&](int it) -> const float * {
+        const int kb = p.kbatches > 1 ? it / ktiles : batch;
+        const int kt = p.kbatches > 1 ? it % ktiles : it;
+        const float *base = p.a + (int64_t)(kb / p.nb2) * p.a_b1 + (int64_t)(kb % p.nb2) * p.a_b2;
+        return A_KC ? base + (int64_t)bm0 * p.lda + kt * BK : base + (int64_t)kt * BK * p.lda + bm0;
+    };
+    auto b_tile = [&](int it) -> const float * {
+        const int kb = p.kbatches > 1 ? it / ktiles : batch;
+        const int kt = p.kbatches > 1 ? it % ktiles : it;
+        const float *base = p.b + (int64_t)(kb / p.nb2) * p.b_b1 + (int64_t)(kb % p.nb2) * p.b_b2;
+        return B_KC ? base + (int64_t)bn0 * p.ldb + kt * BK : base + (int64_t)kt * BK * p.ldb + bn0;
+    };
+    auto k_left = [&](int it) -> int {
+        const int kt = p.kbatches > 1 ? it % ktiles : it;
+        return p.k - kt * BK;
+    };
+
+    LA la;
+    LB lb;
+    const int rows_left = p.m - bm0, cols_left = p.n - bn0;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    if (iters > 0) {
+        la.load(a_tile(0), p.lda, rows_left, k_left(0), tid);
+        lb.load(b_tile(0), p.ldb, cols_left, k_left(0), tid);
+        la.store(As, tid);
+        lb.store(Bs, tid);
+    }
+    __syncthreads();
+
+    // per-lane fragment origins
+    const float *a_frag0 = A_KC ? As + (wm0 + l32) * LA::LDS_ROW + lh * 4 : As + (lh * 4) * LA::LDS_ROW + wm0 + l32;
+    const float *b_frag0 = B_KC ? Bs + (wn0 + l32) * LB::LDS_ROW + lh * 4 : Bs + (lh * 4) * LB::LDS_ROW + wn0 + l32;
+
+    for (int it = 0; it < iters; it++) {
+        const int cur = it & 1;
+        const bool more = it + 1 < iters;
+        if (more) {
+            la.load(a_tile(it + 1), p.lda, rows_left, k_left(it + 1), tid);
+            lb.load(b_tile(it + 1), p.ldb, cols_left, k_left(it + 1), tid);
+        }
+        const float *af_base = a_frag0 + cur * LA::LDS_SIZE;
+        const float *bf_base = b_frag0 + cur * LB::LDS_SIZE;
+#pragma unroll
+        for (int ks = 0; ks < BK / 8; ks++) {
+            float af[TM][4], bf[TN][4];
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                if constexpr (A_KC) {
+                    const f32x4 v = *(const f32x4 *)(af_base + i * 32 * LA::LDS_ROW + ks * 8);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) af[i][e] = v[e];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) af[i][e] = af_base[(ks * 8 + e) * LA::LDS_ROW + i * 32];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                if constexpr (B_KC) {
+                    const f32x4 v = *(const f32x4 *)(bf_base + j * 32 * LB::LDS_ROW + ks * 8);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) bf[j][e] = v[e];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) bf[j][e] = bf_base[(ks * 8 + e) * LB::LDS_ROW + j * 32];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j][e], af[i][e], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            la.store(As + (cur ^ 1) * LA::LDS_SIZE, tid);
+            lb.store(Bs + (cur ^ 1) * LB::LDS_SIZE, tid);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds m = l32 (per tile), n = 8g + 4*lh + 0..3 --------
+    const int cb = p.kbatches > 1 ? 0 : batch;
+    float *cbase = p.c + (int64_t)(cb / p.nb2) * p.c_b1 + (int64_t)(cb % p.nb2) * p.c_b2;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int gm_row = bm0 + wm0 + i * 32 + l32;
+        if (gm_row >= p.m) continue;
+        float *crow = cbase + (int64_t)gm_row * p.ldc;
+        const float rbias = (p.bias_mode == BIAS_PER_ROW) ? p.bias[gm_row] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int gn = bn0 + wn0 + j * 32 + g * 8 + lh * 4;
+                if (gn >= p.n) continue;
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = acc[i][j][g * 4 + e] + rbias;
+                if (p.c_vec) {
+                    if (p.bias_mode == BIAS_PER_COL) v += *(const f32x4 *)(p.bias + gn);
+                    if (p.accumulate) v += *(const f32x4 *)(crow + gn);
+                    *(f32x4 *)(crow + gn) = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (gn + e >= p.n) break;
+                        float x = v[e];
+                        if (p.bias_mode == BIAS_PER_COL) x += p.bias[gn + e];
+                        if (p.accumulate) x += crow[gn + e];
+                        crow[gn + e] = x;
+                    }
+                }
+            }
+        }
+    }
+}
+
+struct Variant {
+    const char *name;
+    int bm, bn, bk, waves_m, waves_n;
+};
+constexpr Variant kVariants[] = {
+    {"256x256x32_w2x4", 256, 256, 32, 2, 4},
+    {"256x256x32_w2x2", 256, 256, 32, 2, 2},
+    {"256x128x32_w2x2", 256, 128, 32, 2, 2},
+    {"128x128x32_w2x2", 128, 128, 32, 2, 2},
+    {"128x64x32_w4x1", 128, 64, 32, 4, 1},
+    {"64x64x32_w2x2", 64, 64, 32, 2, 2},
+};
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+
+template <int BM, int BN, int BK, int WM, int WN>
+hipError_t launch_layout(const Params &p, bool a_kc, bool b_kc, hipStream_t stream) {
+    constexpr int NT = WM * WN * 64;
+    dim3 grid((unsigned)p.total_blocks), block(NT);
+#define DFDX_LAUNCH(AKC, BKC)                                                                                   \
+    do {                                                                                                        \
+        constexpr size_t lds = (size_t)2 * 4 * (Loader<BM, BK, NT, AKC>::LDS_SIZE + Loader<BN, BK, NT, BKC>::LDS_SIZE); \
+        auto kern = gemm_mfma32_kernel<BM, BN, BK, WM, WN, AKC, BKC>;                                           \
+        static bool configured = false;                                                                         \
+        if (!configured) {                                                                                      \
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,   \
+                                               (int)lds);                                                       \
+            if (e != hipSuccess) return e;                                                                      \
+            configured = true;                                                                                  \
+        }                                                                                                       \
+        kern<<<grid, block, lds, stream>>>(p);                                                                  \
+    } while (0)
+    if (a_kc && b_kc) DFDX_LAUNCH(true, true);
+    else if (a_kc && !b_kc) DFDX_LAUNCH(true, false);
+    else if (!a_kc && b_kc) DFDX_LAUNCH(false, true);
+    else DFDX_LAUNCH(false, false);
+#undef DFDX_LAUNCH
+    return hipGetLastError();
+}
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+struct OperandLayout {
+    bool ok, kc;
+    int64_t ld;
+};
+inline OperandLayout classify(int64_t rows, int64_t kdim, int64_t row_stride, int64_t k_stride) {
+    OperandLayout r{false, false, 0};
+    if (k_stride == 1 && kdim % 4 == 0 && (rows == 1 || (row_stride % 4 == 0 && row_stride >= kdim))) {
+        r.ok = true; r.kc = true; r.ld = rows == 1 ? kdim : row_stride;
+    } else if (row_stride == 1 && rows % 4 == 0 && (kdim == 1 || (k_stride % 4 == 0 && k_stride >= rows))) {
+        r.ok = true; r.kc = false; r.ld = kdim == 1 ? rows : k_stride;
+    }
+    return r;
+}
+
+}  // namespace
+
+int mfma32_variant_count() { return kNumVariants; }
+const char *mfma32_variant_name(int v) { return (v >= 1 && v <= kNumVariants) ? kVariants[v - 1].name : "?"; }
+
+bool mfma32_supported(const GemmProblem &p, int variant) {
+    if (p.dtype != DT_F32) return false;
+    if (variant < 1 || variant > kNumVariants) return false;
+    if (p.m < 1 || p.n < 1 || p.k < 1) return false;
+    if (p.m > (1 << 30) || p.n > (1 << 30) || p.k > (1 << 30)) return false;
+    if (p.c_cs != 1 && p.n != 1) return false;
+    if (p.n > 1 && p.m > 1 && p.c_rs < p.n) return false;
+    const OperandLayout la = classify(p.m, p.k, p.a_rs, p.a_cs);
+    const OperandLayout lb = classify(p.n, p.k, p.b_cs, p.b_rs);
+    if (!la.ok || !lb.ok) return false;
+    const Variant &v = kVariants[variant - 1];
+    if (la.ld * (la.kc ? v.bm : v.bk) >= (1ll << 31) || lb.ld * (lb.kc ? v.bn : v.bk) >= (1ll << 31)) return false;
+    if (!aligned16(p.a) || !aligned16(p.b)) return false;
+    if (p.nb1 * p.nb2 > 1) {
+        if (p.a_b1 % 4 || p.a_b2 % 4 || p.b_b1 % 4 || p.b_b2 % 4) return false;
+        if (p.a_b1 < 0 || p.a_b2 < 0 || p.b_b1 < 0 || p.b_b2 < 0) return false;
+    }
+    const int64_t tiles = ((p.m + v.bm - 1) / v.bm) * ((p.n + v.bn - 1) / v.bn);
+    const int64_t blocks = tiles * (p.reduce ? 1 : p.nb1 * p.nb2);
+    if (blocks >= (1ll << 31) || p.nb1 * p.nb2 >= (1ll << 31)) return false;
+    if (p.k * (p.reduce ? p.nb1 * p.nb2 : 1) >= (1ll << 31)) return false;
+    return true;
+}
+
+int mfma32_pick_variant(const GemmProblem &p, int compute_units) {
+    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+    const int order[] = {1, 3, 4, 5, 6};
+    for (int v : order) {
+        const Variant &t = kVariants[v - 1];
+        if (!mfma32_supported(p, v)) continue;
+        if (p.n <= 64 && t.bn > 64) continue;
+        const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
+        if (blocks >= compute_units || v == 6) return v;
+    }
+    return mfma32_supported(p, 6) ? 6 : 0;
+}
+
+hipError_t launch_mfma32(const GemmProblem &g, int variant, hipStream_t stream) {
+    if (!mfma32_supported(g, variant)) return hipErrorInvalidValue;
+    const Variant &v = kVariants[variant - 1];
+    const OperandLayout la = classify(g.m, g.k, g.a_rs, g.a_cs);
+    const OperandLayout lb = classify(g.n, g.k, g.b_cs, g.b_rs);
+    Params p;
+    p.a = (const float *)g.a; p.b = (const float *)g.b; p.c = (float *)g.c; p.bias = (const float *)g.bias;
+    p.m = (int)g.m; p.n = (int)g.n; p.k = (int)g.k;
+    p.lda = (int)la.ld; p.ldb = (int)lb.ld;
+    p.ldc = g.m == 1 ? g.n : g.c_rs;
+    p.a_b1 = g.a_b1; p.a_b2 = g.a_b2; p.b_b1 = g.b_b1; p.b_b2 = g.b_b2; p.c_b1 = g.c_b1; p.c_b2 = g.c_b2;
+    p.nb2 = (int)g.nb2;
+    const int nbatch = (int)(g.nb1 * g.nb2);
+    p.kbatches = g.reduce ? nbatch : 1;
+    p.tiles_m = (int)((g.m + v.bm - 1) / v.bm);
+    p.tiles_n = (int)((g.n + v.bn - 1) / v.bn);
+    p.tiles_per_batch = p.tiles_m * p.tiles_n;
+    p.total_blocks = p.tiles_per_batch * (g.reduce ? 1 : nbatch);
+    p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
+    p.c_vec = (g.n % 4 == 0) && (p.ldc % 4 == 0) && (((uintptr_t)g.c & 15u) == 0) &&
+              (g.c_b1 % 4 == 0) && (g.c_b2 % 4 == 0) && (!g.bias || ((uintptr_t)g.bias & 15u) == 0);
+    p.group_m = 4;
+    switch (variant) {
+    case 1: return launch_layout<256, 256, 32, 2, 4>(p, la.kc, lb.kc, stream);
+    case 2: return launch_layout<256, 256, 32, 2, 2>(p, la.kc, lb.kc, stream);
+    case 3: return launch_layout<256, 128, 32, 2, 2>(p, la.kc, lb.kc, stream);
+    case 4: return launch_layout<128, 128, 32, 2, 2>(p, la.kc, lb.kc, stream);
+    case 5: return launch_layout<128, 64, 32, 4, 1>(p, la.kc, lb.kc, stream);
+    case 6: return launch_layout<64, 64, 32, 2, 2>(p, la.kc, lb.kc, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace dfdx_rocm

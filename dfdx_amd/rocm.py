@@ -1,0 +1,362 @@
+"""``Rocm``: the host-side mirror of a dfdx device for the matmul path.
+
+Method names and argument meaning follow the reference's kernel traits
+(dfdx-core/src/tensor_ops/matmul/mod.rs:116-131,197-212,234-249,273-288):
+``forward(lhs, rhs) -> out`` allocates a fresh contiguous output, and
+``backward(lhs, grad_lhs, rhs, grad_rhs, grad_out)`` accumulates into gradient
+buffers that are laid out like the operands' physical storage.  A tensor is a
+:class:`View`: device storage + shape + strides in elements, which is what a
+dfdx ``Tensor`` hands its kernels (tensor_impls.rs:32-39).  Shape mismatches
+raise ``AssertionError`` before any kernel runs, like the reference's
+``assert_eq!`` (mod.rs:192,229,267-268,306-308).
+
+PyTorch is used for device memory only (allocation, host<->device copies).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+DTYPES = {"f32": 0, "f16": 1, "bf16": 2, "f64": 3}
+ITEMSIZE = {"f32": 4, "f16": 2, "bf16": 2, "f64": 8}
+NP_DTYPES = {"f32": np.float32, "f16": np.float16, "bf16": np.uint16, "f64": np.float64}
+
+KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_GEMV = 0, 1, 2, 3
+
+
+class RocmError(RuntimeError):
+    def __init__(self, code: int, msg: str):
+        super().__init__(f"dfdx_rocm error {code}: {msg}")
+        self.code = code
+
+
+class GemmDesc(ctypes.Structure):
+    """``dfdx_rocm_gemm_desc`` (include/dfdx_rocm.h)."""
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("accumulate", ctypes.c_int32),
+        ("m", ctypes.c_int64), ("n", ctypes.c_int64), ("k", ctypes.c_int64),
+        ("batch1", ctypes.c_int64), ("batch2", ctypes.c_int64),
+        ("a", ctypes.c_void_p), ("a_rs", ctypes.c_int64), ("a_cs", ctypes.c_int64),
+        ("a_b1", ctypes.c_int64), ("a_b2", ctypes.c_int64),
+        ("b", ctypes.c_void_p), ("b_rs", ctypes.c_int64), ("b_cs", ctypes.c_int64),
+        ("b_b1", ctypes.c_int64), ("b_b2", ctypes.c_int64),
+        ("c", ctypes.c_void_p), ("c_rs", ctypes.c_int64), ("c_cs", ctypes.c_int64),
+        ("c_b1", ctypes.c_int64), ("c_b2", ctypes.c_int64),
+        ("bias", ctypes.c_void_p),
+        ("reduce_batch", ctypes.c_int32), ("kernel", ctypes.c_int32),
+        ("variant", ctypes.c_int32), ("reserved", ctypes.c_int32),
+    ]
+
+
+def lib_path() -> str:
+    return os.path.join(_HERE, "lib", "libdfdx_rocm.so")
+
+
+_lib = None
+
+# every symbol include/dfdx_rocm.h declares
+EXPORTS = [
+    "dfdx_rocm_create", "dfdx_rocm_destroy", "dfdx_rocm_strerror", "dfdx_rocm_device_info",
+    "dfdx_rocm_alloc", "dfdx_rocm_free", "dfdx_rocm_memset_zero", "dfdx_rocm_copy_h2d", "dfdx_rocm_copy_d2h",
+    "dfdx_rocm_copy_d2d", "dfdx_rocm_synchronize", "dfdx_rocm_gemm", "dfdx_rocm_gemm_plan",
+    "dfdx_rocm_mfma_variant_count", "dfdx_rocm_gemm_time",
+    "dfdx_rocm_matmat_forward", "dfdx_rocm_matmat_backward",
+    "dfdx_rocm_matmat_br_forward", "dfdx_rocm_matmat_br_backward",
+    "dfdx_rocm_matmat_batch3_forward", "dfdx_rocm_matmat_batch3_backward",
+    "dfdx_rocm_matmat_batch4_forward", "dfdx_rocm_matmat_batch4_backward",
+    "dfdx_rocm_linear_forward",
+]
+
+
+def load_library() -> ctypes.CDLL:
+    """Load the built HIP library; raises if it has not been built (no fallback)."""
+    global _lib
+    if _lib is None:
+        path = lib_path()
+        if not os.path.exists(path):
+            raise FileNotFoundError(
+                f"{path} is missing: build it with `make -C dfdx_amd/csrc` (or __graft_entry__.build())")
+        lib = ctypes.CDLL(path)
+        lib.dfdx_rocm_strerror.restype = ctypes.c_char_p
+        lib.dfdx_rocm_strerror.argtypes = [ctypes.c_int]
+        for name in EXPORTS:
+            fn = getattr(lib, name)
+            if name != "dfdx_rocm_strerror":
+                fn.restype = ctypes.c_int
+        _lib = lib
+    return _lib
+
+
+@dataclass
+class View:
+    """Device storage seen through a shape and element strides (a dfdx tensor's kernel-side face)."""
+    storage: "object"           # torch.uint8 CUDA tensor owning the bytes
+    dtype: str
+    shape: tuple
+    strides: tuple
+    offset: int = 0             # in elements
+
+    @property
+    def ptr(self) -> int:
+        return self.storage.data_ptr() + self.offset * ITEMSIZE[self.dtype]
+
+    def permute(self, *axes) -> "View":
+        """Zero-copy permute (reference: tensor_ops/permute_to.rs:38-52)."""
+        return View(self.storage, self.dtype, tuple(self.shape[a] for a in axes),
+                    tuple(self.strides[a] for a in axes), self.offset)
+
+    def numel_storage(self) -> int:
+        return self.storage.numel() // ITEMSIZE[self.dtype]
+
+
+def _row_major(shape):
+    s = [1] * len(shape)
+    for i in range(len(shape) - 2, -1, -1):
+        s[i] = s[i + 1] * shape[i + 1]
+    return tuple(s)
+
+
+def _i64arr(v: Sequence[int]):
+    return (ctypes.c_int64 * len(v))(*[int(x) for x in v])
+
+
+class Rocm:
+    """One GPU context.  ``Rocm(ordinal)`` ~ ``Cuda::try_build(ordinal, seed)`` (tensor/cuda/device.rs:72-90)."""
+
+    def __init__(self, ordinal: int = 0):
+        import torch
+
+        self._torch = torch
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU visible: the Rocm device needs an MI355X (there is no CPU fallback)")
+        self.lib = load_library()
+        self.ordinal = ordinal
+        self.device = torch.device("cuda", ordinal)
+        torch.cuda.set_device(ordinal)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        ctx = ctypes.c_void_p()
+        self._check(self.lib.dfdx_rocm_create(ordinal, ctypes.c_void_p(stream), ctypes.byref(ctx)))
+        self.ctx = ctx
+
+    def close(self):
+        if getattr(self, "ctx", None):
+            self.lib.dfdx_rocm_destroy(self.ctx)
+            self.ctx = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ------------------------------------------------------------------ misc --
+    def _check(self, code: int):
+        if code != 0:
+            raise RocmError(code, self.lib.dfdx_rocm_strerror(code).decode())
+
+    def synchronize(self):
+        self._check(self.lib.dfdx_rocm_synchronize(self.ctx))
+
+    def device_info(self):
+        name = ctypes.create_string_buffer(128)
+        cus, mhz = ctypes.c_int(), ctypes.c_int()
+        self._check(self.lib.dfdx_rocm_device_info(self.ctx, name, 128, ctypes.byref(cus), ctypes.byref(mhz)))
+        return {"name": name.value.decode(), "compute_units": cus.value, "clock_mhz": mhz.value}
+
+    # --------------------------------------------------------------- storage --
+    def tensor(self, host: np.ndarray, dtype: str, shape=None, strides=None) -> View:
+        """Upload ``host`` (storage order) and view it; bf16 storage is given as uint16 bit patterns."""
+        torch = self._torch
+        host = np.ascontiguousarray(host)
+        if host.dtype != NP_DTYPES[dtype]:
+            raise TypeError(f"{dtype} storage must be numpy {NP_DTYPES[dtype]}, got {host.dtype}")
+        shape = tuple(host.shape) if shape is None else tuple(shape)
+        strides = _row_major(shape) if strides is None else tuple(strides)
+        raw = torch.from_numpy(host.reshape(-1).view(np.uint8).copy()).to(self.device)
+        if raw.numel() == 0:
+            raw = torch.zeros(16, dtype=torch.uint8, device=self.device)
+        return View(raw, dtype, shape, strides)
+
+    def zeros(self, dtype: str, shape, numel_storage: Optional[int] = None, strides=None) -> View:
+        """Zero-filled storage (``Storage::try_alloc_len``, tensor/cuda/device.rs:259-266)."""
+        torch = self._torch
+        shape = tuple(shape)
+        n = int(np.prod(shape, dtype=np.int64)) if numel_storage is None else numel_storage
+        raw = torch.zeros(max(n * ITEMSIZE[dtype], 16), dtype=torch.uint8, device=self.device)
+        return View(raw, dtype, shape, _row_major(shape) if strides is None else tuple(strides))
+
+    def zeros_like_storage(self, v: View) -> View:
+        """A gradient buffer for ``v``: zero-filled, same physical length, same strides (gradients.rs:53-58)."""
+        raw = self._torch.zeros_like(v.storage)
+        return View(raw, v.dtype, v.shape, v.strides, v.offset)
+
+    def to_host(self, v: View) -> np.ndarray:
+        """The storage bytes as a flat numpy array of the storage dtype."""
+        n = v.numel_storage()
+        return v.storage.cpu().numpy().view(NP_DTYPES[v.dtype])[:n].copy()
+
+    # ------------------------------------------------------------------ gemm --
+    def gemm_desc(self, dtype, m, k, n, a, a_strides, b, b_strides, c, c_strides, accumulate=False,
+                  batch=(1, 1), a_batch=(0, 0), b_batch=(0, 0), c_batch=(0, 0), bias=None, reduce_batch=False,
+                  kernel=KERNEL_AUTO, variant=0) -> GemmDesc:
+        d = GemmDesc()
+        d.dtype, d.accumulate = DTYPES[dtype], int(bool(accumulate))
+        d.m, d.n, d.k = m, n, k
+        d.batch1, d.batch2 = batch
+        d.a, d.a_rs, d.a_cs, d.a_b1, d.a_b2 = a, a_strides[0], a_strides[1], a_batch[0], a_batch[1]
+        d.b, d.b_rs, d.b_cs, d.b_b1, d.b_b2 = b, b_strides[0], b_strides[1], b_batch[0], b_batch[1]
+        d.c, d.c_rs, d.c_cs, d.c_b1, d.c_b2 = c, c_strides[0], c_strides[1], c_batch[0], c_batch[1]
+        d.bias = bias
+        d.reduce_batch, d.kernel, d.variant = int(bool(reduce_batch)), kernel, variant
+        return d
+
+    def gemm(self, desc: GemmDesc):
+        """``MatMulImpl::matmul`` / ``Cuda::gemm[_batch]`` (cpu_kernel.rs:38-50, cuda_kernel.rs:153-237)."""
+        self._check(self.lib.dfdx_rocm_gemm(self.ctx, ctypes.byref(desc)))
+
+    def gemm_plan(self, desc: GemmDesc):
+        kernel, variant = ctypes.c_int(), ctypes.c_int()
+        name = ctypes.create_string_buffer(96)
+        self._check(self.lib.dfdx_rocm_gemm_plan(self.ctx, ctypes.byref(desc), ctypes.byref(kernel),
+                                                 ctypes.byref(variant), name, 96))
+        return kernel.value, variant.value, name.value.decode()
+
+    def gemm_time(self, desc: GemmDesc, warmup: int, iters: int) -> float:
+        ms = ctypes.c_float()
+        self._check(self.lib.dfdx_rocm_gemm_time(self.ctx, ctypes.byref(desc), warmup, iters, ctypes.byref(ms)))
+        return ms.value
+
+    def mfma_variant_count(self, dtype: str) -> int:
+        return self.lib.dfdx_rocm_mfma_variant_count(DTYPES[dtype])
+
+    # --------------------------------------------------------- kernel traits --
+    def forward(self, lhs: View, rhs: View) -> View:
+        """Dispatch on rank like ``TryMatMul`` (mod.rs:133-311); rank-1 operands are reshapes (mod.rs:139-174)."""
+        dt = lhs.dtype
+        assert lhs.dtype == rhs.dtype
+        L, R = len(lhs.shape), len(rhs.shape)
+        vp = ctypes.c_void_p
+        if L == 1 and R == 1:      # outer product: (M,1) x (1,N)
+            m, n = lhs.shape[0], rhs.shape[0]
+            out = self.zeros(dt, (m, n))
+            self._check(self.lib.dfdx_rocm_matmat_forward(
+                self.ctx, DTYPES[dt], _c(m), _c(1), _c(n), vp(lhs.ptr), _i64arr((lhs.strides[0], 1)),
+                vp(rhs.ptr), _i64arr((n * rhs.strides[0], rhs.strides[0])), vp(out.ptr)))
+            return out
+        if L == 1 and R == 2:      # (1,K) x (K,N) -> (N,)
+            assert lhs.shape[0] == rhs.shape[0], f"left: {lhs.shape[0]}\n right: {rhs.shape[0]}"
+            k, n = rhs.shape
+            out = self.zeros(dt, (n,))
+            self._check(self.lib.dfdx_rocm_matmat_forward(
+                self.ctx, DTYPES[dt], _c(1), _c(k), _c(n), vp(lhs.ptr), _i64arr((k * lhs.strides[0], lhs.strides[0])),
+                vp(rhs.ptr), _i64arr(rhs.strides), vp(out.ptr)))
+            return out
+        if L == 2 and R == 1:      # (M,K) x (K,1) -> (M,)
+            assert lhs.shape[1] == rhs.shape[0], f"left: {lhs.shape[1]}\n right: {rhs.shape[0]}"
+            m, k = lhs.shape
+            out = self.zeros(dt, (m,))
+            self._check(self.lib.dfdx_rocm_matmat_forward(
+                self.ctx, DTYPES[dt], _c(m), _c(k), _c(1), vp(lhs.ptr), _i64arr(lhs.strides),
+                vp(rhs.ptr), _i64arr((rhs.strides[0], 1)), vp(out.ptr)))
+            return out
+        if L == 2 and R == 2:
+            assert lhs.shape[1] == rhs.shape[0], f"left: {lhs.shape[1]}\n right: {rhs.shape[0]}"
+            (m, k), n = lhs.shape, rhs.shape[1]
+            out = self.zeros(dt, (m, n))
+            self._check(self.lib.dfdx_rocm_matmat_forward(
+                self.ctx, DTYPES[dt], _c(m), _c(k), _c(n), vp(lhs.ptr), _i64arr(lhs.strides),
+                vp(rhs.ptr), _i64arr(rhs.strides), vp(out.ptr)))
+            return out
+        if L == 3 and R == 2:
+            assert lhs.shape[2] == rhs.shape[0], f"left: {lhs.shape[2]}\n right: {rhs.shape[0]}"
+            (b, m, k), n = lhs.shape, rhs.shape[1]
+            out = self.zeros(dt, (b, m, n))
+            self._check(self.lib.dfdx_rocm_matmat_br_forward(
+                self.ctx, DTYPES[dt], _c(b), _c(m), _c(k), _c(n), vp(lhs.ptr), _i64arr(lhs.strides),
+                vp(rhs.ptr), _i64arr(rhs.strides), vp(out.ptr)))
+            return out
+        if L == 3 and R == 3:
+            assert lhs.shape[0] == rhs.shape[0], f"left: {lhs.shape[0]}\n right: {rhs.shape[0]}"
+            assert lhs.shape[2] == rhs.shape[1], f"left: {lhs.shape[2]}\n right: {rhs.shape[1]}"
+            (b, m, k), n = lhs.shape, rhs.shape[2]
+            out = self.zeros(dt, (b, m, n))
+            self._check(self.lib.dfdx_rocm_matmat_batch3_forward(
+                self.ctx, DTYPES[dt], _c(b), _c(m), _c(k), _c(n), vp(lhs.ptr), _i64arr(lhs.strides),
+                vp(rhs.ptr), _i64arr(rhs.strides), vp(out.ptr)))
+            return out
+        if L == 4 and R == 4:
+            assert lhs.shape[0] == rhs.shape[0], f"left: {lhs.shape[0]}\n right: {rhs.shape[0]}"
+            assert lhs.shape[1] == rhs.shape[1], f"left: {lhs.shape[1]}\n right: {rhs.shape[1]}"
+            assert lhs.shape[3] == rhs.shape[2], f"left: {lhs.shape[3]}\n right: {rhs.shape[2]}"
+            (b, s, m, k), n = lhs.shape, rhs.shape[3]
+            out = self.zeros(dt, (b, s, m, n))
+            self._check(self.lib.dfdx_rocm_matmat_batch4_forward(
+                self.ctx, DTYPES[dt], _c(b), _c(s), _c(m), _c(k), _c(n), vp(lhs.ptr), _i64arr(lhs.strides),
+                vp(rhs.ptr), _i64arr(rhs.strides), vp(out.ptr)))
+            return out
+        raise TypeError(f"matmul of rank {L} by rank {R} is not defined (mod.rs:133-311)")
+
+    def backward(self, lhs: View, grad_lhs: View, rhs: View, grad_rhs: View, grad_out: View):
+        """``D::backward(lhs, grad_lhs, rhs, grad_rhs, grad_out)``; grad_out contiguous; grads accumulate."""
+        dt = lhs.dtype
+        L, R = len(lhs.shape), len(rhs.shape)
+        vp = ctypes.c_void_p
+        if L <= 2 and R <= 2:
+            if L == 1 and R == 1:
+                m, k, n = lhs.shape[0], 1, rhs.shape[0]
+                ls, rs = (lhs.strides[0], 1), (n * rhs.strides[0], rhs.strides[0])
+            elif L == 1:
+                (k, n), m = rhs.shape, 1
+                ls, rs = (k * lhs.strides[0], lhs.strides[0]), rhs.strides
+            elif R == 1:
+                (m, k), n = lhs.shape, 1
+                ls, rs = lhs.strides, (rhs.strides[0], 1)
+            else:
+                (m, k), n = lhs.shape, rhs.shape[1]
+                ls, rs = lhs.strides, rhs.strides
+            self._check(self.lib.dfdx_rocm_matmat_backward(
+                self.ctx, DTYPES[dt], _c(m), _c(k), _c(n), vp(lhs.ptr), _i64arr(ls), vp(grad_lhs.ptr),
+                vp(rhs.ptr), _i64arr(rs), vp(grad_rhs.ptr), vp(grad_out.ptr)))
+            return
+        if L == 3 and R == 2:
+            (b, m, k), n = lhs.shape, rhs.shape[1]
+            fn, dims = self.lib.dfdx_rocm_matmat_br_backward, (b, m, k, n)
+        elif L == 3 and R == 3:
+            (b, m, k), n = lhs.shape, rhs.shape[2]
+            fn, dims = self.lib.dfdx_rocm_matmat_batch3_backward, (b, m, k, n)
+        elif L == 4 and R == 4:
+            (b, s, m, k), n = lhs.shape, rhs.shape[3]
+            fn, dims = self.lib.dfdx_rocm_matmat_batch4_backward, (b, s, m, k, n)
+        else:
+            raise TypeError(f"matmul of rank {L} by rank {R} is not defined")
+        self._check(fn(self.ctx, DTYPES[dt], *[_c(d) for d in dims], vp(lhs.ptr), _i64arr(lhs.strides),
+                       vp(grad_lhs.ptr), vp(rhs.ptr), _i64arr(rhs.strides), vp(grad_rhs.ptr), vp(grad_out.ptr)))
+
+    def linear_forward(self, x: View, weight: View, bias: Optional[View]) -> View:
+        """``Linear::try_forward`` (dfdx/src/nn/layers/linear.rs:82-89); weight is the (O, I) storage."""
+        o, i = weight.shape
+        assert weight.strides == (i, 1), "Linear weight storage is (O, I) row-major"
+        assert x.shape[-1] == i, f"left: {x.shape[-1]}\n right: {i}"
+        if len(x.shape) == 1:
+            rows, xs = 1, (i * x.strides[0], x.strides[0])
+        elif len(x.shape) == 2:
+            rows, xs = x.shape[0], x.strides
+        else:
+            assert x.strides == _row_major(x.shape), "batched Linear input must be contiguous to fold its rows"
+            rows, xs = int(np.prod(x.shape[:-1])), (i, 1)
+        out = self.zeros(x.dtype, tuple(x.shape[:-1]) + (o,))
+        self._check(self.lib.dfdx_rocm_linear_forward(
+            self.ctx, DTYPES[x.dtype], _c(rows), _c(i), _c(o), ctypes.c_void_p(x.ptr), _i64arr(xs),
+            ctypes.c_void_p(weight.ptr), ctypes.c_void_p(bias.ptr if bias is not None else None),
+            ctypes.c_void_p(out.ptr)))
+        return out
+
+
+def _c(v: int):
+    return ctypes.c_int64(int(v))

@@ -1,0 +1,193 @@
+/*
+ * dfdx_rocm.h -- C ABI of the MI355X (gfx950) matrix-multiplication backend
+ * for dfdx.
+ *
+ * These are the entry points a `Rocm` device inside dfdx-core binds over FFI in
+ * order to implement the kernel traits its `Cpu` and `Cuda` devices implement
+ * for `matmul`.  Each declaration names the reference interface it stands in
+ * for (paths relative to the dfdx repository, v0.13.0).
+ *
+ * Conventions
+ *   - Every function returns 0 on success.  Positive values are `hipError_t`
+ *     codes, negative values are the DFDX_ROCM_ERR_* codes below;
+ *     dfdx_rocm_strerror() renders either.  Nothing throws or aborts across
+ *     this boundary (the Rust side maps the code into `tensor::Error`,
+ *     dfdx-core/src/tensor/error.rs:5-28).
+ *   - Pointers named a/b/c/lhs/rhs/out/grad_* are DEVICE pointers owned by the
+ *     caller; the library never frees or retains them.
+ *   - Strides and batch strides are in ELEMENTS (not bytes), exactly the
+ *     `strides: [usize; N]` a dfdx `Tensor` carries
+ *     (dfdx-core/src/tensor/tensor_impls.rs:32-39).  Any stride pattern a dfdx
+ *     view can produce is accepted for inputs: transposed, permuted
+ *     (head-interleaved), broadcast (stride 0).
+ *   - Work is asynchronous on the context's stream; dfdx_rocm_synchronize()
+ *     blocks until it is done.
+ *   - f16 and bf16 products accumulate in f32 and round to nearest even once
+ *     on store; f32 accumulates in f32; f64 in f64.
+ */
+#ifndef DFDX_ROCM_H
+#define DFDX_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct dfdx_rocm_ctx dfdx_rocm_ctx;
+
+/* Element types (dfdx-core/src/dtypes/mod.rs:87-116).  `f16` and `AMP<f16>`
+ * are both DFDX_ROCM_F16 (same storage, f32 math: dtypes/amp.rs:8-10). */
+enum {
+    DFDX_ROCM_F32 = 0,
+    DFDX_ROCM_F16 = 1,
+    DFDX_ROCM_BF16 = 2,
+    DFDX_ROCM_F64 = 3
+};
+
+enum {
+    DFDX_ROCM_OK = 0,
+    DFDX_ROCM_ERR_INVALID_ARG = -1,   /* null pointer, negative size, unknown dtype ...          */
+    DFDX_ROCM_ERR_UNSUPPORTED = -2,   /* valid request this build has no kernel for              */
+    DFDX_ROCM_ERR_NO_DEVICE = -3,     /* no usable gfx950 device                                 */
+    DFDX_ROCM_ERR_ALIASED_OUTPUT = -4 /* output view maps several logical elements to one address */
+};
+
+/* Kernel families, for dfdx_rocm_gemm_desc.kernel (0 lets the library choose). */
+enum {
+    DFDX_ROCM_KERNEL_AUTO = 0,
+    DFDX_ROCM_KERNEL_GENERIC = 1, /* any strides, any dtype (scalar loads, LDS tiled)   */
+    DFDX_ROCM_KERNEL_MFMA = 2,    /* matrix-core kernels; variant chosen by `variant`   */
+    DFDX_ROCM_KERNEL_GEMV = 3     /* bandwidth-bound M=1 / N=1 products                 */
+};
+
+/* ---- device context -----------------------------------------------------
+ * Stands in for `Cuda::try_build(ordinal, seed)` and the handles it owns
+ * (dfdx-core/src/tensor/cuda/device.rs:22-33,72-90).  `stream` is a
+ * `hipStream_t` to run on, or NULL for the device's default stream. */
+int dfdx_rocm_create(int ordinal, void *stream, dfdx_rocm_ctx **out);
+int dfdx_rocm_destroy(dfdx_rocm_ctx *ctx);
+const char *dfdx_rocm_strerror(int code);
+/* Device name ("gfx950..."), compute-unit count and clock, for roofline reports. */
+int dfdx_rocm_device_info(dfdx_rocm_ctx *ctx, char *name, size_t name_len, int *compute_units, int *clock_mhz);
+
+/* ---- storage --------------------------------------------------------------
+ * What `Storage::try_alloc_len` (zero-filled; cuda/device.rs:259-266),
+ * `alloc_empty` (cuda/device.rs:97-106), `CopySlice` / `tensor_to_vec`
+ * (tensor/storage_traits.rs:93-96) and `Synchronize` (storage_traits.rs:31-39)
+ * need from the device. */
+int dfdx_rocm_alloc(dfdx_rocm_ctx *ctx, size_t bytes, int zeroed, void **out);
+int dfdx_rocm_free(dfdx_rocm_ctx *ctx, void *ptr);
+int dfdx_rocm_memset_zero(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes);
+int dfdx_rocm_copy_h2d(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes);
+int dfdx_rocm_copy_d2h(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes);
+int dfdx_rocm_copy_d2d(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes);
+int dfdx_rocm_synchronize(dfdx_rocm_ctx *ctx);
+
+/* ---- the strided (batched) GEMM -------------------------------------------
+ * Stands in for `MatMulImpl::matmul` on Cpu
+ * (dfdx-core/src/tensor_ops/matmul/cpu_kernel.rs:38-50) and for `Cuda::gemm` /
+ * `Cuda::gemm_batch` (matmul/cuda_kernel.rs:153-181,184-237), which the conv
+ * ops also call directly (conv2d/cuda_kernel.rs:115-139).
+ *
+ *   for b1 < batch1, b2 < batch2:
+ *     C[b1,b2][i,j] = (accumulate ? C[b1,b2][i,j] : 0) + bias[j]
+ *                     + sum_k A[b1,b2][i,k] * B[b1,b2][k,j]
+ *   X[b1,b2][r,c] lives at x + b1*x_b1 + b2*x_b2 + r*x_rs + c*x_cs.
+ *
+ * `reduce_batch` != 0 sums all batches into ONE C (c_b1, c_b2 ignored): the
+ * shared `grad_rhs` accumulator of the broadcast-rhs backward
+ * (cpu_kernel.rs:339-348), which cuBLAS cannot express
+ * (cuda_kernel.rs:358-371).  `bias` (length n, may be NULL) is the fused
+ * `Bias1D` add of `Linear` (dfdx/src/nn/layers/linear.rs:82-89). */
+typedef struct dfdx_rocm_gemm_desc {
+    int32_t dtype;
+    int32_t accumulate; /* 0: overwrite (forward); 1: add into C (every backward) */
+    int64_t m, n, k;
+    int64_t batch1, batch2; /* >= 1 */
+    const void *a;
+    int64_t a_rs, a_cs, a_b1, a_b2;
+    const void *b;
+    int64_t b_rs, b_cs, b_b1, b_b2;
+    void *c;
+    int64_t c_rs, c_cs, c_b1, c_b2;
+    const void *bias;
+    int32_t reduce_batch;
+    int32_t kernel;  /* DFDX_ROCM_KERNEL_* ; 0 = automatic */
+    int32_t variant; /* tile variant inside the family; 0 = automatic */
+    int32_t reserved;
+} dfdx_rocm_gemm_desc;
+
+int dfdx_rocm_gemm(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc);
+
+/* Which kernel dfdx_rocm_gemm would run for `desc`: writes the family, the
+ * variant and a short name ("mfma16_256x256x64_kc_kc" ...).  No launch. */
+int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int *kernel, int *variant,
+                        char *name, size_t name_len);
+/* Number of MFMA tile variants available for `dtype` (variants are 1..count). */
+int dfdx_rocm_mfma_variant_count(int dtype);
+
+/* Times `iters` back-to-back launches of `desc` with HIP events recorded on
+ * the context's stream (after `warmup` untimed launches) and returns the
+ * average milliseconds per launch.  Benchmark aid; no reference counterpart
+ * (dfdx's benches time with `Instant` around `synchronize`,
+ * dfdx/benches/conv2d.rs:25-45). */
+int dfdx_rocm_gemm_time(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int warmup, int iters, float *avg_ms);
+
+/* ---- the four kernel traits -------------------------------------------------
+ * One function per trait method.  `out` and `grad_out` are contiguous
+ * row-major of the output shape; `grad_lhs` / `grad_rhs` are buffers laid out
+ * like the operand's physical storage and are ACCUMULATED into through the
+ * operand's own strides (cpu_kernel.rs:266-285).  `*_strides` have one entry
+ * per tensor axis. */
+
+/* MatMatKernel (matmul/mod.rs:116-131): (M,K) x (K,N). */
+int dfdx_rocm_matmat_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t m, int64_t k, int64_t n,
+                             const void *lhs, const int64_t lhs_strides[2],
+                             const void *rhs, const int64_t rhs_strides[2], void *out);
+int dfdx_rocm_matmat_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t m, int64_t k, int64_t n,
+                              const void *lhs, const int64_t lhs_strides[2], void *grad_lhs,
+                              const void *rhs, const int64_t rhs_strides[2], void *grad_rhs,
+                              const void *grad_out);
+
+/* MatMatBrKernel (matmul/mod.rs:197-212): (B,M,K) x (K,N), rhs broadcast over the batch. */
+int dfdx_rocm_matmat_br_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t batch, int64_t m, int64_t k, int64_t n,
+                                const void *lhs, const int64_t lhs_strides[3],
+                                const void *rhs, const int64_t rhs_strides[2], void *out);
+int dfdx_rocm_matmat_br_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t batch, int64_t m, int64_t k, int64_t n,
+                                 const void *lhs, const int64_t lhs_strides[3], void *grad_lhs,
+                                 const void *rhs, const int64_t rhs_strides[2], void *grad_rhs,
+                                 const void *grad_out);
+
+/* MatMatBatch3Kernel (matmul/mod.rs:234-249): (B,M,K) x (B,K,N). */
+int dfdx_rocm_matmat_batch3_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t batch, int64_t m, int64_t k, int64_t n,
+                                    const void *lhs, const int64_t lhs_strides[3],
+                                    const void *rhs, const int64_t rhs_strides[3], void *out);
+int dfdx_rocm_matmat_batch3_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t batch, int64_t m, int64_t k, int64_t n,
+                                     const void *lhs, const int64_t lhs_strides[3], void *grad_lhs,
+                                     const void *rhs, const int64_t rhs_strides[3], void *grad_rhs,
+                                     const void *grad_out);
+
+/* MatMatBatch4Kernel (matmul/mod.rs:273-288): (B,S,M,K) x (B,S,K,N). */
+int dfdx_rocm_matmat_batch4_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t batch, int64_t seq, int64_t m, int64_t k,
+                                    int64_t n, const void *lhs, const int64_t lhs_strides[4],
+                                    const void *rhs, const int64_t rhs_strides[4], void *out);
+int dfdx_rocm_matmat_batch4_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t batch, int64_t seq, int64_t m, int64_t k,
+                                     int64_t n, const void *lhs, const int64_t lhs_strides[4], void *grad_lhs,
+                                     const void *rhs, const int64_t rhs_strides[4], void *grad_rhs,
+                                     const void *grad_out);
+
+/* ---- Linear with the bias add fused into the GEMM store ---------------------
+ * `Linear::try_forward` (dfdx/src/nn/layers/linear.rs:82-89): x (rows, I)
+ * with strides x_strides, weight stored (O, I) row-major and consumed through
+ * its zero-copy (I, O) view, bias (O,) or NULL; out (rows, O) contiguous.
+ * A (B, S, I) input is passed with rows = B*S when contiguous. */
+int dfdx_rocm_linear_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t in_dim, int64_t out_dim,
+                             const void *x, const int64_t x_strides[2], const void *weight, const void *bias,
+                             void *out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DFDX_ROCM_H */

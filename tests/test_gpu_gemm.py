@@ -1,0 +1,206 @@
+"""GPU parity: the strided batched GEMM entry (`dfdx_rocm_gemm`) against the CPU oracle.
+
+Every kernel family and every MFMA tile variant is forced in turn, over all operand
+layouts the matmul path produces (NN / TN / NT / TT, row- and column-major C), with
+and without accumulation, on shapes that are not multiples of the tile sizes.
+Tolerance: max|err| <= 1e-5*sqrt(K)*max|a|*max|b| for f32 and 2e-3*sqrt(K)*max|a|*max|b|
+for f16 / bf16 (f32 accumulate), measured against the oracle's float64 shadow result;
+the oracle's own f32-accumulated result must satisfy the same bound.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import assert_within, rng
+from gpu_util import announce, device, make_operand, values
+
+pytestmark = pytest.mark.gpu
+
+from dfdx_amd.rocm import KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA  # noqa: E402
+
+LAYOUTS = {"nn": (False, False), "tn": (True, False), "nt": (False, True), "tt": (True, True)}
+
+
+def run_case(dtype, m, k, n, layout, accumulate, kernel, variant, c_colmajor=False, bias=False, seed=1, pads=(0, 0, 0)):
+    dev = device()
+    g = rng(seed)
+    at, bt = LAYOUTS[layout]
+    a, astr = make_operand(g, m, k, at, dtype, pads[0])
+    b, bstr = make_operand(g, k, n, bt, dtype, pads[1])
+    c, cstr = make_operand(g, m, n, c_colmajor, dtype, pads[2])
+    bias_st = oracle.to_storage(g.standard_normal(n), dtype) if bias else None
+    A, B, C0 = values(a, dtype, (m, k), astr), values(b, dtype, (k, n), bstr), values(c, dtype, (m, n), cstr)
+
+    da, db, dc = dev.tensor(a, dtype), dev.tensor(b, dtype), dev.tensor(c, dtype)
+    dbias = dev.tensor(bias_st, dtype) if bias else None
+    desc = dev.gemm_desc(dtype, m, k, n, da.ptr, astr, db.ptr, bstr, dc.ptr, cstr, accumulate=accumulate,
+                         bias=dbias.ptr if bias else None, kernel=kernel, variant=variant)
+    announce("gemm", dtype, (m, k, n), layout, "acc" if accumulate else "ovw", "kernel", kernel, "variant", variant,
+             "ccol" if c_colmajor else "crow", "bias" if bias else "", dev.gemm_plan(desc)[2])
+    dev.gemm(desc)
+    dev.synchronize()
+    got_st = dev.to_host(dc)
+    got = values(got_st, dtype, (m, n), cstr)
+
+    want = A @ B + (C0 if accumulate else 0.0) + (oracle.to_f64(bias_st, dtype) if bias else 0.0)
+    ulp = {"f32": 2.0 ** -24, "f16": 2.0 ** -11, "bf16": 2.0 ** -8, "f64": 2.0 ** -53}[dtype]
+    assert_within(dtype, k, got, want, A, B, extra=ulp * float(np.max(np.abs(want))), what="gpu vs f64")
+    if not bias:  # the oracle proper (f32 accumulate, same rounding rule) on the same inputs; it has no bias term
+        c_or = c.copy()
+        oracle.gemm(dtype, m, k, n, accumulate, a, astr, b, bstr, c_or, cstr)
+        want_or = values(c_or, dtype, (m, n), cstr)
+        assert_within(dtype, k, got, want_or, A, B, extra=2 * ulp * float(np.max(np.abs(want))), what="gpu vs oracle")
+    # nothing outside the C view is touched
+    mask = np.ones(c.size, dtype=bool)
+    idx = values(np.arange(c.size, dtype=np.float64), "f64", (m, n), cstr).astype(np.int64)
+    mask[idx.reshape(-1)] = False
+    assert np.array_equal(oracle.to_f64(got_st, dtype)[mask], oracle.to_f64(c, dtype)[mask])
+
+
+# ------------------------------------------------------------------ generic --
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16", "f64"])
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_generic_kernel(dtype, layout, accumulate):
+    run_case(dtype, 67, 45, 83, layout, accumulate, KERNEL_GENERIC, 0, pads=(3, 1, 2))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (1, 7, 5), (5, 7, 1), (5, 1, 7), (1, 300, 1), (130, 2, 3)])
+def test_generic_degenerate_shapes(dtype, shape):
+    m, k, n = shape
+    run_case(dtype, m, k, n, "nn", True, KERNEL_GENERIC, 0)
+    run_case(dtype, m, k, n, "tt", False, KERNEL_GENERIC, 0, c_colmajor=True)
+
+
+def test_generic_k_zero_and_empty():
+    dev = device()
+    c = dev.tensor(np.full(6, 7.0, np.float32), "f32")
+    a = dev.tensor(np.zeros(4, np.float32), "f32")
+    announce("gemm k=0")
+    dev.gemm(dev.gemm_desc("f32", 2, 0, 3, a.ptr, (0, 1), a.ptr, (3, 1), c.ptr, (3, 1), accumulate=True))
+    assert np.array_equal(dev.to_host(c), np.full(6, 7.0, np.float32))
+    dev.gemm(dev.gemm_desc("f32", 2, 0, 3, a.ptr, (0, 1), a.ptr, (3, 1), c.ptr, (3, 1), accumulate=False))
+    assert np.array_equal(dev.to_host(c), np.zeros(6, np.float32))
+    dev.gemm(dev.gemm_desc("f32", 0, 4, 3, a.ptr, (4, 1), a.ptr, (3, 1), c.ptr, (3, 1)))  # m = 0: no-op
+
+
+def test_doubly_strided_operand_takes_generic_path():
+    """Neither stride is 1 (reachable through user permutes/slices): Cuda panics there (mod.rs:323), Cpu does not."""
+    dev = device()
+    g = rng(5)
+    m, k, n = 40, 24, 16
+    a = oracle.to_storage(g.standard_normal(m * (2 * k + 3)), "f32")
+    astr = (2 * k + 3, 2)
+    b, bstr = make_operand(g, k, n, False, "f32")
+    c = np.zeros(m * n, np.float32)
+    da, db, dc = dev.tensor(a, "f32"), dev.tensor(b, "f32"), dev.tensor(c, "f32")
+    desc = dev.gemm_desc("f32", m, k, n, da.ptr, astr, db.ptr, bstr, dc.ptr, (n, 1))
+    assert dev.gemm_plan(desc)[0] == KERNEL_GENERIC
+    announce("gemm doubly strided")
+    dev.gemm(desc)
+    A, B = values(a, "f32", (m, k), astr), values(b, "f32", (k, n), bstr)
+    assert_within("f32", k, dev.to_host(dc).astype(np.float64).reshape(m, n), A @ B, A, B, extra=1e-6)
+
+
+def test_aliased_output_is_rejected():
+    from dfdx_amd import RocmError
+
+    dev = device()
+    a = dev.tensor(np.zeros(64, np.float32), "f32")
+    with pytest.raises(RocmError) as e:
+        dev.gemm(dev.gemm_desc("f32", 4, 4, 4, a.ptr, (4, 1), a.ptr, (4, 1), a.ptr, (0, 1)))
+    assert e.value.code == -4
+    with pytest.raises(RocmError):
+        dev.gemm(dev.gemm_desc("f32", -1, 4, 4, a.ptr, (4, 1), a.ptr, (4, 1), a.ptr, (4, 1)))
+
+
+# --------------------------------------------------------------------- MFMA --
+MFMA_SHAPES = [(200, 136, 264), (512, 256, 256), (96, 72, 40)]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+def test_mfma_variants(dtype, variant, layout):
+    for i, (m, k, n) in enumerate(MFMA_SHAPES):
+        run_case(dtype, m, k, n, layout, bool(i % 2), KERNEL_MFMA, variant, seed=10 + i, pads=(8, 16, 8))
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+def test_mfma_column_major_c(dtype, layout):
+    """A permuted operand's gradient is a column-major C (cpu_kernel.rs:283-284): solved as C^T = B^T A^T."""
+    run_case(dtype, 264, 72, 136, layout, True, KERNEL_MFMA, 0, c_colmajor=True, pads=(0, 8, 8))
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_mfma_bias_epilogue(dtype):
+    run_case(dtype, 136, 64, 200, "nt", False, KERNEL_MFMA, 0, bias=True)
+    run_case(dtype, 136, 64, 200, "nt", False, KERNEL_MFMA, 0, bias=True, c_colmajor=True)
+    run_case(dtype, 40, 64, 72, "nn", False, KERNEL_GENERIC, 0, bias=True)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_mfma_small_integer_operands_are_exact(dtype):
+    """Integer operands with exactly representable products and sums: bit-exact whatever the summation order."""
+    dev = device()
+    g = rng(31)
+    m, k, n = 256, 512, 128
+    A = g.integers(-2, 3, (m, k)).astype(np.float64)
+    B = g.integers(-2, 3, (k, n)).astype(np.float64)
+    a, b = oracle.to_storage(A.reshape(-1), dtype), oracle.to_storage(B.reshape(-1), dtype)
+    da, db, dc = dev.tensor(a, dtype), dev.tensor(b, dtype), dev.zeros(dtype, (m, n))
+    for variant in range(1, 7):
+        announce("gemm exact ints", dtype, "variant", variant)
+        dev.gemm(dev.gemm_desc(dtype, m, k, n, da.ptr, (k, 1), db.ptr, (n, 1), dc.ptr, (n, 1), kernel=KERNEL_MFMA, variant=variant))
+        got = oracle.to_f64(dev.to_host(dc), dtype).reshape(m, n)
+        assert np.array_equal(got, A @ B)
+
+
+def test_auto_dispatch_prefers_mfma_when_aligned():
+    dev = device()
+    a = dev.zeros("f16", (256, 256))
+    d = dev.gemm_desc("f16", 256, 256, 256, a.ptr, (256, 1), a.ptr, (256, 1), a.ptr, (256, 1))
+    assert dev.gemm_plan(d)[0] == KERNEL_MFMA
+    d = dev.gemm_desc("f16", 255, 256, 256, a.ptr, (1, 256), a.ptr, (256, 1), a.ptr, (256, 1))
+    assert dev.gemm_plan(d)[0] == KERNEL_GENERIC  # M-contiguous A with M % 8 != 0
+    d = dev.gemm_desc("f64", 256, 256, 256, a.ptr, (256, 1), a.ptr, (256, 1), a.ptr, (256, 1))
+    assert dev.gemm_plan(d)[0] == KERNEL_GENERIC
+
+
+# ------------------------------------------------------------------ batched --
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("kernel", [KERNEL_GENERIC, KERNEL_MFMA])
+def test_batched_and_reduce(dtype, kernel):
+    """Two batch axes with head-interleaved strides, a broadcast (stride 0) B, and the reduce-over-batch mode."""
+    dev = device()
+    g = rng(41)
+    b1, b2, m, k, n = 3, 4, 72, 64, 40
+    # A stored (b1, m, b2, k): batch-2 stride (k) smaller than the row stride (b2*k)
+    a = oracle.to_storage(g.standard_normal(b1 * m * b2 * k), dtype)
+    a_rs, a_cs, a_b1, a_b2 = b2 * k, 1, m * b2 * k, k
+    bmat = oracle.to_storage(g.standard_normal(k * n), dtype)  # shared by all batches
+    c = np.zeros(b1 * b2 * m * n, oracle.NP_DTYPES[dtype])
+    da, db, dc = dev.tensor(a, dtype), dev.tensor(bmat, dtype), dev.tensor(c, dtype)
+    desc = dev.gemm_desc(dtype, m, k, n, da.ptr, (a_rs, a_cs), db.ptr, (n, 1), dc.ptr, (n, 1), batch=(b1, b2),
+                         a_batch=(a_b1, a_b2), b_batch=(0, 0), c_batch=(b2 * m * n, m * n), kernel=kernel)
+    announce("batched", dtype, kernel, dev.gemm_plan(desc)[2])
+    dev.gemm(desc)
+    A = values(a, dtype, (b1, b2, m, k), (a_b1, a_b2, a_rs, a_cs))
+    B = oracle.to_f64(bmat, dtype).reshape(k, n)
+    got = oracle.to_f64(dev.to_host(dc), dtype).reshape(b1, b2, m, n)
+    assert_within(dtype, k, got, A @ B, A, B, extra=2.0 ** -10 * np.abs(A @ B).max())
+
+    # reduce: G (k x n) += sum over batches A[b]^T (k x m) . D[b] (m x n)
+    dmat = oracle.to_storage(g.standard_normal(b1 * b2 * m * n), dtype)
+    gacc = oracle.to_storage(g.standard_normal(k * n), dtype)
+    dd, dg = dev.tensor(dmat, dtype), dev.tensor(gacc, dtype)
+    desc = dev.gemm_desc(dtype, k, m, n, da.ptr, (a_cs, a_rs), dd.ptr, (n, 1), dg.ptr, (n, 1), accumulate=True,
+                         batch=(b1, b2), a_batch=(a_b1, a_b2), b_batch=(b2 * m * n, m * n), reduce_batch=True, kernel=kernel)
+    announce("reduce", dtype, kernel, dev.gemm_plan(desc)[2])
+    dev.gemm(desc)
+    D = oracle.to_f64(dmat, dtype).reshape(b1, b2, m, n)
+    want = oracle.to_f64(gacc, dtype).reshape(k, n) + np.einsum("xymk,xymn->kn", A, D)
+    got = oracle.to_f64(dev.to_host(dg), dtype).reshape(k, n)
+    assert_within(dtype, b1 * b2 * m, got, want, A, D, extra=2.0 ** -10 * np.abs(want).max())
