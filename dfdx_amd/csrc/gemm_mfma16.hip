@@ -20,6 +20,7 @@
 // has one unit stride; pointers, leading strides and batch strides are multiples of
 // 8 elements (16 B) and the contiguous extent is a multiple of 8.
 #include "gemm_internal.h"
+#include <type_traits>
 
 namespace dfdx_rocm {
 namespace {
@@ -73,6 +74,11 @@ __device__ __forceinline__ u32x4 ldg16(const uint16_t *p, bool pred) {
 
 // Loader of one operand tile: ROWS (m or n extent) x BK, NT threads.
 // KC = operand is k-contiguous in global memory.
+//
+// Per-thread element offsets are computed once (init).  Rows beyond the matrix edge are
+// clamped onto the last valid row: they only feed C rows/columns that are never stored, so
+// their values do not matter but their addresses must be valid.  Only the k tail needs
+// zero fill; full k steps take the unpredicated path.
 template <int ROWS, int BK, int NT, bool KC> struct Loader {
     static constexpr int LOADS = ROWS * BK / 8 / NT;  // 16 B loads per thread per k step
     static_assert(LOADS >= 1 && (ROWS * BK / 8) % NT == 0, "tile does not divide over the threads");
@@ -84,44 +90,53 @@ template <int ROWS, int BK, int NT, bool KC> struct Loader {
     static constexpr int LDS_ROW = BK + 8;
 
     u32x4 regs[LOADS];
+    uint32_t goff[LOADS];  // byte offset of each load from the tile origin
+    int koff[LOADS];  // k index of each load inside the tile (for the tail predicate)
+    int soff[KC ? LOADS : UNITS];  // LDS element offset of each store
 
-    // `g` points at element (row0, k0) of the operand; ld = stride of the non-unit axis.
-    __device__ __forceinline__ void load(const uint16_t *g, int ld, int rows_left, int k_left, int tid) {
+    __device__ __forceinline__ void init(int ld, int rows_left, int tid) {
         if constexpr (KC) {
 #pragma unroll
             for (int i = 0; i < LOADS; i++) {
                 const int cid = i * NT + tid;
                 const int row = cid / CPR, ch = cid % CPR;
-                regs[i] = ldg16(g + row * ld + ch * 8, row < rows_left && ch * 8 < k_left);
+                goff[i] = (uint32_t)(min(row, rows_left - 1) * ld + ch * 8) * 2u;
+                koff[i] = ch * 8;
+                soff[i] = row * LDS_ROW + ch * 8;
             }
         } else {
 #pragma unroll
             for (int u = 0; u < UNITS; u++) {
                 const int uid = u * NT + tid;
                 const int kb = uid % NKB, mb = uid / NKB;
+                soff[u] = (mb * 8) * LDS_ROW + kb * KR;
 #pragma unroll
                 for (int r = 0; r < KR; r++) {
-                    const int kk = kb * KR + r;
-                    regs[u * KR + r] = ldg16(g + kk * ld + mb * 8, mb * 8 < rows_left && kk < k_left);
+                    goff[u * KR + r] = (uint32_t)((kb * KR + r) * ld + min(mb * 8, rows_left - 8)) * 2u;
+                    koff[u * KR + r] = kb * KR + r;
                 }
             }
         }
     }
 
-    __device__ __forceinline__ void store(uint16_t *lds, int tid) const {
+    // `g` points at the tile origin (uniform across the workgroup).
+    __device__ __forceinline__ void load(const uint16_t *g) {
+#pragma unroll
+        for (int i = 0; i < LOADS; i++) regs[i] = *(const u32x4 *)((const char *)g + goff[i]);
+    }
+    __device__ __forceinline__ void load_tail(const uint16_t *g, int k_left) {
+#pragma unroll
+        for (int i = 0; i < LOADS; i++) regs[i] = ldg16((const uint16_t *)((const char *)g + goff[i]), koff[i] < k_left);
+    }
+
+    __device__ __forceinline__ void store(uint16_t *lds) const {
         if constexpr (KC) {
 #pragma unroll
-            for (int i = 0; i < LOADS; i++) {
-                const int cid = i * NT + tid;
-                const int row = cid / CPR, ch = cid % CPR;
-                *(u32x4 *)(lds + row * LDS_ROW + ch * 8) = regs[i];
-            }
+            for (int i = 0; i < LOADS; i++) *(u32x4 *)(lds + soff[i]) = regs[i];
         } else {
 #pragma unroll
             for (int u = 0; u < UNITS; u++) {
-                const int uid = u * NT + tid;
-                const int kb = uid % NKB, mb = uid / NKB;
-                uint16_t *dst = lds + (mb * 8) * LDS_ROW + kb * KR;
+                uint16_t *dst = lds + soff[u];
 #pragma unroll
                 for (int j = 0; j < 8; j++) {  // output row j: column mb*8+j of the unit, KR k-values
                     uint32_t w[KR / 2];
@@ -177,27 +192,38 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
     const int ktiles = (p.k + BK - 1) / BK;
     const int iters = ktiles * p.kbatches;
 
-    // uniform pointer to element (bm0, 0) of A / (0, bn0) of B for k-loop step `it`
-    auto a_tile = [&](int it) -> const uint16_t * {
-        const int kb = p.kbatches > 1 ? it / ktiles : batch;
-        const int kt = p.kbatches > 1 ? it % ktiles : it;
+    // Uniform pointers to the origin of the NEXT tile to fetch, advanced incrementally; the
+    // divisions needed to locate a batch run once per batch, not once per k step.
+    auto a_origin = [&](int kb) -> const uint16_t * {
         const uint16_t *base = p.a + (int64_t)(kb / p.nb2) * p.a_b1 + (int64_t)(kb % p.nb2) * p.a_b2;
-        return A_KC ? base + (int64_t)bm0 * p.lda + kt * BK : base + (int64_t)kt * BK * p.lda + bm0;
+        return A_KC ? base + (int64_t)bm0 * p.lda : base + bm0;
     };
-    auto b_tile = [&](int it) -> const uint16_t * {
-        const int kb = p.kbatches > 1 ? it / ktiles : batch;
-        const int kt = p.kbatches > 1 ? it % ktiles : it;
+    auto b_origin = [&](int kb) -> const uint16_t * {
         const uint16_t *base = p.b + (int64_t)(kb / p.nb2) * p.b_b1 + (int64_t)(kb % p.nb2) * p.b_b2;
-        return B_KC ? base + (int64_t)bn0 * p.ldb + kt * BK : base + (int64_t)kt * BK * p.ldb + bn0;
+        return B_KC ? base + (int64_t)bn0 * p.ldb : base + bn0;
     };
-    auto k_left = [&](int it) -> int {
-        const int kt = p.kbatches > 1 ? it % ktiles : it;
-        return p.k - kt * BK;
-    };
+    const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
+    const int64_t b_step = B_KC ? BK : (int64_t)BK * p.ldb;
+    int f_kb = p.kbatches > 1 ? 0 : batch;  // batch of the next tile to fetch
+    int f_kt = 0;                            // its k-tile index
+    const uint16_t *a_next = a_origin(f_kb);
+    const uint16_t *b_next = b_origin(f_kb);
 
     Loader<BM, BK, NT, A_KC> la;
     Loader<BN, BK, NT, B_KC> lb;
-    const int rows_left = p.m - bm0, cols_left = p.n - bn0;
+    la.init(p.lda, p.m - bm0, tid);
+    lb.init(p.ldb, p.n - bn0, tid);
+    auto advance = [&]() {
+        a_next += a_step;
+        b_next += b_step;
+        if (++f_kt == ktiles) {
+            f_kt = 0;
+            if (p.kbatches > 1 && ++f_kb < p.kbatches) {
+                a_next = a_origin(f_kb);
+                b_next = b_origin(f_kb);
+            }
+        }
+    };
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -207,44 +233,57 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    if (iters > 0) {
-        la.load(a_tile(0), p.lda, rows_left, k_left(0), tid);
-        lb.load(b_tile(0), p.ldb, cols_left, k_left(0), tid);
-        la.store(As, tid);
-        lb.store(Bs, tid);
-    }
-    __syncthreads();
-
     const uint16_t *a_frag0 = As + (wm0 + l32) * LDS_ROW + lh * 8;
     const uint16_t *b_frag0 = Bs + (wn0 + l32) * LDS_ROW + lh * 8;
 
-    for (int it = 0; it < iters; it++) {
-        const int cur = it & 1;
-        const bool more = it + 1 < iters;
-        if (more) {
-            la.load(a_tile(it + 1), p.lda, rows_left, k_left(it + 1), tid);
-            lb.load(b_tile(it + 1), p.ldb, cols_left, k_left(it + 1), tid);
-        }
-        const uint16_t *af_base = a_frag0 + cur * BM * LDS_ROW;
-        const uint16_t *bf_base = b_frag0 + cur * BN * LDS_ROW;
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ks++) {
-            u32x4 af[TM], bf[TN];
-#pragma unroll
-            for (int i = 0; i < TM; i++) af[i] = *(const u32x4 *)(af_base + i * 32 * LDS_ROW + ks * 16);
-#pragma unroll
-            for (int j = 0; j < TN; j++) bf[j] = *(const u32x4 *)(bf_base + j * 32 * LDS_ROW + ks * 16);
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++) acc[i][j] = Mma<T>::mfma(bf[j], af[i], acc[i][j]);
-        }
-        if (more) {
-            la.store(As + (cur ^ 1) * BM * LDS_ROW, tid);
-            lb.store(Bs + (cur ^ 1) * BN * LDS_ROW, tid);
+    // The k loop exists twice: K a multiple of BK runs with unpredicated loads only; any
+    // other K runs with the k-tail predicate on every load.
+    auto k_loop = [&](auto tail_tag) {
+        constexpr bool TAIL = decltype(tail_tag)::value;
+        auto fetch = [&]() {
+            if constexpr (TAIL) {
+                const int kl = p.k - f_kt * BK;
+                la.load_tail(a_next, kl);
+                lb.load_tail(b_next, kl);
+            } else {
+                la.load(a_next);
+                lb.load(b_next);
+            }
+            advance();
+        };
+        if (iters > 0) {
+            fetch();
+            la.store(As);
+            lb.store(Bs);
         }
         __syncthreads();
-    }
+        for (int it = 0; it < iters; it++) {
+            const int cur = it & 1;
+            const bool more = it + 1 < iters;
+            if (more) fetch();
+            const uint16_t *af_base = a_frag0 + cur * BM * LDS_ROW;
+            const uint16_t *bf_base = b_frag0 + cur * BN * LDS_ROW;
+#pragma unroll
+            for (int ks = 0; ks < BK / 16; ks++) {
+                u32x4 af[TM], bf[TN];
+#pragma unroll
+                for (int i = 0; i < TM; i++) af[i] = *(const u32x4 *)(af_base + i * 32 * LDS_ROW + ks * 16);
+#pragma unroll
+                for (int j = 0; j < TN; j++) bf[j] = *(const u32x4 *)(bf_base + j * 32 * LDS_ROW + ks * 16);
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) acc[i][j] = Mma<T>::mfma(bf[j], af[i], acc[i][j]);
+            }
+            if (more) {
+                la.store(As + (cur ^ 1) * BM * LDS_ROW);
+                lb.store(Bs + (cur ^ 1) * BN * LDS_ROW);
+            }
+            __syncthreads();
+        }
+    };
+    if (p.k % BK == 0) k_loop(std::false_type{});
+    else k_loop(std::true_type{});
 
     // ---- epilogue: lane holds m = l32 (per tile), n = 8g + 4*lh + 0..3 --------
     const int cb = p.kbatches > 1 ? 0 : batch;
@@ -305,14 +344,23 @@ struct Variant {
     int bm, bn, bk, waves_m, waves_n;
 };
 
-// Variant ids are 1-based indices into this table.
+// Variant ids are 1-based indices into this list: X(id, BM, BN, BK, WAVES_M, WAVES_N).
+#define DFDX_MFMA16_VARIANTS(X) \
+    X(1, 256, 256, 64, 2, 4)    \
+    X(2, 256, 256, 64, 2, 2)    \
+    X(3, 256, 128, 64, 2, 2)    \
+    X(4, 128, 128, 64, 2, 2)    \
+    X(5, 128, 64, 64, 4, 1)     \
+    X(6, 64, 64, 64, 2, 2)      \
+    X(7, 256, 256, 32, 2, 4)    \
+    X(8, 256, 128, 32, 2, 2)    \
+    X(9, 128, 128, 32, 2, 2)    \
+    X(10, 128, 256, 32, 2, 2)
+
 constexpr Variant kVariants[] = {
-    {"256x256x64_w2x4", 256, 256, 64, 2, 4},
-    {"256x256x64_w2x2", 256, 256, 64, 2, 2},
-    {"256x128x64_w2x2", 256, 128, 64, 2, 2},
-    {"128x128x64_w2x2", 128, 128, 64, 2, 2},
-    {"128x64x64_w4x1", 128, 64, 64, 4, 1},
-    {"64x64x64_w2x2", 64, 64, 64, 2, 2},
+#define X(id, bm, bn, bk, wm, wn) {#bm "x" #bn "x" #bk "_w" #wm "x" #wn, bm, bn, bk, wm, wn},
+    DFDX_MFMA16_VARIANTS(X)
+#undef X
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -343,12 +391,10 @@ hipError_t launch_layout(const Params &p, bool a_kc, bool b_kc, hipStream_t stre
 
 template <typename T> hipError_t launch_variant(int variant, const Params &p, bool a_kc, bool b_kc, hipStream_t s) {
     switch (variant) {
-    case 1: return launch_layout<T, 256, 256, 64, 2, 4>(p, a_kc, b_kc, s);
-    case 2: return launch_layout<T, 256, 256, 64, 2, 2>(p, a_kc, b_kc, s);
-    case 3: return launch_layout<T, 256, 128, 64, 2, 2>(p, a_kc, b_kc, s);
-    case 4: return launch_layout<T, 128, 128, 64, 2, 2>(p, a_kc, b_kc, s);
-    case 5: return launch_layout<T, 128, 64, 64, 4, 1>(p, a_kc, b_kc, s);
-    case 6: return launch_layout<T, 64, 64, 64, 2, 2>(p, a_kc, b_kc, s);
+#define X(id, bm, bn, bk, wm, wn) \
+    case id: return launch_layout<T, bm, bn, bk, wm, wn>(p, a_kc, b_kc, s);
+        DFDX_MFMA16_VARIANTS(X)
+#undef X
     default: return hipErrorInvalidValue;
     }
 }
@@ -388,7 +434,7 @@ bool mfma16_supported(const GemmProblem &p, int variant) {
     if (!la.ok || !lb.ok) return false;
     const Variant &v = kVariants[variant - 1];
     // 32-bit offsets inside one tile
-    if (la.ld * (la.kc ? v.bm : v.bk) >= (1ll << 31) || lb.ld * (lb.kc ? v.bn : v.bk) >= (1ll << 31)) return false;
+    if (la.ld * (la.kc ? v.bm : v.bk) >= (1ll << 30) || lb.ld * (lb.kc ? v.bn : v.bk) >= (1ll << 30)) return false;
     if (!aligned16(p.a) || !aligned16(p.b)) return false;
     if (p.nb1 * p.nb2 > 1) {
         if (p.a_b1 % 8 || p.a_b2 % 8 || p.b_b1 % 8 || p.b_b2 % 8) return false;
