@@ -1,0 +1,110 @@
+"""Benchmark of the matmul hot path on one MI355X.
+
+A step is one 4096^3 f16 GEMM (f32 accumulate), C = A.B with row-major operands ~U(-1,1) resident in
+HBM -- the configuration the headline metric is quoted on.  The same launch is also timed for the
+transposed-stride variants and for f32.  One JSON line is printed:
+
+  value       f16 A.B throughput in TFLOP/s over the K timed steps (wall clock, synchronised both sides)
+  roofline    the f16 MFMA kernel's TFLOP/s from HIP events on the launch stream vs the 2.5 PFLOP/s dense peak
+  cpu_baseline  the CPU oracle (a port of dfdx's Cpu matmul semantics) timed on the host cores
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
+N = 4096
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+
+    import numpy as np
+    import torch
+
+    from dfdx_amd import Rocm
+
+    dev = Rocm(0)
+    info = dev.device_info()
+    flop = 2.0 * N ** 3
+    tdt = {"f16": torch.float16, "f32": torch.float32}
+    res = {}
+    headline = None
+    for dtype in ("f16", "f32"):
+        gen = torch.Generator(device="cuda").manual_seed(1234)
+        a = (torch.rand(N, N, device="cuda", generator=gen) * 2 - 1).to(tdt[dtype])
+        b = (torch.rand(N, N, device="cuda", generator=gen) * 2 - 1).to(tdt[dtype])
+        c = torch.zeros(N, N, device="cuda", dtype=tdt[dtype])
+        layouts = {"A.B": ((N, 1), (N, 1)), "At.B": ((1, N), (N, 1)), "A.Bt": ((N, 1), (1, N))}
+        res[dtype] = {}
+        for name, (astr, bstr) in layouts.items():
+            desc = dev.gemm_desc(dtype, N, N, N, a.data_ptr(), astr, b.data_ptr(), bstr, c.data_ptr(), (N, 1))
+            kernel = dev.gemm_plan(desc)[2]
+            for _ in range(args.warmup):
+                dev.gemm(desc)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                dev.gemm(desc)
+            torch.cuda.synchronize()
+            wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+            event_ms = dev.gemm_time(desc, 2, args.steps)   # HIP events on the launch stream
+            res[dtype][name] = {"kernel": kernel, "ms_per_step": round(wall_ms, 5), "tflops": round(flop / wall_ms / 1e9, 2),
+                                "kernel_ms": round(event_ms, 5), "kernel_tflops": round(flop / event_ms / 1e9, 2),
+                                "frac_mfma_peak": round(flop / event_ms / 1e9 / PEAK_TFLOPS[dtype], 4)}
+            if dtype == "f16" and name == "A.B":
+                headline = res[dtype][name]
+        del a, b, c
+
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+
+        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        g = np.random.Generator(np.random.Philox(5))
+        a_h = g.uniform(-1, 1, N * N).astype(np.float16)
+        b_h = g.uniform(-1, 1, N * N).astype(np.float16)
+        c_h = np.zeros(N * N, np.float16)
+        oracle.gemm("f16", 256, N, N, False, a_h, (N, 1), b_h, (N, 1), c_h, (N, 1))   # warm the threads / pages
+        t0 = time.perf_counter()
+        oracle.gemm("f16", N, N, N, False, a_h, (N, 1), b_h, (N, 1), c_h, (N, 1))
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(flop / dt / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+               "sample": f"one full {N}^3 f16 GEMM (f32 accumulate) through the C oracle, OpenMP over rows, {dt:.2f} s"}
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(headline["kernel"])
+
+    line = {
+        "metric": "GEMM TFLOP/s (f16,f32) at 4096^3 + % MFMA peak on 1 MI355X; speedup vs Cpu",
+        "value": headline["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": headline["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[1]: single square GEMM C=A.B, M=N=K=4096, f16 in / f32 accumulate, row-major A and B ~U(-1,1)",
+                   "step": "one GEMM launch (137.44 GFLOP)", "device": info},
+        "roofline": {"bound": "mfma", "achieved": headline["kernel_tflops"], "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
+                     "frac": round(headline["kernel_tflops"] / PEAK_TFLOPS["f16"], 4), "traffic": traffic,
+                     "kernel": headline["kernel"]},
+        "cpu_baseline": cpu,
+        "speedup_vs_cpu": (round(headline["tflops"] / cpu["value"], 1) if cpu else None),
+        "variants": res,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
