@@ -51,6 +51,14 @@ bool mfma16_supported(const GemmProblem &p, int variant);
 int mfma16_pick_variant(const GemmProblem &p, int compute_units);
 hipError_t launch_mfma16(const GemmProblem &p, int variant, hipStream_t stream);
 
+// ---- LDS-DMA MFMA kernels for 16-bit inputs, K % 64 == 0 (gemm_mfma16_dma.hip) ----
+// Reached through the mfma16_* entry points above: their variant ids follow the register-staged ones.
+int mfma16dma_variant_count();
+const char *mfma16dma_variant_name(int variant);
+bool mfma16dma_supported(const GemmProblem &p, int variant);
+int mfma16dma_pick_variant(const GemmProblem &p, int compute_units);
+hipError_t launch_mfma16dma(const GemmProblem &p, int variant, hipStream_t stream);
+
 // ---- MFMA kernels for f32 (gemm_mfma32.hip) ----
 int mfma32_variant_count();
 const char *mfma32_variant_name(int variant);

@@ -419,12 +419,17 @@ inline OperandLayout classify(int64_t rows, int64_t kdim, int64_t row_stride, in
 
 }  // namespace
 
-int mfma16_variant_count() { return kNumVariants; }
-const char *mfma16_variant_name(int v) { return (v >= 1 && v <= kNumVariants) ? kVariants[v - 1].name : "?"; }
+// Variant ids 1..kNumVariants are the register-staged kernels of this file; higher ids are the LDS-DMA kernels.
+int mfma16_variant_count() { return kNumVariants + mfma16dma_variant_count(); }
+const char *mfma16_variant_name(int v) {
+    if (v > kNumVariants) return mfma16dma_variant_name(v - kNumVariants);
+    return (v >= 1) ? kVariants[v - 1].name : "?";
+}
 
 bool mfma16_supported(const GemmProblem &p, int variant) {
+    if (variant > kNumVariants) return mfma16dma_supported(p, variant - kNumVariants);
     if (p.dtype != DT_F16 && p.dtype != DT_BF16) return false;
-    if (variant < 1 || variant > kNumVariants) return false;
+    if (variant < 1) return false;
     if (p.m < 1 || p.n < 1 || p.k < 1) return false;
     if (p.m > (1 << 30) || p.n > (1 << 30) || p.k > (1 << 30)) return false;
     if (p.c_cs != 1 && p.n != 1) return false;
@@ -448,6 +453,7 @@ bool mfma16_supported(const GemmProblem &p, int variant) {
 }
 
 int mfma16_pick_variant(const GemmProblem &p, int compute_units) {
+    if (const int d = mfma16dma_pick_variant(p, compute_units)) return kNumVariants + d;
     // Largest tile that still gives every compute unit at least one workgroup; ties go to the larger tile.
     const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
     const int order[] = {1, 3, 4, 5, 6};
@@ -462,6 +468,7 @@ int mfma16_pick_variant(const GemmProblem &p, int compute_units) {
 }
 
 hipError_t launch_mfma16(const GemmProblem &g, int variant, hipStream_t stream) {
+    if (variant > kNumVariants) return launch_mfma16dma(g, variant - kNumVariants, stream);
     if (!mfma16_supported(g, variant)) return hipErrorInvalidValue;
     const Variant &v = kVariants[variant - 1];
     const OperandLayout la = classify(g.m, g.k, g.a_rs, g.a_cs);

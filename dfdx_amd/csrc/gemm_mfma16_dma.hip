@@ -1,0 +1,495 @@
+// MFMA GEMM for 16-bit inputs (f16 / bf16), f32 accumulate, gfx950 (CDNA4): the fast path for
+// K % 64 == 0.  v_mfma_f32_16x16x32_{f16,bf16}; BM x BN x 64 tile per workgroup of 8 waves.
+//
+// Data movement
+//   * A and B tiles go from global memory straight into LDS with 16 B-per-lane LDS-DMA loads
+//     (global_load_lds_dwordx4): no VGPR staging, no ds_write.  One wave instruction fills 1 KB of
+//     LDS contiguously; WHICH 16 B chunk of the tile a lane fetches is chosen so that the tile lands
+//     XOR-swizzled and every fragment read is bank-conflict free (measured: SQ_LDS_BANK_CONFLICT = 0).
+//   * k-contiguous operand (A row-major, or B stored [N][K]): LDS holds [row][64 k], chunk c of row r at
+//     position c ^ ((r >> 1) & 7); fragments are read with ds_read_b128.
+//   * m/n-contiguous operand (A stored [K][M], or B row-major [K][N]): LDS holds [k][rows] exactly as in
+//     memory (no transpose anywhere); fragments are read with the transposing ds_read_b64_tr_b16, two per
+//     fragment.  Chunk c of k-row k sits at c ^ swz(k) (see mc_swizzle).
+//   * Two LDS stages.  Tile t+1 is requested right after the barrier that retires tile t-1 and has one
+//     full k step of MFMAs to arrive.
+// Schedule per k step (32 wide, two per tile): the A fragments are single buffered in two halves, the B
+// fragments double buffered; the reads for the next step are issued in the middle of the MFMAs of the
+// current one, into registers that are already free, so each read has >= a quarter step of MFMAs to land.
+// One s_barrier per tile.  Stage hand-over uses explicit s_waitcnt vmcnt/lgkmcnt + s_barrier.
+//
+// Rows/columns past the matrix edge are clamped onto valid addresses (they only feed C entries that are
+// never stored).  There is no k tail here: K % 64 != 0 is served by the register-staged kernel.
+#include "gemm_internal.h"
+#include <type_traits>
+
+namespace dfdx_rocm {
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short v4i16 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+#define DFDX_LDS __attribute__((address_space(3)))
+#define DFDX_GLB __attribute__((address_space(1)))
+
+constexpr int BK = 64;
+constexpr int STAGES = 2;
+
+struct Params {
+    const uint16_t *a;
+    const uint16_t *b;
+    uint16_t *c;
+    const uint16_t *bias;
+    int m, n, k;
+    int lda, ldb;
+    int64_t ldc;
+    int64_t a_b1, a_b2, b_b1, b_b2, c_b1, c_b2;
+    int nb2, kbatches;
+    int tiles_m, tiles_n, tiles_per_batch, total_blocks;
+    int accumulate, bias_mode, c_vec;
+    int group_m;
+};
+
+template <typename T> struct Mma;
+template <> struct Mma<_Float16> {
+    static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
+    static __device__ __forceinline__ uint16_t from_f32(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+};
+template <> struct Mma<__bf16> {
+    static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
+    static __device__ __forceinline__ uint16_t from_f32(float v) {
+        uint32_t x = __float_as_uint(v);
+        if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+        return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);  // round to nearest even
+    }
+};
+
+// Swizzle of an m/n-contiguous tile ([k][ROWS] in LDS, ROWS*2 bytes per k-row): XOR applied to the 16 B
+// chunk index of k-row k.  A 16-lane group of a transposing read touches 4 consecutive k-rows x 2 chunks,
+// a second group the same chunks 8 k-rows further: the XOR spreads those over distinct banks.
+template <int ROWS> __device__ __forceinline__ int mc_swizzle(int k) {
+    if constexpr (ROWS >= 128) return (4 * (k & 3)) ^ (2 * ((k >> 3) & 1));
+    else return (4 * ((k >> 1) & 1)) ^ (2 * ((k >> 3) & 1));  // ROWS == 64: bit 3 of the bank slot comes from k & 1
+}
+
+// One operand tile in LDS, filled by LDS-DMA loads (16 B per lane, 1 KB contiguous per wave instruction).
+template <int ROWS, int NWAVES, bool KC> struct DmaTile {
+    static constexpr int BYTES = ROWS * BK * 2;
+    static constexpr int INSTRS = BYTES / 1024;
+    static constexpr int IPW = INSTRS / NWAVES;
+    static_assert(INSTRS % NWAVES == 0 && IPW >= 1, "tile does not divide over the waves");
+    static constexpr int CPR = KC ? BK / 8 : ROWS / 8;  // 16 B chunks per LDS row
+    uint32_t goff[IPW];                                 // byte offset from the tile origin in global memory
+
+    __device__ __forceinline__ void init(int ld, int rows_left, int wave, int lane) {
+#pragma unroll
+        for (int i = 0; i < IPW; i++) {
+            const int slot = (wave * IPW + i) * 64 + lane;  // 16 B slot index inside the tile
+            const int r = slot / CPR, cp = slot % CPR;
+            if constexpr (KC) {
+                const int c = cp ^ ((r >> 1) & 7);
+                goff[i] = (uint32_t)(min(r, rows_left - 1) * ld + c * 8) * 2u;
+            } else {
+                const int c = cp ^ mc_swizzle<ROWS>(r);
+                goff[i] = (uint32_t)(r * ld + min(c * 8, rows_left - 8)) * 2u;
+            }
+        }
+    }
+    __device__ __forceinline__ void issue(const uint16_t *g, uint8_t *lds_tile, int wave) const {
+#pragma unroll
+        for (int i = 0; i < IPW; i++)
+            __builtin_amdgcn_global_load_lds((const DFDX_GLB void *)((const char *)g + goff[i]),
+                                             (DFDX_LDS void *)(lds_tile + (wave * IPW + i) * 1024), 16, 0, 0);
+    }
+};
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(const Params p) {
+    constexpr int NW = WAVES_M * WAVES_N;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 16, TN = WTN / 16;
+    static_assert(WTM % 64 == 0 && WTN % 16 == 0, "wave tile must be a multiple of 64 x 16");
+    constexpr int Q = TM / 4;  // tile rows per quarter of a k step
+    using TA = DmaTile<BM, NW, A_KC>;
+    using TB = DmaTile<BN, NW, B_KC>;
+    constexpr int STAGE_BYTES = TA::BYTES + TB::BYTES;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64, wave = tid / 64;
+    const int wm0 = (wave / WAVES_N) * WTM, wn0 = (wave % WAVES_N) * WTN;
+    const int l16 = lane % 16, lq = lane / 16;
+
+    // ---- which tile -------------------------------------------------------
+    const int work = xcd_remap(blockIdx.x, p.total_blocks);
+    const int batch = work / p.tiles_per_batch;
+    const int tile = work % p.tiles_per_batch;
+    const int gsize = p.group_m * p.tiles_n;
+    const int group = tile / gsize;
+    const int first_m = group * p.group_m;
+    const int gm = min(p.tiles_m - first_m, p.group_m);
+    const int tm_idx = first_m + (tile % gsize) % gm;
+    const int tn_idx = (tile % gsize) / gm;
+    const int bm0 = tm_idx * BM, bn0 = tn_idx * BN;
+
+    const int ktiles = p.k / BK;
+    const int iters = ktiles * p.kbatches;
+
+    // ---- global side: origin of the next tile to request -------------------
+    auto a_origin = [&](int kb) -> const uint16_t * {
+        const uint16_t *base = p.a + (int64_t)(kb / p.nb2) * p.a_b1 + (int64_t)(kb % p.nb2) * p.a_b2;
+        return A_KC ? base + (int64_t)bm0 * p.lda : base + bm0;
+    };
+    auto b_origin = [&](int kb) -> const uint16_t * {
+        const uint16_t *base = p.b + (int64_t)(kb / p.nb2) * p.b_b1 + (int64_t)(kb % p.nb2) * p.b_b2;
+        return B_KC ? base + (int64_t)bn0 * p.ldb : base + bn0;
+    };
+    const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
+    const int64_t b_step = B_KC ? BK : (int64_t)BK * p.ldb;
+    int f_kb = p.kbatches > 1 ? 0 : batch;
+    int f_kt = 0;
+    const uint16_t *a_next = a_origin(f_kb);
+    const uint16_t *b_next = b_origin(f_kb);
+    TA ta;
+    TB tb;
+    ta.init(p.lda, p.m - bm0, wave, lane);
+    tb.init(p.ldb, p.n - bn0, wave, lane);
+    auto issue = [&](int stage) {
+        uint8_t *st = smem + stage * STAGE_BYTES;
+        ta.issue(a_next, st, wave);
+        tb.issue(b_next, st + TA::BYTES, wave);
+        a_next += a_step;
+        b_next += b_step;
+        if (++f_kt == ktiles) {
+            f_kt = 0;
+            if (p.kbatches > 1 && ++f_kb < p.kbatches) {
+                a_next = a_origin(f_kb);
+                b_next = b_origin(f_kb);
+            }
+        }
+    };
+
+    // ---- LDS side: per-lane fragment addresses ------------------------------
+    // k-contiguous: lane reads row w0 + 16*t + l16, logical chunk 4*ks + lq
+    int a_off[2], b_off[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        const int c = ks * 4 + lq;
+        a_off[ks] = (wm0 + l16) * BK * 2 + ((c ^ ((l16 >> 1) & 7)) * 16);
+        b_off[ks] = (wn0 + l16) * BK * 2 + ((c ^ ((l16 >> 1) & 7)) * 16);
+    }
+    // m/n-contiguous: lane 16*g + L supplies the address of X[k = 8*g + L/4 (+32*ks, +4)][col = w0 + 16*t + 4*(L%4)];
+    // the transposing read hands lane L the 4 k-values of column w0 + 16*t + L.
+    const int tr_k = lq * 8 + l16 / 4;
+    const int tr_col = 4 * (l16 % 4);
+    auto tr_frag = [&](const uint8_t *tile_base, auto rows_tag, int ks, int col0) -> u32x4 {
+        constexpr int ROWS = decltype(rows_tag)::value;
+        const int col = col0 + tr_col;
+        const int k = ks * 32 + tr_k;   // k and k+4 share the swizzle (same k & 3 pattern shifted by 4: see below)
+        const int c = col / 8, half = (col / 4) % 2;
+        const int off0 = k * ROWS * 2 + ((c ^ mc_swizzle<ROWS>(k)) * 16) + half * 8;
+        const int off1 = (k + 4) * ROWS * 2 + ((c ^ mc_swizzle<ROWS>(k + 4)) * 16) + half * 8;
+        const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DFDX_LDS v4i16 *)(tile_base + off0));
+        const v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DFDX_LDS v4i16 *)(tile_base + off1));
+        const u32x2 l = __builtin_bit_cast(u32x2, lo), h = __builtin_bit_cast(u32x2, hi);
+        return u32x4{l[0], l[1], h[0], h[1]};
+    };
+
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[i][j][v] = 0.0f;
+
+    u32x4 fa[TM], fb[2][TN];
+    auto read_a = [&](const uint8_t *sa, int ks, int i0, int i1) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            if (i >= i0 && i < i1) {
+                if constexpr (A_KC) fa[i] = *(const u32x4 *)(sa + a_off[ks] + i * 16 * BK * 2);
+                else fa[i] = tr_frag(sa, std::integral_constant<int, BM>{}, ks, wm0 + i * 16);
+            }
+    };
+    auto read_b = [&](const uint8_t *sa, int ks, u32x4(&bf)[TN]) {
+        const uint8_t *sb = sa + TA::BYTES;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            if constexpr (B_KC) bf[j] = *(const u32x4 *)(sb + b_off[ks] + j * 16 * BK * 2);
+            else bf[j] = tr_frag(sb, std::integral_constant<int, BN>{}, ks, wn0 + j * 16);
+        }
+    };
+    // swapped operands: the lane ends up with m = l16 and 4 consecutive n = 4*lq + 0..3 per 16x16 tile
+    auto mma = [&](const u32x4(&bf)[TN], int i0, int i1) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            if (i >= i0 && i < i1) {
+#pragma unroll
+                for (int j = 0; j < TN; j++) acc[i][j] = Mma<T>::mfma(bf[j], fa[i], acc[i][j]);
+            }
+    };
+    // Make tile t visible to every wave, then request tile t+1 into the stage tile t-1 occupied.  Callers
+    // guarantee that this wave has issued all its LDS reads of tile t-1; lgkmcnt(0) makes sure they are done.
+    auto sync_tile = [&](int t) {
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) & lgkmcnt(0)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (t + 1 < iters) issue((t + 1) % STAGES);
+    };
+
+    if (iters > 0) {
+        issue(0);
+        sync_tile(0);
+        read_a(smem, 0, 0, TM);
+        read_b(smem, 0, fb[0]);
+    }
+    auto tile_body = [&](int it, auto has_next_tag) {
+        constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
+        const uint8_t *sa = smem + (it % STAGES) * STAGE_BYTES;
+        const uint8_t *sn = smem + ((it + 1) % STAGES) * STAGE_BYTES;
+        // ---- k step 0 (B buffer 0); prefetch k step 1 of this tile
+        mma(fb[0], 0, Q);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(fb[0], Q, 2 * Q);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(fb[0], 2 * Q, 3 * Q);
+        __builtin_amdgcn_sched_barrier(0);
+        read_a(sa, 1, 0, 2 * Q);
+        read_b(sa, 1, fb[1]);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(fb[0], 3 * Q, TM);
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- k step 1 (B buffer 1); prefetch k step 0 of the next tile
+        mma(fb[1], 0, Q);
+        __builtin_amdgcn_sched_barrier(0);
+        read_a(sa, 1, 2 * Q, TM);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(fb[1], Q, 2 * Q);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(fb[1], 2 * Q, 3 * Q);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (HAS_NEXT) {
+            sync_tile(it + 1);
+            read_a(sn, 0, 0, 2 * Q);
+            read_b(sn, 0, fb[0]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mma(fb[1], 3 * Q, TM);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (HAS_NEXT) read_a(sn, 0, 2 * Q, TM);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    for (int it = 0; it + 1 < iters; it++) tile_body(it, std::true_type{});
+    if (iters > 0) tile_body(iters - 1, std::false_type{});
+
+    // ---- epilogue: lane holds m = l16 (per tile), n = 4*lq + 0..3 -------------
+    const int cb = p.kbatches > 1 ? 0 : batch;
+    uint16_t *cbase = p.c + (int64_t)(cb / p.nb2) * p.c_b1 + (int64_t)(cb % p.nb2) * p.c_b2;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int gm_row = bm0 + wm0 + i * 16 + l16;
+        if (gm_row >= p.m) continue;
+        uint16_t *crow = cbase + (int64_t)gm_row * p.ldc;
+        const float rbias = (p.bias_mode == BIAS_PER_ROW) ? Mma<T>::to_f32(p.bias[gm_row]) : 0.0f;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int gn = bn0 + wn0 + j * 16 + lq * 4;
+            if (gn >= p.n) continue;
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = acc[i][j][e] + rbias;
+            if (p.c_vec) {  // n % 4 == 0 here, so the 4 columns are all in range
+                if (p.bias_mode == BIAS_PER_COL) {
+                    const u32x2 bv = *(const u32x2 *)(p.bias + gn);
+                    v[0] += Mma<T>::to_f32((uint16_t)(bv[0] & 0xffffu));
+                    v[1] += Mma<T>::to_f32((uint16_t)(bv[0] >> 16));
+                    v[2] += Mma<T>::to_f32((uint16_t)(bv[1] & 0xffffu));
+                    v[3] += Mma<T>::to_f32((uint16_t)(bv[1] >> 16));
+                }
+                if (p.accumulate) {
+                    const u32x2 old = *(const u32x2 *)(crow + gn);
+                    v[0] += Mma<T>::to_f32((uint16_t)(old[0] & 0xffffu));
+                    v[1] += Mma<T>::to_f32((uint16_t)(old[0] >> 16));
+                    v[2] += Mma<T>::to_f32((uint16_t)(old[1] & 0xffffu));
+                    v[3] += Mma<T>::to_f32((uint16_t)(old[1] >> 16));
+                }
+                u32x2 o;
+                o[0] = (uint32_t)Mma<T>::from_f32(v[0]) | ((uint32_t)Mma<T>::from_f32(v[1]) << 16);
+                o[1] = (uint32_t)Mma<T>::from_f32(v[2]) | ((uint32_t)Mma<T>::from_f32(v[3]) << 16);
+                *(u32x2 *)(crow + gn) = o;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    if (gn + e >= p.n) break;
+                    float x = v[e];
+                    if (p.bias_mode == BIAS_PER_COL) x += Mma<T>::to_f32(p.bias[gn + e]);
+                    if (p.accumulate) x += Mma<T>::to_f32(crow[gn + e]);
+                    crow[gn + e] = Mma<T>::from_f32(x);
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ host side --
+
+struct Variant {
+    const char *name;
+    int bm, bn, waves_m, waves_n;
+};
+
+// X(id, BM, BN, WAVES_M, WAVES_N); ids are 1-based inside this family.
+#define DFDX_MFMA16_DMA_VARIANTS(X) \
+    X(1, 256, 256, 2, 4)            \
+    X(2, 256, 128, 2, 4)            \
+    X(3, 128, 128, 2, 4)            \
+    X(4, 256, 64, 4, 2)             \
+    X(5, 128, 64, 2, 4)
+
+constexpr Variant kVariants[] = {
+#define X(id, bm, bn, wm, wn) {"dma_" #bm "x" #bn "x64_w" #wm "x" #wn, bm, bn, wm, wn},
+    DFDX_MFMA16_DMA_VARIANTS(X)
+#undef X
+};
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+
+template <typename T, int BM, int BN, int WM, int WN>
+hipError_t launch_layout(const Params &p, bool a_kc, bool b_kc, hipStream_t stream) {
+    constexpr int NT = WM * WN * 64;
+    constexpr size_t lds = (size_t)STAGES * (BM + BN) * BK * 2;
+    dim3 grid((unsigned)p.total_blocks), block(NT);
+#define DFDX_LAUNCH(AKC, BKC)                                                                                  \
+    do {                                                                                                       \
+        auto kern = gemm_mfma16_dma_kernel<T, BM, BN, WM, WN, AKC, BKC>;                                       \
+        static bool configured = false;                                                                        \
+        if (!configured) {                                                                                     \
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                                               (int)lds);                                                      \
+            if (e != hipSuccess) return e;                                                                     \
+            configured = true;                                                                                 \
+        }                                                                                                      \
+        kern<<<grid, block, lds, stream>>>(p);                                                                 \
+    } while (0)
+    if (a_kc && b_kc) DFDX_LAUNCH(true, true);
+    else if (a_kc && !b_kc) DFDX_LAUNCH(true, false);
+    else if (!a_kc && b_kc) DFDX_LAUNCH(false, true);
+    else DFDX_LAUNCH(false, false);
+#undef DFDX_LAUNCH
+    return hipGetLastError();
+}
+
+template <typename T> hipError_t launch_variant(int variant, const Params &p, bool a_kc, bool b_kc, hipStream_t s) {
+    switch (variant) {
+#define X(id, bm, bn, wm, wn) \
+    case id: return launch_layout<T, bm, bn, wm, wn>(p, a_kc, b_kc, s);
+        DFDX_MFMA16_DMA_VARIANTS(X)
+#undef X
+    default: return hipErrorInvalidValue;
+    }
+}
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+struct OperandLayout {
+    bool ok, kc;
+    int64_t ld;
+};
+inline OperandLayout classify(int64_t rows, int64_t kdim, int64_t row_stride, int64_t k_stride) {
+    OperandLayout r{false, false, 0};
+    if (k_stride == 1 && kdim % 8 == 0 && (rows == 1 || (row_stride % 8 == 0 && row_stride >= kdim))) {
+        r.ok = true; r.kc = true; r.ld = rows == 1 ? kdim : row_stride;
+    } else if (row_stride == 1 && rows % 8 == 0 && (kdim == 1 || (k_stride % 8 == 0 && k_stride >= rows))) {
+        r.ok = true; r.kc = false; r.ld = kdim == 1 ? rows : k_stride;
+    }
+    return r;
+}
+
+}  // namespace
+
+int mfma16dma_variant_count() { return kNumVariants; }
+const char *mfma16dma_variant_name(int v) { return (v >= 1 && v <= kNumVariants) ? kVariants[v - 1].name : "?"; }
+
+bool mfma16dma_supported(const GemmProblem &p, int variant) {
+    if (p.dtype != DT_F16 && p.dtype != DT_BF16) return false;
+    if (variant < 1 || variant > kNumVariants) return false;
+    if (p.m < 1 || p.n < 1 || p.k < BK || p.k % BK != 0) return false;
+    if (p.m > (1 << 30) || p.n > (1 << 30) || p.k > (1 << 30)) return false;
+    if (p.c_cs != 1 && p.n != 1) return false;
+    if (p.n > 1 && p.m > 1 && p.c_rs < p.n) return false;
+    const OperandLayout la = classify(p.m, p.k, p.a_rs, p.a_cs);
+    const OperandLayout lb = classify(p.n, p.k, p.b_cs, p.b_rs);
+    if (!la.ok || !lb.ok) return false;
+    const Variant &v = kVariants[variant - 1];
+    if (la.ld * (la.kc ? v.bm : BK) >= (1ll << 30) || lb.ld * (lb.kc ? v.bn : BK) >= (1ll << 30)) return false;
+    if (!aligned16(p.a) || !aligned16(p.b)) return false;
+    if (p.nb1 * p.nb2 > 1) {
+        if (p.a_b1 % 8 || p.a_b2 % 8 || p.b_b1 % 8 || p.b_b2 % 8) return false;
+        if (p.a_b1 < 0 || p.a_b2 < 0 || p.b_b1 < 0 || p.b_b2 < 0) return false;
+    }
+    const int64_t tiles = ((p.m + v.bm - 1) / v.bm) * ((p.n + v.bn - 1) / v.bn);
+    const int64_t blocks = tiles * (p.reduce ? 1 : p.nb1 * p.nb2);
+    if (blocks >= (1ll << 31) || p.nb1 * p.nb2 >= (1ll << 31)) return false;
+    if (p.k * (p.reduce ? p.nb1 * p.nb2 : 1) >= (1ll << 31)) return false;
+    return true;
+}
+
+int mfma16dma_pick_variant(const GemmProblem &p, int compute_units) {
+    // Largest tile that still gives every compute unit a workgroup; BN = 64 tiles only for narrow outputs.
+    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+    const int wide[] = {1, 2, 3}, narrow[] = {4, 5};
+    if (p.n <= 64) {
+        for (int v : narrow) {
+            if (!mfma16dma_supported(p, v)) continue;
+            const Variant &t = kVariants[v - 1];
+            const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
+            if (blocks >= compute_units || v == 5) return v;
+        }
+        return 0;
+    }
+    for (int v : wide) {
+        if (!mfma16dma_supported(p, v)) continue;
+        const Variant &t = kVariants[v - 1];
+        const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
+        if (blocks >= compute_units || v == 3) return v;
+    }
+    return 0;
+}
+
+hipError_t launch_mfma16dma(const GemmProblem &g, int variant, hipStream_t stream) {
+    if (!mfma16dma_supported(g, variant)) return hipErrorInvalidValue;
+    const Variant &v = kVariants[variant - 1];
+    const OperandLayout la = classify(g.m, g.k, g.a_rs, g.a_cs);
+    const OperandLayout lb = classify(g.n, g.k, g.b_cs, g.b_rs);
+    Params p;
+    p.a = (const uint16_t *)g.a; p.b = (const uint16_t *)g.b; p.c = (uint16_t *)g.c; p.bias = (const uint16_t *)g.bias;
+    p.m = (int)g.m; p.n = (int)g.n; p.k = (int)g.k;
+    p.lda = (int)la.ld; p.ldb = (int)lb.ld;
+    p.ldc = g.m == 1 ? g.n : g.c_rs;
+    p.a_b1 = g.a_b1; p.a_b2 = g.a_b2; p.b_b1 = g.b_b1; p.b_b2 = g.b_b2; p.c_b1 = g.c_b1; p.c_b2 = g.c_b2;
+    p.nb2 = (int)g.nb2;
+    const int nbatch = (int)(g.nb1 * g.nb2);
+    p.kbatches = g.reduce ? nbatch : 1;
+    p.tiles_m = (int)((g.m + v.bm - 1) / v.bm);
+    p.tiles_n = (int)((g.n + v.bn - 1) / v.bn);
+    p.tiles_per_batch = p.tiles_m * p.tiles_n;
+    p.total_blocks = p.tiles_per_batch * (g.reduce ? 1 : nbatch);
+    p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
+    p.c_vec = (g.n % 4 == 0) && (p.ldc % 4 == 0) && (((uintptr_t)g.c & 7u) == 0) &&
+              (g.c_b1 % 4 == 0) && (g.c_b2 % 4 == 0) && (!g.bias || ((uintptr_t)g.bias & 7u) == 0);
+    p.group_m = 4;
+    if (g.dtype == DT_F16) return launch_variant<_Float16>(variant, p, la.kc, lb.kc, stream);
+    return launch_variant<__bf16>(variant, p, la.kc, lb.kc, stream);
+}
+
+}  // namespace dfdx_rocm

@@ -16,6 +16,7 @@ from gpu_util import announce, device, make_operand, values
 
 pytestmark = pytest.mark.gpu
 
+from dfdx_amd import RocmError  # noqa: E402
 from dfdx_amd.rocm import KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA  # noqa: E402
 
 LAYOUTS = {"nn": (False, False), "tn": (True, False), "nt": (False, True), "tt": (True, True)}
@@ -116,7 +117,7 @@ def test_aliased_output_is_rejected():
 
 
 # --------------------------------------------------------------------- MFMA --
-MFMA_SHAPES = [(200, 136, 264), (512, 256, 256), (96, 72, 40)]
+MFMA_SHAPES = [(200, 136, 264), (512, 256, 256), (96, 72, 40), (264, 192, 200), (72, 64, 136), (520, 128, 72)]
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
@@ -125,8 +126,15 @@ MFMA_SHAPES = [(200, 136, 264), (512, 256, 256), (96, 72, 40)]
 def test_mfma_variants(dtype, variant, layout):
     if variant > device().mfma_variant_count(dtype):
         pytest.skip("no such tile variant for this dtype")
+    ran = 0
     for i, (m, k, n) in enumerate(MFMA_SHAPES):
-        run_case(dtype, m, k, n, layout, bool(i % 2), KERNEL_MFMA, variant, seed=10 + i, pads=(8, 16, 8))
+        try:
+            run_case(dtype, m, k, n, layout, bool(i % 2), KERNEL_MFMA, variant, seed=10 + i, pads=(8, 16, 8))
+            ran += 1
+        except RocmError as e:   # a variant may not serve a shape (the LDS-DMA kernels need K % 64 == 0)
+            if e.code != -2:
+                raise
+    assert ran >= 2
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
