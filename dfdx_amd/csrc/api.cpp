@@ -16,6 +16,8 @@ struct dfdx_rocm_ctx {
     int clock_mhz;
     char name[128];
     std::mutex mu;
+    void *workspace = nullptr;  // split-k partial sums; grown on demand, owned by the context
+    size_t workspace_bytes = 0;
 };
 
 namespace {
@@ -59,6 +61,8 @@ int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
     p.c = d->c; p.c_rs = d->c_rs; p.c_cs = d->c_cs;
     p.c_b1 = p.reduce ? 0 : d->c_b1; p.c_b2 = p.reduce ? 0 : d->c_b2;
     p.bias = d->bias;
+    p.splits = 1;
+    p.workspace = nullptr;
     // column-major C (a permuted operand's gradient): compute C^T = B^T A^T instead
     if (p.c_cs != 1 && p.c_rs == 1 && p.n > 1) p = transposed(p);
     *out = p;
@@ -66,26 +70,53 @@ int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
 }
 
 struct Plan {
-    int kernel, variant;
+    int kernel, variant, splits;
 };
+
+// Grows the context's workspace; pending work that may still use the old one is drained first.
+int ensure_workspace(dfdx_rocm_ctx *ctx, size_t bytes) {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (bytes <= ctx->workspace_bytes) return DFDX_ROCM_OK;
+    if (ctx->workspace) {
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+        HIP_TRY(hipFree(ctx->workspace));
+        ctx->workspace = nullptr;
+        ctx->workspace_bytes = 0;
+    }
+    bytes = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    HIP_TRY(hipMalloc(&ctx->workspace, bytes));
+    ctx->workspace_bytes = bytes;
+    return DFDX_ROCM_OK;
+}
 
 int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProblem &p, Plan *plan) {
     const bool is16 = p.dtype == DT_F16 || p.dtype == DT_BF16;
     const bool is32 = p.dtype == DT_F32;
+    // split-k: 1 = never (NO_SPLIT_K), n = forced by the caller, 0 = let the planner decide
+    const int forced_splits = (d->flags & DFDX_ROCM_GEMM_NO_SPLIT_K) ? 1 : ((d->flags >> 8) & 0xff);
     switch (d->kernel) {
     case DFDX_ROCM_KERNEL_GENERIC:
-        *plan = {DFDX_ROCM_KERNEL_GENERIC, 0};
+        *plan = {DFDX_ROCM_KERNEL_GENERIC, 0, 1};
         return DFDX_ROCM_OK;
     case DFDX_ROCM_KERNEL_GEMV:
         if (!gemv_supported(p)) return DFDX_ROCM_ERR_UNSUPPORTED;
-        *plan = {DFDX_ROCM_KERNEL_GEMV, 0};
+        *plan = {DFDX_ROCM_KERNEL_GEMV, 0, 1};
         return DFDX_ROCM_OK;
     case DFDX_ROCM_KERNEL_MFMA: {
         int v = d->variant;
+        if (is16 && (v == 0 || v >= mfma16_dma_first_variant())) {  // LDS-DMA family: tile and split count together
+            int dv = 0, splits = 1;
+            mfma16dma_plan_split(p, ctx->compute_units, v ? v - mfma16_dma_first_variant() + 1 : 0, forced_splits, &dv, &splits);
+            if (dv) {
+                *plan = {DFDX_ROCM_KERNEL_MFMA, dv + mfma16_dma_first_variant() - 1, splits};
+                return DFDX_ROCM_OK;
+            }
+            if (v) return DFDX_ROCM_ERR_UNSUPPORTED;
+        }
         if (v == 0) v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units) : 0;
         const bool ok = is16 ? mfma16_supported(p, v) : is32 ? mfma32_supported(p, v) : false;
         if (!ok) return DFDX_ROCM_ERR_UNSUPPORTED;
-        *plan = {DFDX_ROCM_KERNEL_MFMA, v};
+        *plan = {DFDX_ROCM_KERNEL_MFMA, v, 1};
         return DFDX_ROCM_OK;
     }
     case DFDX_ROCM_KERNEL_AUTO:
@@ -94,19 +125,36 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
         return DFDX_ROCM_ERR_INVALID_ARG;
     }
     if (gemv_supported(p)) {
-        *plan = {DFDX_ROCM_KERNEL_GEMV, 0};
+        *plan = {DFDX_ROCM_KERNEL_GEMV, 0, 1};
         return DFDX_ROCM_OK;
+    }
+    if (is16) {
+        int dv = 0, splits = 1;
+        mfma16dma_plan_split(p, ctx->compute_units, 0, forced_splits, &dv, &splits);
+        if (dv) {
+            *plan = {DFDX_ROCM_KERNEL_MFMA, dv + mfma16_dma_first_variant() - 1, splits};
+            return DFDX_ROCM_OK;
+        }
     }
     int v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units) : 0;
     if (v > 0) {
-        *plan = {DFDX_ROCM_KERNEL_MFMA, v};
+        *plan = {DFDX_ROCM_KERNEL_MFMA, v, 1};
         return DFDX_ROCM_OK;
     }
-    *plan = {DFDX_ROCM_KERNEL_GENERIC, 0};
+    *plan = {DFDX_ROCM_KERNEL_GENERIC, 0, 1};
     return DFDX_ROCM_OK;
 }
 
-int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &p, const Plan &plan) {
+int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan) {
+    GemmProblem p = problem;
+    p.splits = 1;
+    p.workspace = nullptr;
+    if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1) {
+        const size_t need = mfma16dma_workspace_bytes(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
+        if (int rc = ensure_workspace(ctx, need)) return rc;
+        p.splits = plan.splits;
+        p.workspace = (float *)ctx->workspace;
+    }
     hipError_t e;
     switch (plan.kernel) {
     case DFDX_ROCM_KERNEL_GENERIC: e = launch_generic(p, ctx->stream); break;
@@ -145,6 +193,11 @@ int dfdx_rocm_create(int ordinal, void *stream, dfdx_rocm_ctx **out) {
 
 int dfdx_rocm_destroy(dfdx_rocm_ctx *ctx) {
     if (!ctx) return DFDX_ROCM_OK;
+    if (ctx->workspace) {
+        (void)hipSetDevice(ctx->device);
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipFree(ctx->workspace);
+    }
     delete ctx;
     return DFDX_ROCM_OK;
 }
@@ -251,13 +304,15 @@ int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int
     if (!ctx) return DFDX_ROCM_ERR_INVALID_ARG;
     GemmProblem p;
     if (int e = make_problem(desc, &p)) return e;
-    Plan plan = {DFDX_ROCM_KERNEL_GENERIC, 0};
+    Plan plan = {DFDX_ROCM_KERNEL_GENERIC, 0, 1};
     if (p.m != 0)
         if (int e = make_plan(ctx, desc, p, &plan)) return e;
     if (kernel) *kernel = plan.kernel;
     if (variant) *variant = plan.variant;
     if (name && name_len) {
-        if (plan.kernel == DFDX_ROCM_KERNEL_MFMA)
+        if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1)
+            std::snprintf(name, name_len, "mfma16_%s_splitk%d", mfma16_variant_name(plan.variant), plan.splits);
+        else if (plan.kernel == DFDX_ROCM_KERNEL_MFMA)
             std::snprintf(name, name_len, "%s_%s", p.dtype == DT_F32 ? "mfma32" : "mfma16",
                           p.dtype == DT_F32 ? mfma32_variant_name(plan.variant) : mfma16_variant_name(plan.variant));
         else

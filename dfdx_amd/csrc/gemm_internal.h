@@ -24,6 +24,9 @@ struct GemmProblem {
     void *c;
     int64_t c_rs, c_cs, c_b1, c_b2;
     const void *bias;
+    // split-k (filled in by the planner): `splits` workgroups share one C tile; f32 partials go to `workspace`
+    int splits;
+    float *workspace;
 };
 
 static inline size_t dtype_size(int dt) { return dt == DT_F32 ? 4 : (dt == DT_F64 ? 8 : 2); }
@@ -49,6 +52,7 @@ int mfma16_variant_count();
 const char *mfma16_variant_name(int variant);
 bool mfma16_supported(const GemmProblem &p, int variant);
 int mfma16_pick_variant(const GemmProblem &p, int compute_units);
+int mfma16_dma_first_variant();  // variant ids >= this are the LDS-DMA kernels
 hipError_t launch_mfma16(const GemmProblem &p, int variant, hipStream_t stream);
 
 // ---- LDS-DMA MFMA kernels for 16-bit inputs, K % 64 == 0 (gemm_mfma16_dma.hip) ----
@@ -58,6 +62,14 @@ const char *mfma16dma_variant_name(int variant);
 bool mfma16dma_supported(const GemmProblem &p, int variant);
 int mfma16dma_pick_variant(const GemmProblem &p, int compute_units);
 hipError_t launch_mfma16dma(const GemmProblem &p, int variant, hipStream_t stream);
+// Split-k planning for the LDS-DMA kernels: picks tile variant and split count together.  `forced_splits`
+// > 0 overrides the count (clamped to what the k extent allows).  Returns the workspace bytes needed.
+void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_variant, int forced_splits, int *variant,
+                          int *splits);
+size_t mfma16dma_workspace_bytes(const GemmProblem &p, int variant, int splits);
+
+// ---- split-k combine (splitk_reduce.hip): C = (accumulate ? C : 0) + bias + sum_s partial[s], s ascending ----
+hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_split_stride, hipStream_t stream);
 
 // ---- MFMA kernels for f32 (gemm_mfma32.hip) ----
 int mfma32_variant_count();

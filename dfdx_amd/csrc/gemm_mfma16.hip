@@ -452,6 +452,8 @@ bool mfma16_supported(const GemmProblem &p, int variant) {
     return true;
 }
 
+int mfma16_dma_first_variant() { return kNumVariants + 1; }
+
 int mfma16_pick_variant(const GemmProblem &p, int compute_units) {
     if (const int d = mfma16dma_pick_variant(p, compute_units)) return kNumVariants + d;
     // Largest tile that still gives every compute unit at least one workgroup; ties go to the larger tile.

@@ -21,6 +21,7 @@
 // Rows/columns past the matrix edge are clamped onto valid addresses (they only feed C entries that are
 // never stored).  There is no k tail here: K % 64 != 0 is served by the register-staged kernel.
 #include "gemm_internal.h"
+#include <algorithm>
 #include <type_traits>
 
 namespace dfdx_rocm {
@@ -51,6 +52,10 @@ struct Params {
     int tiles_m, tiles_n, tiles_per_batch, total_blocks;
     int accumulate, bias_mode, c_vec;
     int group_m;
+    // split-k: `splits` workgroups per C tile, each covering `chunk` k-loop steps, f32 partials in `ws`
+    int splits, chunk;
+    float *ws;
+    int64_t ws_ld, ws_split_stride;
 };
 
 template <typename T> struct Mma;
@@ -142,7 +147,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
     const int bm0 = tm_idx * BM, bn0 = tn_idx * BN;
 
     const int ktiles = p.k / BK;
-    const int iters = ktiles * p.kbatches;
+    // k-loop steps run over (batch, k-tile) pairs; with split-k this workgroup owns steps [it0, it0 + iters)
+    const int split = p.splits > 1 ? batch : 0;
+    const int it0 = split * p.chunk;
+    const int iters = min(ktiles * p.kbatches - it0, p.chunk);
 
     // ---- global side: origin of the next tile to request -------------------
     auto a_origin = [&](int kb) -> const uint16_t * {
@@ -155,10 +163,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
     };
     const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
     const int64_t b_step = B_KC ? BK : (int64_t)BK * p.ldb;
-    int f_kb = p.kbatches > 1 ? 0 : batch;
-    int f_kt = 0;
-    const uint16_t *a_next = a_origin(f_kb);
-    const uint16_t *b_next = b_origin(f_kb);
+    int f_kb = p.kbatches > 1 ? it0 / ktiles : (p.splits > 1 ? 0 : batch);
+    int f_kt = p.kbatches > 1 ? it0 % ktiles : it0;
+    const uint16_t *a_next = a_origin(f_kb) + f_kt * a_step;
+    const uint16_t *b_next = b_origin(f_kb) + f_kt * b_step;
     TA ta;
     TB tb;
     ta.init(p.lda, p.m - bm0, wave, lane);
@@ -294,6 +302,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
     if (iters > 0) tile_body(iters - 1, std::false_type{});
 
     // ---- epilogue: lane holds m = l16 (per tile), n = 4*lq + 0..3 -------------
+    if (p.splits > 1) {  // f32 partial tile into the workspace (padded to whole tiles: no bounds checks)
+        float *wbase = p.ws + split * p.ws_split_stride;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            float *wrow = wbase + (int64_t)(bm0 + wm0 + i * 16 + l16) * p.ws_ld + bn0 + wn0 + lq * 4;
+#pragma unroll
+            for (int j = 0; j < TN; j++) *(f32x4 *)(wrow + j * 16) = acc[i][j];
+        }
+        return;
+    }
     const int cb = p.kbatches > 1 ? 0 : batch;
     uint16_t *cbase = p.c + (int64_t)(cb / p.nb2) * p.c_b1 + (int64_t)(cb % p.nb2) * p.c_b2;
 #pragma unroll
@@ -466,6 +484,58 @@ int mfma16dma_pick_variant(const GemmProblem &p, int compute_units) {
     return 0;
 }
 
+namespace {
+// relative per-CU efficiency of each tile variant (measured at 4096^3 / on the config shapes)
+constexpr double kTileEff[] = {1.0, 0.85, 0.70, 0.60, 0.45};
+}  // namespace
+
+void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_variant, int forced_splits, int *variant,
+                          int *splits) {
+    *variant = 0;
+    *splits = 1;
+    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+    const bool may_split = nbatch == 1 && p.c_cs == 1;
+    const int64_t total_iters = (p.k / BK) * (p.reduce ? p.nb1 * p.nb2 : 1);
+    double best = 1e300;
+    for (int v = 1; v <= kNumVariants; v++) {
+        if (forced_variant > 0 && v != forced_variant) continue;
+        if (!mfma16dma_supported(p, v)) continue;
+        const Variant &t = kVariants[v - 1];
+        if (forced_variant == 0 && ((p.n <= 64) != (t.bn <= 64))) continue;  // BN = 64 tiles only for narrow outputs
+        const int64_t tiles = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
+        const double rate = 4.0e12 * kTileEff[v - 1];  // flop/s of one CU on this tile shape
+        for (int s = 1; s <= 16; s++) {
+            if (forced_splits > 0 && s != std::min<int64_t>(forced_splits, total_iters)) continue;
+            if (s > 1 && (!may_split || (forced_splits == 0 && total_iters / s < 4))) break;
+            const int64_t chunk = (total_iters + s - 1) / s;
+            if ((s - 1) * chunk >= total_iters) continue;  // an empty split
+            const int64_t blocks = tiles * s;
+            const int64_t rounds = (blocks + compute_units - 1) / compute_units;
+            double time = rounds * (chunk * (2.0 * t.bm * t.bn * BK / rate) + 3e-6);
+            if (s > 1) time += 4e-6 + 2.0 * s * (double)p.m * p.n * 4.0 / 3e12;
+            if (time < best) {
+                best = time;
+                *variant = v;
+                *splits = s;
+            }
+        }
+    }
+}
+
+// layout of the split-k workspace: [splits][tiles_m * BM][tiles_n * BN] f32
+static void ws_layout(const GemmProblem &p, int variant, int64_t *ld, int64_t *split_stride) {
+    const Variant &v = kVariants[variant - 1];
+    *ld = ((p.n + v.bn - 1) / v.bn) * v.bn;
+    *split_stride = *ld * (((p.m + v.bm - 1) / v.bm) * v.bm);
+}
+
+size_t mfma16dma_workspace_bytes(const GemmProblem &p, int variant, int splits) {
+    if (splits <= 1) return 0;
+    int64_t ld, stride;
+    ws_layout(p, variant, &ld, &stride);
+    return (size_t)stride * splits * sizeof(float);
+}
+
 hipError_t launch_mfma16dma(const GemmProblem &g, int variant, hipStream_t stream) {
     if (!mfma16dma_supported(g, variant)) return hipErrorInvalidValue;
     const Variant &v = kVariants[variant - 1];
@@ -488,8 +558,21 @@ hipError_t launch_mfma16dma(const GemmProblem &g, int variant, hipStream_t strea
     p.c_vec = (g.n % 4 == 0) && (p.ldc % 4 == 0) && (((uintptr_t)g.c & 7u) == 0) &&
               (g.c_b1 % 4 == 0) && (g.c_b2 % 4 == 0) && (!g.bias || ((uintptr_t)g.bias & 7u) == 0);
     p.group_m = 4;
-    if (g.dtype == DT_F16) return launch_variant<_Float16>(variant, p, la.kc, lb.kc, stream);
-    return launch_variant<__bf16>(variant, p, la.kc, lb.kc, stream);
+    const int total_iters = (p.k / BK) * p.kbatches;
+    p.splits = 1; p.chunk = total_iters; p.ws = nullptr; p.ws_ld = 0; p.ws_split_stride = 0;
+    if (g.splits > 1) {
+        if (!g.workspace || p.total_blocks != p.tiles_per_batch) return hipErrorInvalidValue;
+        p.splits = g.splits;
+        p.chunk = (total_iters + g.splits - 1) / g.splits;
+        if ((int64_t)(g.splits - 1) * p.chunk >= total_iters) return hipErrorInvalidValue;
+        p.ws = g.workspace;
+        ws_layout(g, variant, &p.ws_ld, &p.ws_split_stride);
+        p.total_blocks = p.tiles_per_batch * g.splits;
+    }
+    hipError_t e = (g.dtype == DT_F16) ? launch_variant<_Float16>(variant, p, la.kc, lb.kc, stream)
+                                       : launch_variant<__bf16>(variant, p, la.kc, lb.kc, stream);
+    if (e != hipSuccess || g.splits <= 1) return e;
+    return launch_splitk_reduce(g, p.ws_ld, p.ws_split_stride, stream);
 }
 
 }  // namespace dfdx_rocm

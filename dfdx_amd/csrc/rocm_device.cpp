@@ -80,6 +80,7 @@ int dfdx_rocm_matmat_br_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t batch, in
     }
     d.b = rhs; d.b_rs = rs[0]; d.b_cs = rs[1];  // batch stride 0: shared by every batch
     d.c = out; d.c_rs = n; d.c_cs = 1;
+    d.flags = DFDX_ROCM_GEMM_NO_SPLIT_K;  // same k order as the batched kernels: Br == Batch3 bit for bit (mod.rs:467-472)
     return dfdx_rocm_gemm(ctx, &d);
 }
 
@@ -93,6 +94,7 @@ int dfdx_rocm_matmat_br_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t batch, i
     // grad_lhs[i] (m,k) += grad_out[i] (m,n) . rhs^T (n,k)
     dfdx_rocm_gemm_desc d = blank(dtype, fold ? batch * m : m, n, k);
     d.accumulate = 1;
+    d.flags = DFDX_ROCM_GEMM_NO_SPLIT_K;  // grad_lhs must equal the Batch3 result bit for bit (mod.rs:471)
     d.a = grad_out; d.a_rs = n; d.a_cs = 1;
     d.b = rhs; d.b_rs = rs[1]; d.b_cs = rs[0];
     d.c = grad_lhs; d.c_rs = ls[1]; d.c_cs = ls[2];

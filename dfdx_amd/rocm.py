@@ -50,7 +50,7 @@ class GemmDesc(ctypes.Structure):
         ("c_b1", ctypes.c_int64), ("c_b2", ctypes.c_int64),
         ("bias", ctypes.c_void_p),
         ("reduce_batch", ctypes.c_int32), ("kernel", ctypes.c_int32),
-        ("variant", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("variant", ctypes.c_int32), ("flags", ctypes.c_int32),
     ]
 
 
@@ -204,7 +204,7 @@ class Rocm:
     # ------------------------------------------------------------------ gemm --
     def gemm_desc(self, dtype, m, k, n, a, a_strides, b, b_strides, c, c_strides, accumulate=False,
                   batch=(1, 1), a_batch=(0, 0), b_batch=(0, 0), c_batch=(0, 0), bias=None, reduce_batch=False,
-                  kernel=KERNEL_AUTO, variant=0) -> GemmDesc:
+                  kernel=KERNEL_AUTO, variant=0, no_split_k=False, split_k=0) -> GemmDesc:
         d = GemmDesc()
         d.dtype, d.accumulate = DTYPES[dtype], int(bool(accumulate))
         d.m, d.n, d.k = m, n, k
@@ -214,6 +214,7 @@ class Rocm:
         d.c, d.c_rs, d.c_cs, d.c_b1, d.c_b2 = c, c_strides[0], c_strides[1], c_batch[0], c_batch[1]
         d.bias = bias
         d.reduce_batch, d.kernel, d.variant = int(bool(reduce_batch)), kernel, variant
+        d.flags = (1 if no_split_k else 0) | ((split_k & 0xff) << 8)
         return d
 
     def gemm(self, desc: GemmDesc):

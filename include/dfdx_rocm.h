@@ -116,8 +116,16 @@ typedef struct dfdx_rocm_gemm_desc {
     int32_t reduce_batch;
     int32_t kernel;  /* DFDX_ROCM_KERNEL_* ; 0 = automatic */
     int32_t variant; /* tile variant inside the family; 0 = automatic */
-    int32_t reserved;
+    int32_t flags;   /* DFDX_ROCM_GEMM_* bits below; 0 = defaults */
 } dfdx_rocm_gemm_desc;
+
+/* flags.  Long contractions with few output tiles (weight gradients) are split along k over several
+ * workgroups whose f32 partial sums are combined in a fixed order (deterministic).  NO_SPLIT_K keeps the
+ * plain k-ascending order; the broadcast-rhs forward / grad_lhs use it so that they stay bit-identical to
+ * the batched kernels (dfdx tests assert that equality, matmul/mod.rs:467-472).  SPLIT_K(n) forces n
+ * splits (testing / tuning). */
+#define DFDX_ROCM_GEMM_NO_SPLIT_K 1
+#define DFDX_ROCM_GEMM_SPLIT_K(n) (((n) & 0xff) << 8)
 
 int dfdx_rocm_gemm(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc);
 

@@ -22,7 +22,8 @@ from dfdx_amd.rocm import KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA  # noqa: E402
 LAYOUTS = {"nn": (False, False), "tn": (True, False), "nt": (False, True), "tt": (True, True)}
 
 
-def run_case(dtype, m, k, n, layout, accumulate, kernel, variant, c_colmajor=False, bias=False, seed=1, pads=(0, 0, 0)):
+def run_case(dtype, m, k, n, layout, accumulate, kernel, variant, c_colmajor=False, bias=False, seed=1, pads=(0, 0, 0),
+             split_k=0):
     dev = device()
     g = rng(seed)
     at, bt = LAYOUTS[layout]
@@ -35,7 +36,7 @@ def run_case(dtype, m, k, n, layout, accumulate, kernel, variant, c_colmajor=Fal
     da, db, dc = dev.tensor(a, dtype), dev.tensor(b, dtype), dev.tensor(c, dtype)
     dbias = dev.tensor(bias_st, dtype) if bias else None
     desc = dev.gemm_desc(dtype, m, k, n, da.ptr, astr, db.ptr, bstr, dc.ptr, cstr, accumulate=accumulate,
-                         bias=dbias.ptr if bias else None, kernel=kernel, variant=variant)
+                         bias=dbias.ptr if bias else None, kernel=kernel, variant=variant, split_k=split_k)
     announce("gemm", dtype, (m, k, n), layout, "acc" if accumulate else "ovw", "kernel", kernel, "variant", variant,
              "ccol" if c_colmajor else "crow", "bias" if bias else "", dev.gemm_plan(desc)[2])
     dev.gemm(desc)
@@ -179,6 +180,43 @@ def test_auto_dispatch_prefers_mfma_when_aligned():
     assert dev.gemm_plan(d)[0] == KERNEL_GENERIC
 
 
+# ------------------------------------------------------------------ split-k --
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("layout", ["tn", "nt", "nn"])
+@pytest.mark.parametrize("splits", [2, 3, 8])
+def test_split_k_forced(dtype, layout, splits):
+    """k split over several workgroups, f32 partials combined in a fixed order; with beta = 1, bias, ragged edges."""
+    run_case(dtype, 264, 1024, 200, layout, True, KERNEL_MFMA, 0, split_k=splits, pads=(8, 8, 8))
+    run_case(dtype, 136, 512, 72, layout, False, KERNEL_MFMA, 0, split_k=splits, bias=True)
+    run_case(dtype, 264, 576, 136, layout, True, KERNEL_MFMA, 0, split_k=splits, c_colmajor=True)
+
+
+def test_split_k_is_planned_for_weight_gradients_and_is_deterministic():
+    dev = device()
+    g = rng(77)
+    m, k, n, dtype = 512, 8192, 512, "f16"      # dW-shaped: few output tiles, long contraction
+    a = oracle.to_storage(g.standard_normal(k * m), dtype)      # stored (k, m): the transposed lhs of a weight gradient
+    b = oracle.to_storage(g.standard_normal(k * n), dtype)
+    c0 = oracle.to_storage(g.standard_normal(m * n), dtype)
+    da, db = dev.tensor(a, dtype), dev.tensor(b, dtype)
+    outs = []
+    for _ in range(2):
+        dc = dev.tensor(c0, dtype)
+        desc = dev.gemm_desc(dtype, m, k, n, da.ptr, (1, m), db.ptr, (n, 1), dc.ptr, (n, 1), accumulate=True)
+        name = dev.gemm_plan(desc)[2]
+        assert "splitk" in name, name
+        announce("planned split-k", name)
+        dev.gemm(desc)
+        outs.append(dev.to_host(dc))
+    assert np.array_equal(outs[0], outs[1])
+    A, B = oracle.to_f64(a, dtype).reshape(k, m).T, oracle.to_f64(b, dtype).reshape(k, n)
+    want = A @ B + oracle.to_f64(c0, dtype).reshape(m, n)
+    assert_within(dtype, k, oracle.to_f64(outs[0], dtype).reshape(m, n), want, A, B, extra=2.0 ** -11 * np.abs(want).max())
+    # NO_SPLIT_K keeps the plain kernel
+    desc = dev.gemm_desc(dtype, m, k, n, da.ptr, (1, m), db.ptr, (n, 1), dc.ptr, (n, 1), accumulate=True, no_split_k=True)
+    assert "splitk" not in dev.gemm_plan(desc)[2]
+
+
 # ------------------------------------------------------------------ batched --
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("kernel", [KERNEL_GENERIC, KERNEL_MFMA])
@@ -207,7 +245,8 @@ def test_batched_and_reduce(dtype, kernel):
     gacc = oracle.to_storage(g.standard_normal(k * n), dtype)
     dd, dg = dev.tensor(dmat, dtype), dev.tensor(gacc, dtype)
     desc = dev.gemm_desc(dtype, k, m, n, da.ptr, (a_cs, a_rs), dd.ptr, (n, 1), dg.ptr, (n, 1), accumulate=True,
-                         batch=(b1, b2), a_batch=(a_b1, a_b2), b_batch=(b2 * m * n, m * n), reduce_batch=True, kernel=kernel)
+                         batch=(b1, b2), a_batch=(a_b1, a_b2), b_batch=(b2 * m * n, m * n), reduce_batch=True, kernel=kernel,
+                         split_k=3 if (kernel == KERNEL_MFMA and dtype == "f16") else 0)
     announce("reduce", dtype, kernel, dev.gemm_plan(desc)[2])
     dev.gemm(desc)
     D = oracle.to_f64(dmat, dtype).reshape(b1, b2, m, n)
