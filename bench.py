@@ -27,6 +27,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--probe", action="store_true",
+                    help="counter-collection aid: 3 plain 256 MiB device copies, then 5 headline GEMM launches, nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -38,6 +40,22 @@ def main():
 
     dev = Rocm(0)
     info = dev.device_info()
+    if args.probe:   # for `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`: a copy of known size calibrates the counters
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        a = (torch.rand(N, N, device="cuda") * 2 - 1).half()
+        b = (torch.rand(N, N, device="cuda") * 2 - 1).half()
+        c = torch.zeros(N, N, device="cuda", dtype=torch.float16)
+        desc = dev.gemm_desc("f16", N, N, N, a.data_ptr(), (N, 1), b.data_ptr(), (N, 1), c.data_ptr(), (N, 1))
+        torch.cuda.synchronize()
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            dev.gemm(desc)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "3 x 256 MiB copy, 5 x " + dev.gemm_plan(desc)[2]}))
+        return
     flop = 2.0 * N ** 3
     tdt = {"f16": torch.float16, "f32": torch.float32}
     res = {}
