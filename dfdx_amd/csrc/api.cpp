@@ -155,6 +155,12 @@ int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan) {
         p.splits = plan.splits;
         p.workspace = (float *)ctx->workspace;
     }
+    if (plan.kernel == DFDX_ROCM_KERNEL_GEMV) {
+        if (const size_t need = gemv_workspace_bytes(p)) {
+            if (int rc = ensure_workspace(ctx, need)) return rc;
+            p.workspace = (float *)ctx->workspace;
+        }
+    }
     hipError_t e;
     switch (plan.kernel) {
     case DFDX_ROCM_KERNEL_GENERIC: e = launch_generic(p, ctx->stream); break;

@@ -80,6 +80,7 @@ hipError_t launch_mfma32(const GemmProblem &p, int variant, hipStream_t stream);
 
 // ---- bandwidth-bound vector products (gemv.hip) ----
 bool gemv_supported(const GemmProblem &p);
+size_t gemv_workspace_bytes(const GemmProblem &p);  // f32 partial sums of the k slices (0 when not sliced)
 hipError_t launch_gemv(const GemmProblem &p, hipStream_t stream);
 
 // XCD-aware remap of a linear workgroup id: consecutive ids are dispatched round-robin

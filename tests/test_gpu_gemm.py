@@ -180,6 +180,25 @@ def test_auto_dispatch_prefers_mfma_when_aligned():
     assert dev.gemm_plan(d)[0] == KERNEL_GENERIC
 
 
+# --------------------------------------------------------------------- gemv --
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (1, 520, 264), (1, 8200, 64), (4096, 4096, 1), (264, 520, 1), (72, 16384, 1)])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn"])
+def test_gemv(dtype, shape, layout):
+    """vec.mat (M = 1) and mat.vec (N = 1): the bandwidth-bound kernels, both matrix layouts, beta = 0 / 1, bias."""
+    from dfdx_amd.rocm import KERNEL_GEMV
+    m, k, n = shape
+    dev = device()
+    a = dev.zeros(dtype, (max(m, k), max(m, k)))
+    at, bt = LAYOUTS[layout]
+    astr = (1, m) if at else (k, 1)
+    bstr = (1, k) if bt else (n, 1)
+    plan = dev.gemm_plan(dev.gemm_desc(dtype, m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1)))
+    assert plan[0] == KERNEL_GEMV, plan
+    run_case(dtype, m, k, n, layout, False, KERNEL_AUTO, 0, seed=3)
+    run_case(dtype, m, k, n, layout, True, KERNEL_AUTO, 0, seed=4, bias=(dtype == "f32"))
+
+
 # ------------------------------------------------------------------ split-k --
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("layout", ["tn", "nt", "nn"])
