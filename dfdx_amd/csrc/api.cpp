@@ -63,6 +63,7 @@ int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
     p.bias = d->bias;
     p.splits = 1;
     p.workspace = nullptr;
+    p.compute_units = 0;
     // column-major C (a permuted operand's gradient): compute C^T = B^T A^T instead
     if (p.c_cs != 1 && p.c_rs == 1 && p.n > 1) p = transposed(p);
     *out = p;
@@ -149,6 +150,7 @@ int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan) {
     GemmProblem p = problem;
     p.splits = 1;
     p.workspace = nullptr;
+    p.compute_units = ctx->compute_units;
     if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1) {
         const size_t need = mfma16dma_workspace_bytes(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
         if (int rc = ensure_workspace(ctx, need)) return rc;

@@ -27,6 +27,7 @@ struct GemmProblem {
     // split-k (filled in by the planner): `splits` workgroups share one C tile; f32 partials go to `workspace`
     int splits;
     float *workspace;
+    int compute_units;  // of the device the launch goes to (persistent kernels size their grid with it)
 };
 
 static inline size_t dtype_size(int dt) { return dt == DT_F32 ? 4 : (dt == DT_F64 ? 8 : 2); }

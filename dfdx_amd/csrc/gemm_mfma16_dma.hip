@@ -50,10 +50,11 @@ struct Params {
     int64_t a_b1, a_b2, b_b1, b_b2, c_b1, c_b2;
     int nb2, kbatches;
     int tiles_m, tiles_n, tiles_per_batch, total_blocks;
-    int accumulate, bias_mode, c_vec;
+    int accumulate, bias_mode, c_vec, c_vec8;
     int group_m;
     // split-k: `splits` workgroups per C tile, each covering `chunk` k-loop steps, f32 partials in `ws`
     int splits, chunk;
+    int grid;  // workgroups launched (<= total_blocks: each walks blockIdx.x, blockIdx.x + grid, ...)
     float *ws;
     int64_t ws_ld, ws_split_stride;
 };
@@ -134,55 +135,82 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
     const int wm0 = (wave / WAVES_N) * WTM, wn0 = (wave % WAVES_N) * WTN;
     const int l16 = lane % 16, lq = lane / 16;
 
-    // ---- which tile -------------------------------------------------------
-    const int work = xcd_remap(blockIdx.x, p.total_blocks);
-    const int batch = work / p.tiles_per_batch;
-    const int tile = work % p.tiles_per_batch;
-    const int gsize = p.group_m * p.tiles_n;
-    const int group = tile / gsize;
-    const int first_m = group * p.group_m;
-    const int gm = min(p.tiles_m - first_m, p.group_m);
-    const int tm_idx = first_m + (tile % gsize) % gm;
-    const int tn_idx = (tile % gsize) / gm;
-    const int bm0 = tm_idx * BM, bn0 = tn_idx * BN;
-
+    // ---- work items ---------------------------------------------------------
+    // A work item is one C tile (of one batch, or of one k split).  The workgroup is persistent: it walks the
+    // work items blockIdx.x, blockIdx.x + gridDim.x, ... and keeps ONE load pipeline running across them, so
+    // the stores of a finished tile overlap with the loads (already in flight) and MFMAs of the next one.
+    struct Work {
+        int batch, split, bm0, bn0, it0, iters;
+    };
     const int ktiles = p.k / BK;
-    // k-loop steps run over (batch, k-tile) pairs; with split-k this workgroup owns steps [it0, it0 + iters)
-    const int split = p.splits > 1 ? batch : 0;
-    const int it0 = split * p.chunk;
-    const int iters = min(ktiles * p.kbatches - it0, p.chunk);
+    auto decode = [&](int index) -> Work {
+        Work w;
+        const int work = xcd_remap(index, p.total_blocks);
+        const int bidx = work / p.tiles_per_batch;  // batch, or k split
+        const int tile = work % p.tiles_per_batch;
+        const int gsize = p.group_m * p.tiles_n;
+        const int group = tile / gsize;
+        const int first_m = group * p.group_m;
+        const int gm = min(p.tiles_m - first_m, p.group_m);
+        w.bm0 = (first_m + (tile % gsize) % gm) * BM;
+        w.bn0 = ((tile % gsize) / gm) * BN;
+        w.split = p.splits > 1 ? bidx : 0;
+        w.batch = p.splits > 1 ? 0 : bidx;
+        // k-loop steps run over (batch, k-tile) pairs; with split-k this item owns steps [it0, it0 + iters)
+        w.it0 = w.split * p.chunk;
+        w.iters = min(ktiles * p.kbatches - w.it0, p.chunk);
+        return w;
+    };
 
-    // ---- global side: origin of the next tile to request -------------------
-    auto a_origin = [&](int kb) -> const uint16_t * {
-        const uint16_t *base = p.a + (int64_t)(kb / p.nb2) * p.a_b1 + (int64_t)(kb % p.nb2) * p.a_b2;
-        return A_KC ? base + (int64_t)bm0 * p.lda : base + bm0;
-    };
-    auto b_origin = [&](int kb) -> const uint16_t * {
-        const uint16_t *base = p.b + (int64_t)(kb / p.nb2) * p.b_b1 + (int64_t)(kb % p.nb2) * p.b_b2;
-        return B_KC ? base + (int64_t)bn0 * p.ldb : base + bn0;
-    };
+    // ---- global side: the load pipeline ("fetch" state runs ahead of the compute state) ------------------
     const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
     const int64_t b_step = B_KC ? BK : (int64_t)BK * p.ldb;
-    int f_kb = p.kbatches > 1 ? it0 / ktiles : (p.splits > 1 ? 0 : batch);
-    int f_kt = p.kbatches > 1 ? it0 % ktiles : it0;
-    const uint16_t *a_next = a_origin(f_kb) + f_kt * a_step;
-    const uint16_t *b_next = b_origin(f_kb) + f_kt * b_step;
+    int f_index = blockIdx.x;   // work item whose tiles are being requested
+    Work fw = decode(f_index);
+    int f_left = 0, f_kb = 0, f_kt = 0, f_stage = 0;
+    const uint16_t *a_next = nullptr, *b_next = nullptr;
     TA ta;
     TB tb;
-    ta.init(p.lda, p.m - bm0, wave, lane);
-    tb.init(p.ldb, p.n - bn0, wave, lane);
-    auto issue = [&](int stage) {
-        uint8_t *st = smem + stage * STAGE_BYTES;
+    auto a_origin = [&](const Work &w, int kb) -> const uint16_t * {
+        const uint16_t *base = p.a + (int64_t)(kb / p.nb2) * p.a_b1 + (int64_t)(kb % p.nb2) * p.a_b2;
+        return A_KC ? base + (int64_t)w.bm0 * p.lda : base + w.bm0;
+    };
+    auto b_origin = [&](const Work &w, int kb) -> const uint16_t * {
+        const uint16_t *base = p.b + (int64_t)(kb / p.nb2) * p.b_b1 + (int64_t)(kb % p.nb2) * p.b_b2;
+        return B_KC ? base + (int64_t)w.bn0 * p.ldb : base + w.bn0;
+    };
+    auto begin_fetch = [&]() {  // position the pipeline on the first tile of work item fw
+        f_left = fw.iters;
+        f_kb = p.kbatches > 1 ? fw.it0 / ktiles : fw.batch;
+        f_kt = p.kbatches > 1 ? fw.it0 % ktiles : fw.it0;
+        a_next = a_origin(fw, f_kb) + f_kt * a_step;
+        b_next = b_origin(fw, f_kb) + f_kt * b_step;
+        ta.init(p.lda, p.m - fw.bm0, wave, lane);
+        tb.init(p.ldb, p.n - fw.bn0, wave, lane);
+    };
+    begin_fetch();
+    bool fetching = true;
+    auto issue = [&]() {
+        uint8_t *st = smem + f_stage * STAGE_BYTES;
+        f_stage ^= 1;
         ta.issue(a_next, st, wave);
         tb.issue(b_next, st + TA::BYTES, wave);
+        if (--f_left == 0) {  // next request belongs to the next work item (if any)
+            f_index += gridDim.x;
+            fetching = f_index < p.total_blocks;
+            if (fetching) {
+                fw = decode(f_index);
+                begin_fetch();
+            }
+            return;
+        }
         a_next += a_step;
         b_next += b_step;
         if (++f_kt == ktiles) {
             f_kt = 0;
-            if (p.kbatches > 1 && ++f_kb < p.kbatches) {
-                a_next = a_origin(f_kb);
-                b_next = b_origin(f_kb);
-            }
+            ++f_kb;
+            a_next = a_origin(fw, f_kb);
+            b_next = b_origin(fw, f_kb);
         }
     };
 
@@ -246,26 +274,24 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
                 for (int j = 0; j < TN; j++) acc[i][j] = Mma<T>::mfma(bf[j], fa[i], acc[i][j]);
             }
     };
-    // Make tile t visible to every wave, then request tile t+1 into the stage tile t-1 occupied.  Callers
-    // guarantee that this wave has issued all its LDS reads of tile t-1; lgkmcnt(0) makes sure they are done.
-    auto sync_tile = [&](int t) {
+    // Make the oldest requested tile visible to every wave, then request the next one into the stage that the
+    // previously computed tile occupied.  Callers guarantee that this wave has issued all its LDS reads of
+    // that previous tile; lgkmcnt(0) makes sure they are done.  (vmcnt(0) also covers the stores of a finished
+    // C tile: they had a whole k step to drain.)
+    auto sync_tile = [&]() {
         __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) & lgkmcnt(0)
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (t + 1 < iters) issue((t + 1) % STAGES);
+        if (fetching) issue();
     };
 
-    if (iters > 0) {
-        issue(0);
-        sync_tile(0);
-        read_a(smem, 0, 0, TM);
-        read_b(smem, 0, fb[0]);
-    }
-    auto tile_body = [&](int it, auto has_next_tag) {
+    // one 64-wide k tile from stage `cs`; HAS_NEXT: the next tile belongs to the same work item (hand the stage
+    // over and prefetch its first fragments while the last MFMAs of this tile run)
+    auto tile_body = [&](int cs, auto has_next_tag) {
         constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
-        const uint8_t *sa = smem + (it % STAGES) * STAGE_BYTES;
-        const uint8_t *sn = smem + ((it + 1) % STAGES) * STAGE_BYTES;
+        const uint8_t *sa = smem + cs * STAGE_BYTES;
+        const uint8_t *sn = smem + (cs ^ 1) * STAGE_BYTES;
         // ---- k step 0 (B buffer 0); prefetch k step 1 of this tile
         mma(fb[0], 0, Q);
         __builtin_amdgcn_sched_barrier(0);
@@ -288,7 +314,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
         mma(fb[1], 2 * Q, 3 * Q);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (HAS_NEXT) {
-            sync_tile(it + 1);
+            sync_tile();
             read_a(sn, 0, 0, 2 * Q);
             read_b(sn, 0, fb[0]);
         }
@@ -298,10 +324,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
         if constexpr (HAS_NEXT) read_a(sn, 0, 2 * Q, TM);
         __builtin_amdgcn_sched_barrier(0);
     };
-    for (int it = 0; it + 1 < iters; it++) tile_body(it, std::true_type{});
-    if (iters > 0) tile_body(iters - 1, std::false_type{});
 
-    // ---- epilogue: lane holds m = l16 (per tile), n = 4*lq + 0..3 -------------
+    // ---- epilogue of one work item: lane holds m = l16 (per tile), n = 4*lq + 0..3 -------------
+    auto store_tile = [&](const Work &w) {
+        const int bm0 = w.bm0, bn0 = w.bn0, split = w.split, batch = w.batch;
     if (p.splits > 1) {  // f32 partial tile into the workspace (padded to whole tiles: no bounds checks)
         float *wbase = p.ws + split * p.ws_split_stride;
 #pragma unroll
@@ -314,6 +340,58 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
     }
     const int cb = p.kbatches > 1 ? 0 : batch;
     uint16_t *cbase = p.c + (int64_t)(cb / p.nb2) * p.c_b1 + (int64_t)(cb % p.nb2) * p.c_b2;
+    if constexpr (TN % 2 == 0) {
+        // 16 B per lane: two neighbouring 16x16 tiles exchange halves between the lane rows (16-lane groups) so
+        // that a lane ends up with 8 consecutive columns of one of them.  v_permlane16_swap(x, y) trades lane
+        // rows 1 and 3 of x against lane rows 0 and 2 of y: afterwards lane row lq holds, in (x, y), columns
+        // 8*(lq/2) .. +3 and +4 .. +7 of tile j + (lq & 1).  A wave instruction then writes 64 contiguous
+        // bytes per matrix row instead of 32, which is what the memory system needs to reach its write rate.
+        if (p.c_vec8) {
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                const int gm_row = bm0 + wm0 + i * 16 + l16;
+                const bool row_ok = gm_row < p.m;
+                uint16_t *crow = cbase + (int64_t)gm_row * p.ldc;
+                float rbias = 0.0f;
+                if (p.bias_mode == BIAS_PER_ROW && row_ok) rbias = Mma<T>::to_f32(p.bias[gm_row]);
+#pragma unroll
+                for (int jp = 0; jp < TN / 2; jp++) {
+                    float v[8];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i][2 * jp][e]),
+                                                                        __float_as_uint(acc[i][2 * jp + 1][e]), false, false);
+                        v[e] = __uint_as_float(r[0]) + rbias;
+                        v[4 + e] = __uint_as_float(r[1]) + rbias;
+                    }
+                    const int gn = bn0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8;
+                    if (!row_ok || gn >= p.n) continue;  // n % 8 == 0 here: all 8 columns are in range
+                    if (p.bias_mode == BIAS_PER_COL) {
+                        const u32x4 bv = *(const u32x4 *)(p.bias + gn);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            v[2 * e] += Mma<T>::to_f32((uint16_t)(bv[e] & 0xffffu));
+                            v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(bv[e] >> 16));
+                        }
+                    }
+                    if (p.accumulate) {
+                        const u32x4 old = *(const u32x4 *)(crow + gn);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            v[2 * e] += Mma<T>::to_f32((uint16_t)(old[e] & 0xffffu));
+                            v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(old[e] >> 16));
+                        }
+                    }
+                    u32x4 o;
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        o[e] = (uint32_t)Mma<T>::from_f32(v[2 * e]) | ((uint32_t)Mma<T>::from_f32(v[2 * e + 1]) << 16);
+                    *(u32x4 *)(crow + gn) = o;
+                }
+            }
+            return;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int gm_row = bm0 + wm0 + i * 16 + l16;
@@ -358,7 +436,43 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
             }
         }
     }
+    };
+
+    // ---- compute state ---------------------------------------------------------------------------------------
+    int c_index = blockIdx.x;
+    Work cw = decode(c_index);
+    int c_left = cw.iters, c_stage = 0;
+    issue();
+    sync_tile();
+    read_a(smem, 0, 0, TM);
+    read_b(smem, 0, fb[0]);
+    for (;;) {
+        for (; c_left > 1; --c_left) {
+            tile_body(c_stage, std::true_type{});
+            c_stage ^= 1;
+        }
+        tile_body(c_stage, std::false_type{});
+        c_stage ^= 1;
+        // Work item finished.  Hand the stage over BEFORE the stores are issued: the wait inside sync_tile then
+        // only covers loads, and the stores drain while the next tile is computed.
+        const bool more = c_index + (int)gridDim.x < p.total_blocks;
+        if (more) sync_tile();
+        store_tile(cw);
+        if (!more) break;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) acc[i][j][v] = 0.0f;
+        c_index += gridDim.x;
+        cw = decode(c_index);
+        c_left = cw.iters;
+        read_a(smem + c_stage * STAGE_BYTES, 0, 0, TM);
+        read_b(smem + c_stage * STAGE_BYTES, 0, fb[0]);
+    }
 }
+
 
 // ------------------------------------------------------------------ host side --
 
@@ -382,22 +496,29 @@ constexpr Variant kVariants[] = {
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
+// Persistent launch: as many workgroups as the chip holds at once (what LDS and registers allow per compute
+// unit, rounded to a multiple of the 8 XCDs so that work item i and i + grid land on the same XCD), or one per
+// work item when there are fewer.
 template <typename T, int BM, int BN, int WM, int WN>
-hipError_t launch_layout(const Params &p, bool a_kc, bool b_kc, hipStream_t stream) {
+hipError_t launch_layout(Params p, int compute_units, bool a_kc, bool b_kc, hipStream_t stream) {
     constexpr int NT = WM * WN * 64;
     constexpr size_t lds = (size_t)STAGES * (BM + BN) * BK * 2;
-    dim3 grid((unsigned)p.total_blocks), block(NT);
 #define DFDX_LAUNCH(AKC, BKC)                                                                                  \
     do {                                                                                                       \
         auto kern = gemm_mfma16_dma_kernel<T, BM, BN, WM, WN, AKC, BKC>;                                       \
-        static bool configured = false;                                                                        \
-        if (!configured) {                                                                                     \
+        static int per_cu = 0;                                                                                 \
+        if (per_cu == 0) {                                                                                     \
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,  \
                                                (int)lds);                                                      \
             if (e != hipSuccess) return e;                                                                     \
-            configured = true;                                                                                 \
+            int occ = 0;                                                                                       \
+            e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void *)kern, NT, lds);               \
+            if (e != hipSuccess) return e;                                                                     \
+            per_cu = occ < 1 ? 1 : occ;                                                                        \
         }                                                                                                      \
-        kern<<<grid, block, lds, stream>>>(p);                                                                 \
+        const int resident = (compute_units < 8 ? 8 : compute_units) * per_cu / 8 * 8;                         \
+        p.grid = p.total_blocks <= resident ? p.total_blocks : resident;                                       \
+        kern<<<dim3((unsigned)p.grid), dim3(NT), lds, stream>>>(p);                                            \
     } while (0)
     if (a_kc && b_kc) DFDX_LAUNCH(true, true);
     else if (a_kc && !b_kc) DFDX_LAUNCH(true, false);
@@ -407,10 +528,11 @@ hipError_t launch_layout(const Params &p, bool a_kc, bool b_kc, hipStream_t stre
     return hipGetLastError();
 }
 
-template <typename T> hipError_t launch_variant(int variant, const Params &p, bool a_kc, bool b_kc, hipStream_t s) {
+template <typename T>
+hipError_t launch_variant(int variant, const Params &p, int compute_units, bool a_kc, bool b_kc, hipStream_t s) {
     switch (variant) {
 #define X(id, bm, bn, wm, wn) \
-    case id: return launch_layout<T, bm, bn, wm, wn>(p, a_kc, b_kc, s);
+    case id: return launch_layout<T, bm, bn, wm, wn>(p, compute_units, a_kc, b_kc, s);
         DFDX_MFMA16_DMA_VARIANTS(X)
 #undef X
     default: return hipErrorInvalidValue;
@@ -557,6 +679,8 @@ hipError_t launch_mfma16dma(const GemmProblem &g, int variant, hipStream_t strea
     p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
     p.c_vec = (g.n % 4 == 0) && (p.ldc % 4 == 0) && (((uintptr_t)g.c & 7u) == 0) &&
               (g.c_b1 % 4 == 0) && (g.c_b2 % 4 == 0) && (!g.bias || ((uintptr_t)g.bias & 7u) == 0);
+    p.c_vec8 = p.c_vec && (g.n % 8 == 0) && (p.ldc % 8 == 0) && (((uintptr_t)g.c & 15u) == 0) &&
+               (g.c_b1 % 8 == 0) && (g.c_b2 % 8 == 0) && (!g.bias || ((uintptr_t)g.bias & 15u) == 0);
     p.group_m = 4;
     const int total_iters = (p.k / BK) * p.kbatches;
     p.splits = 1; p.chunk = total_iters; p.ws = nullptr; p.ws_ld = 0; p.ws_split_stride = 0;
@@ -569,8 +693,9 @@ hipError_t launch_mfma16dma(const GemmProblem &g, int variant, hipStream_t strea
         ws_layout(g, variant, &p.ws_ld, &p.ws_split_stride);
         p.total_blocks = p.tiles_per_batch * g.splits;
     }
-    hipError_t e = (g.dtype == DT_F16) ? launch_variant<_Float16>(variant, p, la.kc, lb.kc, stream)
-                                       : launch_variant<__bf16>(variant, p, la.kc, lb.kc, stream);
+    p.grid = 0;  // set per kernel instantiation at launch
+    hipError_t e = (g.dtype == DT_F16) ? launch_variant<_Float16>(variant, p, g.compute_units, la.kc, lb.kc, stream)
+                                       : launch_variant<__bf16>(variant, p, g.compute_units, la.kc, lb.kc, stream);
     if (e != hipSuccess || g.splits <= 1) return e;
     return launch_splitk_reduce(g, p.ws_ld, p.ws_split_stride, stream);
 }
