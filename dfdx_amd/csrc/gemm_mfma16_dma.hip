@@ -606,35 +606,67 @@ int mfma16dma_pick_variant(const GemmProblem &p, int compute_units) {
     return 0;
 }
 
+// Cost model of the planner (seconds), fitted to timings of this kernel family on a 256-CU MI355X.
+//   * a compute unit sustains rate1 / rate2 flop/s on a variant's k tiles when the chip is full; the 128-row tiles
+//     only get there with two workgroups resident per compute unit, and lightly loaded chips clock higher;
+//   * a work item also moves (operands mostly from L2) + (C tile) bytes at the compute unit's share of HBM;
+//   * every work item pays a fixed hand-over cost, every launch a first-load latency and a last C tile;
+//   * split-k adds the workspace round trip, which stays in the last-level cache while it is small.
 namespace {
-// relative per-CU efficiency of each tile variant (measured at 4096^3 / on the config shapes)
-constexpr double kTileEff[] = {1.0, 0.85, 0.70, 0.60, 0.45};
+struct VariantModel {
+    int per_cu;           // workgroups resident per compute unit (LDS and register limits)
+    double rate1, rate2;  // flop/s of a compute unit with 1 / with >= 2 resident workgroups
+};
+constexpr VariantModel kModel[] = {
+    {1, 4.64e12, 4.64e12},  // 256x256
+    {1, 3.81e12, 3.81e12},  // 256x128
+    {2, 2.50e12, 4.25e12},  // 128x128
+    {1, 3.60e12, 3.60e12},  // 256x64
+    {2, 2.20e12, 3.30e12},  // 128x64
+};
+constexpr double kItemOverhead = 3.1e-6, kLaunchLatency = 2e-6, kCuBandwidth = 24e9, kOperandWeight = 0.32;
+constexpr double kIdleBoost = 0.146, kWsBandwidthCached = 9.5e12, kWsBandwidthHbm = 6.1e12, kWsCached = 128e6;
 }  // namespace
 
 void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_variant, int forced_splits, int *variant,
                           int *splits) {
     *variant = 0;
     *splits = 1;
+    const int cus = std::max(1, compute_units);
     const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
     const bool may_split = nbatch == 1 && p.c_cs == 1;
     const int64_t total_iters = (p.k / BK) * (p.reduce ? p.nb1 * p.nb2 : 1);
+    const bool a_kc = classify(p.m, p.k, p.a_rs, p.a_cs).kc, b_kc = classify(p.n, p.k, p.b_cs, p.b_rs).kc;
+    const double elem = 2.0, out_elems = (double)p.m * p.n * nbatch;
     double best = 1e300;
     for (int v = 1; v <= kNumVariants; v++) {
         if (forced_variant > 0 && v != forced_variant) continue;
         if (!mfma16dma_supported(p, v)) continue;
         const Variant &t = kVariants[v - 1];
+        const VariantModel &vm = kModel[v - 1];
         if (forced_variant == 0 && ((p.n <= 64) != (t.bn <= 64))) continue;  // BN = 64 tiles only for narrow outputs
         const int64_t tiles = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
-        const double rate = 4.0e12 * kTileEff[v - 1];  // flop/s of one CU on this tile shape
+        double layout = (a_kc && b_kc) ? 1.0 : (!a_kc && !b_kc) ? 0.955 : 1.0;  // transposing LDS reads cost a little
+        if (v == 2 && !(a_kc && b_kc)) layout *= 0.87;
         for (int s = 1; s <= 16; s++) {
             if (forced_splits > 0 && s != std::min<int64_t>(forced_splits, total_iters)) continue;
             if (s > 1 && (!may_split || (forced_splits == 0 && total_iters / s < 4))) break;
             const int64_t chunk = (total_iters + s - 1) / s;
             if ((s - 1) * chunk >= total_iters) continue;  // an empty split
-            const int64_t blocks = tiles * s;
-            const int64_t rounds = (blocks + compute_units - 1) / compute_units;
-            double time = rounds * (chunk * (2.0 * t.bm * t.bn * BK / rate) + 3e-6);
-            if (s > 1) time += 4e-6 + 2.0 * s * (double)p.m * p.n * 4.0 / 3e12;
+            const int64_t items = tiles * s;
+            const int64_t grid = std::min<int64_t>(items, (int64_t)cus * vm.per_cu);
+            const int64_t conc = (grid + cus - 1) / cus, items_per_wg = (items + grid - 1) / grid;
+            const double active = (double)std::min<int64_t>(grid, cus) / cus;
+            const double cu_rate = (conc >= 2 ? vm.rate2 : vm.rate1) * layout * (1.0 + kIdleBoost * (1.0 - active));
+            const double t_mma = chunk * (2.0 * t.bm * t.bn * BK) / (cu_rate / conc);
+            const double out_bytes = (double)t.bm * t.bn * (s > 1 ? 4.0 : elem * (1 + p.accumulate));
+            const double t_mem = (kOperandWeight * (t.bm + t.bn) * BK * elem * chunk + out_bytes) / (kCuBandwidth / conc);
+            double time = items_per_wg * (std::max(t_mma, t_mem) + kItemOverhead) + kLaunchLatency +
+                          out_bytes / (kCuBandwidth / conc);
+            if (s > 1) {
+                const double ws = s * out_elems * 4.0;
+                time += 3e-6 + (ws + out_elems * elem * (1 + p.accumulate)) / (ws <= kWsCached ? kWsBandwidthCached : kWsBandwidthHbm);
+            }
             if (time < best) {
                 best = time;
                 *variant = v;
