@@ -1,38 +1,38 @@
 // C ABI of the dfdx ROCm matmul backend: context, storage helpers, GEMM dispatch.
-#include "../../include/dfdx_rocm.h"
+#include "ctx_internal.h"
 #include "gemm_internal.h"
 
-#include <hip/hip_runtime.h>
 #include <cstdio>
 #include <cstring>
-#include <mutex>
 
 using namespace dfdx_rocm;
 
-struct dfdx_rocm_ctx {
-    int device;
-    hipStream_t stream;
-    int compute_units;
-    int clock_mhz;
-    char name[128];
-    std::mutex mu;
-    void *workspace = nullptr;  // split-k partial sums; grown on demand, owned by the context
-    size_t workspace_bytes = 0;
-};
-
-namespace {
-
-#define HIP_TRY(expr)                      \
-    do {                                   \
-        hipError_t e__ = (expr);           \
-        if (e__ != hipSuccess) return (int)e__; \
-    } while (0)
+namespace dfdx_rocm {
 
 int bind(dfdx_rocm_ctx *ctx) {
     if (!ctx) return DFDX_ROCM_ERR_INVALID_ARG;
     HIP_TRY(hipSetDevice(ctx->device));
     return DFDX_ROCM_OK;
 }
+
+int ensure_workspace(dfdx_rocm_ctx *ctx, size_t bytes) {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (bytes <= ctx->workspace_bytes) return DFDX_ROCM_OK;
+    if (ctx->workspace) {
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+        HIP_TRY(hipFree(ctx->workspace));
+        ctx->workspace = nullptr;
+        ctx->workspace_bytes = 0;
+    }
+    bytes = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    HIP_TRY(hipMalloc(&ctx->workspace, bytes));
+    ctx->workspace_bytes = bytes;
+    return DFDX_ROCM_OK;
+}
+
+}  // namespace dfdx_rocm
+
+namespace {
 
 // Validates `d` and produces the canonical problem (row-major C whenever the view allows it).
 int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
@@ -73,22 +73,6 @@ int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
 struct Plan {
     int kernel, variant, splits;
 };
-
-// Grows the context's workspace; pending work that may still use the old one is drained first.
-int ensure_workspace(dfdx_rocm_ctx *ctx, size_t bytes) {
-    std::lock_guard<std::mutex> lock(ctx->mu);
-    if (bytes <= ctx->workspace_bytes) return DFDX_ROCM_OK;
-    if (ctx->workspace) {
-        HIP_TRY(hipStreamSynchronize(ctx->stream));
-        HIP_TRY(hipFree(ctx->workspace));
-        ctx->workspace = nullptr;
-        ctx->workspace_bytes = 0;
-    }
-    bytes = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
-    HIP_TRY(hipMalloc(&ctx->workspace, bytes));
-    ctx->workspace_bytes = bytes;
-    return DFDX_ROCM_OK;
-}
 
 int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProblem &p, Plan *plan) {
     const bool is16 = p.dtype == DT_F16 || p.dtype == DT_BF16;

@@ -1,0 +1,32 @@
+// The library context as the host-side sources see it (the C ABI only exposes an opaque pointer).
+#pragma once
+#include "../../include/dfdx_rocm.h"
+
+#include <hip/hip_runtime.h>
+#include <mutex>
+
+struct dfdx_rocm_ctx {
+    int device;
+    hipStream_t stream;
+    int compute_units;
+    int clock_mhz;
+    char name[128];
+    std::mutex mu;
+    void *workspace = nullptr;  // partial sums of split reductions; grown on demand, owned by the context
+    size_t workspace_bytes = 0;
+};
+
+namespace dfdx_rocm {
+
+#define HIP_TRY(expr)                           \
+    do {                                        \
+        hipError_t e__ = (expr);                \
+        if (e__ != hipSuccess) return (int)e__; \
+    } while (0)
+
+// Makes the context's device current for the calling thread.
+int bind(dfdx_rocm_ctx *ctx);
+// Grows the context's workspace to at least `bytes`; work that may still use the old one is drained first.
+int ensure_workspace(dfdx_rocm_ctx *ctx, size_t bytes);
+
+}  // namespace dfdx_rocm

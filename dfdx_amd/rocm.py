@@ -70,7 +70,8 @@ EXPORTS = [
     "dfdx_rocm_matmat_br_forward", "dfdx_rocm_matmat_br_backward",
     "dfdx_rocm_matmat_batch3_forward", "dfdx_rocm_matmat_batch3_backward",
     "dfdx_rocm_matmat_batch4_forward", "dfdx_rocm_matmat_batch4_backward",
-    "dfdx_rocm_linear_forward",
+    "dfdx_rocm_linear_forward", "dfdx_rocm_linear_backward",
+    "dfdx_rocm_bias_forward", "dfdx_rocm_bias_backward",
 ]
 
 
@@ -357,6 +358,49 @@ class Rocm:
             ctypes.c_void_p(weight.ptr), ctypes.c_void_p(bias.ptr if bias is not None else None),
             ctypes.c_void_p(out.ptr)))
         return out
+
+    def _linear_rows(self, x: View, i: int):
+        if len(x.shape) == 1:
+            return 1, (i * x.strides[0], x.strides[0])
+        if len(x.shape) == 2:
+            return x.shape[0], x.strides
+        assert x.strides == _row_major(x.shape), "batched Linear input must be contiguous to fold its rows"
+        return int(np.prod(x.shape[:-1])), (i, 1)
+
+    def linear_backward(self, x: View, grad_x: View, weight: View, grad_weight: View, grad_bias: Optional[View],
+                        grad_out: View):
+        """Backward of ``Linear``: grad_x += go.W, grad_weight += go^T.x, grad_bias += column sums of go."""
+        o, i = weight.shape
+        assert weight.strides == (i, 1), "Linear weight storage is (O, I) row-major"
+        assert x.shape[-1] == i, f"left: {x.shape[-1]}\n right: {i}"
+        assert grad_out.shape == tuple(x.shape[:-1]) + (o,) and grad_out.strides == _row_major(grad_out.shape)
+        rows, xs = self._linear_rows(x, i)
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_linear_backward(
+            self.ctx, DTYPES[x.dtype], _c(rows), _c(i), _c(o), vp(x.ptr), _i64arr(xs), vp(grad_x.ptr),
+            vp(weight.ptr), vp(grad_weight.ptr), vp(grad_bias.ptr if grad_bias is not None else None),
+            vp(grad_out.ptr)))
+
+    def bias_forward(self, x: View, bias: View) -> View:
+        """``Bias1D::try_forward`` (dfdx/src/nn/layers/bias1d.rs:62-78) on a contiguous input."""
+        cols = bias.shape[0]
+        assert x.shape[-1] == cols, f"left: {x.shape[-1]}\n right: {cols}"
+        assert x.strides == _row_major(x.shape) and bias.strides == (1,)
+        rows = int(np.prod(x.shape[:-1], dtype=np.int64))
+        out = self.zeros(x.dtype, x.shape)
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_bias_forward(self.ctx, DTYPES[x.dtype], _c(rows), _c(cols), vp(x.ptr),
+                                                    vp(bias.ptr), vp(out.ptr)))
+        return out
+
+    def bias_backward(self, grad_out: View, grad_bias: View):
+        """grad_bias += column sums of grad_out (the broadcast operand's share of the add's backward)."""
+        cols = grad_bias.shape[0]
+        assert grad_out.shape[-1] == cols and grad_out.strides == _row_major(grad_out.shape)
+        rows = int(np.prod(grad_out.shape[:-1], dtype=np.int64))
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_bias_backward(self.ctx, DTYPES[grad_out.dtype], _c(rows), _c(cols),
+                                                     vp(grad_out.ptr), vp(grad_bias.ptr)))
 
 
 def _c(v: int):

@@ -195,6 +195,30 @@ int dfdx_rocm_linear_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_
                              const void *x, const int64_t x_strides[2], const void *weight, const void *bias,
                              void *out);
 
+/* Backward of the same Linear: grad_x (through x_strides) += grad_out . W,
+ * grad_weight (O, I) += grad_out^T . x, grad_bias (O,) += column sums of
+ * grad_out; grad_out is (rows, O) contiguous.  The two products are the
+ * MatMat backward on the weight's permuted view (linear.rs:85-86 with
+ * matmul/mod.rs:116-131); the bias term is the backward of the broadcast
+ * add (bias1d.rs:62-78).  grad_bias may be NULL. */
+int dfdx_rocm_linear_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t in_dim, int64_t out_dim,
+                              const void *x, const int64_t x_strides[2], void *grad_x, const void *weight,
+                              void *grad_weight, void *grad_bias, const void *grad_out);
+
+/* ---- Bias1D ------------------------------------------------------------------
+ * `Bias1D::try_forward` (dfdx/src/nn/layers/bias1d.rs:62-78): the (cols,)
+ * bias is broadcast over every leading axis of a contiguous input and added;
+ * a (B, S, cols) input is passed with rows = B*S.  out may be x. */
+int dfdx_rocm_bias_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *x, const void *bias,
+                           void *out);
+/* Backward of that add for the broadcast operand (binary-op backward through
+ * a broadcast view, dfdx-core/src/tensor_ops/utilities/cpu_kernels.rs:164-203):
+ * grad_bias[c] += sum over rows of grad_out[r][c].  The reference adds row
+ * after row in the storage type; here the column is summed in f32 and rounded
+ * once.  (grad_x of the add is grad_out itself and needs no kernel.) */
+int dfdx_rocm_bias_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *grad_out,
+                            void *grad_bias);
+
 #ifdef __cplusplus
 }
 #endif
