@@ -1,0 +1,151 @@
+// Reshape of a non-contiguous view: the copy `ReshapeKernel::forward` makes (out, contiguous, takes the view's
+// elements in logical row-major order) and its backward (grad_inp, through the view's strides, += grad_out).
+// HBM-bound gather / scatter; the view's innermost run of contiguous elements is moved 16 bytes at a time when it
+// allows (a head permute of attention keeps rows of head_dim elements contiguous).
+#include "ctx_internal.h"
+#include "elem.h"
+
+namespace dfdx_rocm {
+namespace {
+
+constexpr int MAX_RANK = 6;
+
+struct ViewDims {
+    int rank;
+    uint32_t shape[MAX_RANK];   // innermost axis counted in groups of N elements
+    int64_t stride[MAX_RANK];   // elements
+};
+
+// offset (elements) of the g-th N-element group of the view in logical order
+template <typename Index> __device__ __forceinline__ int64_t view_offset(const ViewDims &d, Index g) {
+    int64_t off = 0;
+#pragma unroll
+    for (int a = MAX_RANK - 1; a >= 0; a--) {
+        if (a < d.rank) {
+            const Index q = g / d.shape[a];
+            off += (int64_t)(g - q * d.shape[a]) * d.stride[a];
+            g = q;
+        }
+    }
+    return off;
+}
+
+template <typename T, int N, typename Index>
+__global__ __launch_bounds__(256) void reshape_forward_kernel(const T *inp, T *out, ViewDims d, Index groups) {
+    for (Index g = (Index)blockIdx.x * 256 + threadIdx.x; g < groups; g += (Index)gridDim.x * 256) {
+        float v[N];
+        load_elems<T, N>(inp + view_offset<Index>(d, g), v);
+        store_elems<T, N>(out + (int64_t)g * N, v);
+    }
+}
+
+template <typename T, int N, typename Index>
+__global__ __launch_bounds__(256) void reshape_backward_kernel(T *grad_inp, const T *grad_out, ViewDims d, Index groups) {
+    for (Index g = (Index)blockIdx.x * 256 + threadIdx.x; g < groups; g += (Index)gridDim.x * 256) {
+        float v[N], old[N];
+        load_elems<T, N>(grad_out + (int64_t)g * N, v);
+        T *dst = grad_inp + view_offset<Index>(d, g);
+        load_elems<T, N>(dst, old);
+#pragma unroll
+        for (int i = 0; i < N; i++) old[i] += v[i];
+        store_elems<T, N>(dst, old);
+    }
+}
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+// Drops size-1 axes and merges neighbours that are contiguous with respect to each other.
+int canonical(int rank, const int64_t *shape, const int64_t *strides, int64_t *cs, int64_t *cst) {
+    int n = 0;
+    for (int a = 0; a < rank; a++) {
+        if (shape[a] == 1) continue;
+        if (n > 0 && cst[n - 1] == strides[a] * shape[a]) {
+            cs[n - 1] *= shape[a];
+            cst[n - 1] = strides[a];
+        } else {
+            cs[n] = shape[a];
+            cst[n] = strides[a];
+            n++;
+        }
+    }
+    if (n == 0) {
+        cs[0] = 1;
+        cst[0] = 1;
+        n = 1;
+    }
+    return n;
+}
+
+template <typename T, bool FWD>
+int launch_t(dfdx_rocm_ctx *ctx, int rank, const int64_t *shape, const int64_t *strides, const void *src, void *dst) {
+    // forward: src = inp (strided), dst = out (contiguous);  backward: src = grad_out (contiguous), dst = grad_inp (strided)
+    int64_t cs[MAX_RANK], cst[MAX_RANK];
+    const int n = canonical(rank, shape, strides, cs, cst);
+    int64_t total = 1;
+    for (int a = 0; a < n; a++) total *= cs[a];
+    constexpr int V = Elem<T>::VEC;
+    const void *strided = FWD ? src : dst;
+    bool vec = cst[n - 1] == 1 && cs[n - 1] % V == 0 && aligned16(src) && aligned16(dst);
+    for (int a = 0; a + 1 < n && vec; a++) vec = cst[a] % V == 0;
+    (void)strided;
+    const int g = vec ? V : 1;
+    ViewDims d;
+    d.rank = n;
+    for (int a = 0; a < MAX_RANK; a++) {
+        d.shape[a] = a < n ? (uint32_t)(a == n - 1 ? cs[a] / g : cs[a]) : 1u;
+        d.stride[a] = a < n ? (a == n - 1 ? cst[a] * g : cst[a]) : 0;
+    }
+    const int64_t groups = total / g;
+    const unsigned grid = (unsigned)std::min<int64_t>((groups + 255) / 256, (int64_t)ctx->compute_units * 16);
+    const bool small = groups < (1ll << 31);
+    hipStream_t s = ctx->stream;
+#define DFDX_RESHAPE(N, IDX)                                                                                       \
+    do {                                                                                                           \
+        if constexpr (FWD) reshape_forward_kernel<T, N, IDX><<<grid, 256, 0, s>>>((const T *)src, (T *)dst, d, (IDX)groups); \
+        else reshape_backward_kernel<T, N, IDX><<<grid, 256, 0, s>>>((T *)dst, (const T *)src, d, (IDX)groups);   \
+    } while (0)
+    if (vec && small) DFDX_RESHAPE(V, uint32_t);
+    else if (vec) DFDX_RESHAPE(V, uint64_t);
+    else if (small) DFDX_RESHAPE(1, uint32_t);
+    else DFDX_RESHAPE(1, uint64_t);
+#undef DFDX_RESHAPE
+    return (int)hipGetLastError();
+}
+
+template <bool FWD>
+int dispatch(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, const int64_t *strides, const void *src, void *dst) {
+    if (int e = bind(ctx)) return e;
+    if (rank < 0 || rank > MAX_RANK || (rank > 0 && (!shape || !strides))) return DFDX_ROCM_ERR_INVALID_ARG;
+    int64_t total = 1;
+    for (int a = 0; a < rank; a++) {
+        if (shape[a] < 0 || strides[a] < 0 || shape[a] >= (1ll << 32)) return DFDX_ROCM_ERR_INVALID_ARG;
+        // a broadcast axis maps several grad_out elements to one grad_inp element: a reduction, not a scatter
+        if (!FWD && shape[a] > 1 && strides[a] == 0) return DFDX_ROCM_ERR_ALIASED_OUTPUT;
+        total *= shape[a];
+    }
+    if (total == 0) return DFDX_ROCM_OK;
+    if (!src || !dst) return DFDX_ROCM_ERR_INVALID_ARG;
+    switch (dtype) {
+    case DFDX_ROCM_F32: return launch_t<float, FWD>(ctx, rank, shape, strides, src, dst);
+    case DFDX_ROCM_F16: return launch_t<_Float16, FWD>(ctx, rank, shape, strides, src, dst);
+    case DFDX_ROCM_BF16: return launch_t<__bf16, FWD>(ctx, rank, shape, strides, src, dst);
+    default: return DFDX_ROCM_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace
+}  // namespace dfdx_rocm
+
+extern "C" {
+
+int dfdx_rocm_reshape_forward(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, const int64_t *inp_strides,
+                              const void *inp, void *out) {
+    return dfdx_rocm::dispatch<true>(ctx, dtype, rank, shape, inp_strides, inp, out);
+}
+
+int dfdx_rocm_reshape_backward(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, const int64_t *inp_strides,
+                               void *grad_inp, const void *grad_out) {
+    return dfdx_rocm::dispatch<false>(ctx, dtype, rank, shape, inp_strides, grad_out, grad_inp);
+}
+
+}  // extern "C"

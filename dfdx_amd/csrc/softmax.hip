@@ -1,0 +1,208 @@
+// Softmax over the last (contiguous) axis of a (rows, cols) matrix and its backward, with an optional scale of
+// the logits folded in (attention's `q.k^T * scalar` followed by softmax).  HBM-bound: the forward reads and
+// writes the matrix once, the backward reads p and grad_out, and reads and writes grad_x.
+//
+// One wave owns a row.  Rows of up to 64 * VEC * MAX_CHUNKS elements stay in registers between the passes; longer
+// rows are walked three times (max, sum, store) from memory.
+#include "ctx_internal.h"
+#include "elem.h"
+
+#include <cfloat>
+
+namespace dfdx_rocm {
+namespace {
+
+constexpr int WAVES = 4;  // rows per workgroup
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// ---- rows held in registers -----------------------------------------------------------------------------------
+// Lane l owns the N-element groups l, l + 64, ... of the row (CH of them; groups past the row end are skipped).
+template <typename T, int N, int CH>
+__global__ __launch_bounds__(WAVES * 64) void softmax_forward_reg_kernel(const T *x, T *out, int64_t rows, int cols, float scale) {
+    const int lane = threadIdx.x % 64;
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const T *src = x + row * cols;
+        float v[CH][N];
+        float m = -FLT_MAX;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+                load_elems<T, N>(src + col, v[c]);
+#pragma unroll
+                for (int i = 0; i < N; i++) {
+                    v[c][i] *= scale;
+                    m = fmaxf(m, v[c][i]);
+                }
+            }
+        }
+        m = wave_max(m);
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) {
+                    v[c][i] = expf(v[c][i] - m);
+                    s += v[c][i];
+                }
+            }
+        }
+        s = wave_sum(s);
+        const float inv = 1.0f / s;
+        T *dst = out + row * cols;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) v[c][i] *= inv;
+                store_elems<T, N>(dst + col, v[c]);
+            }
+        }
+    }
+}
+
+// grad_x += scale * p * (g - sum_j g_j p_j)
+template <typename T, int N, int CH>
+__global__ __launch_bounds__(WAVES * 64) void softmax_backward_reg_kernel(const T *p, const T *go, T *gx, int64_t rows, int cols,
+                                                                          float scale) {
+    const int lane = threadIdx.x % 64;
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const T *ps = p + row * cols, *gs = go + row * cols;
+        float pv[CH][N], gv[CH][N];
+        float dot = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+                load_elems<T, N>(ps + col, pv[c]);
+                load_elems<T, N>(gs + col, gv[c]);
+#pragma unroll
+                for (int i = 0; i < N; i++) dot += pv[c][i] * gv[c][i];
+            }
+        }
+        dot = wave_sum(dot);
+        T *dst = gx + row * cols;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+                float old[N];
+                load_elems<T, N>(dst + col, old);
+#pragma unroll
+                for (int i = 0; i < N; i++) old[i] += scale * (pv[c][i] * (gv[c][i] - dot));
+                store_elems<T, N>(dst + col, old);
+            }
+        }
+    }
+}
+
+// ---- long rows: three passes over memory --------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(WAVES * 64) void softmax_forward_loop_kernel(const T *x, T *out, int64_t rows, int cols, float scale) {
+    const int lane = threadIdx.x % 64;
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const T *src = x + row * cols;
+        float m = -FLT_MAX;
+        for (int c = lane; c < cols; c += 64) m = fmaxf(m, Elem<T>::load(src + c) * scale);
+        m = wave_max(m);
+        float s = 0.0f;
+        for (int c = lane; c < cols; c += 64) s += expf(Elem<T>::load(src + c) * scale - m);
+        s = wave_sum(s);
+        const float inv = 1.0f / s;
+        T *dst = out + row * cols;
+        for (int c = lane; c < cols; c += 64) Elem<T>::store(dst + c, expf(Elem<T>::load(src + c) * scale - m) * inv);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(WAVES * 64) void softmax_backward_loop_kernel(const T *p, const T *go, T *gx, int64_t rows, int cols,
+                                                                           float scale) {
+    const int lane = threadIdx.x % 64;
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const T *ps = p + row * cols, *gs = go + row * cols;
+        float dot = 0.0f;
+        for (int c = lane; c < cols; c += 64) dot += Elem<T>::load(ps + c) * Elem<T>::load(gs + c);
+        dot = wave_sum(dot);
+        T *dst = gx + row * cols;
+        for (int c = lane; c < cols; c += 64)
+            Elem<T>::store(dst + c, Elem<T>::load(dst + c) + scale * (Elem<T>::load(ps + c) * (Elem<T>::load(gs + c) - dot)));
+    }
+}
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+template <typename T, bool FWD>
+int launch_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *a, const void *b, void *c, float scale) {
+    // forward: a = x, c = out;  backward: a = p, b = grad_out, c = grad_x
+    constexpr int V = Elem<T>::VEC;
+    const bool vec = cols % V == 0 && aligned16(a) && aligned16(c) && (FWD || aligned16(b));
+    const unsigned grid = (unsigned)std::min<int64_t>((rows + WAVES - 1) / WAVES, (int64_t)ctx->compute_units * 16);
+    const dim3 block(WAVES * 64);
+    hipStream_t s = ctx->stream;
+    const int n = (int)cols;
+#define DFDX_SOFTMAX_REG(N, CH)                                                                                        \
+    do {                                                                                                               \
+        if constexpr (FWD) softmax_forward_reg_kernel<T, N, CH><<<grid, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale); \
+        else softmax_backward_reg_kernel<T, N, CH><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale); \
+        return (int)hipGetLastError();                                                                                 \
+    } while (0)
+    if (vec) {
+        const int64_t groups = cols / V;
+        if (groups <= 64) DFDX_SOFTMAX_REG(V, 1);
+        if (groups <= 128) DFDX_SOFTMAX_REG(V, 2);
+        if (groups <= 256) DFDX_SOFTMAX_REG(V, 4);
+        if (groups <= 512) DFDX_SOFTMAX_REG(V, 8);
+    } else {
+        if (cols <= 64) DFDX_SOFTMAX_REG(1, 1);
+        if (cols <= 256) DFDX_SOFTMAX_REG(1, 4);
+        if (cols <= 1024) DFDX_SOFTMAX_REG(1, 16);
+    }
+#undef DFDX_SOFTMAX_REG
+    if constexpr (FWD) softmax_forward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale);
+    else softmax_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale);
+    return (int)hipGetLastError();
+}
+
+template <bool FWD>
+int dispatch(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *a, const void *b, void *c, float scale) {
+    if (int e = bind(ctx)) return e;
+    if (rows < 0 || cols < 0 || cols >= (1ll << 31)) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
+    if (!a || !c || (!FWD && !b)) return DFDX_ROCM_ERR_INVALID_ARG;
+    switch (dtype) {
+    case DFDX_ROCM_F32: return launch_t<float, FWD>(ctx, rows, cols, a, b, c, scale);
+    case DFDX_ROCM_F16: return launch_t<_Float16, FWD>(ctx, rows, cols, a, b, c, scale);
+    case DFDX_ROCM_BF16: return launch_t<__bf16, FWD>(ctx, rows, cols, a, b, c, scale);
+    default: return DFDX_ROCM_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace
+}  // namespace dfdx_rocm
+
+extern "C" {
+
+int dfdx_rocm_softmax_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *x, float scale,
+                              void *out) {
+    return dfdx_rocm::dispatch<true>(ctx, dtype, rows, cols, x, nullptr, out, scale);
+}
+
+int dfdx_rocm_softmax_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *out, float scale,
+                               void *grad_x, const void *grad_out) {
+    return dfdx_rocm::dispatch<false>(ctx, dtype, rows, cols, out, grad_out, grad_x, scale);
+}
+
+}  // extern "C"

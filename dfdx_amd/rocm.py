@@ -72,6 +72,9 @@ EXPORTS = [
     "dfdx_rocm_matmat_batch4_forward", "dfdx_rocm_matmat_batch4_backward",
     "dfdx_rocm_linear_forward", "dfdx_rocm_linear_backward",
     "dfdx_rocm_bias_forward", "dfdx_rocm_bias_backward",
+    "dfdx_rocm_scalar_mul_forward", "dfdx_rocm_scalar_mul_backward",
+    "dfdx_rocm_softmax_forward", "dfdx_rocm_softmax_backward",
+    "dfdx_rocm_reshape_forward", "dfdx_rocm_reshape_backward",
 ]
 
 
@@ -401,6 +404,61 @@ class Rocm:
         vp = ctypes.c_void_p
         self._check(self.lib.dfdx_rocm_bias_backward(self.ctx, DTYPES[grad_out.dtype], _c(rows), _c(cols),
                                                      vp(grad_out.ptr), vp(grad_bias.ptr)))
+
+    # ------------------------------------------------- ops between attention's GEMMs --
+    def scalar_mul_forward(self, x: View, scalar: float) -> View:
+        """``x * scalar`` over the physical storage (unary kernel, utilities/cpu_kernels.rs:46-79); same strides."""
+        out = View(self._torch.empty_like(x.storage), x.dtype, x.shape, x.strides, x.offset)
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_scalar_mul_forward(self.ctx, DTYPES[x.dtype], _c(x.numel_storage()),
+                                                          vp(x.storage.data_ptr()), ctypes.c_double(scalar),
+                                                          vp(out.storage.data_ptr())))
+        return out
+
+    def scalar_mul_backward(self, scalar: float, grad_inp: View, grad_out: View):
+        assert grad_inp.numel_storage() == grad_out.numel_storage()
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_scalar_mul_backward(self.ctx, DTYPES[grad_inp.dtype], _c(grad_inp.numel_storage()),
+                                                           ctypes.c_double(scalar), vp(grad_inp.storage.data_ptr()),
+                                                           vp(grad_out.storage.data_ptr())))
+
+    def softmax_forward(self, x: View, scale: float = 1.0) -> View:
+        """softmax(scale * x) over the last axis of a contiguous tensor (softmax.rs:70-83)."""
+        assert x.strides == _row_major(x.shape), "softmax input must be contiguous"
+        cols = x.shape[-1]
+        rows = int(np.prod(x.shape[:-1], dtype=np.int64))
+        out = View(self._torch.empty_like(x.storage), x.dtype, x.shape, x.strides)
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_softmax_forward(self.ctx, DTYPES[x.dtype], _c(rows), _c(cols), vp(x.ptr),
+                                                       ctypes.c_float(scale), vp(out.ptr)))
+        return out
+
+    def softmax_backward(self, out: View, grad_x: View, grad_out: View, scale: float = 1.0):
+        assert out.strides == _row_major(out.shape) and grad_out.shape == out.shape and grad_x.shape == out.shape
+        cols = out.shape[-1]
+        rows = int(np.prod(out.shape[:-1], dtype=np.int64))
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_softmax_backward(self.ctx, DTYPES[out.dtype], _c(rows), _c(cols), vp(out.ptr),
+                                                        ctypes.c_float(scale), vp(grad_x.ptr), vp(grad_out.ptr)))
+
+    def reshape_forward(self, x: View, new_shape) -> View:
+        """``try_reshape_like`` (reshape_to/mod.rs:90-115): free for a contiguous tensor, a copy otherwise."""
+        new_shape = tuple(int(d) for d in new_shape)
+        assert int(np.prod(x.shape, dtype=np.int64)) == int(np.prod(new_shape, dtype=np.int64)), \
+            f"left: {int(np.prod(x.shape))}\n right: {int(np.prod(new_shape))}"
+        if x.strides == _row_major(x.shape):
+            return View(x.storage, x.dtype, new_shape, _row_major(new_shape), x.offset)
+        out = self.zeros(x.dtype, new_shape)
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_reshape_forward(self.ctx, DTYPES[x.dtype], len(x.shape), _i64arr(x.shape),
+                                                       _i64arr(x.strides), vp(x.ptr), vp(out.ptr)))
+        return out
+
+    def reshape_backward(self, x: View, grad_inp: View, grad_out: View):
+        """Backward of a copying reshape: grad_inp (laid out like x's storage) += grad_out through x's strides."""
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_reshape_backward(self.ctx, DTYPES[x.dtype], len(x.shape), _i64arr(x.shape),
+                                                        _i64arr(x.strides), vp(grad_inp.ptr), vp(grad_out.ptr)))
 
 
 def _c(v: int):

@@ -219,6 +219,46 @@ int dfdx_rocm_bias_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t 
 int dfdx_rocm_bias_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *grad_out,
                             void *grad_bias);
 
+/* ---- The ops between attention's GEMMs ---------------------------------------
+ * MultiHeadAttention::try_forward (dfdx/src/nn/layers/multi_head_attention.rs:
+ * 105-146) runs, between its matmuls, a multiplication by a scalar, a softmax
+ * over the last axis and one reshape of a permuted tensor.  These entry points
+ * keep those on the device. */
+
+/* `t * scalar` (ScalarMulKernelOp, dfdx-core/src/tensor_ops/mul/cpu_kernel.rs:
+ * 5-17, run by the unary kernel over the tensor's physical storage,
+ * utilities/cpu_kernels.rs:46-109): out[i] = x[i] * s for i < len, with s
+ * rounded to the element type first; out may be x.  Backward:
+ * grad_inp[i] += s * grad_out[i]. */
+int dfdx_rocm_scalar_mul_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const void *x, double scalar, void *out);
+int dfdx_rocm_scalar_mul_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, double scalar, void *grad_inp,
+                                  const void *grad_out);
+
+/* Softmax over the last axis of a contiguous (rows, cols) matrix
+ * (`try_softmax::<Axis<3>>`, dfdx-core/src/tensor_ops/softmax.rs:70-83:
+ * exp(t - max) / sum exp(t - max)), applied to scale * x so that attention's
+ * scalar multiplication can be folded in (scale = 1 for a plain softmax).
+ * The reference composes it from max / sub / exp / sum / div kernels, each
+ * rounding to the element type; here a row is processed in f32 and rounded
+ * once.  out may be x.  Backward of the composition, from the saved output:
+ * grad_x[r][c] += scale * out[r][c] * (grad_out[r][c] - sum_j grad_out[r][j] * out[r][j]). */
+int dfdx_rocm_softmax_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *x, float scale,
+                              void *out);
+int dfdx_rocm_softmax_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *out, float scale,
+                               void *grad_x, const void *grad_out);
+
+/* ReshapeKernel (dfdx-core/src/tensor_ops/reshape_to/mod.rs:90-115,
+ * cpu_kernel.rs:7-35) for a view that is not contiguous: forward copies the
+ * view's elements, in logical row-major order, into the contiguous `out`;
+ * backward adds grad_out (contiguous) into grad_inp through the view's
+ * strides.  rank <= 6, strides in elements.  A zero stride on an axis longer
+ * than 1 is accepted by forward and answered with
+ * DFDX_ROCM_ERR_ALIASED_OUTPUT by backward. */
+int dfdx_rocm_reshape_forward(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, const int64_t *inp_strides,
+                              const void *inp, void *out);
+int dfdx_rocm_reshape_backward(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, const int64_t *inp_strides,
+                               void *grad_inp, const void *grad_out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -50,3 +50,102 @@ def bias_backward(grad_out: np.ndarray, grad_bias: np.ndarray, dtype: str, faith
     for r in range(go.shape[0]):
         acc = round_to(acc + go[r], dtype)
     return acc
+
+
+# ------------------------------------------------------------------------------------------ scalar mul --
+
+def scalar_mul_forward(x: np.ndarray, scalar: float, dtype: str) -> np.ndarray:
+    """``t * scalar`` (ScalarMulKernelOp::f, tensor_ops/mul/cpu_kernel.rs:5-11, applied to every element of the
+    storage by the unary kernel, utilities/cpu_kernels.rs:73-78); the scalar is held in the element type."""
+    s = round_to(np.float64(scalar), dtype)
+    return round_to(np.asarray(x, np.float64) * s, dtype)
+
+
+def scalar_mul_backward(scalar: float, grad_inp: np.ndarray, grad_out: np.ndarray, dtype: str) -> np.ndarray:
+    """``*x += df * grad_out[i]`` with the constant df = scalar (utilities/cpu_kernels.rs:89-93): the product and
+    the add each round to the element type."""
+    s = round_to(np.float64(scalar), dtype)
+    return round_to(np.asarray(grad_inp, np.float64) + round_to(s * np.asarray(grad_out, np.float64), dtype), dtype)
+
+
+# --------------------------------------------------------------------------------------------- softmax --
+
+def _seq_sum_last(x: np.ndarray, dtype: str) -> np.ndarray:
+    """Sum over the last axis the way the Cpu reduction does it for f32 / plain f16: one accumulator of the
+    element type per output, elements added in index order (tensor_ops/sum_to/cpu_kernel.rs:72-103).  (The
+    AMP<f16> impl, :8-41, keeps that accumulator in f32 instead.)"""
+    acc = np.zeros(x.shape[:-1], np.float64)
+    for j in range(x.shape[-1]):
+        acc = round_to(acc + x[..., j], dtype)
+    return acc
+
+
+def softmax_forward(x: np.ndarray, dtype: str, faithful: bool = True) -> np.ndarray:
+    """``try_softmax`` over the last axis (tensor_ops/softmax.rs:70-83): m = max, tm = t - m, e = exp(tm),
+    s = sum(e), out = e / s, every step a kernel that rounds to the element type.  ``faithful=False`` evaluates the
+    same formula in float64 and rounds once."""
+    x = np.asarray(x, np.float64)
+    m = x.max(axis=-1, keepdims=True)
+    if not faithful:
+        e = np.exp(x - m)
+        return round_to(e / e.sum(axis=-1, keepdims=True), dtype)
+    tm = round_to(x - m, dtype)
+    e = round_to(np.exp(tm), dtype)
+    s = _seq_sum_last(e, dtype)[..., None]
+    return round_to(e / s, dtype)
+
+
+def softmax_backward(x: np.ndarray, grad_out: np.ndarray, dtype: str, faithful: bool = True) -> np.ndarray:
+    """Gradient of that composition w.r.t. t, as the tape replays it (softmax.rs:70-83 with the binary div, the
+    broadcast sum and exp backward ops): with e, s as above,
+        g_e  = g / s                       (div backward, lhs; utilities/cpu_kernels.rs:164-187)
+        g_s  = sum_j( -e_j / s^2 * g_j )   (div backward, broadcast rhs: accumulated element by element)
+        g_e += g_s                         (sum backward: broadcast add)
+        g_t  = g_e * e                     (exp backward, df = f(x))
+    ``faithful=False`` returns out * (g - sum_j g_j out_j) evaluated in float64, rounded once."""
+    x = np.asarray(x, np.float64)
+    g = np.asarray(grad_out, np.float64)
+    m = x.max(axis=-1, keepdims=True)
+    if not faithful:
+        e = np.exp(x - m)
+        p = e / e.sum(axis=-1, keepdims=True)
+        return round_to(p * (g - (g * p).sum(axis=-1, keepdims=True)), dtype)
+    tm = round_to(x - m, dtype)
+    e = round_to(np.exp(tm), dtype)
+    s = _seq_sum_last(e, dtype)[..., None]
+    g_e = round_to(round_to(1.0 / s, dtype) * g, dtype)
+    contrib = round_to(round_to(-e / round_to(s * s, dtype), dtype) * g, dtype)
+    g_s = _seq_sum_last(contrib, dtype)[..., None]
+    g_e = round_to(g_e + g_s, dtype)
+    return round_to(e * g_e, dtype)
+
+
+# --------------------------------------------------------------------------------------------- reshape --
+
+def _view_indices(shape, strides) -> np.ndarray:
+    idx = np.zeros(tuple(shape), dtype=np.int64)
+    for ax, (n, s) in enumerate(zip(shape, strides)):
+        sh = [1] * len(shape)
+        sh[ax] = n
+        idx = idx + (np.arange(n, dtype=np.int64) * s).reshape(sh)
+    return idx.reshape(-1)
+
+
+def reshape_forward(storage: np.ndarray, shape, strides) -> np.ndarray:
+    """``ReshapeKernel::forward`` (tensor_ops/reshape_to/cpu_kernel.rs:8-21): the view's elements in logical
+    row-major order, copied into a fresh contiguous buffer."""
+    return np.asarray(storage).reshape(-1)[_view_indices(shape, strides)].copy()
+
+
+def reshape_backward(shape, strides, grad_inp: np.ndarray, grad_out: np.ndarray, dtype: str) -> np.ndarray:
+    """``ReshapeKernel::backward`` (cpu_kernel.rs:22-34): ``grad_inp[i] += grad_out[o]`` walking both index
+    sequences together; a repeated i (broadcast view) accumulates in visiting order."""
+    out = np.asarray(grad_inp, np.float64).copy().reshape(-1)
+    go = np.asarray(grad_out, np.float64).reshape(-1)
+    idx = _view_indices(shape, strides)
+    if len(np.unique(idx)) == len(idx):
+        out[idx] = round_to(out[idx] + go, dtype)
+        return out
+    for o, i in enumerate(idx):
+        out[i] = round_to(out[i] + go[o], dtype)
+    return out
