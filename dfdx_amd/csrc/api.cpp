@@ -15,20 +15,23 @@ int bind(dfdx_rocm_ctx *ctx) {
     return DFDX_ROCM_OK;
 }
 
-int ensure_workspace(dfdx_rocm_ctx *ctx, size_t bytes) {
+static int grow(dfdx_rocm_ctx *ctx, void **buf, size_t *have, size_t bytes) {
     std::lock_guard<std::mutex> lock(ctx->mu);
-    if (bytes <= ctx->workspace_bytes) return DFDX_ROCM_OK;
-    if (ctx->workspace) {
+    if (bytes <= *have) return DFDX_ROCM_OK;
+    if (*buf) {
         HIP_TRY(hipStreamSynchronize(ctx->stream));
-        HIP_TRY(hipFree(ctx->workspace));
-        ctx->workspace = nullptr;
-        ctx->workspace_bytes = 0;
+        HIP_TRY(hipFree(*buf));
+        *buf = nullptr;
+        *have = 0;
     }
     bytes = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
-    HIP_TRY(hipMalloc(&ctx->workspace, bytes));
-    ctx->workspace_bytes = bytes;
+    HIP_TRY(hipMalloc(buf, bytes));
+    *have = bytes;
     return DFDX_ROCM_OK;
 }
+
+int ensure_workspace(dfdx_rocm_ctx *ctx, size_t bytes) { return grow(ctx, &ctx->workspace, &ctx->workspace_bytes, bytes); }
+int ensure_patches(dfdx_rocm_ctx *ctx, size_t bytes) { return grow(ctx, &ctx->patches, &ctx->patches_bytes, bytes); }
 
 }  // namespace dfdx_rocm
 
@@ -185,10 +188,11 @@ int dfdx_rocm_create(int ordinal, void *stream, dfdx_rocm_ctx **out) {
 
 int dfdx_rocm_destroy(dfdx_rocm_ctx *ctx) {
     if (!ctx) return DFDX_ROCM_OK;
-    if (ctx->workspace) {
+    if (ctx->workspace || ctx->patches) {
         (void)hipSetDevice(ctx->device);
         (void)hipStreamSynchronize(ctx->stream);
-        (void)hipFree(ctx->workspace);
+        if (ctx->workspace) (void)hipFree(ctx->workspace);
+        if (ctx->patches) (void)hipFree(ctx->patches);
     }
     delete ctx;
     return DFDX_ROCM_OK;

@@ -1,0 +1,251 @@
+// conv2d as unfold + batched GEMM: the images (forward) or the output gradients (backward) are unfolded into patch
+// matrices by HBM-bound gather kernels, and every product is one call of the library's strided batched GEMM --
+// filters with batch stride 0 over the images, groups as the second batch axis, the filter gradient as a GEMM
+// that reduces over the batch.
+#include "ctx_internal.h"
+#include "elem.h"
+
+#include <cstring>
+
+namespace dfdx_rocm {
+namespace {
+
+struct Op {  // dfdx_rocm_conv2d_op narrowed to 32 bits (validated on entry)
+    int kernel, stride, padding, dilation, groups, batch, chan_in, chan_out, h_in, h_out, w_in, w_out;
+};
+
+// patches[b][c][k1][k2][oh][ow] = img[b][c][oh*stride + dilation*k1 - padding][ow*stride + dilation*k2 - padding],
+// zero outside the image.  One thread writes N consecutive ow (w_out % N == 0).
+template <typename T, int N>
+__global__ __launch_bounds__(256) void unfold_input_kernel(Op op, const T *img, T *patches, uint32_t groups) {
+    const uint32_t wg = (uint32_t)op.w_out / N;
+    for (uint32_t t = blockIdx.x * 256 + threadIdx.x; t < groups; t += gridDim.x * 256) {
+        uint32_t r = t;
+        const int ow0 = (int)(r % wg) * N; r /= wg;
+        const int oh = (int)(r % op.h_out); r /= op.h_out;
+        const int k2 = (int)(r % op.kernel); r /= op.kernel;
+        const int k1 = (int)(r % op.kernel); r /= op.kernel;  // r = b * chan_in + c
+        const int y = oh * op.stride + op.dilation * k1 - op.padding;
+        const T *row = img + ((int64_t)r * op.h_in + y) * op.w_in;
+        float v[N];
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int x = (ow0 + i) * op.stride + op.dilation * k2 - op.padding;
+            v[i] = (y >= 0 && y < op.h_in && x >= 0 && x < op.w_in) ? Elem<T>::load(row + x) : 0.0f;
+        }
+        store_elems<T, N>(patches + (int64_t)t * N, v);
+    }
+}
+
+// patches[b][o][k1][k2][y][x] = grad_out[b][o][oh][ow] where oh*stride = y + padding - dilation*k1 (likewise ow),
+// zero when no output position reads image pixel (y, x) through filter tap (k1, k2).
+template <typename T, int N>
+__global__ __launch_bounds__(256) void unfold_output_kernel(Op op, const T *grad_out, T *patches, uint32_t groups) {
+    const uint32_t wg = (uint32_t)op.w_in / N;
+    for (uint32_t t = blockIdx.x * 256 + threadIdx.x; t < groups; t += gridDim.x * 256) {
+        uint32_t r = t;
+        const int x0 = (int)(r % wg) * N; r /= wg;
+        const int y = (int)(r % op.h_in); r /= op.h_in;
+        const int k2 = (int)(r % op.kernel); r /= op.kernel;
+        const int k1 = (int)(r % op.kernel); r /= op.kernel;  // r = b * chan_out + o
+        int oh = y + op.padding - op.dilation * k1;
+        const bool row_ok = oh >= 0 && oh % op.stride == 0 && oh / op.stride < op.h_out;
+        oh /= op.stride;
+        const T *row = grad_out + ((int64_t)r * op.h_out + oh) * op.w_out;
+        float v[N];
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int ow = x0 + i + op.padding - op.dilation * k2;
+            const bool ok = row_ok && ow >= 0 && ow % op.stride == 0 && ow / op.stride < op.w_out;
+            v[i] = ok ? Elem<T>::load(row + ow / op.stride) : 0.0f;
+        }
+        store_elems<T, N>(patches + (int64_t)t * N, v);
+    }
+}
+
+// filters (G*O/G, C/G, K, K) <-> transposed (G, C/G, O/G, K*K).  ADD_BACK: filters[..] += transposed[..].
+template <typename T, bool ADD_BACK>
+__global__ __launch_bounds__(256) void filter_transpose_kernel(Op op, T *filters, T *transposed, int total) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int kk = op.kernel * op.kernel, og = op.chan_out / op.groups, cg = op.chan_in / op.groups;
+    int r = i;
+    const int tap = r % kk; r /= kk;
+    const int o = r % og; r /= og;
+    const int c = r % cg;
+    const int g = r / cg;
+    T *f = filters + (((int64_t)(g * og + o) * cg + c) * kk + tap);
+    if constexpr (ADD_BACK) Elem<T>::store(f, Elem<T>::load(f) + Elem<T>::load(transposed + i));
+    else transposed[i] = *f;
+}
+
+template <typename T> __global__ __launch_bounds__(256) void zero_kernel(T *p, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) Elem<T>::store(p + i, 0.0f);
+}
+
+constexpr size_t kPatchBudget = size_t(1) << 30;  // bytes of patches per batch chunk
+
+template <typename T> unsigned grid_for(dfdx_rocm_ctx *ctx, uint64_t threads) {
+    return (unsigned)std::min<uint64_t>((threads + 255) / 256, (uint64_t)ctx->compute_units * 32);
+}
+
+inline int narrow(const dfdx_rocm_conv2d_op *o, Op *op) {
+    const size_t f[12] = {o->kernel, o->stride, o->padding, o->dilation, o->groups, o->batch,
+                          o->chan_in, o->chan_out, o->h_in, o->h_out, o->w_in, o->w_out};
+    for (size_t v : f)
+        if (v >= (size_t(1) << 30)) return DFDX_ROCM_ERR_INVALID_ARG;
+    *op = {(int)f[0], (int)f[1], (int)f[2], (int)f[3], (int)f[4], (int)f[5], (int)f[6], (int)f[7], (int)f[8], (int)f[9], (int)f[10], (int)f[11]};
+    if (op->kernel < 1 || op->stride < 1 || op->dilation < 1 || op->groups < 1) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (op->chan_in % op->groups || op->chan_out % op->groups) return DFDX_ROCM_ERR_INVALID_ARG;
+    // the output size must be the one the reference derives (conv2d/mod.rs:143-160)
+    const int64_t span = (int64_t)op->dilation * (op->kernel - 1) + 1;
+    if (op->h_in + 2ll * op->padding < span || op->w_in + 2ll * op->padding < span) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (op->h_out != (op->h_in + 2ll * op->padding - span) / op->stride + 1) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (op->w_out != (op->w_in + 2ll * op->padding - span) / op->stride + 1) return DFDX_ROCM_ERR_INVALID_ARG;
+    return DFDX_ROCM_OK;
+}
+
+dfdx_rocm_gemm_desc blank_desc(int dtype, int64_t m, int64_t k, int64_t n) {
+    dfdx_rocm_gemm_desc d;
+    std::memset(&d, 0, sizeof(d));
+    d.dtype = dtype;
+    d.m = m; d.k = k; d.n = n;
+    d.batch1 = 1; d.batch2 = 1;
+    return d;
+}
+
+template <typename T>
+int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void *filters, void *out) {
+    const int64_t kk = (int64_t)op.kernel * op.kernel, n = (int64_t)op.h_out * op.w_out;
+    const int64_t m = op.chan_out / op.groups, k = (op.chan_in / op.groups) * kk;
+    const int64_t per_image = (int64_t)op.chan_in * kk * n;  // patch elements of one image
+    if (per_image == 0 || m == 0) return DFDX_ROCM_OK;
+    if (per_image >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
+    int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
+    chunk = std::min<int64_t>(std::min<int64_t>(chunk, op.batch), ((1ll << 31) - 1) / per_image);
+    if (int rc = ensure_patches(ctx, (size_t)(chunk * per_image) * sizeof(T))) return rc;
+    T *patches = (T *)ctx->patches;
+    constexpr int V = Elem<T>::VEC;
+    const bool vec = op.w_out % V == 0;
+    for (int64_t b0 = 0; b0 < op.batch; b0 += chunk) {
+        const int64_t nb = std::min<int64_t>(chunk, op.batch - b0);
+        Op sub = op;
+        sub.batch = (int)nb;
+        const T *src = (const T *)img + b0 * op.chan_in * op.h_in * op.w_in;
+        const uint64_t elems = (uint64_t)nb * per_image;
+        if (vec) unfold_input_kernel<T, V><<<grid_for<T>(ctx, elems / V), 256, 0, ctx->stream>>>(sub, src, patches, (uint32_t)(elems / V));
+        else unfold_input_kernel<T, 1><<<grid_for<T>(ctx, elems), 256, 0, ctx->stream>>>(sub, src, patches, (uint32_t)elems);
+        HIP_TRY(hipGetLastError());
+        // filters (G, O/G, C/G*K*K) . patches (B, G, C/G*K*K, OH*OW) -> out (B, G, O/G, OH*OW)
+        dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
+        d.batch1 = nb; d.batch2 = op.groups;
+        d.a = filters; d.a_rs = k; d.a_cs = 1; d.a_b1 = 0; d.a_b2 = m * k;
+        d.b = patches; d.b_rs = n; d.b_cs = 1; d.b_b1 = op.groups * k * n; d.b_b2 = k * n;
+        d.c = (T *)out + b0 * op.chan_out * n; d.c_rs = n; d.c_cs = 1; d.c_b1 = op.chan_out * n; d.c_b2 = m * n;
+        if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+    }
+    return DFDX_ROCM_OK;
+}
+
+template <typename T>
+int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad_img, const void *filters, void *grad_filters,
+               const void *grad_out) {
+    const int64_t kk = (int64_t)op.kernel * op.kernel, hw = (int64_t)op.h_in * op.w_in, ohw = (int64_t)op.h_out * op.w_out;
+    const int64_t cg = op.chan_in / op.groups, og = op.chan_out / op.groups;
+    const int64_t per_image = (int64_t)op.chan_out * kk * hw;
+    const int64_t f_elems = (int64_t)op.groups * cg * og * kk;
+    if (per_image == 0 || f_elems == 0 || ohw == 0) return DFDX_ROCM_OK;
+    if (per_image >= (1ll << 31) || f_elems >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
+    int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
+    chunk = std::min<int64_t>(std::min<int64_t>(chunk, op.batch), ((1ll << 31) - 1) / per_image);
+    // patch buffer: [chunk][O*K*K][H*W], then the transposed filters and their gradient
+    const size_t patch_bytes = ((size_t)(chunk * per_image) * sizeof(T) + 255) & ~size_t(255);
+    const size_t f_bytes = ((size_t)f_elems * sizeof(T) + 255) & ~size_t(255);
+    if (int rc = ensure_patches(ctx, patch_bytes + 2 * f_bytes)) return rc;
+    T *patches = (T *)ctx->patches;
+    T *f_tr = (T *)((char *)ctx->patches + patch_bytes);
+    T *grad_f_tr = (T *)((char *)ctx->patches + patch_bytes + f_bytes);
+    const unsigned fgrid = (unsigned)((f_elems + 255) / 256);
+    filter_transpose_kernel<T, false><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)const_cast<void *>(filters), f_tr, (int)f_elems);
+    HIP_TRY(hipGetLastError());
+    zero_kernel<T><<<fgrid, 256, 0, ctx->stream>>>(grad_f_tr, (int)f_elems);
+    HIP_TRY(hipGetLastError());
+    constexpr int V = Elem<T>::VEC;
+    const bool vec = op.w_in % V == 0;
+    for (int64_t b0 = 0; b0 < op.batch; b0 += chunk) {
+        const int64_t nb = std::min<int64_t>(chunk, op.batch - b0);
+        Op sub = op;
+        sub.batch = (int)nb;
+        const T *go = (const T *)grad_out + b0 * op.chan_out * ohw;
+        const uint64_t elems = (uint64_t)nb * per_image;
+        if (vec) unfold_output_kernel<T, V><<<grid_for<T>(ctx, elems / V), 256, 0, ctx->stream>>>(sub, go, patches, (uint32_t)(elems / V));
+        else unfold_output_kernel<T, 1><<<grid_for<T>(ctx, elems), 256, 0, ctx->stream>>>(sub, go, patches, (uint32_t)elems);
+        HIP_TRY(hipGetLastError());
+        {   // grad_img (B, G, C/G, H*W) += filters^T (G, C/G, O/G*K*K) . patches (B, G, O/G*K*K, H*W)
+            const int64_t m = cg, k = og * kk, n = hw;
+            dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
+            d.accumulate = 1;
+            d.batch1 = nb; d.batch2 = op.groups;
+            d.a = f_tr; d.a_rs = k; d.a_cs = 1; d.a_b1 = 0; d.a_b2 = m * k;
+            d.b = patches; d.b_rs = n; d.b_cs = 1; d.b_b1 = op.groups * k * n; d.b_b2 = k * n;
+            d.c = (T *)grad_img + b0 * op.chan_in * hw; d.c_rs = n; d.c_cs = 1; d.c_b1 = op.chan_in * hw; d.c_b2 = m * n;
+            if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+        }
+        for (int g = 0; g < op.groups; g++) {
+            // grad_filters^T (C/G, O/G*K*K) += sum over images of img (C/G, H*W) . patches^T (H*W, O/G*K*K)
+            const int64_t m = cg, k = hw, n = og * kk;
+            dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
+            d.accumulate = 1;
+            d.reduce_batch = 1;
+            d.batch1 = nb;
+            d.a = (const T *)img + (b0 * op.chan_in + g * cg) * hw; d.a_rs = k; d.a_cs = 1; d.a_b1 = op.chan_in * hw;
+            d.b = patches + g * n * k; d.b_rs = 1; d.b_cs = k; d.b_b1 = per_image;
+            d.c = grad_f_tr + g * m * n; d.c_rs = n; d.c_cs = 1;
+            if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+        }
+    }
+    filter_transpose_kernel<T, true><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)grad_filters, grad_f_tr, (int)f_elems);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+}  // namespace dfdx_rocm
+
+using namespace dfdx_rocm;
+
+extern "C" {
+
+int dfdx_rocm_conv2d_forward(dfdx_rocm_ctx *ctx, int dtype, const dfdx_rocm_conv2d_op *op, const void *img,
+                             const void *filters, void *out) {
+    if (int e = bind(ctx)) return e;
+    Op o;
+    if (!op) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (int e = narrow(op, &o)) return e;
+    if (o.batch == 0 || o.chan_out == 0 || o.h_out == 0 || o.w_out == 0) return DFDX_ROCM_OK;
+    if (!img || !filters || !out) return DFDX_ROCM_ERR_INVALID_ARG;
+    switch (dtype) {
+    case DFDX_ROCM_F32: return forward_t<float>(ctx, dtype, o, img, filters, out);
+    case DFDX_ROCM_F16: return forward_t<_Float16>(ctx, dtype, o, img, filters, out);
+    case DFDX_ROCM_BF16: return forward_t<__bf16>(ctx, dtype, o, img, filters, out);
+    default: return DFDX_ROCM_ERR_UNSUPPORTED;
+    }
+}
+
+int dfdx_rocm_conv2d_backward(dfdx_rocm_ctx *ctx, int dtype, const dfdx_rocm_conv2d_op *op, const void *img, void *grad_img,
+                              const void *filters, void *grad_filters, const void *grad_out) {
+    if (int e = bind(ctx)) return e;
+    Op o;
+    if (!op) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (int e = narrow(op, &o)) return e;
+    if (o.batch == 0 || o.chan_out == 0 || o.chan_in == 0) return DFDX_ROCM_OK;
+    if (!img || !grad_img || !filters || !grad_filters || !grad_out) return DFDX_ROCM_ERR_INVALID_ARG;
+    switch (dtype) {
+    case DFDX_ROCM_F32: return backward_t<float>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out);
+    case DFDX_ROCM_F16: return backward_t<_Float16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out);
+    case DFDX_ROCM_BF16: return backward_t<__bf16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out);
+    default: return DFDX_ROCM_ERR_UNSUPPORTED;
+    }
+}
+
+}  // extern "C"

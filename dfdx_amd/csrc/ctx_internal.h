@@ -14,6 +14,8 @@ struct dfdx_rocm_ctx {
     std::mutex mu;
     void *workspace = nullptr;  // partial sums of split reductions; grown on demand, owned by the context
     size_t workspace_bytes = 0;
+    void *patches = nullptr;  // unfolded images of conv2d (alive across the GEMMs that may regrow `workspace`)
+    size_t patches_bytes = 0;
 };
 
 namespace dfdx_rocm {
@@ -28,5 +30,7 @@ namespace dfdx_rocm {
 int bind(dfdx_rocm_ctx *ctx);
 // Grows the context's workspace to at least `bytes`; work that may still use the old one is drained first.
 int ensure_workspace(dfdx_rocm_ctx *ctx, size_t bytes);
+// Same for the conv2d patch buffer.
+int ensure_patches(dfdx_rocm_ctx *ctx, size_t bytes);
 
 }  // namespace dfdx_rocm

@@ -54,6 +54,12 @@ class GemmDesc(ctypes.Structure):
     ]
 
 
+class Conv2DOp(ctypes.Structure):
+    """Mirrors ``dfdx_rocm_conv2d_op`` == the reference's ``Conv2DOp`` (conv2d/mod.rs:14-29)."""
+    _fields_ = [(n, ctypes.c_size_t) for n in ("kernel", "stride", "padding", "dilation", "groups", "batch",
+                                               "chan_in", "chan_out", "h_in", "h_out", "w_in", "w_out")]
+
+
 def lib_path() -> str:
     return os.path.join(_HERE, "lib", "libdfdx_rocm.so")
 
@@ -75,6 +81,7 @@ EXPORTS = [
     "dfdx_rocm_scalar_mul_forward", "dfdx_rocm_scalar_mul_backward",
     "dfdx_rocm_softmax_forward", "dfdx_rocm_softmax_backward",
     "dfdx_rocm_reshape_forward", "dfdx_rocm_reshape_backward",
+    "dfdx_rocm_conv2d_forward", "dfdx_rocm_conv2d_backward",
 ]
 
 
@@ -459,6 +466,39 @@ class Rocm:
         vp = ctypes.c_void_p
         self._check(self.lib.dfdx_rocm_reshape_backward(self.ctx, DTYPES[x.dtype], len(x.shape), _i64arr(x.shape),
                                                         _i64arr(x.strides), vp(grad_inp.ptr), vp(grad_out.ptr)))
+
+    # ---------------------------------------------------------------- conv2d --
+    def _conv2d_op(self, img: View, filters: View, stride, padding, dilation, groups) -> Conv2DOp:
+        """Shape checks and output size of ``try_conv2d`` (conv2d/mod.rs:143-160, 279-308)."""
+        shape = img.shape if len(img.shape) == 4 else (1,) + tuple(img.shape)
+        batch, chan_in, h, w = shape
+        chan_out, cg, kernel, k2 = filters.shape
+        assert chan_in == cg * groups, f"left: {chan_in}\n right: {cg * groups}"
+        assert kernel == k2, f"left: {kernel}\n right: {k2}"
+        assert chan_out % groups == 0
+        if img.strides != _row_major(img.shape) or filters.strides != _row_major(filters.shape):
+            raise ValueError("Image & filter inputs to conv2d must be contiguous")
+        size = lambda d: (d + 2 * padding - 1 - dilation * (kernel - 1)) // stride + 1
+        assert h + 2 * padding - 1 >= dilation * (kernel - 1) and w + 2 * padding - 1 >= dilation * (kernel - 1)
+        return Conv2DOp(kernel, stride, padding, dilation, groups, batch, chan_in, chan_out, h, size(h), w, size(w))
+
+    def conv2d_forward(self, img: View, filters: View, stride=1, padding=0, dilation=1, groups=1) -> View:
+        """``(img, filters).conv2d(stride, padding, dilation, groups)``; img (B, C, H, W) or (C, H, W)."""
+        op = self._conv2d_op(img, filters, stride, padding, dilation, groups)
+        lead = (op.batch,) if len(img.shape) == 4 else ()
+        out = self.zeros(img.dtype, lead + (op.chan_out, op.h_out, op.w_out))
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_conv2d_forward(self.ctx, DTYPES[img.dtype], ctypes.byref(op), vp(img.ptr),
+                                                      vp(filters.ptr), vp(out.ptr)))
+        return out
+
+    def conv2d_backward(self, img: View, grad_img: View, filters: View, grad_filters: View, grad_out: View,
+                        stride=1, padding=0, dilation=1, groups=1):
+        op = self._conv2d_op(img, filters, stride, padding, dilation, groups)
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_conv2d_backward(self.ctx, DTYPES[img.dtype], ctypes.byref(op), vp(img.ptr),
+                                                       vp(grad_img.ptr), vp(filters.ptr), vp(grad_filters.ptr),
+                                                       vp(grad_out.ptr)))
 
 
 def _c(v: int):

@@ -259,6 +259,24 @@ int dfdx_rocm_reshape_forward(dfdx_rocm_ctx *ctx, int dtype, int rank, const int
 int dfdx_rocm_reshape_backward(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, const int64_t *inp_strides,
                                void *grad_inp, const void *grad_out);
 
+/* ---- conv2d as unfold + batched GEMM ---------------------------------------
+ * Conv2DKernel (dfdx-core/src/tensor_ops/conv2d/mod.rs:31-55; Cpu impl
+ * cpu_kernel.rs:40-278, Cuda impl cuda_kernel.rs:62-281).  The op struct has
+ * the fields and order of the reference's #[repr(C)] Conv2DOp (mod.rs:14-29),
+ * so the Rust side passes its own value by pointer.  img is (batch, chan_in,
+ * h_in, w_in), filters (chan_out, chan_in/groups, kernel, kernel), out
+ * (batch, chan_out, h_out, w_out), all contiguous as the reference requires
+ * (mod.rs:290-292); an unbatched image is batch = 1.  Forward overwrites out;
+ * backward accumulates into grad_img and grad_filters. */
+typedef struct dfdx_rocm_conv2d_op {
+    size_t kernel, stride, padding, dilation, groups, batch, chan_in, chan_out, h_in, h_out, w_in, w_out;
+} dfdx_rocm_conv2d_op;
+
+int dfdx_rocm_conv2d_forward(dfdx_rocm_ctx *ctx, int dtype, const dfdx_rocm_conv2d_op *op, const void *img,
+                             const void *filters, void *out);
+int dfdx_rocm_conv2d_backward(dfdx_rocm_ctx *ctx, int dtype, const dfdx_rocm_conv2d_op *op, const void *img,
+                              void *grad_img, const void *filters, void *grad_filters, const void *grad_out);
+
 #ifdef __cplusplus
 }
 #endif

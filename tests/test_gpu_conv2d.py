@@ -1,0 +1,149 @@
+"""GPU parity of conv2d (unfold kernels + the library's batched GEMM) against the PyTorch-produced literals of
+the reference's tests (conv2d/tests.rs) and the CPU restatement of cpu_kernel.rs on seeded inputs."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle.conv2d import Conv2DOp, conv2d_backward, conv2d_forward
+from helpers import assert_within, logical, rng
+from gpu_util import announce, device
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+CONV = json.load(open(os.path.join(GOLD, "conv2d_literals.json")))
+ULP = {"f32": 2.0 ** -23, "f16": 2.0 ** -10, "bf16": 2.0 ** -7}
+
+
+def host(dev, view):
+    return logical(oracle.to_f64(dev.to_host(view), view.dtype), view.shape, view.strides, view.offset)
+
+
+def upload(dev, values, dtype):
+    values = np.asarray(values, dtype=np.float64)
+    return dev.tensor(oracle.to_storage(values.reshape(-1), dtype).reshape(values.shape), dtype)
+
+
+@pytest.mark.parametrize("case", CONV["cases"], ids=lambda c: c["name"])
+def test_conv2d_literals(case):
+    dev = device()
+    announce("conv2d literal", case["name"])
+    x, w = upload(dev, case["x"], "f32"), upload(dev, case["weight"], "f32")
+    kw = dict(stride=case["stride"], padding=case["padding"], dilation=case["dilation"], groups=case["groups"])
+    y = host(dev, dev.conv2d_forward(x, w, **kw))
+    if "bias" in case:
+        y = y + np.asarray(case["bias"]).reshape(-1, 1, 1)
+    np.testing.assert_allclose(y, case["out"], rtol=0, atol=2e-6)
+    gy = {"exp_mean": np.exp(y) / y.size, "mean": np.full(y.shape, 1.0 / y.size)}[case["loss"]]
+    gx, gw = dev.zeros_like_storage(x), dev.zeros_like_storage(w)
+    dev.conv2d_backward(x, gx, w, gw, upload(dev, gy, "f32"), **kw)
+    np.testing.assert_allclose(host(dev, gx), case["grad_x"], rtol=0, atol=2e-6)
+    np.testing.assert_allclose(host(dev, gw), case["grad_weight"], rtol=0, atol=2e-6)
+
+
+CONFIGS = [
+    # batch, chan_in, chan_out, h, w, kernel, stride, padding, dilation, groups
+    (2, 4, 6, 7, 6, 3, 2, 1, 1, 2),
+    (1, 3, 5, 9, 8, 2, 1, 2, 3, 1),
+    (3, 6, 3, 5, 5, 1, 1, 0, 1, 3),
+    (1, 5, 3, 7, 6, 2, 4, 3, 1, 1),
+    (10, 3, 5, 28, 28, 6, 3, 2, 1, 1),     # the shape of the reference's batched test (conv2d/tests.rs:219-250)
+    (2, 9, 15, 14, 14, 3, 1, 0, 1, 3),     # the shape of its grouped-slices test (:405-464)
+    (4, 64, 64, 28, 28, 3, 1, 1, 1, 1),    # k = 576, n = 784: the MFMA kernels
+    (2, 64, 128, 32, 32, 3, 2, 1, 1, 2),
+    (3, 32, 64, 24, 40, 5, 1, 2, 2, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("cfg", CONFIGS, ids=lambda c: "x".join(map(str, c)))
+def test_conv2d_seeded(cfg, dtype):
+    dev, g = device(), rng(501)
+    batch, cin, cout, h, w_, kernel, stride, padding, dilation, groups = cfg
+    announce("conv2d", cfg, dtype)
+    op = Conv2DOp.make(batch, cin, cout, h, w_, kernel, stride, padding, dilation, groups)
+    kw = dict(stride=stride, padding=padding, dilation=dilation, groups=groups)
+    x = upload(dev, g.standard_normal((batch, cin, h, w_)), dtype)
+    w = upload(dev, g.standard_normal((cout, cin // groups, kernel, kernel)) / np.sqrt(cin // groups * kernel * kernel), dtype)
+    y = dev.conv2d_forward(x, w, **kw)
+    assert y.shape == (batch, cout, op.h_out, op.w_out)
+    x_h, w_h = dev.to_host(x).reshape(-1), dev.to_host(w).reshape(-1)
+    X, W = oracle.to_f64(x_h, dtype), oracle.to_f64(w_h, dtype)
+    want = oracle.to_f64(conv2d_forward(dtype, op, x_h, w_h), dtype)
+    kf = cin // groups * kernel * kernel
+    assert_within(dtype, kf, host(dev, y).reshape(-1), want, X, W, extra=ULP[dtype] * float(np.abs(want).max()), what="out")
+    go = upload(dev, g.standard_normal(y.shape), dtype)
+    gx0, gw0 = upload(dev, g.standard_normal(x.shape), dtype), upload(dev, g.standard_normal(w.shape), dtype)
+    gx, gw = dev.tensor(dev.to_host(gx0), dtype), dev.tensor(dev.to_host(gw0), dtype)
+    dev.conv2d_backward(x, gx, w, gw, go, **kw)
+    go_h = dev.to_host(go).reshape(-1)
+    ogx, ogw = dev.to_host(gx0).reshape(-1).copy(), dev.to_host(gw0).reshape(-1).copy()
+    conv2d_backward(dtype, op, x_h, ogx, w_h, ogw, go_h)
+    GO = oracle.to_f64(go_h, dtype)
+    wgx, wgw = oracle.to_f64(ogx, dtype), oracle.to_f64(ogw, dtype)
+    assert_within(dtype, cout // groups * kernel * kernel, host(dev, gx).reshape(-1), wgx, GO, W,
+                  extra=2 * ULP[dtype] * float(np.abs(wgx).max()), what="grad_img")
+    # the restatement rounds the filter gradient to the element type after every image, the device once per chunk
+    assert_within(dtype, batch * h * w_, host(dev, gw).reshape(-1), wgw, GO, X,
+                  extra=(batch + 2) * ULP[dtype] * float(np.abs(wgw).max()), what="grad_filters")
+
+
+def test_conv2d_unbatched_equals_batch_of_one():
+    dev, g = device(), rng(502)
+    announce("conv2d unbatched")
+    x3 = upload(dev, g.standard_normal((3, 12, 12)), "f32")
+    w = upload(dev, g.standard_normal((4, 3, 3, 3)), "f32")
+    y3 = dev.conv2d_forward(x3, w, padding=1)
+    x4 = dev.tensor(dev.to_host(x3).reshape(1, 3, 12, 12), "f32")
+    y4 = dev.conv2d_forward(x4, w, padding=1)
+    assert y3.shape == (4, 12, 12) and y4.shape == (1, 4, 12, 12)
+    np.testing.assert_array_equal(host(dev, y3), host(dev, y4)[0])
+
+
+def test_conv2d_shape_checks():
+    dev = device()
+    x = dev.zeros("f32", (1, 4, 8, 8))
+    with pytest.raises(AssertionError, match="left: 4\n right: 6"):
+        dev.conv2d_forward(x, dev.zeros("f32", (2, 3, 3, 3)), groups=2)
+    with pytest.raises(ValueError, match="must be contiguous"):
+        dev.conv2d_forward(x.permute(0, 1, 3, 2), dev.zeros("f32", (2, 4, 3, 3)))
+
+
+def test_conv2d_batch_larger_than_one_patch_chunk():
+    """A batch whose unfolded patches exceed the per-launch patch budget is processed in several chunks; every
+    chunk boundary must be seamless (outputs of all images, gradients summed over all of them)."""
+    dev, g = device(), rng(503)
+    dtype, (batch, c, h, w_) = "f16", (80, 64, 112, 112)
+    announce("conv2d chunked batch", batch, c, h, w_)
+    cout = 64  # forward patches 14.4 MB per image, backward patches the same: both exceed the budget at batch 80
+    op = Conv2DOp.make(batch, c, cout, h, w_, 3, 1, 1, 1, 1)
+    x = upload(dev, g.standard_normal((batch, c, h, w_)).astype(np.float32), dtype)
+    w = upload(dev, g.standard_normal((cout, c, 3, 3)) / 24.0, dtype)
+    y = dev.conv2d_forward(x, w, padding=1)
+    go = upload(dev, g.standard_normal(y.shape).astype(np.float32), dtype)
+    gx, gw = dev.zeros_like_storage(x), dev.zeros_like_storage(w)
+    dev.conv2d_backward(x, gx, w, gw, go, padding=1)
+    x_h, w_h, go_h = (dev.to_host(t).reshape(-1) for t in (x, w, go))
+    y_h, gx_h = dev.to_host(y).reshape(batch, -1), dev.to_host(gx).reshape(batch, -1)
+    op1 = Conv2DOp.make(1, c, cout, h, w_, 3, 1, 1, 1, 1)
+    per_x, per_y = c * h * w_, cout * h * w_
+    W = oracle.to_f64(w_h, dtype)
+    gw_sum = np.zeros(w_h.size)
+    for b in range(batch):
+        xb, gob = x_h[b * per_x:(b + 1) * per_x], go_h[b * per_y:(b + 1) * per_y]
+        ogx, ogw = np.zeros(per_x, np.float16), np.zeros(w_h.size, np.float32)
+        if b in (0, 36, 37, 73, 74, 79):  # around the chunk boundaries
+            want = oracle.to_f64(conv2d_forward(dtype, op1, xb, w_h), dtype)
+            assert_within(dtype, c * 9, oracle.to_f64(y_h[b], dtype), want, oracle.to_f64(xb, dtype), W, extra=ULP[dtype] * 8, what=f"out[{b}]")
+            conv2d_backward(dtype, op1, xb, ogx, w_h, np.zeros_like(w_h), gob)
+            assert_within(dtype, cout * 9, oracle.to_f64(gx_h[b], dtype), oracle.to_f64(ogx, dtype), oracle.to_f64(gob, dtype), W, extra=ULP[dtype] * 8, what=f"grad_img[{b}]")
+        # filter gradient in float32 per image (exact enough), summed in float64
+        conv2d_backward("f32", op1, oracle.to_f64(xb, dtype).astype(np.float32), np.zeros(per_x, np.float32),
+                        W.astype(np.float32), ogw, oracle.to_f64(gob, dtype).astype(np.float32))
+        gw_sum += ogw
+    got = oracle.to_f64(dev.to_host(gw).reshape(-1), dtype)
+    tol = 2e-3 * np.sqrt(batch * h * w_) * 5.0 * 5.0
+    assert float(np.abs(got - gw_sum).max()) <= tol + 4 * ULP[dtype] * float(np.abs(gw_sum).max())
