@@ -104,7 +104,7 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
         if (v == 0) v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units) : 0;
         const bool ok = is16 ? mfma16_supported(p, v) : is32 ? mfma32_supported(p, v) : false;
         if (!ok) return DFDX_ROCM_ERR_UNSUPPORTED;
-        *plan = {DFDX_ROCM_KERNEL_MFMA, v, 1};
+        *plan = {DFDX_ROCM_KERNEL_MFMA, v, is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
         return DFDX_ROCM_OK;
     }
     case DFDX_ROCM_KERNEL_AUTO:
@@ -126,7 +126,7 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
     }
     int v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units) : 0;
     if (v > 0) {
-        *plan = {DFDX_ROCM_KERNEL_MFMA, v, 1};
+        *plan = {DFDX_ROCM_KERNEL_MFMA, v, is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
         return DFDX_ROCM_OK;
     }
     *plan = {DFDX_ROCM_KERNEL_GENERIC, 0, 1};
@@ -139,7 +139,8 @@ int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan) {
     p.workspace = nullptr;
     p.compute_units = ctx->compute_units;
     if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1) {
-        const size_t need = mfma16dma_workspace_bytes(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
+        const size_t need = p.dtype == DT_F32 ? mfma32_workspace_bytes(p, plan.variant, plan.splits)
+                                              : mfma16dma_workspace_bytes(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
         if (int rc = ensure_workspace(ctx, need)) return rc;
         p.splits = plan.splits;
         p.workspace = (float *)ctx->workspace;
@@ -307,7 +308,8 @@ int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int
     if (variant) *variant = plan.variant;
     if (name && name_len) {
         if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1)
-            std::snprintf(name, name_len, "mfma16_%s_splitk%d", mfma16_variant_name(plan.variant), plan.splits);
+            std::snprintf(name, name_len, "%s_%s_splitk%d", p.dtype == DT_F32 ? "mfma32" : "mfma16",
+                          p.dtype == DT_F32 ? mfma32_variant_name(plan.variant) : mfma16_variant_name(plan.variant), plan.splits);
         else if (plan.kernel == DFDX_ROCM_KERNEL_MFMA)
             std::snprintf(name, name_len, "%s_%s", p.dtype == DT_F32 ? "mfma32" : "mfma16",
                           p.dtype == DT_F32 ? mfma32_variant_name(plan.variant) : mfma16_variant_name(plan.variant));

@@ -33,6 +33,10 @@ struct Params {
     int tiles_m, tiles_n, tiles_per_batch, total_blocks;
     int accumulate, bias_mode, c_vec;
     int group_m;
+    // split-k: k-loop steps [split * chunk, +chunk) per workgroup, f32 partial tiles to ws[split][row][col]
+    int splits, chunk;
+    float *ws;
+    int64_t ws_ld, ws_split_stride;
 };
 
 __device__ __forceinline__ f32x4 ldg4(const float *p, bool pred) {
@@ -86,7 +90,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
     const int l32 = lane % 32, lh = lane / 32;
 
     const int work = xcd_remap(blockIdx.x, p.total_blocks);
-    const int batch = work / p.tiles_per_batch;
+    const int bidx = work / p.tiles_per_batch;  // batch, or k split
+    const int batch = p.splits > 1 ? 0 : bidx;
+    const int split = p.splits > 1 ? bidx : 0;
     const int tile = work % p.tiles_per_batch;
     const int gsize = p.group_m * p.tiles_n;
     const int group = tile / gsize;
@@ -97,7 +103,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
     const int bm0 = tm_idx * BM, bn0 = tn_idx * BN;
 
     const int ktiles = (p.k + BK - 1) / BK;
-    const int iters = ktiles * p.kbatches;
+    const int it0 = split * p.chunk;
+    const int iters = min(ktiles * p.kbatches - it0, p.chunk);
 
     auto a_tile = [&](int it) -> const float * {
         const int kb = p.kbatches > 1 ? it / ktiles : batch;
@@ -129,8 +136,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     if (iters > 0) {
-        la.load(a_tile(0), p.lda, rows_left, k_left(0), tid);
-        lb.load(b_tile(0), p.ldb, cols_left, k_left(0), tid);
+        la.load(a_tile(it0), p.lda, rows_left, k_left(it0), tid);
+        lb.load(b_tile(it0), p.ldb, cols_left, k_left(it0), tid);
         la.store(As, tid);
         lb.store(Bs, tid);
     }
@@ -144,8 +151,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
         const int cur = it & 1;
         const bool more = it + 1 < iters;
         if (more) {
-            la.load(a_tile(it + 1), p.lda, rows_left, k_left(it + 1), tid);
-            lb.load(b_tile(it + 1), p.ldb, cols_left, k_left(it + 1), tid);
+            la.load(a_tile(it0 + it + 1), p.lda, rows_left, k_left(it0 + it + 1), tid);
+            lb.load(b_tile(it0 + it + 1), p.ldb, cols_left, k_left(it0 + it + 1), tid);
         }
         const float *af_base = a_frag0 + cur * LA::LDS_SIZE;
         const float *bf_base = b_frag0 + cur * LB::LDS_SIZE;
@@ -190,6 +197,23 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
     }
 
     // ---- epilogue: lane holds m = l32 (per tile), n = 8g + 4*lh + 0..3 --------
+    if (p.splits > 1) {  // f32 partial tile into the workspace (padded to whole tiles: no bounds checks)
+        float *wbase = p.ws + split * p.ws_split_stride;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            float *wrow = wbase + (int64_t)(bm0 + wm0 + i * 32 + l32) * p.ws_ld + bn0 + wn0 + lh * 4;
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    f32x4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = acc[i][j][g * 4 + e];
+                    *(f32x4 *)(wrow + j * 32 + g * 8) = v;
+                }
+        }
+        return;
+    }
     const int cb = p.kbatches > 1 ? 0 : batch;
     float *cbase = p.c + (int64_t)(cb / p.nb2) * p.c_b1 + (int64_t)(cb % p.nb2) * p.c_b2;
 #pragma unroll
@@ -310,6 +334,38 @@ bool mfma32_supported(const GemmProblem &p, int variant) {
     return true;
 }
 
+// Split-k for small outputs with a long reduction (weight gradients): when the chosen tile shape leaves most of
+// the chip idle, the k loop is cut into up to 16 slices of at least 4 steps each.
+int mfma32_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits) {
+    if (variant < 1 || variant > (int)(sizeof(kVariants) / sizeof(kVariants[0]))) return 1;
+    const Variant &t = kVariants[variant - 1];
+    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+    const int64_t total_iters = ((p.k + t.bk - 1) / t.bk) * (p.reduce ? p.nb1 * p.nb2 : 1);
+    if (nbatch != 1 || p.c_cs != 1 || total_iters < 2) return 1;
+    if (forced_splits > 0) {
+        int64_t s = std::min<int64_t>(forced_splits, total_iters);
+        while (s > 1 && (s - 1) * ((total_iters + s - 1) / s) >= total_iters) s--;  // no empty split
+        return (int)s;
+    }
+    const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn);
+    int64_t s = std::min<int64_t>(std::min<int64_t>(16, compute_units / std::max<int64_t>(1, blocks)), total_iters / 4);
+    while (s > 1 && (s - 1) * ((total_iters + s - 1) / s) >= total_iters) s--;
+    return (int)std::max<int64_t>(1, s);
+}
+
+static void ws_layout32(const GemmProblem &p, int variant, int64_t *ld, int64_t *split_stride) {
+    const Variant &v = kVariants[variant - 1];
+    *ld = ((p.n + v.bn - 1) / v.bn) * v.bn;
+    *split_stride = *ld * (((p.m + v.bm - 1) / v.bm) * v.bm);
+}
+
+size_t mfma32_workspace_bytes(const GemmProblem &p, int variant, int splits) {
+    if (splits <= 1) return 0;
+    int64_t ld, stride;
+    ws_layout32(p, variant, &ld, &stride);
+    return (size_t)stride * splits * sizeof(float);
+}
+
 int mfma32_pick_variant(const GemmProblem &p, int compute_units) {
     const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
     const int order[] = {1, 3, 4, 5, 6};
@@ -322,6 +378,8 @@ int mfma32_pick_variant(const GemmProblem &p, int compute_units) {
     }
     return mfma32_supported(p, 6) ? 6 : 0;
 }
+
+static hipError_t launch_tiles(const Params &p, int variant, bool a_kc, bool b_kc, hipStream_t stream);
 
 hipError_t launch_mfma32(const GemmProblem &g, int variant, hipStream_t stream) {
     if (!mfma32_supported(g, variant)) return hipErrorInvalidValue;
@@ -345,6 +403,24 @@ hipError_t launch_mfma32(const GemmProblem &g, int variant, hipStream_t stream) 
     p.c_vec = (g.n % 4 == 0) && (p.ldc % 4 == 0) && (((uintptr_t)g.c & 15u) == 0) &&
               (g.c_b1 % 4 == 0) && (g.c_b2 % 4 == 0) && (!g.bias || ((uintptr_t)g.bias & 15u) == 0);
     p.group_m = 4;
+    const int total_iters = (int)(((g.k + v.bk - 1) / v.bk) * p.kbatches);
+    p.splits = 1; p.chunk = total_iters; p.ws = nullptr; p.ws_ld = 0; p.ws_split_stride = 0;
+    if (g.splits > 1) {
+        if (!g.workspace || p.total_blocks != p.tiles_per_batch) return hipErrorInvalidValue;
+        p.splits = g.splits;
+        p.chunk = (total_iters + g.splits - 1) / g.splits;
+        if ((int64_t)(g.splits - 1) * p.chunk >= total_iters) return hipErrorInvalidValue;
+        p.ws = g.workspace;
+        ws_layout32(g, variant, &p.ws_ld, &p.ws_split_stride);
+        p.total_blocks = p.tiles_per_batch * g.splits;
+    }
+    hipError_t e = launch_tiles(p, variant, la.kc, lb.kc, stream);
+    if (e != hipSuccess || g.splits <= 1) return e;
+    return launch_splitk_reduce(g, p.ws_ld, p.ws_split_stride, stream);
+}
+
+static hipError_t launch_tiles(const Params &p, int variant, bool a_kc, bool b_kc, hipStream_t stream) {
+    struct { bool kc; } la{a_kc}, lb{b_kc};
     switch (variant) {
     case 1: return launch_layout<256, 256, 32, 2, 4>(p, la.kc, lb.kc, stream);
     case 2: return launch_layout<256, 256, 32, 2, 2>(p, la.kc, lb.kc, stream);

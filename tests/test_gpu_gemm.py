@@ -200,7 +200,7 @@ def test_gemv(dtype, shape, layout):
 
 
 # ------------------------------------------------------------------ split-k --
-@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("layout", ["tn", "nt", "nn"])
 @pytest.mark.parametrize("splits", [2, 3, 8])
 def test_split_k_forced(dtype, layout, splits):
@@ -233,6 +233,33 @@ def test_split_k_is_planned_for_weight_gradients_and_is_deterministic():
     assert_within(dtype, k, oracle.to_f64(outs[0], dtype).reshape(m, n), want, A, B, extra=2.0 ** -11 * np.abs(want).max())
     # NO_SPLIT_K keeps the plain kernel
     desc = dev.gemm_desc(dtype, m, k, n, da.ptr, (1, m), db.ptr, (n, 1), dc.ptr, (n, 1), accumulate=True, no_split_k=True)
+    assert "splitk" not in dev.gemm_plan(desc)[2]
+
+
+def test_split_k_f32_planned_for_long_reductions():
+    """f32: a small output with a long contraction (weight gradient, reduce-over-batch) is cut along k, gives the
+    same bits on every run and stays within the f32 tolerance; NO_SPLIT_K switches it off."""
+    dev, g = device(), rng(78)
+    m, k, n, nb, dtype = 64, 3136, 576, 8, "f32"
+    a = oracle.to_storage(g.standard_normal(nb * m * k), dtype)
+    b = oracle.to_storage(g.standard_normal(nb * n * k), dtype)     # stored (nb, n, k): B^T per batch
+    da, db = dev.tensor(a, dtype), dev.tensor(b, dtype)
+    outs = []
+    for _ in range(2):
+        dc = dev.zeros(dtype, (m, n))
+        desc = dev.gemm_desc(dtype, m, k, n, da.ptr, (k, 1), db.ptr, (1, k), dc.ptr, (n, 1), accumulate=True,
+                             batch=(nb, 1), a_batch=(m * k, 0), b_batch=(n * k, 0), reduce_batch=True)
+        name = dev.gemm_plan(desc)[2]
+        assert "mfma32" in name and "splitk" in name, name
+        announce("planned f32 split-k", name)
+        dev.gemm(desc)
+        outs.append(dev.to_host(dc))
+    assert np.array_equal(outs[0], outs[1])
+    A, B = oracle.to_f64(a, dtype).reshape(nb, m, k), oracle.to_f64(b, dtype).reshape(nb, n, k)
+    want = np.einsum("bmk,bnk->mn", A, B)
+    assert_within(dtype, nb * k, oracle.to_f64(outs[0], dtype).reshape(m, n), want, A, B)
+    desc = dev.gemm_desc(dtype, m, k, n, da.ptr, (k, 1), db.ptr, (1, k), dc.ptr, (n, 1), accumulate=True,
+                         batch=(nb, 1), a_batch=(m * k, 0), b_batch=(n * k, 0), reduce_batch=True, no_split_k=True)
     assert "splitk" not in dev.gemm_plan(desc)[2]
 
 
