@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Per-GEMM timings of the five workload configurations on one MI355X, plus the ops around them.
+
+`bench.py` reports the headline metric (4096^3); this companion times every GEMM shape the configurations contain
+(Linear forward / dX / dW at small f32 size, broadcast-rhs f16, attention-shaped batched f16, the encoder block's
+bf16 Linears, vec.mat / mat.vec), the HBM-bound ops between them (softmax, bias, reshape) and a few conv2d
+layers.  GEMMs are timed with HIP events on the library's stream (dfdx_rocm_gemm_time), the other ops with
+events around a loop of calls.  One line per case on stdout; `--json FILE` also writes them as JSON.
+
+Synthetic inputs, resident in HBM before timing.  Nothing here touches the CPU oracle.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--json", default=None, help="also write the rows to this file")
+    ap.add_argument("--iters", type=int, default=30)
+    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,gemv,glue,conv")
+    args = ap.parse_args()
+    import torch
+    from dfdx_amd import Rocm
+    from dfdx_amd.rocm import View
+
+    if not torch.cuda.is_available():
+        sys.exit("bench_configs.py needs a GPU")
+    dev = Rocm(0)
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
+    esz = {"f16": 2, "bf16": 2, "f32": 4}
+    only = set(filter(None, args.only.split(",")))
+    rows = []
+
+    def want(group):
+        return not only or group in only
+
+    def rnd(shape, dtype, scale=1.0):
+        return (torch.randn(*shape, device="cuda") * scale).to(tdt[dtype])
+
+    def zeros(shape, dtype):
+        return torch.zeros(*shape, device="cuda", dtype=tdt[dtype])
+
+    def view(t, dtype):
+        return View(t.view(torch.uint8).reshape(-1), dtype, tuple(t.shape), tuple(t.stride()))
+
+    def report(group, name, flop, nbytes, ms, kernel):
+        row = {"group": group, "case": name, "kernel": kernel, "us": round(ms * 1e3, 2),
+               "tflops": round(flop / ms / 1e9, 1) if flop else None,
+               "gbps": round(nbytes / ms / 1e6, 1) if nbytes else None}
+        rows.append(row)
+        print(f"{group:5s} {name:44s} {kernel:40s} {row['us']:9.1f} us "
+              f"{(str(row['tflops']) + ' TFLOP/s') if flop else '':>16s} {(str(row['gbps']) + ' GB/s') if nbytes else '':>14s}",
+              flush=True)
+
+    def gemm(group, name, desc, flop, nbytes, iters=None):
+        ms = dev.gemm_time(desc, 5, iters or args.iters)
+        report(group, name, flop, nbytes, ms, dev.gemm_plan(desc)[2])
+
+    def timed(group, name, fn, flop, nbytes, kernel):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        report(group, name, flop, nbytes, e0.elapsed_time(e1) / args.iters, kernel)
+
+    P = lambda t: t.data_ptr()
+
+    # ---- config 1: Linear 512 -> 256 on 64 rows, f32 (latency-bound) ------------------------------------------
+    if want("c1"):
+        dt, (r, i, o), es = "f32", (64, 512, 256), 4
+        x, w, go = rnd((r, i), dt), rnd((o, i), dt, 0.04), rnd((r, o), dt)
+        y, gx, gw = zeros((r, o), dt), zeros((r, i), dt), zeros((o, i), dt)
+        fl = 2 * r * i * o
+        gemm("c1", "Linear fwd 64x512x256 NT", dev.gemm_desc(dt, r, i, o, P(x), (i, 1), P(w), (1, i), P(y), (o, 1)),
+             fl, es * (r * i + i * o + r * o), 200)
+        gemm("c1", "dX 64x256x512 NN acc", dev.gemm_desc(dt, r, o, i, P(go), (o, 1), P(w), (i, 1), P(gx), (i, 1), accumulate=True),
+             fl, es * (r * o + i * o + 2 * r * i), 200)
+        gemm("c1", "dW 512x64x256 TN col-major C acc",
+             dev.gemm_desc(dt, i, r, o, P(x), (1, i), P(go), (o, 1), P(gw), (1, i), accumulate=True),
+             fl, es * (r * o + r * i + 2 * i * o), 200)
+
+    # ---- config 3: [32,512,1024] x [1024,1024], f16, broadcast rhs ---------------------------------------------
+    if want("c3"):
+        dt, (B, M, K, N), es = "f16", (32, 512, 1024, 1024), 2
+        lhs, rhs, go = rnd((B, M, K), dt), rnd((K, N), dt, 1 / 32), rnd((B, M, N), dt)
+        out, gl, gr = zeros((B, M, N), dt), zeros((B, M, K), dt), zeros((K, N), dt)
+        fl = 2 * B * M * K * N
+        gemm("c3", "fwd 16384x1024x1024 NN", dev.gemm_desc(dt, B * M, K, N, P(lhs), (K, 1), P(rhs), (N, 1), P(out), (N, 1)),
+             fl, es * (B * M * K + K * N + B * M * N))
+        gemm("c3", "fwd, rhs = Linear weight view NT",
+             dev.gemm_desc(dt, B * M, K, N, P(lhs), (K, 1), P(rhs), (1, K), P(out), (N, 1)), fl, es * (B * M * K + K * N + B * M * N))
+        gemm("c3", "dX 16384x1024x1024 NT acc",
+             dev.gemm_desc(dt, B * M, N, K, P(go), (N, 1), P(rhs), (1, N), P(gl), (K, 1), accumulate=True),
+             fl, es * (B * M * N + K * N + 2 * B * M * K))
+        gemm("c3", "dW 1024x16384x1024 TN acc",
+             dev.gemm_desc(dt, K, B * M, N, P(lhs), (1, K), P(go), (N, 1), P(gr), (N, 1), accumulate=True),
+             fl, es * (B * M * K + B * M * N + 2 * K * N))
+        lv, rv, gov, glv, grv = (view(t, dt) for t in (lhs, rhs, go, gl, gr))
+        timed("c3", "MatMatBr forward (trait call, allocates out)", lambda: dev.forward(lv, rv), fl, 0, "br_forward")
+        timed("c3", "MatMatBr backward (trait call, dX + dW)", lambda: dev.backward(lv, glv, rv, grv, gov), 2 * fl, 0, "br_backward")
+        del lhs, rhs, go, out, gl, gr
+
+    # ---- config 4: attention-shaped Rank-4, f16 -----------------------------------------------------------------
+    if want("c4"):
+        dt, (Bq, H, S, D), es = "f16", (8, 16, 1024, 64), 2
+        q, k, v, d_o = (rnd((Bq, H, S, D), dt) for _ in range(4))
+        sc = zeros((Bq, H, S, S), dt)
+        p = torch.softmax(torch.randn(Bq, H, S, S, device="cuda"), -1).to(tdt[dt])
+        o, gp, gv, gq, gk = zeros((Bq, H, S, D), dt), zeros((Bq, H, S, S), dt), zeros((Bq, H, S, D), dt), zeros((Bq, H, S, D), dt), zeros((Bq, H, S, D), dt)
+        nb = Bq * H
+        sSD, sSS = (H * S * D, S * D), (H * S * S, S * S)
+        fl = 2 * nb * S * S * D
+
+        def d4(m, kk, n, a, astr, ab, b, bstr, bb, c, cstr, cb, acc):
+            return dev.gemm_desc(dt, m, kk, n, P(a), astr, P(b), bstr, P(c), cstr, accumulate=acc, batch=(Bq, H),
+                                 a_batch=ab, b_batch=bb, c_batch=cb)
+
+        gemm("c4", "scores Q.K^T 1024x64x1024 NT", d4(S, D, S, q, (D, 1), sSD, k, (1, D), sSD, sc, (S, 1), sSS, False),
+             fl, es * nb * (2 * S * D + S * S))
+        gemm("c4", "out P.V 1024x1024x64 NN", d4(S, S, D, p, (S, 1), sSS, v, (D, 1), sSD, o, (D, 1), sSD, False),
+             fl, es * nb * (S * S + 2 * S * D))
+        gemm("c4", "dP dO.V^T NT acc", d4(S, D, S, d_o, (D, 1), sSD, v, (1, D), sSD, gp, (S, 1), sSS, True),
+             fl, es * nb * (2 * S * D + 2 * S * S))
+        gemm("c4", "dV P^T.dO TN acc", d4(S, S, D, p, (1, S), sSS, d_o, (D, 1), sSD, gv, (D, 1), sSD, True),
+             fl, es * nb * (S * S + 3 * S * D))
+        gemm("c4", "dQ dS.K NN acc", d4(S, S, D, gp, (S, 1), sSS, k, (D, 1), sSD, gq, (D, 1), sSD, True),
+             fl, es * nb * (S * S + 3 * S * D))
+        gemm("c4", "dK^T Q^T.dS col-major C acc", d4(D, S, S, q, (1, D), sSD, gp, (S, 1), sSS, gk, (1, D), sSD, True),
+             fl, es * nb * (S * S + 3 * S * D))
+        if want("glue"):
+            scv, pv, gpv, ov = view(sc, dt), view(p, dt), view(gp, dt), view(o, dt)
+            mat = nb * S * S * es
+            timed("glue", "softmax fwd (8,16,1024,1024) f16, scale folded", lambda: dev.softmax_forward(scv, 0.125), 0, 2 * mat, "softmax_forward")
+            gsv = view(zeros((Bq, H, S, S), dt), dt)
+            timed("glue", "softmax bwd (8,16,1024,1024) f16", lambda: dev.softmax_backward(pv, gsv, gpv, 0.125), 0, 4 * mat, "softmax_backward")
+            tok = nb * S * D * es
+            timed("glue", "reshape copy (B,H,S,D)->(B,S,H*D) f16", lambda: dev.reshape_forward(ov.permute(0, 2, 1, 3), (Bq, S, H * D)), 0, 2 * tok, "reshape_forward")
+            gt = view(rnd((Bq, S, H * D), dt), dt)
+            gov = view(zeros((Bq, H, S, D), dt), dt)
+            timed("glue", "reshape backward (scatter-add) f16", lambda: dev.reshape_backward(ov.permute(0, 2, 1, 3), gov, gt), 0, 3 * tok, "reshape_backward")
+        del sc, p, gp
+
+    # ---- config 5: the encoder block's Linears, bf16, 8192 tokens ----------------------------------------------
+    if want("c5"):
+        dt, T = "bf16", 8192
+        for name, kin, nout in (("qkv / out proj", 1024, 1024), ("ff1", 1024, 4096), ("ff2", 4096, 1024)):
+            x, w, go = rnd((T, kin), dt), rnd((nout, kin), dt, 0.02), rnd((T, nout), dt)
+            y, gx, gw = zeros((T, nout), dt), zeros((T, kin), dt), zeros((nout, kin), dt)
+            fl = 2 * T * kin * nout
+            gemm("c5", f"{name} fwd {T}x{kin}x{nout} NT", dev.gemm_desc(dt, T, kin, nout, P(x), (kin, 1), P(w), (1, kin), P(y), (nout, 1)), fl, 0)
+            gemm("c5", f"{name} dX NN acc", dev.gemm_desc(dt, T, nout, kin, P(go), (nout, 1), P(w), (kin, 1), P(gx), (kin, 1), accumulate=True), fl, 0)
+            gemm("c5", f"{name} dW TN col-major C acc",
+                 dev.gemm_desc(dt, kin, T, nout, P(x), (1, kin), P(go), (nout, 1), P(gw), (1, kin), accumulate=True), fl, 0)
+            if want("glue"):
+                gov, gbv, bv = view(go, dt), view(zeros((nout,), dt), dt), view(rnd((nout,), dt), dt)
+                timed("glue", f"bias backward {T}x{nout} bf16", lambda: dev.bias_backward(gov, gbv), 0, T * nout * 2, "bias_backward")
+
+    # ---- vec.mat / mat.vec: HBM roofline ------------------------------------------------------------------------
+    if want("gemv"):
+        for dt in ("f16", "f32"):
+            es = esz[dt]
+            for n_ in (4096, 16384):
+                W, xv, yv = rnd((n_, n_), dt), rnd((n_,), dt), zeros((n_,), dt)
+                gemm("gemv", f"vec.mat {dt} (1,{n_})x({n_},{n_})", dev.gemm_desc(dt, 1, n_, n_, P(xv), (n_, 1), P(W), (n_, 1), P(yv), (n_, 1)), 2 * n_ * n_, es * n_ * n_, 100)
+                gemm("gemv", f"vec.mat {dt}, Linear weight view", dev.gemm_desc(dt, 1, n_, n_, P(xv), (n_, 1), P(W), (1, n_), P(yv), (n_, 1)), 2 * n_ * n_, es * n_ * n_, 100)
+                gemm("gemv", f"mat.vec {dt} ({n_},{n_})x({n_},)", dev.gemm_desc(dt, n_, n_, 1, P(W), (n_, 1), P(xv), (1, 1), P(yv), (1, 1)), 2 * n_ * n_, es * n_ * n_, 100)
+                del W
+
+    # ---- conv2d (unfold + batched GEMM) -------------------------------------------------------------------------
+    if want("conv"):
+        for dt, (B, C, O, H, W_, K, s, pad) in (("f16", (64, 64, 64, 56, 56, 3, 1, 1)), ("f16", (64, 128, 128, 28, 28, 3, 1, 1)),
+                                                ("f32", (32, 64, 64, 56, 56, 3, 1, 1))):
+            x, w = rnd((B, C, H, W_), dt), rnd((O, C, K, K), dt, 1 / 24)
+            xv, wv = view(x, dt), view(w, dt)
+            y = dev.conv2d_forward(xv, wv, stride=s, padding=pad)
+            gov = view(rnd(y.shape, dt), dt)
+            gxv, gwv = view(zeros((B, C, H, W_), dt), dt), view(zeros((O, C, K, K), dt), dt)
+            fl = 2.0 * B * O * C * K * K * y.shape[2] * y.shape[3]
+            tag = f"{dt} B{B} {C}->{O} {H}x{W_} k{K}"
+            timed("conv", f"conv2d fwd {tag}", lambda: dev.conv2d_forward(xv, wv, stride=s, padding=pad), fl, 0, "unfold + gemm")
+            timed("conv", f"conv2d bwd {tag}", lambda: dev.conv2d_backward(xv, gxv, wv, gwv, gov, stride=s, padding=pad), 2 * fl, 0, "unfold + 2 gemm")
+
+    if args.json:
+        with open(args.json, "w") as f:
+            json.dump({"device": dev.device_info(), "rows": rows}, f, indent=1)
+
+
+if __name__ == "__main__":
+    main()
