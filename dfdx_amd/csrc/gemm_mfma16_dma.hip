@@ -31,6 +31,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short v4i16 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 #define DFDX_LDS __attribute__((address_space(3)))
@@ -66,6 +67,10 @@ template <> struct Mma<_Float16> {
     }
     static __device__ __forceinline__ float to_f32(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
     static __device__ __forceinline__ uint16_t from_f32(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // v_cvt_pk_f16_f32: RNE, lo in bits 15:0
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, h2));
+    }
 };
 template <> struct Mma<__bf16> {
     static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
@@ -76,6 +81,10 @@ template <> struct Mma<__bf16> {
         uint32_t x = __float_as_uint(v);
         if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
         return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);  // round to nearest even
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // v_cvt_pk_bf16_f32: RNE, quiet NaNs
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, b2));
     }
 };
 
@@ -347,48 +356,62 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
         // 8*(lq/2) .. +3 and +4 .. +7 of tile j + (lq & 1).  A wave instruction then writes 64 contiguous
         // bytes per matrix row instead of 32, which is what the memory system needs to reach its write rate.
         if (p.c_vec8) {
+            // PLAIN: the tile lies inside C and the store is a pure overwrite -- no bounds checks, no bias, no
+            // read of C (every forward product of whole tiles; the k = 64 products of attention above all).
+            auto rows = [&](auto plain_tag) {
+                constexpr bool PLAIN = decltype(plain_tag)::value;
 #pragma unroll
-            for (int i = 0; i < TM; i++) {
-                const int gm_row = bm0 + wm0 + i * 16 + l16;
-                const bool row_ok = gm_row < p.m;
-                uint16_t *crow = cbase + (int64_t)gm_row * p.ldc;
-                float rbias = 0.0f;
-                if (p.bias_mode == BIAS_PER_ROW && row_ok) rbias = Mma<T>::to_f32(p.bias[gm_row]);
+                for (int i = 0; i < TM; i++) {
+                    const int gm_row = bm0 + wm0 + i * 16 + l16;
+                    const bool row_ok = PLAIN || gm_row < p.m;
+                    uint16_t *crow = cbase + (int64_t)gm_row * p.ldc;
+                    float rbias = 0.0f;
+                    if constexpr (!PLAIN)
+                        if (p.bias_mode == BIAS_PER_ROW && row_ok) rbias = Mma<T>::to_f32(p.bias[gm_row]);
 #pragma unroll
-                for (int jp = 0; jp < TN / 2; jp++) {
-                    float v[8];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i][2 * jp][e]),
-                                                                        __float_as_uint(acc[i][2 * jp + 1][e]), false, false);
-                        v[e] = __uint_as_float(r[0]) + rbias;
-                        v[4 + e] = __uint_as_float(r[1]) + rbias;
-                    }
-                    const int gn = bn0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8;
-                    if (!row_ok || gn >= p.n) continue;  // n % 8 == 0 here: all 8 columns are in range
-                    if (p.bias_mode == BIAS_PER_COL) {
-                        const u32x4 bv = *(const u32x4 *)(p.bias + gn);
+                    for (int jp = 0; jp < TN / 2; jp++) {
+                        float v[8];
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            v[2 * e] += Mma<T>::to_f32((uint16_t)(bv[e] & 0xffffu));
-                            v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(bv[e] >> 16));
+                            const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i][2 * jp][e]),
+                                                                            __float_as_uint(acc[i][2 * jp + 1][e]), false, false);
+                            v[e] = __uint_as_float(r[0]);
+                            v[4 + e] = __uint_as_float(r[1]);
                         }
-                    }
-                    if (p.accumulate) {
-                        const u32x4 old = *(const u32x4 *)(crow + gn);
+                        const int gn = bn0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8;
+                        if constexpr (!PLAIN) {
+                            if (!row_ok || gn >= p.n) continue;  // n % 8 == 0 here: all 8 columns are in range
+                            if (p.bias_mode == BIAS_PER_ROW) {
 #pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            v[2 * e] += Mma<T>::to_f32((uint16_t)(old[e] & 0xffffu));
-                            v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(old[e] >> 16));
+                                for (int e = 0; e < 8; e++) v[e] += rbias;
+                            }
+                            if (p.bias_mode == BIAS_PER_COL) {
+                                const u32x4 bv = *(const u32x4 *)(p.bias + gn);
+#pragma unroll
+                                for (int e = 0; e < 4; e++) {
+                                    v[2 * e] += Mma<T>::to_f32((uint16_t)(bv[e] & 0xffffu));
+                                    v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(bv[e] >> 16));
+                                }
+                            }
+                            if (p.accumulate) {
+                                const u32x4 old = *(const u32x4 *)(crow + gn);
+#pragma unroll
+                                for (int e = 0; e < 4; e++) {
+                                    v[2 * e] += Mma<T>::to_f32((uint16_t)(old[e] & 0xffffu));
+                                    v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(old[e] >> 16));
+                                }
+                            }
                         }
-                    }
-                    u32x4 o;
+                        u32x4 o;
 #pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        o[e] = (uint32_t)Mma<T>::from_f32(v[2 * e]) | ((uint32_t)Mma<T>::from_f32(v[2 * e + 1]) << 16);
-                    *(u32x4 *)(crow + gn) = o;
+                        for (int e = 0; e < 4; e++) o[e] = Mma<T>::pack2(v[2 * e], v[2 * e + 1]);
+                        *(u32x4 *)(crow + gn) = o;
+                    }
                 }
-            }
+            };
+            const bool plain = bm0 + BM <= p.m && bn0 + BN <= p.n && p.bias_mode == BIAS_NONE && !p.accumulate;
+            if (plain) rows(std::true_type{});
+            else rows(std::false_type{});
             return;
         }
     }
