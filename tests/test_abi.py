@@ -33,7 +33,9 @@ def test_every_declaration_cites_the_reference():
     """Each block of declarations names the reference interface it replaces (file:line)."""
     text = open(HEADER).read()
     for needle in ("cpu_kernel.rs:38-50", "cuda_kernel.rs:153-181", "matmul/mod.rs:116-131", "matmul/mod.rs:197-212",
-                   "matmul/mod.rs:234-249", "matmul/mod.rs:273-288", "linear.rs:82-89", "cuda/device.rs:259-266"):
+                   "matmul/mod.rs:234-249", "matmul/mod.rs:273-288", "linear.rs:82-89", "cuda/device.rs:259-266",
+                   "bias1d.rs:62-78", "utilities/cpu_kernels.rs:164-203", "softmax.rs:70-83", "mul/cpu_kernel.rs:\n * 5-17",
+                   "reshape_to/mod.rs:90-115", "conv2d/mod.rs:31-55", "multi_head_attention.rs:\n * 105-146"):
         assert needle in text, needle
 
 
@@ -52,6 +54,24 @@ def test_desc_struct_layout_matches_c(tmp_path):
     want = [ctypes.sizeof(GemmDesc), GemmDesc.m.offset, GemmDesc.a.offset, GemmDesc.b.offset, GemmDesc.c.offset,
             GemmDesc.bias.offset, GemmDesc.kernel.offset]
     assert got == want
+
+
+def test_conv2d_op_layout_matches_c(tmp_path):
+    """dfdx_rocm_conv2d_op is twelve size_t in the reference's field order (conv2d/mod.rs:14-29)."""
+    from dfdx_amd.rocm import Conv2DOp
+
+    src = tmp_path / "conv.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "dfdx_rocm.h"\n'
+        "int main(void){printf(\"%zu %zu %zu %zu %zu\\n\", sizeof(dfdx_rocm_conv2d_op), offsetof(dfdx_rocm_conv2d_op,kernel),"
+        "offsetof(dfdx_rocm_conv2d_op,groups), offsetof(dfdx_rocm_conv2d_op,chan_in), offsetof(dfdx_rocm_conv2d_op,w_out));return 0;}\n")
+    exe = tmp_path / "conv"
+    subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
+    got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    assert got == [ctypes.sizeof(Conv2DOp), Conv2DOp.kernel.offset, Conv2DOp.groups.offset, Conv2DOp.chan_in.offset,
+                   Conv2DOp.w_out.offset]
+    assert [n for n, _ in Conv2DOp._fields_] == ["kernel", "stride", "padding", "dilation", "groups", "batch", "chan_in",
+                                                 "chan_out", "h_in", "h_out", "w_in", "w_out"]
 
 
 def test_header_compiles_as_c_and_cxx(tmp_path):
@@ -77,6 +97,14 @@ def test_calls_fail_cleanly_without_a_device():
     assert ctx.value is None
     assert lib.dfdx_rocm_gemm(None, None) == -1
     assert lib.dfdx_rocm_synchronize(None) == -1
+    # the entry points around the matmuls refuse a null context the same way
+    i64, vp = ctypes.c_int64, ctypes.c_void_p
+    assert lib.dfdx_rocm_bias_forward(None, 0, i64(1), i64(1), vp(), vp(), vp()) == -1
+    assert lib.dfdx_rocm_bias_backward(None, 0, i64(1), i64(1), vp(), vp()) == -1
+    assert lib.dfdx_rocm_softmax_forward(None, 0, i64(1), i64(1), vp(), ctypes.c_float(1.0), vp()) == -1
+    assert lib.dfdx_rocm_reshape_forward(None, 0, 1, vp(), vp(), vp(), vp()) == -1
+    assert lib.dfdx_rocm_scalar_mul_forward(None, 0, i64(1), vp(), ctypes.c_double(1.0), vp()) == -1
+    assert lib.dfdx_rocm_conv2d_forward(None, 0, vp(), vp(), vp(), vp()) == -1
     assert b"gfx950" in lib.dfdx_rocm_strerror(-3)
     assert lib.dfdx_rocm_mfma_variant_count(1) >= 6
     with pytest.raises(RuntimeError):  # the Python mirror refuses too: there is no CPU fallback
