@@ -151,11 +151,20 @@ template <typename T> __global__ __launch_bounds__(256) void gemv_dots_kernel(co
     }
 }
 
-template <typename T> __global__ __launch_bounds__(256) void gemv_combine_kernel(const Params p) {
-    const int j = blockIdx.x * 256 + threadIdx.x;
+template <typename T> __global__ __launch_bounds__(64) void gemv_combine_kernel(const Params p) {
+    const int j = blockIdx.x * 64 + threadIdx.x;
     if (j >= p.j) return;
-    float v = p.ws[j];
-    for (int s = 1; s < p.kslices; s++) v += p.ws[(int64_t)s * p.j + j];
+    const float *src = p.ws + j;
+    float v = 0.0f;
+    int s = 0;
+    for (; s + 8 <= p.kslices; s += 8) {  // eight loads in flight, added in slice order
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) t[u] = src[(int64_t)(s + u) * p.j];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v += t[u];
+    }
+    for (; s < p.kslices; s++) v += src[(int64_t)s * p.j];
     finish<T>(p, j, v);
 }
 
@@ -210,7 +219,7 @@ void plan_slices(Shape &s, int dtype) {
     int slices = 1;
     if (s.cols) {
         slices = (p.k + KCHUNK_MAX - 1) / KCHUNK_MAX;  // the vector slice must fit the LDS buffer
-        while (blocks_j * slices < 256 && p.k / (slices * 2) >= 256) slices *= 2;
+        while (blocks_j * slices < 512 && p.k / (slices * 2) >= 128) slices *= 2;
     } else {
         while (blocks_j * slices < 512 && p.k / (slices * 2) >= 64 * vec) slices *= 2;
     }
@@ -231,7 +240,7 @@ template <typename T> hipError_t launch_t(const Shape &s, hipStream_t stream) {
         dim3 grid((unsigned)((p.j + 3) / 4), (unsigned)p.kslices);
         gemv_dots_kernel<T><<<grid, 256, 0, stream>>>(p);
     }
-    if (p.kslices > 1) gemv_combine_kernel<T><<<dim3((unsigned)((p.j + 255) / 256)), 256, 0, stream>>>(p);
+    if (p.kslices > 1) gemv_combine_kernel<T><<<dim3((unsigned)((p.j + 63) / 64)), 64, 0, stream>>>(p);
     return hipGetLastError();
 }
 
