@@ -16,7 +16,7 @@ int bind(dfdx_rocm_ctx *ctx) {
 }
 
 static int grow(dfdx_rocm_ctx *ctx, void **buf, size_t *have, size_t bytes) {
-    std::lock_guard<std::mutex> lock(ctx->mu);
+    CtxLock lock(ctx->mu);
     if (bytes <= *have) return DFDX_ROCM_OK;
     if (*buf) {
         HIP_TRY(hipStreamSynchronize(ctx->stream));
@@ -134,6 +134,7 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
 }
 
 int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan) {
+    CtxLock lock(ctx->mu);  // a split plan is two launches around the shared workspace
     GemmProblem p = problem;
     p.splits = 1;
     p.workspace = nullptr;

@@ -119,6 +119,7 @@ int bias_backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *
     slices = std::min<int64_t>(slices, 65535);
     const int64_t rows_per_slice = (rows + slices - 1) / slices;
     slices = (rows + rows_per_slice - 1) / rows_per_slice;
+    CtxLock lock(ctx->mu);  // two launches around the shared workspace
     float *partial = nullptr;
     if (slices > 1) {
         if (int rc = ensure_workspace(ctx, (size_t)slices * cols * sizeof(float))) return rc;

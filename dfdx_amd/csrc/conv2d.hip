@@ -122,6 +122,7 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
     const int64_t per_image = (int64_t)op.chan_in * kk * n;  // patch elements of one image
     if (per_image == 0 || m == 0) return DFDX_ROCM_OK;
     if (per_image >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
+    CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
     int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
     chunk = std::min<int64_t>(std::min<int64_t>(chunk, op.batch), ((1ll << 31) - 1) / per_image);
     if (int rc = ensure_patches(ctx, (size_t)(chunk * per_image) * sizeof(T))) return rc;
@@ -157,6 +158,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     const int64_t f_elems = (int64_t)op.groups * cg * og * kk;
     if (per_image == 0 || f_elems == 0 || ohw == 0) return DFDX_ROCM_OK;
     if (per_image >= (1ll << 31) || f_elems >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
+    CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
     int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
     chunk = std::min<int64_t>(std::min<int64_t>(chunk, op.batch), ((1ll << 31) - 1) / per_image);
     // patch buffer: [chunk][O*K*K][H*W], then the transposed filters and their gradient

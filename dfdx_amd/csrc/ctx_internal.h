@@ -11,7 +11,9 @@ struct dfdx_rocm_ctx {
     int compute_units;
     int clock_mhz;
     char name[128];
-    std::mutex mu;
+    // Serialises every call sequence that uses `workspace` or `patches` (several launches that must not
+    // interleave with another host thread's on the same stream); recursive because conv2d holds it across its GEMMs.
+    std::recursive_mutex mu;
     void *workspace = nullptr;  // partial sums of split reductions; grown on demand, owned by the context
     size_t workspace_bytes = 0;
     void *patches = nullptr;  // unfolded images of conv2d (alive across the GEMMs that may regrow `workspace`)
@@ -25,6 +27,8 @@ namespace dfdx_rocm {
         hipError_t e__ = (expr);                \
         if (e__ != hipSuccess) return (int)e__; \
     } while (0)
+
+typedef std::lock_guard<std::recursive_mutex> CtxLock;
 
 // Makes the context's device current for the calling thread.
 int bind(dfdx_rocm_ctx *ctx);

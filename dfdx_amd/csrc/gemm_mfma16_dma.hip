@@ -507,7 +507,7 @@ struct Variant {
 // X(id, BM, BN, WAVES_M, WAVES_N); ids are 1-based inside this family.
 #define DFDX_MFMA16_DMA_VARIANTS(X) \
     X(1, 256, 256, 2, 4)            \
-    X(2, 256, 128, 2, 4)            \
+    X(2, 256, 128, 4, 2)            \
     X(3, 128, 128, 2, 4)            \
     X(4, 256, 64, 4, 2)             \
     X(5, 128, 64, 2, 4)
