@@ -233,21 +233,44 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
         b_off[ks] = (wn0 + l16) * BK * 2 + ((c ^ ((l16 >> 1) & 7)) * 16);
     }
     // m/n-contiguous: lane 16*g + L supplies the address of X[k = 8*g + L/4 (+32*ks, +4)][col = w0 + 16*t + 4*(L%4)];
-    // the transposing read hands lane L the 4 k-values of column w0 + 16*t + L.
+    // the transposing read hands lane L the 4 k-values of column w0 + 16*t + L.  k + 4 and k + 32 leave the
+    // swizzle bits of k alone, so the four reads of one 16-column tile (two k steps x two halves) differ only by
+    // immediate offsets from one per-lane address.
+    //
+    // These reads are issued from inline asm: the compiler puts a vmcnt(0) in front of every transposing-read
+    // builtin while an LDS-DMA load is outstanding (it cannot see that the load targets the other stage), which
+    // would make the prefetched tile arrive half a tile early.  The price is that the compiler does not track
+    // their completion either: every consumer sits behind an explicit `fence` (see below).
     const int tr_k = lq * 8 + l16 / 4;
     const int tr_col = 4 * (l16 % 4);
-    auto tr_frag = [&](const uint8_t *tile_base, auto rows_tag, int ks, int col0) -> u32x4 {
+    auto tr_base = [&](auto rows_tag, int col0) -> uint32_t {  // byte offset inside the operand tile, k step 0, low half
         constexpr int ROWS = decltype(rows_tag)::value;
         const int col = col0 + tr_col;
-        const int k = ks * 32 + tr_k;   // k and k+4 share the swizzle (same k & 3 pattern shifted by 4: see below)
         const int c = col / 8, half = (col / 4) % 2;
-        const int off0 = k * ROWS * 2 + ((c ^ mc_swizzle<ROWS>(k)) * 16) + half * 8;
-        const int off1 = (k + 4) * ROWS * 2 + ((c ^ mc_swizzle<ROWS>(k + 4)) * 16) + half * 8;
-        const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DFDX_LDS v4i16 *)(tile_base + off0));
-        const v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DFDX_LDS v4i16 *)(tile_base + off1));
-        const u32x2 l = __builtin_bit_cast(u32x2, lo), h = __builtin_bit_cast(u32x2, hi);
+        return (uint32_t)(tr_k * ROWS * 2 + ((c ^ mc_swizzle<ROWS>(tr_k)) * 16) + half * 8);
+    };
+    uint32_t a_tr[A_KC ? 1 : TM], b_tr[B_KC ? 1 : TN];
+    if constexpr (!A_KC) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) a_tr[i] = tr_base(std::integral_constant<int, BM>{}, wm0 + i * 16);
+    }
+    if constexpr (!B_KC) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) b_tr[j] = TA::BYTES + tr_base(std::integral_constant<int, BN>{}, wn0 + j * 16);
+    }
+    auto lds_addr = [](const uint8_t *p) -> uint32_t { return (uint32_t)(uintptr_t)(DFDX_LDS const uint8_t *)p; };
+    auto tr_frag = [&](uint32_t addr, auto rows_tag, auto ks_tag) -> u32x4 {
+        constexpr int OFF = decltype(ks_tag)::value * 32 * decltype(rows_tag)::value * 2;
+        constexpr int HI = 4 * decltype(rows_tag)::value * 2;
+        u32x2 l, h;
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(l) : "v"(addr), "i"(OFF));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(h) : "v"(addr), "i"(OFF + HI));
         return u32x4{l[0], l[1], h[0], h[1]};
     };
+    // `fence<N>(x...)`: at most N LDS operations issued by this wave may still be outstanding (they complete in
+    // order); the fragments passed in are re-defined by the asm so that nothing that uses them can move above it.
+    auto tie = [](u32x4 &x) { asm volatile("" : "+v"(x)); };
+    constexpr int OPS_A = A_KC ? 1 : 2, OPS_B = B_KC ? 1 : 2;  // LDS instructions per fragment
 
     f32x4 acc[TM][TN];
 #pragma unroll
@@ -258,20 +281,43 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
             for (int v = 0; v < 4; v++) acc[i][j][v] = 0.0f;
 
     u32x4 fa[TM], fb[2][TN];
-    auto read_a = [&](const uint8_t *sa, int ks, int i0, int i1) {
+    auto read_a = [&](const uint8_t *sa, auto ks_tag, int i0, int i1) {
+        constexpr int ks = decltype(ks_tag)::value;
+        [[maybe_unused]] const uint32_t base = lds_addr(sa);
 #pragma unroll
         for (int i = 0; i < TM; i++)
             if (i >= i0 && i < i1) {
                 if constexpr (A_KC) fa[i] = *(const u32x4 *)(sa + a_off[ks] + i * 16 * BK * 2);
-                else fa[i] = tr_frag(sa, std::integral_constant<int, BM>{}, ks, wm0 + i * 16);
+                else fa[i] = tr_frag(base + a_tr[i], std::integral_constant<int, BM>{}, ks_tag);
             }
     };
-    auto read_b = [&](const uint8_t *sa, int ks, u32x4(&bf)[TN]) {
+    auto read_b = [&](const uint8_t *sa, auto ks_tag, u32x4(&bf)[TN]) {
+        constexpr int ks = decltype(ks_tag)::value;
         const uint8_t *sb = sa + TA::BYTES;
+        [[maybe_unused]] const uint32_t base = lds_addr(sa);
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             if constexpr (B_KC) bf[j] = *(const u32x4 *)(sb + b_off[ks] + j * 16 * BK * 2);
-            else bf[j] = tr_frag(sb, std::integral_constant<int, BN>{}, ks, wn0 + j * 16);
+            else bf[j] = tr_frag(base + b_tr[j], std::integral_constant<int, BN>{}, ks_tag);
+        }
+    };
+    // Completion of the asm-issued (transposing) reads.  `left` = LDS instructions issued after the youngest one
+    // that must be complete; the hardware counter saturates the wait at 15.
+    auto fence_a = [&](auto left_tag, int i0, int i1) {
+        if constexpr (!A_KC) {
+            constexpr int LEFT = decltype(left_tag)::value > 15 ? 15 : decltype(left_tag)::value;
+            asm volatile("s_waitcnt lgkmcnt(%0)" ::"i"(LEFT));
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                if (i >= i0 && i < i1) tie(fa[i]);
+        }
+    };
+    auto fence_b = [&](auto left_tag, u32x4(&bf)[TN]) {
+        if constexpr (!B_KC) {
+            constexpr int LEFT = decltype(left_tag)::value > 15 ? 15 : decltype(left_tag)::value;
+            asm volatile("s_waitcnt lgkmcnt(%0)" ::"i"(LEFT));
+#pragma unroll
+            for (int j = 0; j < TN; j++) tie(bf[j]);
         }
     };
     // swapped operands: the lane ends up with m = l16 and 4 consecutive n = 4*lq + 0..3 per 16x16 tile
@@ -297,40 +343,62 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
 
     // one 64-wide k tile from stage `cs`; HAS_NEXT: the next tile belongs to the same work item (hand the stage
     // over and prefetch its first fragments while the last MFMAs of this tile run)
+    // LDS instructions per group of reads, as issued below: half of the A fragments, all B fragments of a k step
+    constexpr int RA = 2 * Q * OPS_A, RB = TN * OPS_B;
+    constexpr std::integral_constant<int, 0> K0{};
+    constexpr std::integral_constant<int, 1> K1{};
+#define DFDX_LEFT(n) std::integral_constant<int, (n)> {}
+    // First fragments of a tile, in the order the fences of tile_body assume: A rows [0, 2Q), B, A rows [2Q, TM).
+    auto read_first = [&](const uint8_t *st) {
+        read_a(st, K0, 0, 2 * Q);
+        read_b(st, K0, fb[0]);
+        read_a(st, K0, 2 * Q, TM);
+    };
     auto tile_body = [&](int cs, auto has_next_tag) {
         constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
         const uint8_t *sa = smem + cs * STAGE_BYTES;
         const uint8_t *sn = smem + (cs ^ 1) * STAGE_BYTES;
-        // ---- k step 0 (B buffer 0); prefetch k step 1 of this tile
+        // ---- k step 0 (B buffer 0); prefetch k step 1 of this tile.  Outstanding on entry, oldest first:
+        //      A[0,2Q), B, A[2Q,TM) of this k step.
+        fence_b(DFDX_LEFT(RA), fb[0]);
+        fence_a(DFDX_LEFT(RA / 2 + RB + RA), 0, Q);
         mma(fb[0], 0, Q);
         __builtin_amdgcn_sched_barrier(0);
+        fence_a(DFDX_LEFT(RB + RA), Q, 2 * Q);
         mma(fb[0], Q, 2 * Q);
         __builtin_amdgcn_sched_barrier(0);
+        fence_a(DFDX_LEFT(RA / 2), 2 * Q, 3 * Q);
         mma(fb[0], 2 * Q, 3 * Q);
         __builtin_amdgcn_sched_barrier(0);
-        read_a(sa, 1, 0, 2 * Q);
-        read_b(sa, 1, fb[1]);
+        read_a(sa, K1, 0, 2 * Q);
+        read_b(sa, K1, fb[1]);
         __builtin_amdgcn_sched_barrier(0);
+        fence_a(DFDX_LEFT(RA + RB), 3 * Q, TM);
         mma(fb[0], 3 * Q, TM);
         __builtin_amdgcn_sched_barrier(0);
         // ---- k step 1 (B buffer 1); prefetch k step 0 of the next tile
+        fence_b(DFDX_LEFT(0), fb[1]);
+        fence_a(DFDX_LEFT(RA / 2 + RB), 0, Q);
         mma(fb[1], 0, Q);
         __builtin_amdgcn_sched_barrier(0);
-        read_a(sa, 1, 2 * Q, TM);
+        read_a(sa, K1, 2 * Q, TM);
         __builtin_amdgcn_sched_barrier(0);
+        fence_a(DFDX_LEFT(RB + RA), Q, 2 * Q);
         mma(fb[1], Q, 2 * Q);
         __builtin_amdgcn_sched_barrier(0);
+        fence_a(DFDX_LEFT(RA / 2), 2 * Q, 3 * Q);
         mma(fb[1], 2 * Q, 3 * Q);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (HAS_NEXT) {
             sync_tile();
-            read_a(sn, 0, 0, 2 * Q);
-            read_b(sn, 0, fb[0]);
+            read_a(sn, K0, 0, 2 * Q);
+            read_b(sn, K0, fb[0]);
         }
         __builtin_amdgcn_sched_barrier(0);
+        fence_a(DFDX_LEFT(HAS_NEXT ? RA + RB : 0), 3 * Q, TM);
         mma(fb[1], 3 * Q, TM);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (HAS_NEXT) read_a(sn, 0, 2 * Q, TM);
+        if constexpr (HAS_NEXT) read_a(sn, K0, 2 * Q, TM);
         __builtin_amdgcn_sched_barrier(0);
     };
 
@@ -467,8 +535,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
     int c_left = cw.iters, c_stage = 0;
     issue();
     sync_tile();
-    read_a(smem, 0, 0, TM);
-    read_b(smem, 0, fb[0]);
+    read_first(smem);
     for (;;) {
         for (; c_left > 1; --c_left) {
             tile_body(c_stage, std::true_type{});
@@ -491,11 +558,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
         c_index += gridDim.x;
         cw = decode(c_index);
         c_left = cw.iters;
-        read_a(smem + c_stage * STAGE_BYTES, 0, 0, TM);
-        read_b(smem + c_stage * STAGE_BYTES, 0, fb[0]);
+        read_first(smem + c_stage * STAGE_BYTES);
     }
 }
 
+
+#undef DFDX_LEFT
 
 // ------------------------------------------------------------------ host side --
 
