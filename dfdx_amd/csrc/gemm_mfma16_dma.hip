@@ -737,8 +737,7 @@ void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_va
         const VariantModel &vm = kModel[v - 1];
         if (forced_variant == 0 && ((p.n <= 64) != (t.bn <= 64))) continue;  // BN = 64 tiles only for narrow outputs
         const int64_t tiles = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
-        double layout = (a_kc && b_kc) ? 1.0 : (!a_kc && !b_kc) ? 0.955 : 1.0;  // transposing LDS reads cost a little
-        if (v == 2 && !(a_kc && b_kc)) layout *= 0.87;
+        const double layout = (a_kc && b_kc) ? 1.0 : (!a_kc && !b_kc) ? 0.98 : 0.99;  // transposing LDS reads cost a little
         for (int s = 1; s <= 16; s++) {
             if (forced_splits > 0 && s != std::min<int64_t>(forced_splits, total_iters)) continue;
             if (s > 1 && (!may_split || (forced_splits == 0 && total_iters / s < 4))) break;
