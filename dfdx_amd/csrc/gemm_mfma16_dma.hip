@@ -51,7 +51,7 @@ struct Params {
     int64_t a_b1, a_b2, b_b1, b_b2, c_b1, c_b2;
     int nb2, kbatches;
     int tiles_m, tiles_n, tiles_per_batch, total_blocks;
-    int accumulate, bias_mode, c_vec, c_vec8;
+    int accumulate, bias_mode;
     int group_m;
     // split-k: `splits` workgroups per C tile, each covering `chunk` k-loop steps, f32 partials in `ws`
     int splits, chunk;
@@ -423,7 +423,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
         // rows 1 and 3 of x against lane rows 0 and 2 of y: afterwards lane row lq holds, in (x, y), columns
         // 8*(lq/2) .. +3 and +4 .. +7 of tile j + (lq & 1).  A wave instruction then writes 64 contiguous
         // bytes per matrix row instead of 32, which is what the memory system needs to reach its write rate.
-        if (p.c_vec8) {
+        {
             // PLAIN: the tile lies inside C and the store is a pure overwrite -- no bounds checks, no bias, no
             // read of C (every forward product of whole tiles; the k = 64 products of attention above all).
             auto rows = [&](auto plain_tag) {
@@ -483,20 +483,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
             return;
         }
     }
+    if constexpr (TN % 2 != 0) {  // a single 16-column tile per wave: 8 B per lane (the host guarantees n % 4 == 0 etc.)
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-        const int gm_row = bm0 + wm0 + i * 16 + l16;
-        if (gm_row >= p.m) continue;
-        uint16_t *crow = cbase + (int64_t)gm_row * p.ldc;
-        const float rbias = (p.bias_mode == BIAS_PER_ROW) ? Mma<T>::to_f32(p.bias[gm_row]) : 0.0f;
+        for (int i = 0; i < TM; i++) {
+            const int gm_row = bm0 + wm0 + i * 16 + l16;
+            if (gm_row >= p.m) continue;
+            uint16_t *crow = cbase + (int64_t)gm_row * p.ldc;
+            const float rbias = (p.bias_mode == BIAS_PER_ROW) ? Mma<T>::to_f32(p.bias[gm_row]) : 0.0f;
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int gn = bn0 + wn0 + j * 16 + lq * 4;
-            if (gn >= p.n) continue;
-            float v[4];
+            for (int j = 0; j < TN; j++) {
+                const int gn = bn0 + wn0 + j * 16 + lq * 4;
+                if (gn >= p.n) continue;  // n % 4 == 0: the 4 columns are all in range
+                float v[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = acc[i][j][e] + rbias;
-            if (p.c_vec) {  // n % 4 == 0 here, so the 4 columns are all in range
+                for (int e = 0; e < 4; e++) v[e] = acc[i][j][e] + rbias;
                 if (p.bias_mode == BIAS_PER_COL) {
                     const u32x2 bv = *(const u32x2 *)(p.bias + gn);
                     v[0] += Mma<T>::to_f32((uint16_t)(bv[0] & 0xffffu));
@@ -511,19 +511,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
                     v[2] += Mma<T>::to_f32((uint16_t)(old[1] & 0xffffu));
                     v[3] += Mma<T>::to_f32((uint16_t)(old[1] >> 16));
                 }
-                u32x2 o;
-                o[0] = (uint32_t)Mma<T>::from_f32(v[0]) | ((uint32_t)Mma<T>::from_f32(v[1]) << 16);
-                o[1] = (uint32_t)Mma<T>::from_f32(v[2]) | ((uint32_t)Mma<T>::from_f32(v[3]) << 16);
-                *(u32x2 *)(crow + gn) = o;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    if (gn + e >= p.n) break;
-                    float x = v[e];
-                    if (p.bias_mode == BIAS_PER_COL) x += Mma<T>::to_f32(p.bias[gn + e]);
-                    if (p.accumulate) x += Mma<T>::to_f32(crow[gn + e]);
-                    crow[gn + e] = Mma<T>::from_f32(x);
-                }
+                *(u32x2 *)(crow + gn) = u32x2{Mma<T>::pack2(v[0], v[1]), Mma<T>::pack2(v[2], v[3])};
             }
         }
     }
@@ -664,6 +652,13 @@ bool mfma16dma_supported(const GemmProblem &p, int variant) {
     const Variant &v = kVariants[variant - 1];
     if (la.ld * (la.kc ? v.bm : BK) >= (1ll << 30) || lb.ld * (lb.kc ? v.bn : BK) >= (1ll << 30)) return false;
     if (!aligned16(p.a) || !aligned16(p.b)) return false;
+    {   // the epilogue stores whole 16 B (8 B for the 16-column wave tile) pieces of C rows and nothing narrower
+        const int vecw = (v.bn / v.waves_n) % 32 == 0 ? 8 : 4;
+        const int64_t ldc = p.m == 1 ? p.n : p.c_rs;
+        const uintptr_t mask = (uintptr_t)vecw * 2 - 1;
+        if (p.n % vecw || ldc % vecw || ((uintptr_t)p.c & mask) || p.c_b1 % vecw || p.c_b2 % vecw) return false;
+        if (p.bias && ((uintptr_t)p.bias & mask)) return false;
+    }
     if (p.nb1 * p.nb2 > 1) {
         if (p.a_b1 % 8 || p.a_b2 % 8 || p.b_b1 % 8 || p.b_b2 % 8) return false;
         if (p.a_b1 < 0 || p.a_b2 < 0 || p.b_b1 < 0 || p.b_b2 < 0) return false;
@@ -799,10 +794,6 @@ hipError_t launch_mfma16dma(const GemmProblem &g, int variant, hipStream_t strea
     p.tiles_per_batch = p.tiles_m * p.tiles_n;
     p.total_blocks = p.tiles_per_batch * (g.reduce ? 1 : nbatch);
     p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
-    p.c_vec = (g.n % 4 == 0) && (p.ldc % 4 == 0) && (((uintptr_t)g.c & 7u) == 0) &&
-              (g.c_b1 % 4 == 0) && (g.c_b2 % 4 == 0) && (!g.bias || ((uintptr_t)g.bias & 7u) == 0);
-    p.c_vec8 = p.c_vec && (g.n % 8 == 0) && (p.ldc % 8 == 0) && (((uintptr_t)g.c & 15u) == 0) &&
-               (g.c_b1 % 8 == 0) && (g.c_b2 % 8 == 0) && (!g.bias || ((uintptr_t)g.bias & 15u) == 0);
     p.group_m = 4;
     const int total_iters = (p.k / BK) * p.kbatches;
     p.splits = 1; p.chunk = total_iters; p.ws = nullptr; p.ws_ld = 0; p.ws_split_stride = 0;
