@@ -15,51 +15,80 @@ struct Op {  // dfdx_rocm_conv2d_op narrowed to 32 bits (validated on entry)
 };
 
 // patches[b][c][k1][k2][oh][ow] = img[b][c][oh*stride + dilation*k1 - padding][ow*stride + dilation*k2 - padding],
-// zero outside the image.  One thread writes N consecutive ow (w_out % N == 0).
+// zero outside the image.  One workgroup per (b, c, k1, k2) slab, so that the index arithmetic per element is a
+// row counter: a thread owns one group of N consecutive ow (w_out % N == 0) and walks down the output rows.
 template <typename T, int N>
-__global__ __launch_bounds__(256) void unfold_input_kernel(Op op, const T *img, T *patches, uint32_t groups) {
-    const uint32_t wg = (uint32_t)op.w_out / N;
-    for (uint32_t t = blockIdx.x * 256 + threadIdx.x; t < groups; t += gridDim.x * 256) {
-        uint32_t r = t;
-        const int ow0 = (int)(r % wg) * N; r /= wg;
-        const int oh = (int)(r % op.h_out); r /= op.h_out;
-        const int k2 = (int)(r % op.kernel); r /= op.kernel;
-        const int k1 = (int)(r % op.kernel); r /= op.kernel;  // r = b * chan_in + c
+__global__ __launch_bounds__(256) void unfold_input_kernel(Op op, const T *img, T *patches) {
+    const uint32_t slab = blockIdx.x;
+    const int kk = op.kernel * op.kernel;
+    const int k2 = (int)(slab % op.kernel), k1 = (int)((slab / op.kernel) % op.kernel);
+    const uint32_t r = slab / kk;  // b * chan_in + c
+    const int wg = op.w_out / N;
+    const T *plane = img + (int64_t)r * op.h_in * op.w_in;
+    T *dst = patches + (int64_t)slab * op.h_out * op.w_out;
+    auto emit = [&](int oh, int owg) {
         const int y = oh * op.stride + op.dilation * k1 - op.padding;
-        const T *row = img + ((int64_t)r * op.h_in + y) * op.w_in;
+        const T *row = plane + (int64_t)y * op.w_in;
         float v[N];
+        const int x0 = owg * N * op.stride + op.dilation * k2 - op.padding;
+        if (N > 1 && op.stride == 1 && y >= 0 && y < op.h_in && x0 >= 0 && x0 + N <= op.w_in) {
+            load_elems_unaligned<T, N>(row + x0, v);  // unit stride, window inside the row: N consecutive pixels
+        } else {
 #pragma unroll
-        for (int i = 0; i < N; i++) {
-            const int x = (ow0 + i) * op.stride + op.dilation * k2 - op.padding;
-            v[i] = (y >= 0 && y < op.h_in && x >= 0 && x < op.w_in) ? Elem<T>::load(row + x) : 0.0f;
+            for (int i = 0; i < N; i++) {
+                const int x = x0 + i * op.stride;
+                v[i] = (y >= 0 && y < op.h_in && x >= 0 && x < op.w_in) ? Elem<T>::load(row + x) : 0.0f;
+            }
         }
-        store_elems<T, N>(patches + (int64_t)t * N, v);
+        store_elems<T, N>(dst + (int64_t)oh * op.w_out + owg * N, v);
+    };
+    const int step_rows = 256 / wg;  // rows covered per pass; 0 when a row has more than 256 groups
+    if (step_rows) {
+        if ((int)threadIdx.x >= step_rows * wg) return;
+        const int owg = (int)threadIdx.x % wg;
+        for (int oh = (int)threadIdx.x / wg; oh < op.h_out; oh += step_rows) emit(oh, owg);
+    } else {
+        for (int g = threadIdx.x; g < op.h_out * wg; g += 256) emit(g / wg, g % wg);
     }
 }
 
 // patches[b][o][k1][k2][y][x] = grad_out[b][o][oh][ow] where oh*stride = y + padding - dilation*k1 (likewise ow),
-// zero when no output position reads image pixel (y, x) through filter tap (k1, k2).
+// zero when no output position reads image pixel (y, x) through filter tap (k1, k2).  Same slab mapping.
 template <typename T, int N>
-__global__ __launch_bounds__(256) void unfold_output_kernel(Op op, const T *grad_out, T *patches, uint32_t groups) {
-    const uint32_t wg = (uint32_t)op.w_in / N;
-    for (uint32_t t = blockIdx.x * 256 + threadIdx.x; t < groups; t += gridDim.x * 256) {
-        uint32_t r = t;
-        const int x0 = (int)(r % wg) * N; r /= wg;
-        const int y = (int)(r % op.h_in); r /= op.h_in;
-        const int k2 = (int)(r % op.kernel); r /= op.kernel;
-        const int k1 = (int)(r % op.kernel); r /= op.kernel;  // r = b * chan_out + o
+__global__ __launch_bounds__(256) void unfold_output_kernel(Op op, const T *grad_out, T *patches) {
+    const uint32_t slab = blockIdx.x;
+    const int kk = op.kernel * op.kernel;
+    const int k2 = (int)(slab % op.kernel), k1 = (int)((slab / op.kernel) % op.kernel);
+    const uint32_t r = slab / kk;  // b * chan_out + o
+    const int wg = op.w_in / N;
+    const T *plane = grad_out + (int64_t)r * op.h_out * op.w_out;
+    T *dst = patches + (int64_t)slab * op.h_in * op.w_in;
+    auto emit = [&](int y, int xg) {
         int oh = y + op.padding - op.dilation * k1;
         const bool row_ok = oh >= 0 && oh % op.stride == 0 && oh / op.stride < op.h_out;
         oh /= op.stride;
-        const T *row = grad_out + ((int64_t)r * op.h_out + oh) * op.w_out;
+        const T *row = plane + (int64_t)oh * op.w_out;
         float v[N];
+        const int ow0 = xg * N + op.padding - op.dilation * k2;
+        if (N > 1 && op.stride == 1 && row_ok && ow0 >= 0 && ow0 + N <= op.w_out) {
+            load_elems_unaligned<T, N>(row + ow0, v);  // unit stride, window inside the row
+        } else {
 #pragma unroll
-        for (int i = 0; i < N; i++) {
-            const int ow = x0 + i + op.padding - op.dilation * k2;
-            const bool ok = row_ok && ow >= 0 && ow % op.stride == 0 && ow / op.stride < op.w_out;
-            v[i] = ok ? Elem<T>::load(row + ow / op.stride) : 0.0f;
+            for (int i = 0; i < N; i++) {
+                const int ow = ow0 + i;
+                const bool ok = row_ok && ow >= 0 && ow % op.stride == 0 && ow / op.stride < op.w_out;
+                v[i] = ok ? Elem<T>::load(row + ow / op.stride) : 0.0f;
+            }
         }
-        store_elems<T, N>(patches + (int64_t)t * N, v);
+        store_elems<T, N>(dst + (int64_t)y * op.w_in + xg * N, v);
+    };
+    const int step_rows = 256 / wg;
+    if (step_rows) {
+        if ((int)threadIdx.x >= step_rows * wg) return;
+        const int xg = (int)threadIdx.x % wg;
+        for (int y = (int)threadIdx.x / wg; y < op.h_in; y += step_rows) emit(y, xg);
+    } else {
+        for (int g = threadIdx.x; g < op.h_in * wg; g += 256) emit(g / wg, g % wg);
     }
 }
 
@@ -134,9 +163,9 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
         Op sub = op;
         sub.batch = (int)nb;
         const T *src = (const T *)img + b0 * op.chan_in * op.h_in * op.w_in;
-        const uint64_t elems = (uint64_t)nb * per_image;
-        if (vec) unfold_input_kernel<T, V><<<grid_for<T>(ctx, elems / V), 256, 0, ctx->stream>>>(sub, src, patches, (uint32_t)(elems / V));
-        else unfold_input_kernel<T, 1><<<grid_for<T>(ctx, elems), 256, 0, ctx->stream>>>(sub, src, patches, (uint32_t)elems);
+        const unsigned slabs = (unsigned)(nb * op.chan_in * kk);
+        if (vec) unfold_input_kernel<T, V><<<slabs, 256, 0, ctx->stream>>>(sub, src, patches);
+        else unfold_input_kernel<T, 1><<<slabs, 256, 0, ctx->stream>>>(sub, src, patches);
         HIP_TRY(hipGetLastError());
         // filters (G, O/G, C/G*K*K) . patches (B, G, C/G*K*K, OH*OW) -> out (B, G, O/G, OH*OW)
         dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
@@ -180,9 +209,9 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         Op sub = op;
         sub.batch = (int)nb;
         const T *go = (const T *)grad_out + b0 * op.chan_out * ohw;
-        const uint64_t elems = (uint64_t)nb * per_image;
-        if (vec) unfold_output_kernel<T, V><<<grid_for<T>(ctx, elems / V), 256, 0, ctx->stream>>>(sub, go, patches, (uint32_t)(elems / V));
-        else unfold_output_kernel<T, 1><<<grid_for<T>(ctx, elems), 256, 0, ctx->stream>>>(sub, go, patches, (uint32_t)elems);
+        const unsigned slabs = (unsigned)(nb * op.chan_out * kk);
+        if (vec) unfold_output_kernel<T, V><<<slabs, 256, 0, ctx->stream>>>(sub, go, patches);
+        else unfold_output_kernel<T, 1><<<slabs, 256, 0, ctx->stream>>>(sub, go, patches);
         HIP_TRY(hipGetLastError());
         {   // grad_img (B, G, C/G, H*W) += filters^T (G, C/G, O/G*K*K) . patches (B, G, O/G*K*K, H*W)
             const int64_t m = cg, k = og * kk, n = hw;

@@ -43,6 +43,21 @@ template <typename T, int N> __device__ __forceinline__ void load_elems(const T 
         for (int i = 0; i < N; i++) v[i] = Elem<T>::load(p + i);
     }
 }
+// The same from an address that is only element-aligned (one unaligned 16-byte load; global memory allows it).
+template <typename T, int N> __device__ __forceinline__ void load_elems_unaligned(const T *p, float (&v)[N]) {
+    if constexpr (N == Elem<T>::VEC) {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
+        const u32x4 raw = *(const u32x4_unaligned *)p;
+        T tmp[N];
+        __builtin_memcpy(tmp, &raw, 16);
+#pragma unroll
+        for (int i = 0; i < N; i++) v[i] = Elem<T>::load(&tmp[i]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; i++) v[i] = Elem<T>::load(p + i);
+    }
+}
 template <typename T, int N> __device__ __forceinline__ void store_elems(T *p, const float (&v)[N]) {
     if constexpr (N == Elem<T>::VEC) {
         typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
