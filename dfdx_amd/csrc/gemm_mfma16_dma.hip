@@ -477,8 +477,51 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
                     }
                 }
             };
-            const bool plain = bm0 + BM <= p.m && bn0 + BN <= p.n && p.bias_mode == BIAS_NONE && !p.accumulate;
-            if (plain) rows(std::true_type{});
+            // beta = 1 on an interior tile without bias (every gradient product of whole tiles): all old values are
+            // requested before the first store goes out.  While loads and stores are outstanding together the
+            // compiler can only wait for everything (the two kinds may complete out of order), so the interleaved
+            // form of `rows` drains the stores of the tile sixteen times; here the loads overlap each other and
+            // are waited for in issue order.
+            auto rows_accumulate = [&]() {
+                constexpr int IG = TM * (TN / 2) > 8 ? TM / 2 : TM;  // tile rows per batch: at most 8 vectors in flight
+                // wave-uniform base (scalar registers) + one 32-bit per-lane byte offset: no address VGPRs per access
+                const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+                const int wm0_u = (wave_u / WAVES_N) * WTM, wn0_u = (wave_u % WAVES_N) * WTN;
+                char *base = (char *)(cbase + (int64_t)(bm0 + wm0_u) * p.ldc + bn0 + wn0_u);
+                const uint32_t lane_off = (uint32_t)(l16 * (int)p.ldc + (lq & 1) * 16 + (lq >> 1) * 8) * 2u;
+                const int64_t row_step = p.ldc * 32;  // 16 rows, bytes
+#pragma unroll
+                for (int i0 = 0; i0 < TM; i0 += IG) {
+                    u32x4 old[IG][TN / 2];
+#pragma unroll
+                    for (int i = 0; i < IG; i++)
+#pragma unroll
+                        for (int jp = 0; jp < TN / 2; jp++)
+                            old[i][jp] = *(const u32x4 *)(base + (i0 + i) * row_step + jp * 64 + lane_off);
+#pragma unroll
+                    for (int i = 0; i < IG; i++)
+#pragma unroll
+                        for (int jp = 0; jp < TN / 2; jp++) {
+                            float v[8];
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i0 + i][2 * jp][e]),
+                                                                                __float_as_uint(acc[i0 + i][2 * jp + 1][e]), false, false);
+                                v[e] = __uint_as_float(r[0]);
+                                v[4 + e] = __uint_as_float(r[1]);
+                            }
+                            u32x4 o;
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                o[e] = Mma<T>::pack2(v[2 * e] + Mma<T>::to_f32((uint16_t)(old[i][jp][e] & 0xffffu)),
+                                                     v[2 * e + 1] + Mma<T>::to_f32((uint16_t)(old[i][jp][e] >> 16)));
+                            *(u32x4 *)(base + (i0 + i) * row_step + jp * 64 + lane_off) = o;
+                        }
+                }
+            };
+            const bool interior = bm0 + BM <= p.m && bn0 + BN <= p.n && p.bias_mode == BIAS_NONE;
+            if (interior && !p.accumulate) rows(std::true_type{});
+            else if (interior && p.ldc < (1 << 26)) rows_accumulate();
             else rows(std::false_type{});
             return;
         }
