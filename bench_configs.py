@@ -157,6 +157,9 @@ def main():
             y, gx, gw = zeros((T, nout), dt), zeros((T, kin), dt), zeros((nout, kin), dt)
             fl = 2 * T * kin * nout
             gemm("c5", f"{name} fwd {T}x{kin}x{nout} NT", dev.gemm_desc(dt, T, kin, nout, P(x), (kin, 1), P(w), (1, kin), P(y), (nout, 1)), fl, 0)
+            bvec = rnd((nout,), dt)
+            gemm("c5", f"{name} fwd with fused bias (Linear)",
+                 dev.gemm_desc(dt, T, kin, nout, P(x), (kin, 1), P(w), (1, kin), P(y), (nout, 1), bias=P(bvec)), fl, 0)
             gemm("c5", f"{name} dX NN acc", dev.gemm_desc(dt, T, nout, kin, P(go), (nout, 1), P(w), (kin, 1), P(gx), (kin, 1), accumulate=True), fl, 0)
             gemm("c5", f"{name} dW TN col-major C acc",
                  dev.gemm_desc(dt, kin, T, nout, P(x), (1, kin), P(go), (nout, 1), P(gw), (1, kin), accumulate=True), fl, 0)

@@ -424,18 +424,31 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
         // 8*(lq/2) .. +3 and +4 .. +7 of tile j + (lq & 1).  A wave instruction then writes 64 contiguous
         // bytes per matrix row instead of 32, which is what the memory system needs to reach its write rate.
         {
-            // PLAIN: the tile lies inside C and the store is a pure overwrite -- no bounds checks, no bias, no
-            // read of C (every forward product of whole tiles; the k = 64 products of attention above all).
+            // PLAIN: the tile lies inside C and the store is a pure overwrite, optionally with a per-column bias --
+            // no bounds checks, no read of C (every forward product of whole tiles, Linear's fused bias included).
             auto rows = [&](auto plain_tag) {
                 constexpr bool PLAIN = decltype(plain_tag)::value;
+                // The bias values depend on the column (or row) only: they are fetched before the first store, so
+                // that a fused Linear forward has no load waiting behind its own stores.
+                u32x4 cbias[TN / 2];
+                float rbias_all[PLAIN ? 1 : TM];
+                if (p.bias_mode == BIAS_PER_COL) {
+#pragma unroll
+                    for (int jp = 0; jp < TN / 2; jp++)
+                        cbias[jp] = *(const u32x4 *)(p.bias + min(bn0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8, p.n - 8));
+                }
+                if constexpr (!PLAIN) {
+                    if (p.bias_mode == BIAS_PER_ROW) {
+#pragma unroll
+                        for (int i = 0; i < TM; i++) rbias_all[i] = Mma<T>::to_f32(p.bias[min(bm0 + wm0 + i * 16 + l16, p.m - 1)]);
+                    }
+                }
 #pragma unroll
                 for (int i = 0; i < TM; i++) {
                     const int gm_row = bm0 + wm0 + i * 16 + l16;
                     const bool row_ok = PLAIN || gm_row < p.m;
                     uint16_t *crow = cbase + (int64_t)gm_row * p.ldc;
-                    float rbias = 0.0f;
-                    if constexpr (!PLAIN)
-                        if (p.bias_mode == BIAS_PER_ROW && row_ok) rbias = Mma<T>::to_f32(p.bias[gm_row]);
+                    [[maybe_unused]] const float rbias = PLAIN ? 0.0f : rbias_all[PLAIN ? 0 : i];
 #pragma unroll
                     for (int jp = 0; jp < TN / 2; jp++) {
                         float v[8];
@@ -453,14 +466,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
 #pragma unroll
                                 for (int e = 0; e < 8; e++) v[e] += rbias;
                             }
-                            if (p.bias_mode == BIAS_PER_COL) {
-                                const u32x4 bv = *(const u32x4 *)(p.bias + gn);
+                        }
+                        if (p.bias_mode == BIAS_PER_COL) {
+                            const u32x4 bv = cbias[jp];
 #pragma unroll
-                                for (int e = 0; e < 4; e++) {
-                                    v[2 * e] += Mma<T>::to_f32((uint16_t)(bv[e] & 0xffffu));
-                                    v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(bv[e] >> 16));
-                                }
+                            for (int e = 0; e < 4; e++) {
+                                v[2 * e] += Mma<T>::to_f32((uint16_t)(bv[e] & 0xffffu));
+                                v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(bv[e] >> 16));
                             }
+                        }
+                        if constexpr (!PLAIN) {
                             if (p.accumulate) {
                                 const u32x4 old = *(const u32x4 *)(crow + gn);
 #pragma unroll
@@ -519,9 +534,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
                         }
                 }
             };
-            const bool interior = bm0 + BM <= p.m && bn0 + BN <= p.n && p.bias_mode == BIAS_NONE;
+            const bool interior = bm0 + BM <= p.m && bn0 + BN <= p.n && p.bias_mode != BIAS_PER_ROW;
             if (interior && !p.accumulate) rows(std::true_type{});
-            else if (interior && p.ldc < (1 << 26)) rows_accumulate();
+            else if (interior && p.bias_mode == BIAS_NONE && p.ldc < (1 << 26)) rows_accumulate();
             else rows(std::false_type{});
             return;
         }
