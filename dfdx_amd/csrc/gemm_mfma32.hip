@@ -222,6 +222,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
         if (gm_row >= p.m) continue;
         float *crow = cbase + (int64_t)gm_row * p.ldc;
         const float rbias = (p.bias_mode == BIAS_PER_ROW) ? p.bias[gm_row] : 0.0f;
+        // beta = 1: the old values of this row block are all requested before its first store (clamped addresses);
+        // a load issued behind a store can only be waited for together with every outstanding store
+        f32x4 old[TN][4];
+        if (p.c_vec && p.accumulate) {
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) old[j][g] = *(const f32x4 *)(crow + min(bn0 + wn0 + j * 32 + g * 8 + lh * 4, p.n - 4));
+        }
 #pragma unroll
         for (int j = 0; j < TN; j++) {
 #pragma unroll
@@ -233,7 +242,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
                 for (int e = 0; e < 4; e++) v[e] = acc[i][j][g * 4 + e] + rbias;
                 if (p.c_vec) {
                     if (p.bias_mode == BIAS_PER_COL) v += *(const f32x4 *)(p.bias + gn);
-                    if (p.accumulate) v += *(const f32x4 *)(crow + gn);
+                    if (p.accumulate) v += old[j][g];
                     *(f32x4 *)(crow + gn) = v;
                 } else {
 #pragma unroll
