@@ -29,6 +29,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection aid: 3 plain 256 MiB device copies, then 5 headline GEMM launches, nothing else")
+    ap.add_argument("--probe-variants", action="store_true",
+                    help="counter-collection aid: 3 launches of the headline GEMM with every f16 MFMA tile variant forced in turn")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -55,6 +57,22 @@ def main():
             dev.gemm(desc)
         torch.cuda.synchronize()
         print(json.dumps({"probe": "3 x 256 MiB copy, 5 x " + dev.gemm_plan(desc)[2]}))
+        return
+    if args.probe_variants:   # for `rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES ...`: one tile shape per kernel name in the output
+        from dfdx_amd.rocm import KERNEL_MFMA
+
+        a = (torch.rand(N, N, device="cuda") * 2 - 1).half()
+        b = (torch.rand(N, N, device="cuda") * 2 - 1).half()
+        c = torch.zeros(N, N, device="cuda", dtype=torch.float16)
+        names = []
+        for v in range(1, dev.mfma_variant_count("f16") + 1):
+            desc = dev.gemm_desc("f16", N, N, N, a.data_ptr(), (N, 1), b.data_ptr(), (N, 1), c.data_ptr(), (N, 1),
+                                 kernel=KERNEL_MFMA, variant=v, no_split_k=True)
+            names.append(dev.gemm_plan(desc)[2])
+            for _ in range(3):
+                dev.gemm(desc)
+            torch.cuda.synchronize()
+        print(json.dumps({"probe": names}))
         return
     flop = 2.0 * N ** 3
     tdt = {"f16": torch.float16, "f32": torch.float32}
