@@ -127,8 +127,17 @@ template <int ROWS, int NWAVES, bool KC> struct DmaTile {
     }
 };
 
+// Waves per SIMD that the two LDS stages of a BM x BN x 64 tile let a CU hold (160 KB of LDS, 8-wave workgroups on 4
+// SIMDs): the register budget the kernel is compiled for, so that a scalar-register spill into vector lanes cannot
+// push the 128 x 128 tile past 128 VGPRs and halve its occupancy.
+constexpr int dma_waves_per_simd(int bm, int bn, int waves) {
+    const int wgs = 163840 / (2 * (bm + bn) * 64 * 2);
+    const int w = (wgs < 1 ? 1 : wgs) * waves / 4;
+    return w < 2 ? 2 : (w > 6 ? 6 : w);
+}
+
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(const Params p) {
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, WAVES_M *WAVES_N)) void gemm_mfma16_dma_kernel(const Params p) {
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
     constexpr int TM = WTM / 16, TN = WTN / 16;
@@ -424,31 +433,25 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
         // 8*(lq/2) .. +3 and +4 .. +7 of tile j + (lq & 1).  A wave instruction then writes 64 contiguous
         // bytes per matrix row instead of 32, which is what the memory system needs to reach its write rate.
         {
-            // PLAIN: the tile lies inside C and the store is a pure overwrite, optionally with a per-column bias --
-            // no bounds checks, no read of C (every forward product of whole tiles, Linear's fused bias included).
-            auto rows = [&](auto plain_tag) {
-                constexpr bool PLAIN = decltype(plain_tag)::value;
-                // The bias values depend on the column (or row) only: they are fetched before the first store, so
-                // that a fused Linear forward has no load waiting behind its own stores.
+            // The general form: bounds checks, either bias, beta = 1 with the old value loaded where it is used (edge
+            // tiles, per-row bias, very large ldc).
+            auto rows = [&]() {
                 u32x4 cbias[TN / 2];
-                float rbias_all[PLAIN ? 1 : TM];
+                float rbias_all[TM];
                 if (p.bias_mode == BIAS_PER_COL) {
 #pragma unroll
                     for (int jp = 0; jp < TN / 2; jp++)
                         cbias[jp] = *(const u32x4 *)(p.bias + min(bn0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8, p.n - 8));
                 }
-                if constexpr (!PLAIN) {
-                    if (p.bias_mode == BIAS_PER_ROW) {
+                if (p.bias_mode == BIAS_PER_ROW) {
 #pragma unroll
-                        for (int i = 0; i < TM; i++) rbias_all[i] = Mma<T>::to_f32(p.bias[min(bm0 + wm0 + i * 16 + l16, p.m - 1)]);
-                    }
+                    for (int i = 0; i < TM; i++) rbias_all[i] = Mma<T>::to_f32(p.bias[min(bm0 + wm0 + i * 16 + l16, p.m - 1)]);
                 }
 #pragma unroll
                 for (int i = 0; i < TM; i++) {
                     const int gm_row = bm0 + wm0 + i * 16 + l16;
-                    const bool row_ok = PLAIN || gm_row < p.m;
+                    const bool row_ok = gm_row < p.m;
                     uint16_t *crow = cbase + (int64_t)gm_row * p.ldc;
-                    [[maybe_unused]] const float rbias = PLAIN ? 0.0f : rbias_all[PLAIN ? 0 : i];
 #pragma unroll
                     for (int jp = 0; jp < TN / 2; jp++) {
                         float v[8];
@@ -460,12 +463,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
                             v[4 + e] = __uint_as_float(r[1]);
                         }
                         const int gn = bn0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8;
-                        if constexpr (!PLAIN) {
-                            if (!row_ok || gn >= p.n) continue;  // n % 8 == 0 here: all 8 columns are in range
-                            if (p.bias_mode == BIAS_PER_ROW) {
+                        if (!row_ok || gn >= p.n) continue;  // n % 8 == 0 here: all 8 columns are in range
+                        if (p.bias_mode == BIAS_PER_ROW) {
 #pragma unroll
-                                for (int e = 0; e < 8; e++) v[e] += rbias;
-                            }
+                            for (int e = 0; e < 8; e++) v[e] += rbias_all[i];
                         }
                         if (p.bias_mode == BIAS_PER_COL) {
                             const u32x4 bv = cbias[jp];
@@ -475,14 +476,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
                                 v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(bv[e] >> 16));
                             }
                         }
-                        if constexpr (!PLAIN) {
-                            if (p.accumulate) {
-                                const u32x4 old = *(const u32x4 *)(crow + gn);
+                        if (p.accumulate) {
+                            const u32x4 old = *(const u32x4 *)(crow + gn);
 #pragma unroll
-                                for (int e = 0; e < 4; e++) {
-                                    v[2 * e] += Mma<T>::to_f32((uint16_t)(old[e] & 0xffffu));
-                                    v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(old[e] >> 16));
-                                }
+                            for (int e = 0; e < 4; e++) {
+                                v[2 * e] += Mma<T>::to_f32((uint16_t)(old[e] & 0xffffu));
+                                v[2 * e + 1] += Mma<T>::to_f32((uint16_t)(old[e] >> 16));
                             }
                         }
                         u32x4 o;
@@ -492,6 +491,51 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
                     }
                 }
             };
+            // Interior tiles address C as wave-uniform base (scalar registers) + one 32-bit per-lane byte offset
+            // + immediate: no address arithmetic in vector registers per access.
+            const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+            char *const tile_base = (char *)(cbase + (int64_t)(bm0 + (wave_u / WAVES_N) * WTM) * p.ldc + bn0 + (wave_u % WAVES_N) * WTN);
+            const uint32_t lane_off = (uint32_t)(l16 * (int)p.ldc + (lq & 1) * 16 + (lq >> 1) * 8) * 2u;
+            const int64_t row_step = p.ldc * 32;  // 16 rows, bytes
+            // Pure overwrite of an interior tile, optionally with a per-column bias (every forward product of whole
+            // tiles, Linear's fused bias included): no bounds checks, no read of C; the bias values are fetched and
+            // widened once, before the first store.
+            auto rows_plain = [&](auto bias_tag) {
+                constexpr bool BIAS = decltype(bias_tag)::value;
+                [[maybe_unused]] float cb[TN / 2][8];
+                if constexpr (BIAS) {
+#pragma unroll
+                    for (int jp = 0; jp < TN / 2; jp++) {
+                        const u32x4 bv = *(const u32x4 *)(p.bias + bn0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            cb[jp][2 * e] = Mma<T>::to_f32((uint16_t)(bv[e] & 0xffffu));
+                            cb[jp][2 * e + 1] = Mma<T>::to_f32((uint16_t)(bv[e] >> 16));
+                        }
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int jp = 0; jp < TN / 2; jp++) {
+                        float v[8];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i][2 * jp][e]),
+                                                                            __float_as_uint(acc[i][2 * jp + 1][e]), false, false);
+                            v[e] = __uint_as_float(r[0]);
+                            v[4 + e] = __uint_as_float(r[1]);
+                        }
+                        if constexpr (BIAS) {
+#pragma unroll
+                            for (int e = 0; e < 8; e++) v[e] += cb[jp][e];
+                        }
+                        u32x4 o;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) o[e] = Mma<T>::pack2(v[2 * e], v[2 * e + 1]);
+                        *(u32x4 *)(tile_base + i * row_step + jp * 64 + lane_off) = o;
+                    }
+            };
             // beta = 1 on an interior tile without bias (every gradient product of whole tiles): all old values are
             // requested before the first store goes out.  While loads and stores are outstanding together the
             // compiler can only wait for everything (the two kinds may complete out of order), so the interleaved
@@ -499,12 +543,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
             // are waited for in issue order.
             auto rows_accumulate = [&]() {
                 constexpr int IG = TM * (TN / 2) > 8 ? TM / 2 : TM;  // tile rows per batch: at most 8 vectors in flight
-                // wave-uniform base (scalar registers) + one 32-bit per-lane byte offset: no address VGPRs per access
-                const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-                const int wm0_u = (wave_u / WAVES_N) * WTM, wn0_u = (wave_u % WAVES_N) * WTN;
-                char *base = (char *)(cbase + (int64_t)(bm0 + wm0_u) * p.ldc + bn0 + wn0_u);
-                const uint32_t lane_off = (uint32_t)(l16 * (int)p.ldc + (lq & 1) * 16 + (lq >> 1) * 8) * 2u;
-                const int64_t row_step = p.ldc * 32;  // 16 rows, bytes
+                char *const base = tile_base;
 #pragma unroll
                 for (int i0 = 0; i0 < TM; i0 += IG) {
                     u32x4 old[IG][TN / 2];
@@ -534,10 +573,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_dma_kernel(
                         }
                 }
             };
-            const bool interior = bm0 + BM <= p.m && bn0 + BN <= p.n && p.bias_mode != BIAS_PER_ROW;
-            if (interior && !p.accumulate) rows(std::true_type{});
-            else if (interior && p.bias_mode == BIAS_NONE && p.ldc < (1 << 26)) rows_accumulate();
-            else rows(std::false_type{});
+            const bool interior = bm0 + BM <= p.m && bn0 + BN <= p.n && p.bias_mode != BIAS_PER_ROW && p.ldc < (1 << 26);
+            if (interior && !p.accumulate) {
+                if (p.bias_mode == BIAS_PER_COL) rows_plain(std::true_type{});
+                else rows_plain(std::false_type{});
+            } else if (interior && p.bias_mode == BIAS_NONE) rows_accumulate();
+            else rows();
             return;
         }
     }
