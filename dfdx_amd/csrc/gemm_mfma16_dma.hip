@@ -88,6 +88,12 @@ template <> struct Mma<__bf16> {
     }
 };
 
+// DPP row rotation by 8 lanes: the lanes of the 4-lane banks selected by BANK_MASK (bit b = lanes 4b..4b+3 of every
+// 16-lane row) receive `src` of the lane 8 places away in their row, the other lanes keep `keep`.
+template <int BANK_MASK> __device__ __forceinline__ uint32_t lane8_trade(uint32_t keep, uint32_t src) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)keep, (int)src, 0x128 /* row_ror:8 */, 0xF, BANK_MASK, false);
+}
+
 // Swizzle of an m/n-contiguous tile ([k][ROWS] in LDS, ROWS*2 bytes per k-row): XOR applied to the 16 B
 // chunk index of k-row k.  A 16-lane group of a transposing read touches 4 consecutive k-rows x 2 chunks,
 // a second group the same chunks 8 k-rows further: the XOR spreads those over distinct banks.
@@ -497,6 +503,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
             char *const tile_base = (char *)(cbase + (int64_t)(bm0 + (wave_u / WAVES_N) * WTM) * p.ldc + bn0 + (wave_u % WAVES_N) * WTN);
             const uint32_t lane_off = (uint32_t)(l16 * (int)p.ldc + (lq & 1) * 16 + (lq >> 1) * 8) * 2u;
             const int64_t row_step = p.ldc * 32;  // 16 rows, bytes
+            // A wave tile that is 64 columns wide (TN == 4) writes whole 128 B lines: after the 16-lane swaps a lane
+            // row holds the left 64 B of matrix row l16 in one register set and the right 64 B in another; lanes
+            // l16 < 8 and l16 >= 8 then trade one set each (DPP row rotation by 8), so that one store instruction
+            // covers rows 0..7 x 128 B and a second one rows 8..15.  Measured on the device with plain store kernels,
+            // a CU retires 134 GB/s of whole-line stores but only 38 GB/s when every line arrives as two 64 B
+            // halves from different instructions (and 19 GB/s in 32 B pieces); with half lines the stores of a
+            // K = 64 work item take longer to leave the CU than its MFMAs take to compute.
+            [[maybe_unused]] const uint32_t line_off =
+                (uint32_t)((l16 & 7) * (int)p.ldc * 2 + (l16 >> 3) * 64 + ((lq & 1) * 2 + (lq >> 1)) * 16);
+            [[maybe_unused]] const int64_t half_step = p.ldc * 16;  // 8 rows, bytes
             // Pure overwrite of an interior tile, optionally with a per-column bias (every forward product of whole
             // tiles, Linear's fused bias included): no bounds checks, no read of C; the bias values are fetched and
             // widened once, before the first store.
@@ -515,7 +531,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
                     }
                 }
 #pragma unroll
-                for (int i = 0; i < TM; i++)
+                for (int i = 0; i < TM; i++) {
+                    u32x4 o[TN / 2];
 #pragma unroll
                     for (int jp = 0; jp < TN / 2; jp++) {
                         float v[8];
@@ -530,11 +547,23 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
 #pragma unroll
                             for (int e = 0; e < 8; e++) v[e] += cb[jp][e];
                         }
-                        u32x4 o;
 #pragma unroll
-                        for (int e = 0; e < 4; e++) o[e] = Mma<T>::pack2(v[2 * e], v[2 * e + 1]);
-                        *(u32x4 *)(tile_base + i * row_step + jp * 64 + lane_off) = o;
+                        for (int e = 0; e < 4; e++) o[jp][e] = Mma<T>::pack2(v[2 * e], v[2 * e + 1]);
                     }
+                    if constexpr (TN == 4) {
+                        u32x4 lo, hi;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            hi[e] = lane8_trade<0x3>(o[1][e], o[0][e]);  // rows 8..15: left halves come from lanes + 8
+                            lo[e] = lane8_trade<0xC>(o[0][e], o[1][e]);  // rows 0..7: right halves come from lanes - 8
+                        }
+                        *(u32x4 *)(tile_base + i * row_step + line_off) = lo;
+                        *(u32x4 *)(tile_base + i * row_step + half_step + line_off) = hi;
+                    } else {
+#pragma unroll
+                        for (int jp = 0; jp < TN / 2; jp++) *(u32x4 *)(tile_base + i * row_step + jp * 64 + lane_off) = o[jp];
+                    }
+                }
             };
             // beta = 1 on an interior tile without bias (every gradient product of whole tiles): all old values are
             // requested before the first store goes out.  While loads and stores are outstanding together the
@@ -550,27 +579,41 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
 #pragma unroll
                     for (int i = 0; i < IG; i++)
 #pragma unroll
-                        for (int jp = 0; jp < TN / 2; jp++)
-                            old[i][jp] = *(const u32x4 *)(base + (i0 + i) * row_step + jp * 64 + lane_off);
-#pragma unroll
-                    for (int i = 0; i < IG; i++)
-#pragma unroll
                         for (int jp = 0; jp < TN / 2; jp++) {
-                            float v[8];
+                            if constexpr (TN == 4) old[i][jp] = *(const u32x4 *)(base + (i0 + i) * row_step + jp * half_step + line_off);
+                            else old[i][jp] = *(const u32x4 *)(base + (i0 + i) * row_step + jp * 64 + lane_off);
+                        }
+#pragma unroll
+                    for (int i = 0; i < IG; i++) {
+                        float v[TN / 2][8];
+#pragma unroll
+                        for (int jp = 0; jp < TN / 2; jp++)
 #pragma unroll
                             for (int e = 0; e < 4; e++) {
                                 const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i0 + i][2 * jp][e]),
                                                                                 __float_as_uint(acc[i0 + i][2 * jp + 1][e]), false, false);
-                                v[e] = __uint_as_float(r[0]);
-                                v[4 + e] = __uint_as_float(r[1]);
+                                v[jp][e] = __uint_as_float(r[0]);
+                                v[jp][4 + e] = __uint_as_float(r[1]);
                             }
+                        if constexpr (TN == 4) {  // whole lines: v[0] becomes rows 0..7, v[1] rows 8..15 (see line_off)
+#pragma unroll
+                            for (int e = 0; e < 8; e++) {
+                                const uint32_t left = __float_as_uint(v[0][e]), right = __float_as_uint(v[1][e]);
+                                v[1][e] = __uint_as_float(lane8_trade<0x3>(right, left));
+                                v[0][e] = __uint_as_float(lane8_trade<0xC>(left, right));
+                            }
+                        }
+#pragma unroll
+                        for (int jp = 0; jp < TN / 2; jp++) {
                             u32x4 o;
 #pragma unroll
                             for (int e = 0; e < 4; e++)
-                                o[e] = Mma<T>::pack2(v[2 * e] + Mma<T>::to_f32((uint16_t)(old[i][jp][e] & 0xffffu)),
-                                                     v[2 * e + 1] + Mma<T>::to_f32((uint16_t)(old[i][jp][e] >> 16)));
-                            *(u32x4 *)(base + (i0 + i) * row_step + jp * 64 + lane_off) = o;
+                                o[e] = Mma<T>::pack2(v[jp][2 * e] + Mma<T>::to_f32((uint16_t)(old[i][jp][e] & 0xffffu)),
+                                                     v[jp][2 * e + 1] + Mma<T>::to_f32((uint16_t)(old[i][jp][e] >> 16)));
+                            if constexpr (TN == 4) *(u32x4 *)(base + (i0 + i) * row_step + jp * half_step + line_off) = o;
+                            else *(u32x4 *)(base + (i0 + i) * row_step + jp * 64 + lane_off) = o;
                         }
+                    }
                 }
             };
             const bool interior = bm0 + BM <= p.m && bn0 + BN <= p.n && p.bias_mode != BIAS_PER_ROW && p.ldc < (1 << 26);
@@ -631,7 +674,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
         tile_body(c_stage, std::false_type{});
         c_stage ^= 1;
         // Work item finished.  Hand the stage over BEFORE the stores are issued: the wait inside sync_tile then
-        // only covers loads, and the stores drain while the next tile is computed.
+        // covers the next tile's loads and the stores of the PREVIOUS item only, and this item's stores drain while
+        // the next tile is computed.  (Converting the accumulators before that wait was tried: it costs registers
+        // inside the k loop and lost.)
         const bool more = c_index + (int)gridDim.x < p.total_blocks;
         if (more) sync_tile();
         store_tile(cw);
