@@ -18,14 +18,16 @@ struct Op {  // dfdx_rocm_conv2d_op narrowed to 32 bits (validated on entry)
 // zero outside the image.  One workgroup per (b, c, k1, k2) slab, so that the index arithmetic per element is a
 // row counter: a thread owns one group of N consecutive ow (w_out % N == 0) and walks down the output rows.
 template <typename T, int N>
-__global__ __launch_bounds__(256) void unfold_input_kernel(Op op, const T *img, T *patches) {
+__global__ __launch_bounds__(256) void unfold_input_kernel(Op op, const T *img, T *patches, int slab_stride) {
     const uint32_t slab = blockIdx.x;
     const int kk = op.kernel * op.kernel;
     const int k2 = (int)(slab % op.kernel), k1 = (int)((slab / op.kernel) % op.kernel);
     const uint32_t r = slab / kk;  // b * chan_in + c
     const int wg = op.w_out / N;
     const T *plane = img + (int64_t)r * op.h_in * op.w_in;
-    T *dst = patches + (int64_t)slab * op.h_out * op.w_out;
+    T *dst = patches + (int64_t)slab * slab_stride;
+    // rows padded to the GEMM's vector width end in zeros (they are k or dropped n positions of the products)
+    if ((int)threadIdx.x < slab_stride - op.h_out * op.w_out) Elem<T>::store(dst + op.h_out * op.w_out + threadIdx.x, 0.0f);
     auto emit = [&](int oh, int owg) {
         const int y = oh * op.stride + op.dilation * k1 - op.padding;
         const T *row = plane + (int64_t)y * op.w_in;
@@ -55,14 +57,15 @@ __global__ __launch_bounds__(256) void unfold_input_kernel(Op op, const T *img, 
 // patches[b][o][k1][k2][y][x] = grad_out[b][o][oh][ow] where oh*stride = y + padding - dilation*k1 (likewise ow),
 // zero when no output position reads image pixel (y, x) through filter tap (k1, k2).  Same slab mapping.
 template <typename T, int N>
-__global__ __launch_bounds__(256) void unfold_output_kernel(Op op, const T *grad_out, T *patches) {
+__global__ __launch_bounds__(256) void unfold_output_kernel(Op op, const T *grad_out, T *patches, int slab_stride) {
     const uint32_t slab = blockIdx.x;
     const int kk = op.kernel * op.kernel;
     const int k2 = (int)(slab % op.kernel), k1 = (int)((slab / op.kernel) % op.kernel);
     const uint32_t r = slab / kk;  // b * chan_out + o
     const int wg = op.w_in / N;
     const T *plane = grad_out + (int64_t)r * op.h_out * op.w_out;
-    T *dst = patches + (int64_t)slab * op.h_in * op.w_in;
+    T *dst = patches + (int64_t)slab * slab_stride;
+    if ((int)threadIdx.x < slab_stride - op.h_in * op.w_in) Elem<T>::store(dst + op.h_in * op.w_in + threadIdx.x, 0.0f);
     auto emit = [&](int y, int xg) {
         int oh = y + op.padding - op.dilation * k1;
         const bool row_ok = oh >= 0 && oh % op.stride == 0 && oh / op.stride < op.h_out;
@@ -92,6 +95,70 @@ __global__ __launch_bounds__(256) void unfold_output_kernel(Op op, const T *grad
     }
 }
 
+// The same two gathers for row widths that are not a multiple of the vector width, and for small images: a thread owns
+// one 16-byte vector of the patch buffer, i.e. V consecutive positions of a flattened (row, column) slab -- they may
+// straddle two rows -- whatever the slab size (a 7x7 slab would leave 249 of a workgroup's 256 threads idle);
+// positions behind the slab's last element (the row padding) are zeros.
+template <typename T>
+__global__ __launch_bounds__(256) void unfold_input_flat_kernel(Op op, const T *img, T *patches, int slab_stride, uint32_t vectors) {
+    constexpr int V = Elem<T>::VEC;
+    const uint32_t item = blockIdx.x * 256 + threadIdx.x;  // one 16-byte vector of the patch buffer per thread
+    if (item >= vectors) return;
+    const uint32_t per_slab = (uint32_t)slab_stride / V, slab = item / per_slab;
+    const int kk = op.kernel * op.kernel, n = op.h_out * op.w_out;
+    const int k2 = (int)(slab % op.kernel), k1 = (int)((slab / op.kernel) % op.kernel);
+    const T *plane = img + (int64_t)(slab / kk) * op.h_in * op.w_in;
+    T *dst = patches + (int64_t)slab * slab_stride;
+    {
+        const int pos0 = (int)(item - slab * per_slab) * V;
+        int oh = pos0 / op.w_out, ow = pos0 - oh * op.w_out;
+        float v[V];
+        const int y0 = oh * op.stride + op.dilation * k1 - op.padding, x0 = ow * op.stride + op.dilation * k2 - op.padding;
+        if (op.stride == 1 && ow + V <= op.w_out && pos0 + V <= n && y0 >= 0 && y0 < op.h_in && x0 >= 0 && x0 + V <= op.w_in) {
+            load_elems_unaligned<T, V>(plane + (int64_t)y0 * op.w_in + x0, v);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const int y = oh * op.stride + op.dilation * k1 - op.padding, x = ow * op.stride + op.dilation * k2 - op.padding;
+                const bool ok = pos0 + i < n && y >= 0 && y < op.h_in && x >= 0 && x < op.w_in;
+                v[i] = ok ? Elem<T>::load(plane + (int64_t)y * op.w_in + x) : 0.0f;
+                if (++ow == op.w_out) { ow = 0; ++oh; }
+            }
+        }
+        store_elems<T, V>(dst + pos0, v);
+    }
+}
+template <typename T>
+__global__ __launch_bounds__(256) void unfold_output_flat_kernel(Op op, const T *grad_out, T *patches, int slab_stride, uint32_t vectors) {
+    constexpr int V = Elem<T>::VEC;
+    const uint32_t item = blockIdx.x * 256 + threadIdx.x;
+    if (item >= vectors) return;
+    const uint32_t per_slab = (uint32_t)slab_stride / V, slab = item / per_slab;
+    const int kk = op.kernel * op.kernel, n = op.h_in * op.w_in;
+    const int k2 = (int)(slab % op.kernel), k1 = (int)((slab / op.kernel) % op.kernel);
+    const T *plane = grad_out + (int64_t)(slab / kk) * op.h_out * op.w_out;
+    T *dst = patches + (int64_t)slab * slab_stride;
+    {
+        const int pos0 = (int)(item - slab * per_slab) * V;
+        int y = pos0 / op.w_in, x = pos0 - y * op.w_in;
+        float v[V];
+        const int oh0 = y + op.padding - op.dilation * k1, ow0 = x + op.padding - op.dilation * k2;
+        if (op.stride == 1 && x + V <= op.w_in && pos0 + V <= n && oh0 >= 0 && oh0 < op.h_out && ow0 >= 0 && ow0 + V <= op.w_out) {
+            load_elems_unaligned<T, V>(plane + (int64_t)oh0 * op.w_out + ow0, v);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const int oh = y + op.padding - op.dilation * k1, ow = x + op.padding - op.dilation * k2;
+                const bool ok = pos0 + i < n && oh >= 0 && oh % op.stride == 0 && oh / op.stride < op.h_out && ow >= 0 &&
+                                ow % op.stride == 0 && ow / op.stride < op.w_out;
+                v[i] = ok ? Elem<T>::load(plane + (int64_t)(oh / op.stride) * op.w_out + ow / op.stride) : 0.0f;
+                if (++x == op.w_in) { x = 0; ++y; }
+            }
+        }
+        store_elems<T, V>(dst + pos0, v);
+    }
+}
+
 // filters (G*O/G, C/G, K, K) <-> transposed (G, C/G, O/G, K*K).  ADD_BACK: filters[..] += transposed[..].
 template <typename T, bool ADD_BACK>
 __global__ __launch_bounds__(256) void filter_transpose_kernel(Op op, T *filters, T *transposed, int total) {
@@ -113,7 +180,26 @@ template <typename T> __global__ __launch_bounds__(256) void zero_kernel(T *p, i
     if (i < n) Elem<T>::store(p + i, 0.0f);
 }
 
+// Rows of `len` elements <-> rows padded to `padded` elements (zeros behind the data).  When the spatial size of a
+// product (OH*OW forward, H*W backward) is not a multiple of the GEMM's vector width, the matrices on that side get
+// padded rows in the patch buffer, so that the matrix-core kernels apply instead of the scalar fallback.
+template <typename T> __global__ __launch_bounds__(256) void pad_rows_kernel(const T *src, T *dst, int len, int padded, int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into dst
+    if (i >= total) return;
+    const int64_t row = i / padded;
+    const int col = (int)(i - row * padded);
+    if (col < len) dst[i] = src[row * len + col];
+    else Elem<T>::store(dst + i, 0.0f);
+}
+template <typename T> __global__ __launch_bounds__(256) void unpad_rows_kernel(const T *src, T *dst, int len, int padded, int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into dst
+    if (i >= total) return;
+    const int64_t row = i / len;
+    dst[i] = src[row * padded + (i - row * len)];
+}
+
 constexpr size_t kPatchBudget = size_t(1) << 30;  // bytes of patches per batch chunk
+inline size_t round256(size_t b) { return (b + 255) & ~size_t(255); }
 
 template <typename T> unsigned grid_for(dfdx_rocm_ctx *ctx, uint64_t threads) {
     return (unsigned)std::min<uint64_t>((threads + 255) / 256, (uint64_t)ctx->compute_units * 32);
@@ -146,34 +232,48 @@ dfdx_rocm_gemm_desc blank_desc(int dtype, int64_t m, int64_t k, int64_t n) {
 
 template <typename T>
 int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void *filters, void *out) {
+    constexpr int V = Elem<T>::VEC;
     const int64_t kk = (int64_t)op.kernel * op.kernel, n = (int64_t)op.h_out * op.w_out;
+    const int64_t np = (n + V - 1) / V * V;  // row length of the patch matrix (and of a padded output)
     const int64_t m = op.chan_out / op.groups, k = (op.chan_in / op.groups) * kk;
-    const int64_t per_image = (int64_t)op.chan_in * kk * n;  // patch elements of one image
+    const int64_t per_image = (int64_t)op.chan_in * kk * np;  // patch elements of one image
     if (per_image == 0 || m == 0) return DFDX_ROCM_OK;
-    if (per_image >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
+    if (per_image >= (1ll << 31) || (int64_t)op.chan_out * np >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
     CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
     int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
     chunk = std::min<int64_t>(std::min<int64_t>(chunk, op.batch), ((1ll << 31) - 1) / per_image);
-    if (int rc = ensure_patches(ctx, (size_t)(chunk * per_image) * sizeof(T))) return rc;
+    const bool padded = np != n;  // the product goes to a padded copy of the output, which is then compacted
+    const size_t patch_bytes = round256((size_t)(chunk * per_image) * sizeof(T));
+    const size_t out_bytes = padded ? round256((size_t)(chunk * op.chan_out * np) * sizeof(T)) : 0;
+    if (int rc = ensure_patches(ctx, patch_bytes + out_bytes)) return rc;
     T *patches = (T *)ctx->patches;
-    constexpr int V = Elem<T>::VEC;
-    const bool vec = op.w_out % V == 0;
+    T *out_p = (T *)((char *)ctx->patches + patch_bytes);
+    const bool vec = op.w_out % V == 0 && n >= 256 * V;  // whole workgroups per slab only when a slab fills one
     for (int64_t b0 = 0; b0 < op.batch; b0 += chunk) {
         const int64_t nb = std::min<int64_t>(chunk, op.batch - b0);
         Op sub = op;
         sub.batch = (int)nb;
         const T *src = (const T *)img + b0 * op.chan_in * op.h_in * op.w_in;
         const unsigned slabs = (unsigned)(nb * op.chan_in * kk);
-        if (vec) unfold_input_kernel<T, V><<<slabs, 256, 0, ctx->stream>>>(sub, src, patches);
-        else unfold_input_kernel<T, 1><<<slabs, 256, 0, ctx->stream>>>(sub, src, patches);
+        if (vec) unfold_input_kernel<T, V><<<slabs, 256, 0, ctx->stream>>>(sub, src, patches, (int)np);
+        else {
+            const uint32_t vectors = (uint32_t)(slabs * (np / V));  // < 2^28: the chunk's patches stay below 2^31 elements
+            unfold_input_flat_kernel<T><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, src, patches, (int)np, vectors);
+        }
         HIP_TRY(hipGetLastError());
         // filters (G, O/G, C/G*K*K) . patches (B, G, C/G*K*K, OH*OW) -> out (B, G, O/G, OH*OW)
-        dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
+        T *dst = (T *)out + b0 * op.chan_out * n;
+        dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, np);
         d.batch1 = nb; d.batch2 = op.groups;
         d.a = filters; d.a_rs = k; d.a_cs = 1; d.a_b1 = 0; d.a_b2 = m * k;
-        d.b = patches; d.b_rs = n; d.b_cs = 1; d.b_b1 = op.groups * k * n; d.b_b2 = k * n;
-        d.c = (T *)out + b0 * op.chan_out * n; d.c_rs = n; d.c_cs = 1; d.c_b1 = op.chan_out * n; d.c_b2 = m * n;
+        d.b = patches; d.b_rs = np; d.b_cs = 1; d.b_b1 = op.groups * k * np; d.b_b2 = k * np;
+        d.c = padded ? out_p : dst; d.c_rs = np; d.c_cs = 1; d.c_b1 = op.chan_out * np; d.c_b2 = m * np;
         if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+        if (padded) {
+            const int64_t total = nb * op.chan_out * n;
+            unpad_rows_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(out_p, dst, (int)n, (int)np, total);
+            HIP_TRY(hipGetLastError());
+        }
     }
     return DFDX_ROCM_OK;
 }
@@ -181,56 +281,85 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
 template <typename T>
 int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad_img, const void *filters, void *grad_filters,
                const void *grad_out) {
+    constexpr int V = Elem<T>::VEC;
     const int64_t kk = (int64_t)op.kernel * op.kernel, hw = (int64_t)op.h_in * op.w_in, ohw = (int64_t)op.h_out * op.w_out;
+    // Row length of the patch matrix and of the padded image-side matrices.  H*W is the n of the image-gradient
+    // product and the k of the filter-gradient product; for the 16-bit types that k is rounded up to the k tile of the
+    // split-k capable kernels -- a filter gradient has few output tiles and a long reduction over batch * H*W.
+    const int64_t align = sizeof(T) == 2 ? 64 : V;
+    const int64_t hp = (hw + align - 1) / align * align;
     const int64_t cg = op.chan_in / op.groups, og = op.chan_out / op.groups;
-    const int64_t per_image = (int64_t)op.chan_out * kk * hw;
+    const int64_t per_image = (int64_t)op.chan_out * kk * hp;
     const int64_t f_elems = (int64_t)op.groups * cg * og * kk;
     if (per_image == 0 || f_elems == 0 || ohw == 0) return DFDX_ROCM_OK;
-    if (per_image >= (1ll << 31) || f_elems >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
+    if (per_image >= (1ll << 31) || f_elems >= (1ll << 31) || (int64_t)op.chan_in * hp >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
     CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
     int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
     chunk = std::min<int64_t>(std::min<int64_t>(chunk, op.batch), ((1ll << 31) - 1) / per_image);
-    // patch buffer: [chunk][O*K*K][H*W], then the transposed filters and their gradient
-    const size_t patch_bytes = ((size_t)(chunk * per_image) * sizeof(T) + 255) & ~size_t(255);
-    const size_t f_bytes = ((size_t)f_elems * sizeof(T) + 255) & ~size_t(255);
-    if (int rc = ensure_patches(ctx, patch_bytes + 2 * f_bytes)) return rc;
+    // H*W not a multiple of the vector width: the image and its gradient take part as padded copies
+    // (zeros behind every row; the gradient copy starts from grad_img, so beta = 1 rounds exactly as without it).
+    const bool padded = hp != hw;
+    // patch buffer: [chunk][O*K*K][hp], the transposed filters and their gradient, then the padded copies
+    const size_t patch_bytes = round256((size_t)(chunk * per_image) * sizeof(T));
+    const size_t f_bytes = round256((size_t)f_elems * sizeof(T));
+    const size_t img_bytes = padded ? round256((size_t)(chunk * op.chan_in * hp) * sizeof(T)) : 0;
+    if (int rc = ensure_patches(ctx, patch_bytes + 2 * f_bytes + 2 * img_bytes)) return rc;
     T *patches = (T *)ctx->patches;
     T *f_tr = (T *)((char *)ctx->patches + patch_bytes);
     T *grad_f_tr = (T *)((char *)ctx->patches + patch_bytes + f_bytes);
+    T *img_p = (T *)((char *)ctx->patches + patch_bytes + 2 * f_bytes);
+    T *grad_img_p = (T *)((char *)ctx->patches + patch_bytes + 2 * f_bytes + img_bytes);
     const unsigned fgrid = (unsigned)((f_elems + 255) / 256);
     filter_transpose_kernel<T, false><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)const_cast<void *>(filters), f_tr, (int)f_elems);
     HIP_TRY(hipGetLastError());
     zero_kernel<T><<<fgrid, 256, 0, ctx->stream>>>(grad_f_tr, (int)f_elems);
     HIP_TRY(hipGetLastError());
-    constexpr int V = Elem<T>::VEC;
-    const bool vec = op.w_in % V == 0;
+    const bool vec = op.w_in % V == 0 && hw >= 256 * V;
     for (int64_t b0 = 0; b0 < op.batch; b0 += chunk) {
         const int64_t nb = std::min<int64_t>(chunk, op.batch - b0);
         Op sub = op;
         sub.batch = (int)nb;
         const T *go = (const T *)grad_out + b0 * op.chan_out * ohw;
         const unsigned slabs = (unsigned)(nb * op.chan_out * kk);
-        if (vec) unfold_output_kernel<T, V><<<slabs, 256, 0, ctx->stream>>>(sub, go, patches);
-        else unfold_output_kernel<T, 1><<<slabs, 256, 0, ctx->stream>>>(sub, go, patches);
+        if (vec) unfold_output_kernel<T, V><<<slabs, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
+        else {
+            const uint32_t vectors = (uint32_t)(slabs * (hp / V));
+            unfold_output_flat_kernel<T><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp, vectors);
+        }
         HIP_TRY(hipGetLastError());
+        const T *img_b = (const T *)img + b0 * op.chan_in * hw;
+        T *grad_img_b = (T *)grad_img + b0 * op.chan_in * hw;
+        const int64_t rows_p = nb * op.chan_in * hp;
+        if (padded) {
+            const unsigned g = (unsigned)((rows_p + 255) / 256);
+            pad_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(img_b, img_p, (int)hw, (int)hp, rows_p);
+            HIP_TRY(hipGetLastError());
+            pad_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(grad_img_b, grad_img_p, (int)hw, (int)hp, rows_p);
+            HIP_TRY(hipGetLastError());
+        }
         {   // grad_img (B, G, C/G, H*W) += filters^T (G, C/G, O/G*K*K) . patches (B, G, O/G*K*K, H*W)
-            const int64_t m = cg, k = og * kk, n = hw;
+            const int64_t m = cg, k = og * kk, n = hp;
             dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
             d.accumulate = 1;
             d.batch1 = nb; d.batch2 = op.groups;
             d.a = f_tr; d.a_rs = k; d.a_cs = 1; d.a_b1 = 0; d.a_b2 = m * k;
             d.b = patches; d.b_rs = n; d.b_cs = 1; d.b_b1 = op.groups * k * n; d.b_b2 = k * n;
-            d.c = (T *)grad_img + b0 * op.chan_in * hw; d.c_rs = n; d.c_cs = 1; d.c_b1 = op.chan_in * hw; d.c_b2 = m * n;
+            d.c = padded ? grad_img_p : grad_img_b; d.c_rs = n; d.c_cs = 1; d.c_b1 = op.chan_in * n; d.c_b2 = m * n;
             if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+        }
+        if (padded) {
+            const int64_t total = nb * op.chan_in * hw;
+            unpad_rows_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(grad_img_p, grad_img_b, (int)hw, (int)hp, total);
+            HIP_TRY(hipGetLastError());
         }
         for (int g = 0; g < op.groups; g++) {
             // grad_filters^T (C/G, O/G*K*K) += sum over images of img (C/G, H*W) . patches^T (H*W, O/G*K*K)
-            const int64_t m = cg, k = hw, n = og * kk;
+            const int64_t m = cg, k = hp, n = og * kk;
             dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
             d.accumulate = 1;
             d.reduce_batch = 1;
             d.batch1 = nb;
-            d.a = (const T *)img + (b0 * op.chan_in + g * cg) * hw; d.a_rs = k; d.a_cs = 1; d.a_b1 = op.chan_in * hw;
+            d.a = (padded ? (const T *)img_p : img_b) + g * cg * k; d.a_rs = k; d.a_cs = 1; d.a_b1 = op.chan_in * k;
             d.b = patches + g * n * k; d.b_rs = 1; d.b_cs = k; d.b_b1 = per_image;
             d.c = grad_f_tr + g * m * n; d.c_rs = n; d.c_cs = 1;
             if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;

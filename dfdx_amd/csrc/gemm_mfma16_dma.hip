@@ -877,8 +877,9 @@ void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_va
         if (forced_variant == 0 && ((p.n <= 64) != (t.bn <= 64))) continue;  // BN = 64 tiles only for narrow outputs
         const int64_t tiles = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
         const double layout = (a_kc && b_kc) ? 1.0 : (!a_kc && !b_kc) ? 0.98 : 0.99;  // transposing LDS reads cost a little
-        for (int s = 1; s <= 16; s++) {
-            if (forced_splits > 0 && s != std::min<int64_t>(forced_splits, total_iters)) continue;
+        // candidates 1..16, 20..32, 40..64 (filter gradients of convolutions: a handful of tiles, thousands of k steps)
+        const int forced_s = forced_splits > 0 ? (int)std::min<int64_t>(forced_splits, total_iters) : 0;
+        for (int s = forced_s ? forced_s : 1; s <= (forced_s ? forced_s : 64); s += (s < 16 ? 1 : s < 32 ? 4 : 8)) {
             if (s > 1 && (!may_split || (forced_splits == 0 && total_iters / s < 4))) break;
             const int64_t chunk = (total_iters + s - 1) / s;
             if ((s - 1) * chunk >= total_iters) continue;  // an empty split
