@@ -14,91 +14,113 @@ struct Op {  // dfdx_rocm_conv2d_op narrowed to 32 bits (validated on entry)
     int kernel, stride, padding, dilation, groups, batch, chan_in, chan_out, h_in, h_out, w_in, w_out;
 };
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
+
+// A 16-byte vector moved by `bits` towards element 0 (bits > 0) or away from it (bits < 0), zeros moving in.
+__device__ __forceinline__ u32x4 shift128(u32x4 r, int bits) {
+    uint64_t lo = r[0] | ((uint64_t)r[1] << 32), hi = r[2] | ((uint64_t)r[3] << 32);
+    if (bits >= 0) {
+        const unsigned s = (unsigned)bits;
+        if (s >= 64) { lo = hi; hi = 0; }
+        const unsigned t = s & 63;
+        if (t) { lo = (lo >> t) | (hi << (64 - t)); hi >>= t; }
+        if (s >= 128) lo = 0;
+    } else {
+        const unsigned s = (unsigned)(-bits);
+        if (s >= 64) { hi = lo; lo = 0; }
+        const unsigned t = s & 63;
+        if (t) { hi = (hi << t) | (lo >> (64 - t)); lo <<= t; }
+        if (s >= 128) hi = 0;
+    }
+    return u32x4{(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
+}
+// N = 16 bytes of elements of one image row starting at column x0, zeros outside [0, width): one (unaligned) vector
+// load from the nearest window inside the row, then a shift -- no per-element path for the lanes at the image border,
+// which a wave would otherwise execute in full next to the vector path of its interior lanes.  width >= N.
+template <typename T> __device__ __forceinline__ u32x4 row_window(const T *row, bool row_ok, int x0, int width) {
+    constexpr int N = Elem<T>::VEC;
+    const int x0c = min(max(x0, 0), width - N);
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (row_ok) raw = *(const u32x4_unaligned *)(row + x0c);
+    return shift128(raw, (x0 - x0c) * (int)(8 * sizeof(T)));
+}
+
 // patches[b][c][k1][k2][oh][ow] = img[b][c][oh*stride + dilation*k1 - padding][ow*stride + dilation*k2 - padding],
-// zero outside the image.  One workgroup per (b, c, k1, k2) slab, so that the index arithmetic per element is a
-// row counter: a thread owns one group of N consecutive ow (w_out % N == 0) and walks down the output rows.
-template <typename T, int N>
-__global__ __launch_bounds__(256) void unfold_input_kernel(Op op, const T *img, T *patches, int slab_stride) {
-    const uint32_t slab = blockIdx.x;
-    const int kk = op.kernel * op.kernel;
-    const int k2 = (int)(slab % op.kernel), k1 = (int)((slab / op.kernel) % op.kernel);
-    const uint32_t r = slab / kk;  // b * chan_in + c
-    const int wg = op.w_out / N;
-    const T *plane = img + (int64_t)r * op.h_in * op.w_in;
-    T *dst = patches + (int64_t)slab * slab_stride;
-    // rows padded to the GEMM's vector width end in zeros (they are k or dropped n positions of the products)
-    if ((int)threadIdx.x < slab_stride - op.h_out * op.w_out) Elem<T>::store(dst + op.h_out * op.w_out + threadIdx.x, 0.0f);
-    auto emit = [&](int oh, int owg) {
-        const int y = oh * op.stride + op.dilation * k1 - op.padding;
-        const T *row = plane + (int64_t)y * op.w_in;
-        float v[N];
-        const int x0 = owg * N * op.stride + op.dilation * k2 - op.padding;
-        if (N > 1 && op.stride == 1 && y >= 0 && y < op.h_in && x0 >= 0 && x0 + N <= op.w_in) {
-            load_elems_unaligned<T, N>(row + x0, v);  // unit stride, window inside the row: N consecutive pixels
-        } else {
+// zero outside the image.  Unit stride, output width a multiple of the vector: one workgroup per (b, c) plane writes
+// the K*K slabs of that plane; a thread owns a vector position (oh, V consecutive ow) and moves one window per tap --
+// with a compile-time K the loads of all taps are in flight before the first store.  Each slab is `slab_stride`
+// elements long: the rows of the patch matrix may be padded, and the padding is zeros.
+template <typename T, int KS>
+__global__ __launch_bounds__(256) void unfold_input_plane_kernel(Op op, const T *__restrict__ img, T *__restrict__ patches,
+                                                                 int slab_stride) {
+    constexpr int V = Elem<T>::VEC;
+    const int K = KS ? KS : op.kernel, kk = K * K, n = op.h_out * op.w_out, wg = op.w_out / V;
+    const T *plane = img + (int64_t)blockIdx.x * op.h_in * op.w_in;
+    T *dst = patches + (int64_t)blockIdx.x * kk * slab_stride;
+    if ((int)threadIdx.x < slab_stride - n)
+        for (int tap = 0; tap < kk; tap++) Elem<T>::store(dst + (int64_t)tap * slab_stride + n + threadIdx.x, 0.0f);
+    for (int g = threadIdx.x; g < n / V; g += 256) {
+        const int oh = g / wg, ow = (g - oh * wg) * V;
 #pragma unroll
-            for (int i = 0; i < N; i++) {
-                const int x = x0 + i * op.stride;
-                v[i] = (y >= 0 && y < op.h_in && x >= 0 && x < op.w_in) ? Elem<T>::load(row + x) : 0.0f;
+        for (int k1 = 0; k1 < (KS ? KS : 1); k1++)
+#pragma unroll
+            for (int k2 = 0; k2 < (KS ? KS : 1); k2++) {
+                if constexpr (KS != 0) {
+                    const int y = oh + op.dilation * k1 - op.padding;
+                    *(u32x4 *)(dst + (int64_t)(k1 * K + k2) * slab_stride + g * V) =
+                        row_window<T>(plane + (int64_t)y * op.w_in, y >= 0 && y < op.h_in, ow + op.dilation * k2 - op.padding, op.w_in);
+                }
+            }
+        if constexpr (KS == 0) {
+            for (int tap = 0; tap < kk; tap++) {
+                const int t1 = tap / K, t2 = tap - t1 * K;
+                const int y = oh + op.dilation * t1 - op.padding;
+                *(u32x4 *)(dst + (int64_t)tap * slab_stride + g * V) =
+                    row_window<T>(plane + (int64_t)y * op.w_in, y >= 0 && y < op.h_in, ow + op.dilation * t2 - op.padding, op.w_in);
             }
         }
-        store_elems<T, N>(dst + (int64_t)oh * op.w_out + owg * N, v);
-    };
-    const int step_rows = 256 / wg;  // rows covered per pass; 0 when a row has more than 256 groups
-    if (step_rows) {
-        if ((int)threadIdx.x >= step_rows * wg) return;
-        const int owg = (int)threadIdx.x % wg;
-        for (int oh = (int)threadIdx.x / wg; oh < op.h_out; oh += step_rows) emit(oh, owg);
-    } else {
-        for (int g = threadIdx.x; g < op.h_out * wg; g += 256) emit(g / wg, g % wg);
     }
 }
 
 // patches[b][o][k1][k2][y][x] = grad_out[b][o][oh][ow] where oh*stride = y + padding - dilation*k1 (likewise ow),
-// zero when no output position reads image pixel (y, x) through filter tap (k1, k2).  Same slab mapping.
-template <typename T, int N>
-__global__ __launch_bounds__(256) void unfold_output_kernel(Op op, const T *grad_out, T *patches, int slab_stride) {
-    const uint32_t slab = blockIdx.x;
-    const int kk = op.kernel * op.kernel;
-    const int k2 = (int)(slab % op.kernel), k1 = (int)((slab / op.kernel) % op.kernel);
-    const uint32_t r = slab / kk;  // b * chan_out + o
-    const int wg = op.w_in / N;
-    const T *plane = grad_out + (int64_t)r * op.h_out * op.w_out;
-    T *dst = patches + (int64_t)slab * slab_stride;
-    if ((int)threadIdx.x < slab_stride - op.h_in * op.w_in) Elem<T>::store(dst + op.h_in * op.w_in + threadIdx.x, 0.0f);
-    auto emit = [&](int y, int xg) {
-        int oh = y + op.padding - op.dilation * k1;
-        const bool row_ok = oh >= 0 && oh % op.stride == 0 && oh / op.stride < op.h_out;
-        oh /= op.stride;
-        const T *row = plane + (int64_t)oh * op.w_out;
-        float v[N];
-        const int ow0 = xg * N + op.padding - op.dilation * k2;
-        if (N > 1 && op.stride == 1 && row_ok && ow0 >= 0 && ow0 + N <= op.w_out) {
-            load_elems_unaligned<T, N>(row + ow0, v);  // unit stride, window inside the row
-        } else {
+// zero when no output position reads image pixel (y, x) through filter tap (k1, k2).  Same mapping, unit stride.
+template <typename T, int KS>
+__global__ __launch_bounds__(256) void unfold_output_plane_kernel(Op op, const T *__restrict__ grad_out, T *__restrict__ patches,
+                                                                  int slab_stride) {
+    constexpr int V = Elem<T>::VEC;
+    const int K = KS ? KS : op.kernel, kk = K * K, n = op.h_in * op.w_in, wg = op.w_in / V;
+    const T *plane = grad_out + (int64_t)blockIdx.x * op.h_out * op.w_out;
+    T *dst = patches + (int64_t)blockIdx.x * kk * slab_stride;
+    if ((int)threadIdx.x < slab_stride - n)
+        for (int tap = 0; tap < kk; tap++) Elem<T>::store(dst + (int64_t)tap * slab_stride + n + threadIdx.x, 0.0f);
+    for (int g = threadIdx.x; g < n / V; g += 256) {
+        const int y = g / wg, x = (g - y * wg) * V;
 #pragma unroll
-            for (int i = 0; i < N; i++) {
-                const int ow = ow0 + i;
-                const bool ok = row_ok && ow >= 0 && ow % op.stride == 0 && ow / op.stride < op.w_out;
-                v[i] = ok ? Elem<T>::load(row + ow / op.stride) : 0.0f;
+        for (int k1 = 0; k1 < (KS ? KS : 1); k1++)
+#pragma unroll
+            for (int k2 = 0; k2 < (KS ? KS : 1); k2++) {
+                if constexpr (KS != 0) {
+                    const int oh = y + op.padding - op.dilation * k1;
+                    *(u32x4 *)(dst + (int64_t)(k1 * K + k2) * slab_stride + g * V) =
+                        row_window<T>(plane + (int64_t)oh * op.w_out, oh >= 0 && oh < op.h_out, x + op.padding - op.dilation * k2, op.w_out);
+                }
+            }
+        if constexpr (KS == 0) {
+            for (int tap = 0; tap < kk; tap++) {
+                const int t1 = tap / K, t2 = tap - t1 * K;
+                const int oh = y + op.padding - op.dilation * t1;
+                *(u32x4 *)(dst + (int64_t)tap * slab_stride + g * V) =
+                    row_window<T>(plane + (int64_t)oh * op.w_out, oh >= 0 && oh < op.h_out, x + op.padding - op.dilation * t2, op.w_out);
             }
         }
-        store_elems<T, N>(dst + (int64_t)y * op.w_in + xg * N, v);
-    };
-    const int step_rows = 256 / wg;
-    if (step_rows) {
-        if ((int)threadIdx.x >= step_rows * wg) return;
-        const int xg = (int)threadIdx.x % wg;
-        for (int y = (int)threadIdx.x / wg; y < op.h_in; y += step_rows) emit(y, xg);
-    } else {
-        for (int g = threadIdx.x; g < op.h_in * wg; g += 256) emit(g / wg, g % wg);
     }
 }
 
-// The same two gathers for row widths that are not a multiple of the vector width, and for small images: a thread owns
-// one 16-byte vector of the patch buffer, i.e. V consecutive positions of a flattened (row, column) slab -- they may
-// straddle two rows -- whatever the slab size (a 7x7 slab would leave 249 of a workgroup's 256 threads idle);
-// positions behind the slab's last element (the row padding) are zeros.
+// The same two gathers for every other case (any stride, row widths that are not a multiple of the vector width, small
+// images): a thread owns one 16-byte vector of the patch buffer, i.e. V consecutive positions of a flattened (row,
+// column) slab -- they may straddle two rows -- whatever the slab size (a 7x7 slab would leave 249 of a workgroup's
+// 256 threads idle); positions behind the slab's last element (the row padding) are zeros.
 template <typename T>
 __global__ __launch_bounds__(256) void unfold_input_flat_kernel(Op op, const T *img, T *patches, int slab_stride, uint32_t vectors) {
     constexpr int V = Elem<T>::VEC;
@@ -248,14 +270,16 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
     if (int rc = ensure_patches(ctx, patch_bytes + out_bytes)) return rc;
     T *patches = (T *)ctx->patches;
     T *out_p = (T *)((char *)ctx->patches + patch_bytes);
-    const bool vec = op.w_out % V == 0 && n >= 256 * V;  // whole workgroups per slab only when a slab fills one
+    // a workgroup per image plane when its K*K slabs give the 256 threads a few vectors each
+    const bool planes = op.stride == 1 && op.w_out % V == 0 && op.w_in >= V && (n / V) * kk >= 512;
     for (int64_t b0 = 0; b0 < op.batch; b0 += chunk) {
         const int64_t nb = std::min<int64_t>(chunk, op.batch - b0);
         Op sub = op;
         sub.batch = (int)nb;
         const T *src = (const T *)img + b0 * op.chan_in * op.h_in * op.w_in;
         const unsigned slabs = (unsigned)(nb * op.chan_in * kk);
-        if (vec) unfold_input_kernel<T, V><<<slabs, 256, 0, ctx->stream>>>(sub, src, patches, (int)np);
+        if (planes && op.kernel == 3) unfold_input_plane_kernel<T, 3><<<slabs / 9, 256, 0, ctx->stream>>>(sub, src, patches, (int)np);
+        else if (planes) unfold_input_plane_kernel<T, 0><<<(unsigned)(slabs / kk), 256, 0, ctx->stream>>>(sub, src, patches, (int)np);
         else {
             const uint32_t vectors = (uint32_t)(slabs * (np / V));  // < 2^28: the chunk's patches stay below 2^31 elements
             unfold_input_flat_kernel<T><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, src, patches, (int)np, vectors);
@@ -314,14 +338,15 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     HIP_TRY(hipGetLastError());
     zero_kernel<T><<<fgrid, 256, 0, ctx->stream>>>(grad_f_tr, (int)f_elems);
     HIP_TRY(hipGetLastError());
-    const bool vec = op.w_in % V == 0 && hw >= 256 * V;
+    const bool planes = op.stride == 1 && op.w_in % V == 0 && op.w_out >= V && (hw / V) * kk >= 512;
     for (int64_t b0 = 0; b0 < op.batch; b0 += chunk) {
         const int64_t nb = std::min<int64_t>(chunk, op.batch - b0);
         Op sub = op;
         sub.batch = (int)nb;
         const T *go = (const T *)grad_out + b0 * op.chan_out * ohw;
         const unsigned slabs = (unsigned)(nb * op.chan_out * kk);
-        if (vec) unfold_output_kernel<T, V><<<slabs, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
+        if (planes && op.kernel == 3) unfold_output_plane_kernel<T, 3><<<slabs / 9, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
+        else if (planes) unfold_output_plane_kernel<T, 0><<<(unsigned)(slabs / kk), 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
         else {
             const uint32_t vectors = (uint32_t)(slabs * (hp / V));
             unfold_output_flat_kernel<T><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp, vectors);
