@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256) void unfold_input_flat_kernel(Op op, const T *
         store_elems<T, V>(dst + pos0, v);
     }
 }
-template <typename T>
+template <typename T, bool UNIT_STRIDE>
 __global__ __launch_bounds__(256) void unfold_output_flat_kernel(Op op, const T *grad_out, T *patches, int slab_stride, uint32_t vectors) {
     constexpr int V = Elem<T>::VEC;
     const uint32_t item = blockIdx.x * 256 + threadIdx.x;
@@ -171,9 +171,14 @@ __global__ __launch_bounds__(256) void unfold_output_flat_kernel(Op op, const T 
 #pragma unroll
             for (int i = 0; i < V; i++) {
                 const int oh = y + op.padding - op.dilation * k1, ow = x + op.padding - op.dilation * k2;
-                const bool ok = pos0 + i < n && oh >= 0 && oh % op.stride == 0 && oh / op.stride < op.h_out && ow >= 0 &&
-                                ow % op.stride == 0 && ow / op.stride < op.w_out;
-                v[i] = ok ? Elem<T>::load(plane + (int64_t)(oh / op.stride) * op.w_out + ow / op.stride) : 0.0f;
+                if constexpr (UNIT_STRIDE) {  // no divisions
+                    const bool ok = pos0 + i < n && oh >= 0 && oh < op.h_out && ow >= 0 && ow < op.w_out;
+                    v[i] = ok ? Elem<T>::load(plane + (int64_t)oh * op.w_out + ow) : 0.0f;
+                } else {
+                    const bool ok = pos0 + i < n && oh >= 0 && oh % op.stride == 0 && oh / op.stride < op.h_out && ow >= 0 &&
+                                    ow % op.stride == 0 && ow / op.stride < op.w_out;
+                    v[i] = ok ? Elem<T>::load(plane + (int64_t)(oh / op.stride) * op.w_out + ow / op.stride) : 0.0f;
+                }
                 if (++x == op.w_in) { x = 0; ++y; }
             }
         }
@@ -349,7 +354,8 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         else if (planes) unfold_output_plane_kernel<T, 0><<<(unsigned)(slabs / kk), 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
         else {
             const uint32_t vectors = (uint32_t)(slabs * (hp / V));
-            unfold_output_flat_kernel<T><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp, vectors);
+            if (op.stride == 1) unfold_output_flat_kernel<T, true><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp, vectors);
+            else unfold_output_flat_kernel<T, false><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp, vectors);
         }
         HIP_TRY(hipGetLastError());
         const T *img_b = (const T *)img + b0 * op.chan_in * hw;

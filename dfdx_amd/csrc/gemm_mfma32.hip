@@ -357,7 +357,8 @@ int mfma32_plan_splits(const GemmProblem &p, int variant, int compute_units, int
         return (int)s;
     }
     const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn);
-    int64_t s = std::min<int64_t>(std::min<int64_t>(16, compute_units / std::max<int64_t>(1, blocks)), total_iters / 4);
+    // enough work items for two workgroups per compute unit, at least four k steps each
+    int64_t s = std::min<int64_t>(std::min<int64_t>(64, 2 * compute_units / std::max<int64_t>(1, blocks)), total_iters / 4);
     while (s > 1 && (s - 1) * ((total_iters + s - 1) / s) >= total_iters) s--;
     return (int)std::max<int64_t>(1, s);
 }
