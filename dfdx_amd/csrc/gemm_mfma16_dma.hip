@@ -878,7 +878,8 @@ void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_va
         const int64_t tiles = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
         const double layout = (a_kc && b_kc) ? 1.0 : (!a_kc && !b_kc) ? 0.98 : 0.99;  // transposing LDS reads cost a little
         // candidates 1..16, 20..32, 40..64 (filter gradients of convolutions: a handful of tiles, thousands of k steps)
-        const int forced_s = forced_splits > 0 ? (int)std::min<int64_t>(forced_splits, total_iters) : 0;
+        int forced_s = forced_splits > 0 ? (int)std::min<int64_t>(forced_splits, total_iters) : 0;
+        while (forced_s > 1 && (forced_s - 1) * ((total_iters + forced_s - 1) / forced_s) >= total_iters) forced_s--;  // no empty split
         for (int s = forced_s ? forced_s : 1; s <= (forced_s ? forced_s : 64); s += (s < 16 ? 1 : s < 32 ? 4 : 8)) {
             if (s > 1 && (!may_split || (forced_splits == 0 && total_iters / s < 4))) break;
             const int64_t chunk = (total_iters + s - 1) / s;

@@ -263,6 +263,35 @@ def test_split_k_f32_planned_for_long_reductions():
     assert "splitk" not in dev.gemm_plan(desc)[2]
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+def test_split_k_many_ways_for_filter_gradient_shapes(dtype):
+    """A convolution's filter gradient: one or two output tiles and a reduction over batch x pixels.  The planner cuts
+    it into more than 16 pieces; forced counts beyond the planner's candidates (40, 64, 100) work too; every count
+    gives the same bits on every run and stays within tolerance."""
+    dev, g = device(), rng(79)
+    m, k, n, nb = 64, 1024, 192, 48
+    a = oracle.to_storage(g.standard_normal(nb * m * k), dtype)
+    b = oracle.to_storage(g.standard_normal(nb * n * k), dtype)     # stored (nb, n, k): B^T per batch
+    da, db = dev.tensor(a, dtype), dev.tensor(b, dtype)
+    A, B = oracle.to_f64(a, dtype).reshape(nb, m, k), oracle.to_f64(b, dtype).reshape(nb, n, k)
+    want = np.einsum("bmk,bnk->mn", A, B)
+    ulp = {"f16": 2.0 ** -11, "bf16": 2.0 ** -8, "f32": 2.0 ** -24}[dtype]
+    for split_k in (0, 40, 64, 100):
+        outs = []
+        for _ in range(2):
+            dc = dev.zeros(dtype, (m, n))
+            desc = dev.gemm_desc(dtype, m, k, n, da.ptr, (k, 1), db.ptr, (1, k), dc.ptr, (n, 1), accumulate=True,
+                                 batch=(nb, 1), a_batch=(m * k, 0), b_batch=(n * k, 0), reduce_batch=True, split_k=split_k)
+            name = dev.gemm_plan(desc)[2]
+            announce("filter-gradient split-k", dtype, split_k, name)
+            splits = int(name.rsplit("splitk", 1)[1]) if "splitk" in name else 1
+            assert 16 < splits <= (split_k or 64), name      # a forced count shrinks until no piece is empty
+            dev.gemm(desc)
+            outs.append(dev.to_host(dc))
+        assert np.array_equal(outs[0], outs[1])
+        assert_within(dtype, nb * k, oracle.to_f64(outs[0], dtype).reshape(m, n), want, A, B, extra=ulp * np.abs(want).max())
+
+
 # ------------------------------------------------------------------ batched --
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("kernel", [KERNEL_GENERIC, KERNEL_MFMA])
