@@ -167,6 +167,30 @@ def main():
                 gov, gbv, bv = view(go, dt), view(zeros((nout,), dt), dt), view(rnd((nout,), dt), dt)
                 timed("glue", f"bias backward {T}x{nout} bf16", lambda: dev.bias_backward(gov, gbv), 0, T * nout * 2, "bias_backward")
 
+        # the block's attention products: heads interleaved in the token rows (batch-2 stride 64 < row stride 1024),
+        # as MultiHeadAttention's reshape + permute hands them over (multi_head_attention.rs:105-146)
+        Bq, H, S, D, es = 16, 16, 512, 64, 2
+        nb = Bq * H
+        q, k, v, d_o = (rnd((Bq, S, H * D), dt) for _ in range(4))
+        sc, p_, gp = zeros((Bq, H, S, S), dt), rnd((Bq, H, S, S), dt, 0.05), zeros((Bq, H, S, S), dt)
+        o, gv = zeros((Bq, H, S, D), dt), zeros((Bq, S, H * D), dt)
+        tok, sSS, sSD = (S * H * D, D), (H * S * S, S * S), (H * S * D, S * D)
+        fl = 2 * nb * S * S * D
+
+        def d5(m, kk, n, a, astr, ab, b, bstr, bb, c, cstr, cb, acc):
+            return dev.gemm_desc(dt, m, kk, n, P(a), astr, P(b), bstr, P(c), cstr, accumulate=acc, batch=(Bq, H),
+                                 a_batch=ab, b_batch=bb, c_batch=cb)
+
+        gemm("c5", "attn scores Q.K^T 512x64x512 interleaved", d5(S, D, S, q, (H * D, 1), tok, k, (1, H * D), tok, sc, (S, 1), sSS, False),
+             fl, es * nb * (2 * S * D + S * S))
+        gemm("c5", "attn out P.V 512x512x64 interleaved V", d5(S, S, D, p_, (S, 1), sSS, v, (H * D, 1), tok, o, (D, 1), sSD, False),
+             fl, es * nb * (S * S + 2 * S * D))
+        gemm("c5", "attn dP dO.V^T acc", d5(S, D, S, d_o, (D, 1), sSD, v, (1, H * D), tok, gp, (S, 1), sSS, True),
+             fl, es * nb * (2 * S * D + 2 * S * S))
+        gemm("c5", "attn dV P^T.dO acc, interleaved rows", d5(S, S, D, p_, (1, S), sSS, d_o, (D, 1), sSD, gv, (H * D, 1), tok, True),
+             fl, es * nb * (S * S + 3 * S * D))
+        del sc, p_, gp
+
     # ---- vec.mat / mat.vec: HBM roofline ------------------------------------------------------------------------
     if want("gemv"):
         for dt in ("f16", "f32"):
