@@ -4,7 +4,8 @@ A step is one 4096^3 f16 GEMM (f32 accumulate), C = A.B with row-major operands 
 HBM -- the configuration the headline metric is quoted on.  The same launch is also timed for the
 transposed-stride variants and for f32.  One JSON line is printed:
 
-  value       f16 A.B throughput in TFLOP/s over the K timed steps (wall clock, synchronised both sides)
+  value       f16 A.B throughput in TFLOP/s over the K timed steps (wall clock, synchronised both sides; the device is
+              first brought to its sustained clock by --spinup-ms of untimed launches, then the W warm-up steps run)
   roofline    the f16 MFMA kernel's TFLOP/s from HIP events on the launch stream vs the 2.5 PFLOP/s dense peak
   cpu_baseline  the CPU oracle (a port of dfdx's Cpu matmul semantics) timed on the host cores
 """
@@ -27,6 +28,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--spinup-ms", type=float, default=300.0,
+                    help="untimed device spin-up before the first warm-up step (0 disables it)")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection aid: 3 plain 256 MiB device copies, then 5 headline GEMM launches, nothing else")
     ap.add_argument("--probe-variants", action="store_true",
@@ -78,6 +81,19 @@ def main():
     tdt = {"f16": torch.float16, "f32": torch.float32}
     res = {}
     headline = None
+    if args.spinup_ms > 0:
+        # An idle MI355X needs about 30 ms of load to reach its sustained clock (launches 150 -> 118 us over the first
+        # ~250): run the headline launch untimed for a fixed wall-clock span first, so that a short --warmup does not
+        # put the clock ramp into the timed steps.  The W warm-up and K timed steps below follow as asked.
+        sa = (torch.rand(N, N, device="cuda") * 2 - 1).half()
+        sc = torch.zeros(N, N, device="cuda", dtype=torch.float16)
+        sd = dev.gemm_desc("f16", N, N, N, sa.data_ptr(), (N, 1), sa.data_ptr(), (N, 1), sc.data_ptr(), (N, 1))
+        t_end = time.perf_counter() + args.spinup_ms * 1e-3
+        while time.perf_counter() < t_end:
+            for _ in range(50):
+                dev.gemm(sd)
+            torch.cuda.synchronize()
+        del sa, sc
     for dtype in ("f16", "f32"):
         gen = torch.Generator(device="cuda").manual_seed(1234)
         a = (torch.rand(N, N, device="cuda", generator=gen) * 2 - 1).to(tdt[dtype])
