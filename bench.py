@@ -78,7 +78,7 @@ def main():
         print(json.dumps({"probe": names}))
         return
     flop = 2.0 * N ** 3
-    tdt = {"f16": torch.float16, "f32": torch.float32}
+    tdt = {"f16": torch.float16, "f32": torch.float32, "bf16": torch.bfloat16}
     res = {}
     headline = None
     if args.spinup_ms > 0:
@@ -94,12 +94,14 @@ def main():
                 dev.gemm(sd)
             torch.cuda.synchronize()
         del sa, sc
-    for dtype in ("f16", "f32"):
+    for dtype in ("f16", "f32", "bf16"):
         gen = torch.Generator(device="cuda").manual_seed(1234)
         a = (torch.rand(N, N, device="cuda", generator=gen) * 2 - 1).to(tdt[dtype])
         b = (torch.rand(N, N, device="cuda", generator=gen) * 2 - 1).to(tdt[dtype])
         c = torch.zeros(N, N, device="cuda", dtype=tdt[dtype])
         layouts = {"A.B": ((N, 1), (N, 1)), "At.B": ((1, N), (N, 1)), "A.Bt": ((N, 1), (1, N))}
+        if dtype == "bf16":
+            layouts = {"A.B": layouts["A.B"]}   # same kernel as f16; one layout as a cross-check
         res[dtype] = {}
         for name, (astr, bstr) in layouts.items():
             desc = dev.gemm_desc(dtype, N, N, N, a.data_ptr(), astr, b.data_ptr(), bstr, c.data_ptr(), (N, 1))
