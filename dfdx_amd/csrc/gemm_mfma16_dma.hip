@@ -856,6 +856,7 @@ constexpr VariantModel kModel[] = {
 };
 constexpr double kItemOverhead = 3.1e-6, kLaunchLatency = 2e-6, kCuBandwidth = 24e9, kOperandWeight = 0.32;
 constexpr double kIdleBoost = 0.146, kWsBandwidthCached = 9.5e12, kWsBandwidthHbm = 6.1e12, kWsCached = 128e6;
+constexpr double kSplitLaunch = 7e-6, kSplitPerPiece = 0.25e-6;  // 1024^3: 12.4 us unsplit, 15.9 / 18.0 us in 2 / 4 pieces
 }  // namespace
 
 void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_variant, int forced_splits, int *variant,
@@ -896,7 +897,9 @@ void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_va
                           out_bytes / (kCuBandwidth / conc);
             if (s > 1) {
                 const double ws = s * out_elems * 4.0;
-                time += 3e-6 + (ws + out_elems * elem * (1 + p.accumulate)) / (ws <= kWsCached ? kWsBandwidthCached : kWsBandwidthHbm);
+                // second launch + the reduce kernel's chain of s dependent partial-tile reads, then the workspace round trip
+                time += kSplitLaunch + kSplitPerPiece * s +
+                        (ws + out_elems * elem * (1 + p.accumulate)) / (ws <= kWsCached ? kWsBandwidthCached : kWsBandwidthHbm);
             }
             if (time < best) {
                 best = time;
