@@ -850,9 +850,9 @@ struct VariantModel {
 constexpr VariantModel kModel[] = {
     {1, 4.64e12, 4.64e12},  // 256x256
     {1, 3.81e12, 3.81e12},  // 256x128
-    {2, 2.50e12, 4.25e12},  // 128x128
+    {2, 3.00e12, 4.25e12},  // 128x128
     {1, 3.60e12, 3.60e12},  // 256x64
-    {2, 2.20e12, 3.30e12},  // 128x64
+    {2, 2.20e12, 2.90e12},  // 128x64
 };
 constexpr double kItemOverhead = 3.1e-6, kLaunchLatency = 2e-6, kCuBandwidth = 24e9, kOperandWeight = 0.32;
 constexpr double kIdleBoost = 0.146, kWsBandwidthCached = 9.5e12, kWsBandwidthHbm = 6.1e12, kWsCached = 128e6;
@@ -875,7 +875,9 @@ void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_va
         if (!mfma16dma_supported(p, v)) continue;
         const Variant &t = kVariants[v - 1];
         const VariantModel &vm = kModel[v - 1];
-        if (forced_variant == 0 && ((p.n <= 64) != (t.bn <= 64))) continue;  // BN = 64 tiles only for narrow outputs
+        // narrow outputs take the BN = 64 tiles; wide ones may take the small 128 x 64 tile (more workgroups for a
+        // problem of a few tiles), never the 256 x 64 one
+        if (forced_variant == 0 && (p.n <= 64 ? t.bn > 64 : (t.bn <= 64 && t.bm > 128))) continue;
         const int64_t tiles = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
         const double layout = (a_kc && b_kc) ? 1.0 : (!a_kc && !b_kc) ? 0.98 : 0.99;  // transposing LDS reads cost a little
         // candidates 1..16, 20..32, 40..64 (filter gradients of convolutions: a handful of tiles, thousands of k steps)
