@@ -101,7 +101,7 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
             }
             if (v) return DFDX_ROCM_ERR_UNSUPPORTED;
         }
-        if (v == 0) v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units) : 0;
+        if (v == 0) v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units, forced_splits) : 0;
         const bool ok = is16 ? mfma16_supported(p, v) : is32 ? mfma32_supported(p, v) : false;
         if (!ok) return DFDX_ROCM_ERR_UNSUPPORTED;
         *plan = {DFDX_ROCM_KERNEL_MFMA, v, is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
@@ -124,7 +124,7 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
             return DFDX_ROCM_OK;
         }
     }
-    int v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units) : 0;
+    int v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units, forced_splits) : 0;
     if (v > 0) {
         *plan = {DFDX_ROCM_KERNEL_MFMA, v, is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
         return DFDX_ROCM_OK;

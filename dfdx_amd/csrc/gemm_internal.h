@@ -76,7 +76,7 @@ hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_
 int mfma32_variant_count();
 const char *mfma32_variant_name(int variant);
 bool mfma32_supported(const GemmProblem &p, int variant);
-int mfma32_pick_variant(const GemmProblem &p, int compute_units);
+int mfma32_pick_variant(const GemmProblem &p, int compute_units, int forced_splits);
 int mfma32_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits);
 size_t mfma32_workspace_bytes(const GemmProblem &p, int variant, int splits);
 hipError_t launch_mfma32(const GemmProblem &p, int variant, hipStream_t stream);

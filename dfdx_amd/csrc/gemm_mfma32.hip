@@ -345,22 +345,64 @@ bool mfma32_supported(const GemmProblem &p, int variant) {
 
 // Split-k for small outputs with a long reduction (weight gradients): when the chosen tile shape leaves most of
 // the chip idle, the k loop is cut into up to 16 slices of at least 4 steps each.
-int mfma32_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits) {
-    if (variant < 1 || variant > (int)(sizeof(kVariants) / sizeof(kVariants[0]))) return 1;
-    const Variant &t = kVariants[variant - 1];
+// Planner of the f32 family: estimated time of (tile variant, k pieces) = rounds of workgroups x k steps x the time of
+// one step at the variant's measured rate (relative to 256x256 at 4096^3: 128 / 130 TFLOP/s down to 101 for 64x64,
+// shared by the workgroups a compute unit holds), plus, for a split, the second launch and the workspace round trip.
+// Measured against forced sweeps: a per-image convolution GEMM with 64 output channels runs 3.4x faster on 64-row
+// tiles than on the largest tile that fills the chip; long-k weight gradients want the big tile cut 16 ways.
+namespace {
+constexpr double kRate32[kNumVariants] = {1.0, 0.97, 0.90, 0.91, 0.80, 0.78};
+constexpr int kPerCu32[kNumVariants] = {1, 1, 1, 2, 2, 4};  // workgroups a compute unit holds (LDS)
+constexpr double kCuFlops32 = 130e12 / 256, kSplitLaunch32 = 2.5e-6, kWorkspaceBw32 = 4.5e12;
+constexpr double kStepLatency32 = 1.0e-6;  // a k step of a lone small workgroup is bound by its load -> LDS -> MFMA chain
+
+double plan_time32(const GemmProblem &p, int v, int64_t s, int compute_units) {
+    const Variant &t = kVariants[v - 1];
     const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
     const int64_t total_iters = ((p.k + t.bk - 1) / t.bk) * (p.reduce ? p.nb1 * p.nb2 : 1);
-    if (nbatch != 1 || p.c_cs != 1 || total_iters < 2) return 1;
+    const int64_t items = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch * s;
+    const int64_t slots = (int64_t)std::max(1, compute_units) * kPerCu32[v - 1];
+    const double rounds = std::max(1.0, (double)items / (double)slots);  // workgroups are handed out as others finish
+    const int64_t conc = std::min<int64_t>(kPerCu32[v - 1], (items + compute_units - 1) / std::max(1, compute_units));
+    const double step = std::max(kStepLatency32, 2.0 * t.bm * t.bn * t.bk / (kRate32[v - 1] * kCuFlops32 / (double)conc));
+    double time = rounds * (double)((total_iters + s - 1) / s) * step + 4e-6;
+    if (s > 1) time += kSplitLaunch32 + (double)s * (double)p.m * (double)p.n * 4.0 * 2.0 / kWorkspaceBw32;
+    return time;
+}
+
+// best number of pieces for one variant (1 when it may not be split)
+int64_t plan_pieces32(const GemmProblem &p, int v, int compute_units, int forced_splits, double *time) {
+    const Variant &t = kVariants[v - 1];
+    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+    const int64_t total_iters = ((p.k + t.bk - 1) / t.bk) * (p.reduce ? p.nb1 * p.nb2 : 1);
+    const bool may_split = nbatch == 1 && p.c_cs == 1 && total_iters >= 2;
+    auto valid = [&](int64_t s) { return s == 1 || (s - 1) * ((total_iters + s - 1) / s) < total_iters; };  // no empty piece
     if (forced_splits > 0) {
-        int64_t s = std::min<int64_t>(forced_splits, total_iters);
-        while (s > 1 && (s - 1) * ((total_iters + s - 1) / s) >= total_iters) s--;  // no empty split
-        return (int)s;
+        int64_t s = may_split ? std::min<int64_t>(forced_splits, total_iters) : 1;
+        while (!valid(s)) s--;
+        if (time) *time = plan_time32(p, v, s, compute_units);
+        return s;
     }
-    const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn);
-    // enough work items for two workgroups per compute unit, at least four k steps each
-    int64_t s = std::min<int64_t>(std::min<int64_t>(64, 2 * compute_units / std::max<int64_t>(1, blocks)), total_iters / 4);
-    while (s > 1 && (s - 1) * ((total_iters + s - 1) / s) >= total_iters) s--;
-    return (int)std::max<int64_t>(1, s);
+    int64_t best = 1;
+    double best_time = plan_time32(p, v, 1, compute_units);
+    constexpr int kCandidates[] = {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
+    for (int s : kCandidates) {
+        if (!may_split || total_iters / s < 4) break;
+        if (!valid(s)) continue;
+        const double tm = plan_time32(p, v, s, compute_units);
+        if (tm < best_time) {
+            best_time = tm;
+            best = s;
+        }
+    }
+    if (time) *time = best_time;
+    return best;
+}
+}  // namespace
+
+int mfma32_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits) {
+    if (variant < 1 || variant > kNumVariants) return 1;
+    return (int)plan_pieces32(p, variant, compute_units, forced_splits, nullptr);
 }
 
 static void ws_layout32(const GemmProblem &p, int variant, int64_t *ld, int64_t *split_stride) {
@@ -376,22 +418,15 @@ size_t mfma32_workspace_bytes(const GemmProblem &p, int variant, int splits) {
     return (size_t)stride * splits * sizeof(float);
 }
 
-int mfma32_pick_variant(const GemmProblem &p, int compute_units) {
-    // Least estimated time: the work of the padded tiles over the variant's measured rate (relative to 256x256 at
-    // 4096^3: 128 / 130 TFLOP/s down to 101 for 64x64) and over the share of the chip its workgroups fill.  A
-    // per-image convolution GEMM with 64 output channels runs 3.4x faster on 64-row tiles than on 256-row ones.
-    constexpr double kRate[kNumVariants] = {1.0, 0.97, 0.90, 0.91, 0.80, 0.78};
-    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+int mfma32_pick_variant(const GemmProblem &p, int compute_units, int forced_splits) {
     int best = 0;
     double best_time = 1e300;
     for (int v = 1; v <= kNumVariants; v++) {
         if (!mfma32_supported(p, v)) continue;
-        const Variant &t = kVariants[v - 1];
-        const double blocks = (double)((p.m + t.bm - 1) / t.bm) * (double)((p.n + t.bn - 1) / t.bn) * (double)nbatch;
-        const double fill = std::min(1.0, blocks / std::max(1, compute_units));
-        const double time = blocks * t.bm * t.bn / (kRate[v - 1] * fill);
-        if (time < best_time) {
-            best_time = time;
+        double tm;
+        plan_pieces32(p, v, compute_units, forced_splits, &tm);
+        if (tm < best_time) {
+            best_time = tm;
             best = v;
         }
     }
