@@ -456,17 +456,28 @@ int mfma16_dma_first_variant() { return kNumVariants + 1; }
 
 int mfma16_pick_variant(const GemmProblem &p, int compute_units) {
     if (const int d = mfma16dma_pick_variant(p, compute_units)) return kNumVariants + d;
-    // Largest tile that still gives every compute unit at least one workgroup; ties go to the larger tile.
+    // Least estimated time among the BK = 64 tiles: the work of the padded tiles over the tile's rate (measured at
+    // 4096^3 relative to 256x256: 821 TFLOP/s down to 377 for 64x64) and over the share of the chip its workgroups
+    // fill.  Per-image convolution GEMMs with 64 or 96 rows run 1.5-1.8x faster on the small tiles than on the
+    // largest tile that fills the chip.
     const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
-    const int order[] = {1, 3, 4, 5, 6};
-    for (int v : order) {
-        const Variant &t = kVariants[v - 1];
+    const int candidates[] = {1, 3, 4, 5, 6};
+    const double rate[] = {1.0, 0.60, 0.73, 0.54, 0.46};
+    int best = 0;
+    double best_time = 1e300;
+    for (int i = 0; i < 5; i++) {
+        const int v = candidates[i];
         if (!mfma16_supported(p, v)) continue;
-        if (p.n <= 64 && t.bn > 64) continue;
-        const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch;
-        if (blocks >= compute_units || v == 6) return v;
+        const Variant &t = kVariants[v - 1];
+        const double blocks = (double)((p.m + t.bm - 1) / t.bm) * (double)((p.n + t.bn - 1) / t.bn) * (double)nbatch;
+        const double fill = std::min(1.0, blocks / std::max(1, compute_units));
+        const double time = blocks * t.bm * t.bn / (rate[i] * fill);
+        if (time < best_time) {
+            best_time = time;
+            best = v;
+        }
     }
-    return mfma16_supported(p, 6) ? 6 : 0;
+    return best;
 }
 
 hipError_t launch_mfma16(const GemmProblem &g, int variant, hipStream_t stream) {
