@@ -206,6 +206,7 @@ def main():
     if want("conv"):
         for dt, (B, C, O, H, W_, K, s, pad) in (("f16", (64, 64, 64, 56, 56, 3, 1, 1)), ("f16", (64, 128, 128, 28, 28, 3, 1, 1)),
                                                 ("f16", (64, 256, 256, 14, 14, 3, 1, 1)), ("f16", (64, 512, 512, 7, 7, 3, 1, 1)),
+                                                ("f16", (64, 256, 64, 56, 56, 1, 1, 0)),
                                                 ("f32", (32, 64, 64, 56, 56, 3, 1, 1))):
             x, w = rnd((B, C, H, W_), dt), rnd((O, C, K, K), dt, 1 / 24)
             xv, wv = view(x, dt), view(w, dt)

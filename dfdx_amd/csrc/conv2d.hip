@@ -270,7 +270,10 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
     int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
     chunk = std::min<int64_t>(std::min<int64_t>(chunk, op.batch), ((1ll << 31) - 1) / per_image);
     const bool padded = np != n;  // the product goes to a padded copy of the output, which is then compacted
-    const size_t patch_bytes = round256((size_t)(chunk * per_image) * sizeof(T));
+    // 1x1 filters at unit stride without padding: the patch matrix IS the image -- no gather, one product for the batch
+    const bool pointwise = op.kernel == 1 && op.stride == 1 && op.padding == 0 && !padded && ((uintptr_t)img & 15u) == 0;
+    if (pointwise) chunk = op.batch;
+    const size_t patch_bytes = pointwise ? 0 : round256((size_t)(chunk * per_image) * sizeof(T));
     const size_t out_bytes = padded ? round256((size_t)(chunk * op.chan_out * np) * sizeof(T)) : 0;
     if (int rc = ensure_patches(ctx, patch_bytes + out_bytes)) return rc;
     T *patches = (T *)ctx->patches;
@@ -283,7 +286,8 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
         sub.batch = (int)nb;
         const T *src = (const T *)img + b0 * op.chan_in * op.h_in * op.w_in;
         const unsigned slabs = (unsigned)(nb * op.chan_in * kk);
-        if (planes && op.kernel == 3) unfold_input_plane_kernel<T, 3><<<slabs / 9, 256, 0, ctx->stream>>>(sub, src, patches, (int)np);
+        if (pointwise) patches = const_cast<T *>(src);
+        else if (planes && op.kernel == 3) unfold_input_plane_kernel<T, 3><<<slabs / 9, 256, 0, ctx->stream>>>(sub, src, patches, (int)np);
         else if (planes) unfold_input_plane_kernel<T, 0><<<(unsigned)(slabs / kk), 256, 0, ctx->stream>>>(sub, src, patches, (int)np);
         else {
             const uint32_t vectors = (uint32_t)(slabs * (np / V));  // < 2^28: the chunk's patches stay below 2^31 elements
@@ -329,7 +333,10 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     // (zeros behind every row; the gradient copy starts from grad_img, so beta = 1 rounds exactly as without it).
     const bool padded = hp != hw;
     // patch buffer: [chunk][O*K*K][hp], the transposed filters and their gradient, then the padded copies
-    const size_t patch_bytes = round256((size_t)(chunk * per_image) * sizeof(T));
+    // 1x1 filters at unit stride without padding: the patch matrix IS grad_out
+    const bool pointwise = op.kernel == 1 && op.stride == 1 && op.padding == 0 && !padded && ((uintptr_t)grad_out & 15u) == 0;
+    if (pointwise) chunk = op.batch;
+    const size_t patch_bytes = pointwise ? 0 : round256((size_t)(chunk * per_image) * sizeof(T));
     const size_t f_bytes = round256((size_t)f_elems * sizeof(T));
     const size_t img_bytes = padded ? round256((size_t)(chunk * op.chan_in * hp) * sizeof(T)) : 0;
     if (int rc = ensure_patches(ctx, patch_bytes + 2 * f_bytes + 2 * img_bytes)) return rc;
@@ -350,7 +357,8 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         sub.batch = (int)nb;
         const T *go = (const T *)grad_out + b0 * op.chan_out * ohw;
         const unsigned slabs = (unsigned)(nb * op.chan_out * kk);
-        if (planes && op.kernel == 3) unfold_output_plane_kernel<T, 3><<<slabs / 9, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
+        if (pointwise) patches = const_cast<T *>(go);
+        else if (planes && op.kernel == 3) unfold_output_plane_kernel<T, 3><<<slabs / 9, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
         else if (planes) unfold_output_plane_kernel<T, 0><<<(unsigned)(slabs / kk), 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
         else {
             const uint32_t vectors = (uint32_t)(slabs * (hp / V));

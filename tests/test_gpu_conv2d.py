@@ -54,6 +54,8 @@ CONFIGS = [
     (2, 9, 15, 14, 14, 3, 1, 0, 1, 3),     # the shape of its grouped-slices test (:405-464)
     (4, 64, 64, 28, 28, 3, 1, 1, 1, 1),    # k = 576, n = 784: the MFMA kernels
     (2, 64, 128, 32, 32, 3, 2, 1, 1, 2),
+    (4, 64, 128, 8, 8, 1, 1, 0, 1, 1),     # 1x1 filters: the image / grad_out are the patch matrices, no gather
+    (2, 64, 64, 16, 16, 1, 1, 0, 1, 2),    # the same with groups
     (4, 64, 64, 14, 14, 3, 1, 1, 1, 1),    # n = 196: rows padded to the vector width inside the patch buffer
     (2, 32, 48, 7, 7, 3, 1, 1, 1, 1),      # n = 49
     (2, 16, 32, 15, 13, 3, 2, 1, 1, 1),    # input 195 and output 56 positions: only the backward side is padded
