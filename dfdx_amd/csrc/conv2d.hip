@@ -4,6 +4,7 @@
 // that reduces over the batch.
 #include "ctx_internal.h"
 #include "elem.h"
+#include "gemm_internal.h"
 
 #include <cstring>
 
@@ -13,38 +14,6 @@ namespace {
 struct Op {  // dfdx_rocm_conv2d_op narrowed to 32 bits (validated on entry)
     int kernel, stride, padding, dilation, groups, batch, chan_in, chan_out, h_in, h_out, w_in, w_out;
 };
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
-
-// A 16-byte vector moved by `bits` towards element 0 (bits > 0) or away from it (bits < 0), zeros moving in.
-__device__ __forceinline__ u32x4 shift128(u32x4 r, int bits) {
-    uint64_t lo = r[0] | ((uint64_t)r[1] << 32), hi = r[2] | ((uint64_t)r[3] << 32);
-    if (bits >= 0) {
-        const unsigned s = (unsigned)bits;
-        if (s >= 64) { lo = hi; hi = 0; }
-        const unsigned t = s & 63;
-        if (t) { lo = (lo >> t) | (hi << (64 - t)); hi >>= t; }
-        if (s >= 128) lo = 0;
-    } else {
-        const unsigned s = (unsigned)(-bits);
-        if (s >= 64) { hi = lo; lo = 0; }
-        const unsigned t = s & 63;
-        if (t) { hi = (hi << t) | (lo >> (64 - t)); lo <<= t; }
-        if (s >= 128) hi = 0;
-    }
-    return u32x4{(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
-}
-// N = 16 bytes of elements of one image row starting at column x0, zeros outside [0, width): one (unaligned) vector
-// load from the nearest window inside the row, then a shift -- no per-element path for the lanes at the image border,
-// which a wave would otherwise execute in full next to the vector path of its interior lanes.  width >= N.
-template <typename T> __device__ __forceinline__ u32x4 row_window(const T *row, bool row_ok, int x0, int width) {
-    constexpr int N = Elem<T>::VEC;
-    const int x0c = min(max(x0, 0), width - N);
-    u32x4 raw = {0u, 0u, 0u, 0u};
-    if (row_ok) raw = *(const u32x4_unaligned *)(row + x0c);
-    return shift128(raw, (x0 - x0c) * (int)(8 * sizeof(T)));
-}
 
 // patches[b][c][k1][k2][oh][ow] = img[b][c][oh*stride + dilation*k1 - padding][ow*stride + dilation*k2 - padding],
 // zero outside the image.  Unit stride, output width a multiple of the vector: one workgroup per (b, c) plane writes
@@ -257,6 +226,35 @@ dfdx_rocm_gemm_desc blank_desc(int dtype, int64_t m, int64_t k, int64_t n) {
     return d;
 }
 
+// Unit-stride forward convolutions of the 16-bit types without a patch matrix in memory: the GEMM kernel forms its B
+// tiles from the image planes themselves (one window load per 8 pixels, zeros where the window leaves the image), so
+// the K*K-fold copy of the image is neither written nor read back.  Returns false when the shape does not fit (the
+// caller then unfolds as for every other case).  The backward pass keeps the patch matrix: the filter gradient needs
+// it anyway, and reading it back for the image gradient costs less than forming the windows a second time (57 vs
+// 81 us at 64 channels, 56x56).
+template <typename T>
+bool implicit_forward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *filters, const void *img, void *out, int *rc) {
+    if (sizeof(T) != 2 || op.stride != 1) return false;
+    const int64_t kk = (int64_t)op.kernel * op.kernel, hw = (int64_t)op.h_in * op.w_in, ohw = (int64_t)op.h_out * op.w_out;
+    const int64_t cg = op.chan_in / op.groups, og = op.chan_out / op.groups;
+    GemmProblem g{};  // out (B, G, O/G, OH*OW) = filters (G, O/G, C/G*K*K) . patches of img
+    g.dtype = dtype == DFDX_ROCM_F16 ? DT_F16 : DT_BF16;
+    g.m = og; g.k = cg * kk; g.n = ohw;
+    g.nb1 = op.batch; g.nb2 = op.groups;
+    g.a = filters; g.a_rs = g.k; g.a_cs = 1; g.a_b1 = 0; g.a_b2 = g.m * g.k;
+    g.b = img; g.b_b1 = op.chan_in * hw; g.b_b2 = cg * hw;
+    g.c = out; g.c_rs = ohw; g.c_cs = 1; g.c_b1 = op.chan_out * ohw; g.c_b2 = og * ohw;
+    g.compute_units = ctx->compute_units;
+    ConvPatches cv{};
+    cv.taps = (int)kk; cv.ksize = op.kernel;
+    cv.w_dst = op.w_out; cv.h_src = op.h_in; cv.w_src = op.w_in; cv.plane = hw;
+    cv.off_y = cv.off_x = -op.padding; cv.step_y = cv.step_x = op.dilation;
+    const hipError_t e = launch_mfma16_conv(g, cv, ctx->compute_units, ctx->stream);
+    if (e == hipErrorNotSupported) return false;
+    *rc = (int)e;
+    return true;
+}
+
 template <typename T>
 int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void *filters, void *out) {
     constexpr int V = Elem<T>::VEC;
@@ -266,6 +264,10 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
     const int64_t per_image = (int64_t)op.chan_in * kk * np;  // patch elements of one image
     if (per_image == 0 || m == 0) return DFDX_ROCM_OK;
     if (per_image >= (1ll << 31) || (int64_t)op.chan_out * np >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
+    if (op.kernel > 1) {  // (1x1 filters have no patch matrix to avoid: see `pointwise` below)
+        int rc = 0;
+        if (implicit_forward<T>(ctx, dtype, op, filters, img, out, &rc)) return rc;
+    }
     CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
     int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
     chunk = std::min<int64_t>(std::min<int64_t>(chunk, op.batch), ((1ll << 31) - 1) / per_image);

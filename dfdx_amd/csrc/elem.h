@@ -73,4 +73,40 @@ template <typename T, int N> __device__ __forceinline__ void store_elems(T *p, c
     }
 }
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
+
+// A 16-byte vector moved by `bits` towards element 0 (bits > 0) or away from it (bits < 0), zeros moving in.
+__device__ __forceinline__ u32x4 shift128(u32x4 r, int bits) {
+    uint64_t lo = r[0] | ((uint64_t)r[1] << 32), hi = r[2] | ((uint64_t)r[3] << 32);
+    if (bits >= 0) {
+        const unsigned s = (unsigned)bits;
+        if (s >= 64) { lo = hi; hi = 0; }
+        const unsigned t = s & 63;
+        if (t) { lo = (lo >> t) | (hi << (64 - t)); hi >>= t; }
+        if (s >= 128) lo = 0;
+    } else {
+        const unsigned s = (unsigned)(-bits);
+        if (s >= 64) { hi = lo; lo = 0; }
+        const unsigned t = s & 63;
+        if (t) { hi = (hi << t) | (lo >> (64 - t)); lo <<= t; }
+        if (s >= 128) hi = 0;
+    }
+    return u32x4{(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
+}
+// 16 bytes of elements (ELEM_BYTES each) of one image row starting at column x0, zeros outside [0, width): one
+// (unaligned) vector load from the nearest window inside the row, then a shift -- no per-element path for the lanes at
+// the image border, which a wave would otherwise execute in full next to the vector path of its interior lanes.
+// width >= 16 / ELEM_BYTES.
+template <int ELEM_BYTES> __device__ __forceinline__ u32x4 row_window_bytes(const void *row, bool row_ok, int x0, int width) {
+    constexpr int N = 16 / ELEM_BYTES;
+    const int x0c = min(max(x0, 0), width - N);
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (row_ok) raw = *(const u32x4_unaligned *)((const char *)row + (int64_t)x0c * ELEM_BYTES);
+    return shift128(raw, (x0 - x0c) * (8 * ELEM_BYTES));
+}
+template <typename T> __device__ __forceinline__ u32x4 row_window(const T *row, bool row_ok, int x0, int width) {
+    return row_window_bytes<(int)sizeof(T)>(row, row_ok, x0, width);
+}
+
 }  // namespace dfdx_rocm

@@ -30,6 +30,17 @@ struct GemmProblem {
     int compute_units;  // of the device the launch goes to (persistent kernels size their grid with it)
 };
 
+// The patch matrix of a unit-stride convolution as the B operand of a GEMM, never materialised: row k = (channel,
+// tap (k1, k2)), column = pixel (r, x) of a `w_dst`-wide grid; element = plane[channel][r + off_y + step_y * k1]
+// [x + off_x + step_x * k2], zero outside the h_src x w_src plane.
+struct ConvPatches {
+    int taps, ksize;     // K*K, K
+    int w_dst;           // pixels per row of the column index space (a multiple of 8)
+    int h_src, w_src;    // the planes the windows come from (w_src >= 8)
+    int off_y, off_x, step_y, step_x;
+    int64_t plane;       // elements between channels
+};
+
 static inline size_t dtype_size(int dt) { return dt == DT_F32 ? 4 : (dt == DT_F64 ? 8 : 2); }
 
 // Swap the roles of the operands: C^T = B^T A^T.  Used to turn a column-major C into a row-major one.
@@ -55,6 +66,10 @@ bool mfma16_supported(const GemmProblem &p, int variant);
 int mfma16_pick_variant(const GemmProblem &p, int compute_units);
 int mfma16_dma_first_variant();  // variant ids >= this are the LDS-DMA kernels
 hipError_t launch_mfma16(const GemmProblem &p, int variant, hipStream_t stream);
+// The same product with B given as a patch matrix (`p.b` = channel 0 of the first image, b_b1 / b_b2 = image and group
+// strides, b_rs / b_cs unused): register-staged kernels only, tile chosen inside.  Returns hipErrorNotSupported when
+// the shape does not fit (the caller then unfolds).
+hipError_t launch_mfma16_conv(const GemmProblem &p, const ConvPatches &conv, int compute_units, hipStream_t stream);
 
 // ---- LDS-DMA MFMA kernels for 16-bit inputs, K % 64 == 0 (gemm_mfma16_dma.hip) ----
 // Reached through the mfma16_* entry points above: their variant ids follow the register-staged ones.

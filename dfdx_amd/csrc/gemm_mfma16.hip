@@ -20,6 +20,7 @@
 // has one unit stride; pointers, leading strides and batch strides are multiples of
 // 8 elements (16 B) and the contiguous extent is a multiple of 8.
 #include "gemm_internal.h"
+#include "elem.h"
 #include <type_traits>
 
 namespace dfdx_rocm {
@@ -45,6 +46,7 @@ struct Params {
     int tiles_m, tiles_n, tiles_per_batch, total_blocks;
     int accumulate, bias_mode, c_vec;
     int group_m;
+    ConvPatches conv;  // CONV_B kernels: B is the patch matrix of a unit-stride convolution, formed on the fly
 };
 
 template <typename T> struct Mma;
@@ -119,6 +121,38 @@ template <int ROWS, int BK, int NT, bool KC> struct Loader {
         }
     }
 
+    // Patch-matrix form of an m/n-contiguous operand (convolutions at unit stride): row k = (channel, tap) of the
+    // matrix is the channel's plane moved by the tap, zero where the window leaves the image; column = pixel.  A
+    // unit's 8 columns are 8 consecutive pixels of one image row (the row width is a multiple of 8), so a load is one
+    // window of that row.  `planes` points at channel 0 of the image (uniform), k0 is the tile's first k.
+    int py[KC ? 1 : UNITS], px[KC ? 1 : UNITS];
+    __device__ __forceinline__ void init_conv(const ConvPatches &cv, int col0, int cols_left, int tid) {
+        if constexpr (!KC) {
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) {
+                const int mb = (u * NT + tid) / NKB;
+                const int col = col0 + min(mb * 8, cols_left - 8);
+                py[u] = col / cv.w_dst;
+                px[u] = col - py[u] * cv.w_dst;
+            }
+        }
+    }
+    __device__ __forceinline__ void load_conv(const ConvPatches &cv, const uint16_t *planes, int k0, int k_total) {
+        if constexpr (!KC) {
+#pragma unroll
+            for (int i = 0; i < LOADS; i++) {
+                const int k = k0 + koff[i], u = i / KR;
+                const int c = cv.taps == 9 ? k / 9 : (cv.taps == 1 ? k : k / cv.taps);
+                const int tap = k - c * cv.taps;
+                const int k1 = cv.ksize == 3 ? tap / 3 : (cv.ksize == 1 ? 0 : tap / cv.ksize);
+                const int k2 = tap - k1 * cv.ksize;
+                const int y = py[u] + cv.off_y + cv.step_y * k1;
+                regs[i] = row_window_bytes<2>(planes + (int64_t)c * cv.plane + (int64_t)y * cv.w_src,
+                                              k < k_total && y >= 0 && y < cv.h_src, px[u] + cv.off_x + cv.step_x * k2, cv.w_src);
+            }
+        }
+    }
+
     // `g` points at the tile origin (uniform across the workgroup).
     __device__ __forceinline__ void load(const uint16_t *g) {
 #pragma unroll
@@ -160,8 +194,9 @@ template <int ROWS, int BK, int NT, bool KC> struct Loader {
     }
 };
 
-template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool CONV_B = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(const Params p) {
+    static_assert(!CONV_B || !B_KC, "the patch-matrix form is an n-contiguous B");
     constexpr int NT = WAVES_M * WAVES_N * 64;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -200,6 +235,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
     };
     auto b_origin = [&](int kb) -> const uint16_t * {
         const uint16_t *base = p.b + (int64_t)(kb / p.nb2) * p.b_b1 + (int64_t)(kb % p.nb2) * p.b_b2;
+        if constexpr (CONV_B) return base;  // channel 0 of this batch's image
         return B_KC ? base + (int64_t)bn0 * p.ldb : base + bn0;
     };
     const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
@@ -213,9 +249,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
     Loader<BN, BK, NT, B_KC> lb;
     la.init(p.lda, p.m - bm0, tid);
     lb.init(p.ldb, p.n - bn0, tid);
+    if constexpr (CONV_B) lb.init_conv(p.conv, bn0, p.n - bn0, tid);
     auto advance = [&]() {
         a_next += a_step;
-        b_next += b_step;
+        if constexpr (!CONV_B) b_next += b_step;
         if (++f_kt == ktiles) {
             f_kt = 0;
             if (p.kbatches > 1 && ++f_kb < p.kbatches) {
@@ -244,11 +281,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
             if constexpr (TAIL) {
                 const int kl = p.k - f_kt * BK;
                 la.load_tail(a_next, kl);
-                lb.load_tail(b_next, kl);
+                if constexpr (!CONV_B) lb.load_tail(b_next, kl);
             } else {
                 la.load(a_next);
-                lb.load(b_next);
+                if constexpr (!CONV_B) lb.load(b_next);
             }
+            if constexpr (CONV_B) lb.load_conv(p.conv, b_next, f_kt * BK, p.k);
             advance();
         };
         if (iters > 0) {
@@ -389,6 +427,31 @@ hipError_t launch_layout(const Params &p, bool a_kc, bool b_kc, hipStream_t stre
     return hipGetLastError();
 }
 
+// The patch-matrix kernels: A k-contiguous (filters), B formed from image planes.
+template <typename T, int BM, int BN, int BK, int WM, int WN> hipError_t launch_conv_layout(const Params &p, hipStream_t stream) {
+    constexpr int NT = WM * WN * 64;
+    constexpr size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * 2;
+    auto kern = gemm_mfma16_kernel<T, BM, BN, BK, WM, WN, true, false, true>;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    kern<<<dim3((unsigned)p.total_blocks), dim3(NT), lds, stream>>>(p);
+    return hipGetLastError();
+}
+template <typename T> hipError_t launch_conv_variant(int variant, const Params &p, hipStream_t s) {
+    switch (variant) {
+    case 1: return launch_conv_layout<T, 256, 256, 64, 2, 4>(p, s);
+    case 3: return launch_conv_layout<T, 256, 128, 64, 2, 2>(p, s);
+    case 4: return launch_conv_layout<T, 128, 128, 64, 2, 2>(p, s);
+    case 5: return launch_conv_layout<T, 128, 64, 64, 4, 1>(p, s);
+    case 6: return launch_conv_layout<T, 64, 64, 64, 2, 2>(p, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 template <typename T> hipError_t launch_variant(int variant, const Params &p, bool a_kc, bool b_kc, hipStream_t s) {
     switch (variant) {
 #define X(id, bm, bn, bk, wm, wn) \
@@ -454,12 +517,18 @@ bool mfma16_supported(const GemmProblem &p, int variant) {
 
 int mfma16_dma_first_variant() { return kNumVariants + 1; }
 
+static int pick_staged(const GemmProblem &p, int compute_units, bool check_support);
+
 int mfma16_pick_variant(const GemmProblem &p, int compute_units) {
     if (const int d = mfma16dma_pick_variant(p, compute_units)) return kNumVariants + d;
     // Least estimated time among the BK = 64 tiles: the work of the padded tiles over the tile's rate (measured at
     // 4096^3 relative to 256x256: 821 TFLOP/s down to 377 for 64x64) and over the share of the chip its workgroups
     // fill.  Per-image convolution GEMMs with 64 or 96 rows run 1.5-1.8x faster on the small tiles than on the
     // largest tile that fills the chip.
+    return pick_staged(p, compute_units, true);
+}
+
+static int pick_staged(const GemmProblem &p, int compute_units, bool check_support) {
     const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
     const int candidates[] = {1, 3, 4, 5, 6};
     const double rate[] = {1.0, 0.60, 0.73, 0.54, 0.46};
@@ -467,7 +536,7 @@ int mfma16_pick_variant(const GemmProblem &p, int compute_units) {
     double best_time = 1e300;
     for (int i = 0; i < 5; i++) {
         const int v = candidates[i];
-        if (!mfma16_supported(p, v)) continue;
+        if (check_support && !mfma16_supported(p, v)) continue;
         const Variant &t = kVariants[v - 1];
         const double blocks = (double)((p.m + t.bm - 1) / t.bm) * (double)((p.n + t.bn - 1) / t.bn) * (double)nbatch;
         const double fill = std::min(1.0, blocks / std::max(1, compute_units));
@@ -503,8 +572,45 @@ hipError_t launch_mfma16(const GemmProblem &g, int variant, hipStream_t stream) 
     p.c_vec = (g.n % 4 == 0) && (p.ldc % 4 == 0) && (((uintptr_t)g.c & 7u) == 0) &&
               (g.c_b1 % 4 == 0) && (g.c_b2 % 4 == 0) && (!g.bias || ((uintptr_t)g.bias & 7u) == 0);
     p.group_m = 4;
+    p.conv = ConvPatches{};
     if (g.dtype == DT_F16) return launch_variant<_Float16>(variant, p, la.kc, lb.kc, stream);
     return launch_variant<__bf16>(variant, p, la.kc, lb.kc, stream);
+}
+
+hipError_t launch_mfma16_conv(const GemmProblem &g, const ConvPatches &conv, int compute_units, hipStream_t stream) {
+    if (g.dtype != DT_F16 && g.dtype != DT_BF16) return hipErrorNotSupported;
+    if (g.reduce || g.bias || g.m < 1 || g.n < 8 || g.k < 8) return hipErrorNotSupported;
+    if (g.m >= (1 << 30) || g.n >= (1 << 30) || g.k >= (1 << 30) || g.nb1 * g.nb2 >= (1ll << 31)) return hipErrorNotSupported;
+    const OperandLayout la = classify(g.m, g.k, g.a_rs, g.a_cs);
+    if (!la.ok || !la.kc || !aligned16(g.a) || g.a_b1 % 8 || g.a_b2 % 8 || g.a_b1 < 0 || g.a_b2 < 0) return hipErrorNotSupported;
+    if (g.c_cs != 1 || g.n % 8 || g.c_rs % 8 || g.c_rs < g.n || ((uintptr_t)g.c & 15u) || g.c_b1 % 8 || g.c_b2 % 8) return hipErrorNotSupported;
+    if (conv.w_dst < 8 || conv.w_dst % 8 || g.n % conv.w_dst || conv.w_src < 8 || conv.taps != conv.ksize * conv.ksize ||
+        g.k % conv.taps || g.b_b1 < 0 || g.b_b2 < 0 || ((uintptr_t)g.b & 1u))
+        return hipErrorNotSupported;
+    if ((int64_t)(g.k / conv.taps) * conv.plane >= (1ll << 31)) return hipErrorNotSupported;
+    const int variant = pick_staged(g, compute_units, false);
+    const Variant &v = kVariants[variant - 1];
+    if (la.ld * v.bm >= (1ll << 30)) return hipErrorNotSupported;
+    Params p;
+    p.a = (const uint16_t *)g.a; p.b = (const uint16_t *)g.b; p.c = (uint16_t *)g.c; p.bias = nullptr;
+    p.m = (int)g.m; p.n = (int)g.n; p.k = (int)g.k;
+    p.lda = (int)la.ld; p.ldb = 0;
+    p.ldc = g.c_rs;
+    p.a_b1 = g.a_b1; p.a_b2 = g.a_b2; p.b_b1 = g.b_b1; p.b_b2 = g.b_b2; p.c_b1 = g.c_b1; p.c_b2 = g.c_b2;
+    p.nb2 = (int)g.nb2;
+    p.kbatches = 1;
+    p.tiles_m = (int)((g.m + v.bm - 1) / v.bm);
+    p.tiles_n = (int)((g.n + v.bn - 1) / v.bn);
+    p.tiles_per_batch = p.tiles_m * p.tiles_n;
+    const int64_t blocks = (int64_t)p.tiles_per_batch * g.nb1 * g.nb2;
+    if (blocks >= (1ll << 31)) return hipErrorNotSupported;
+    p.total_blocks = (int)blocks;
+    p.accumulate = g.accumulate; p.bias_mode = BIAS_NONE;
+    p.c_vec = 1;
+    p.group_m = 4;
+    p.conv = conv;
+    if (g.dtype == DT_F16) return launch_conv_variant<_Float16>(variant, p, stream);
+    return launch_conv_variant<__bf16>(variant, p, stream);
 }
 
 }  // namespace dfdx_rocm

@@ -54,6 +54,10 @@ CONFIGS = [
     (2, 9, 15, 14, 14, 3, 1, 0, 1, 3),     # the shape of its grouped-slices test (:405-464)
     (4, 64, 64, 28, 28, 3, 1, 1, 1, 1),    # k = 576, n = 784: the MFMA kernels
     (2, 64, 128, 32, 32, 3, 2, 1, 1, 2),
+    (3, 16, 24, 16, 16, 3, 1, 1, 1, 1),    # unit stride, output width a multiple of 8: forward without a patch matrix
+    (2, 32, 32, 12, 24, 3, 1, 2, 2, 2),    # the same with dilation and groups
+    (2, 8, 16, 12, 20, 5, 1, 0, 1, 1),     # the same, no padding, k = 200 (a k tail in the 64-wide steps)
+    (2, 64, 64, 56, 56, 3, 1, 1, 1, 1),    # the same at a ResNet shape
     (4, 64, 128, 8, 8, 1, 1, 0, 1, 1),     # 1x1 filters: the image / grad_out are the patch matrices, no gather
     (2, 64, 64, 16, 16, 1, 1, 0, 1, 2),    # the same with groups
     (4, 64, 64, 14, 14, 3, 1, 1, 1, 1),    # n = 196: rows padded to the vector width inside the patch buffer
