@@ -215,8 +215,8 @@ def main():
             gxv, gwv = view(zeros((B, C, H, W_), dt), dt), view(zeros((O, C, K, K), dt), dt)
             fl = 2.0 * B * O * C * K * K * y.shape[2] * y.shape[3]
             tag = f"{dt} B{B} {C}->{O} {H}x{W_} k{K}"
-            timed("conv", f"conv2d fwd {tag}", lambda: dev.conv2d_forward(xv, wv, stride=s, padding=pad), fl, 0, "unfold + gemm")
-            timed("conv", f"conv2d bwd {tag}", lambda: dev.conv2d_backward(xv, gxv, wv, gwv, gov, stride=s, padding=pad), 2 * fl, 0, "unfold + 2 gemm")
+            timed("conv", f"conv2d fwd {tag}", lambda: dev.conv2d_forward(xv, wv, stride=s, padding=pad), fl, 0, "conv2d_forward")
+            timed("conv", f"conv2d bwd {tag}", lambda: dev.conv2d_backward(xv, gxv, wv, gwv, gov, stride=s, padding=pad), 2 * fl, 0, "conv2d_backward")
 
     if args.json:
         with open(args.json, "w") as f:
