@@ -235,6 +235,9 @@ dfdx_rocm_gemm_desc blank_desc(int dtype, int64_t m, int64_t k, int64_t n) {
 template <typename T>
 bool implicit_forward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *filters, const void *img, void *out, int *rc) {
     if (sizeof(T) != 2 || op.stride != 1) return false;
+    // narrow rows that are not a multiple of 8 pixels wide make half of the window loads straddle two rows and leave
+    // much of a tile past the last pixel: 14x14 runs 118 us this way against 74 us through the patch matrix
+    if (op.w_out % 8 != 0 && op.w_out < 24) return false;
     const int64_t kk = (int64_t)op.kernel * op.kernel, hw = (int64_t)op.h_in * op.w_in, ohw = (int64_t)op.h_out * op.w_out;
     const int64_t cg = op.chan_in / op.groups, og = op.chan_out / op.groups;
     GemmProblem g{};  // out (B, G, O/G, OH*OW) = filters (G, O/G, C/G*K*K) . patches of img

@@ -35,7 +35,7 @@ struct GemmProblem {
 // [x + off_x + step_x * k2], zero outside the h_src x w_src plane.
 struct ConvPatches {
     int taps, ksize;     // K*K, K
-    int w_dst;           // pixels per row of the column index space (a multiple of 8)
+    int w_dst;           // pixels per row of the column index space (>= 8)
     int h_src, w_src;    // the planes the windows come from (w_src >= 8)
     int off_y, off_x, step_y, step_x;
     int64_t plane;       // elements between channels

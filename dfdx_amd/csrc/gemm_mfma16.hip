@@ -123,15 +123,17 @@ template <int ROWS, int BK, int NT, bool KC> struct Loader {
 
     // Patch-matrix form of an m/n-contiguous operand (convolutions at unit stride): row k = (channel, tap) of the
     // matrix is the channel's plane moved by the tap, zero where the window leaves the image; column = pixel.  A
-    // unit's 8 columns are 8 consecutive pixels of one image row (the row width is a multiple of 8), so a load is one
-    // window of that row.  `planes` points at channel 0 of the image (uniform), k0 is the tile's first k.
+    // unit's 8 columns are 8 consecutive pixels: one window of an image row, or -- when the row width is not a
+    // multiple of 8 -- the end of one row and the start of the next (rows are at least 8 pixels wide).  Columns past
+    // the last pixel only feed C columns that are never stored.  `planes` points at channel 0 of the image (uniform),
+    // k0 is the tile's first k.
     int py[KC ? 1 : UNITS], px[KC ? 1 : UNITS];
     __device__ __forceinline__ void init_conv(const ConvPatches &cv, int col0, int cols_left, int tid) {
         if constexpr (!KC) {
 #pragma unroll
             for (int u = 0; u < UNITS; u++) {
                 const int mb = (u * NT + tid) / NKB;
-                const int col = col0 + min(mb * 8, cols_left - 8);
+                const int col = col0 + min(mb * 8, ((cols_left + 7) & ~7) - 8);
                 py[u] = col / cv.w_dst;
                 px[u] = col - py[u] * cv.w_dst;
             }
@@ -146,9 +148,19 @@ template <int ROWS, int BK, int NT, bool KC> struct Loader {
                 const int tap = k - c * cv.taps;
                 const int k1 = cv.ksize == 3 ? tap / 3 : (cv.ksize == 1 ? 0 : tap / cv.ksize);
                 const int k2 = tap - k1 * cv.ksize;
-                const int y = py[u] + cv.off_y + cv.step_y * k1;
-                regs[i] = row_window_bytes<2>(planes + (int64_t)c * cv.plane + (int64_t)y * cv.w_src,
-                                              k < k_total && y >= 0 && y < cv.h_src, px[u] + cv.off_x + cv.step_x * k2, cv.w_src);
+                const int y = py[u] + cv.off_y + cv.step_y * k1, x = cv.off_x + cv.step_x * k2;
+                const uint16_t *row = planes + (int64_t)c * cv.plane + (int64_t)y * cv.w_src;
+                u32x4 w = row_window_bytes<2>(row, k < k_total && y >= 0 && y < cv.h_src, px[u] + x, cv.w_src);
+                const int n1 = cv.w_dst - px[u];  // pixels left in this image row
+                if (n1 < 8) {  // the other 8 - n1 pixels start the next row
+                    const u32x4 w2 = row_window_bytes<2>(row + cv.w_src, k < k_total && y + 1 >= 0 && y + 1 < cv.h_src, x, cv.w_src);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) w[j] &= n1 >= 2 * j + 2 ? 0xffffffffu : (n1 == 2 * j + 1 ? 0x0000ffffu : 0u);
+                    const u32x4 hi = shift128(w2, -16 * n1);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) w[j] |= hi[j];
+                }
+                regs[i] = w;
             }
         }
     }
@@ -583,8 +595,8 @@ hipError_t launch_mfma16_conv(const GemmProblem &g, const ConvPatches &conv, int
     if (g.m >= (1 << 30) || g.n >= (1 << 30) || g.k >= (1 << 30) || g.nb1 * g.nb2 >= (1ll << 31)) return hipErrorNotSupported;
     const OperandLayout la = classify(g.m, g.k, g.a_rs, g.a_cs);
     if (!la.ok || !la.kc || !aligned16(g.a) || g.a_b1 % 8 || g.a_b2 % 8 || g.a_b1 < 0 || g.a_b2 < 0) return hipErrorNotSupported;
-    if (g.c_cs != 1 || g.n % 8 || g.c_rs % 8 || g.c_rs < g.n || ((uintptr_t)g.c & 15u) || g.c_b1 % 8 || g.c_b2 % 8) return hipErrorNotSupported;
-    if (conv.w_dst < 8 || conv.w_dst % 8 || g.n % conv.w_dst || conv.w_src < 8 || conv.taps != conv.ksize * conv.ksize ||
+    if (g.c_cs != 1 || g.n % 4 || g.c_rs % 4 || g.c_rs < g.n || ((uintptr_t)g.c & 7u) || g.c_b1 % 4 || g.c_b2 % 4) return hipErrorNotSupported;
+    if (conv.w_dst < 8 || g.n % conv.w_dst || conv.w_src < 8 || conv.taps != conv.ksize * conv.ksize ||
         g.k % conv.taps || g.b_b1 < 0 || g.b_b2 < 0 || ((uintptr_t)g.b & 1u))
         return hipErrorNotSupported;
     if ((int64_t)(g.k / conv.taps) * conv.plane >= (1ll << 31)) return hipErrorNotSupported;

@@ -58,6 +58,8 @@ CONFIGS = [
     (2, 32, 32, 12, 24, 3, 1, 2, 2, 2),    # the same with dilation and groups
     (2, 8, 16, 12, 20, 5, 1, 0, 1, 1),     # the same, no padding, k = 200 (a k tail in the 64-wide steps)
     (2, 64, 64, 56, 56, 3, 1, 1, 1, 1),    # the same at a ResNet shape
+    (2, 16, 16, 9, 28, 3, 1, 1, 1, 1),     # the same with rows of 28 pixels: windows that straddle two image rows
+    (2, 8, 8, 5, 30, 3, 1, 0, 1, 1),       # output 3 x 28 = 84 pixels (n % 8 = 4), no padding
     (4, 64, 128, 8, 8, 1, 1, 0, 1, 1),     # 1x1 filters: the image / grad_out are the patch matrices, no gather
     (2, 64, 64, 16, 16, 1, 1, 0, 1, 2),    # the same with groups
     (4, 64, 64, 14, 14, 3, 1, 1, 1, 1),    # n = 196: rows padded to the vector width inside the patch buffer
