@@ -518,16 +518,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
             // widened once, before the first store.
             auto rows_plain = [&](auto bias_tag) {
                 constexpr bool BIAS = decltype(bias_tag)::value;
-                [[maybe_unused]] float cb[TN / 2][8];
+                // Rounded to the 16-bit type first, the lane rows then trade PACKED pairs: half as many cross-lane
+                // instructions as trading the f32 values (the conversions and trades of a K = 64 work item cost
+                // the vector ALU more cycles than its MFMAs cost the matrix core).
+                [[maybe_unused]] float cb[TN][4];  // bias of the columns the lane holds before the trade
                 if constexpr (BIAS) {
 #pragma unroll
-                    for (int jp = 0; jp < TN / 2; jp++) {
-                        const u32x4 bv = *(const u32x4 *)(p.bias + bn0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8);
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            cb[jp][2 * e] = Mma<T>::to_f32((uint16_t)(bv[e] & 0xffffu));
-                            cb[jp][2 * e + 1] = Mma<T>::to_f32((uint16_t)(bv[e] >> 16));
-                        }
+                    for (int j = 0; j < TN; j++) {
+                        const u32x2 bv = *(const u32x2 *)(p.bias + bn0 + wn0 + j * 16 + lq * 4);
+                        cb[j][0] = Mma<T>::to_f32((uint16_t)(bv[0] & 0xffffu));
+                        cb[j][1] = Mma<T>::to_f32((uint16_t)(bv[0] >> 16));
+                        cb[j][2] = Mma<T>::to_f32((uint16_t)(bv[1] & 0xffffu));
+                        cb[j][3] = Mma<T>::to_f32((uint16_t)(bv[1] >> 16));
                     }
                 }
 #pragma unroll
@@ -535,20 +537,24 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
                     u32x4 o[TN / 2];
 #pragma unroll
                     for (int jp = 0; jp < TN / 2; jp++) {
-                        float v[8];
+                        uint32_t pk[2][2];  // [tile 2jp / 2jp + 1][columns 4*lq + 0,1 / 2,3]
 #pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i][2 * jp][e]),
-                                                                            __float_as_uint(acc[i][2 * jp + 1][e]), false, false);
-                            v[e] = __uint_as_float(r[0]);
-                            v[4 + e] = __uint_as_float(r[1]);
+                        for (int t = 0; t < 2; t++)
+#pragma unroll
+                            for (int h = 0; h < 2; h++) {
+                                float x = acc[i][2 * jp + t][2 * h], y = acc[i][2 * jp + t][2 * h + 1];
+                                if constexpr (BIAS) {
+                                    x += cb[2 * jp + t][2 * h];
+                                    y += cb[2 * jp + t][2 * h + 1];
+                                }
+                                pk[t][h] = Mma<T>::pack2(x, y);
+                            }
+#pragma unroll
+                        for (int h = 0; h < 2; h++) {
+                            const auto r = __builtin_amdgcn_permlane16_swap(pk[0][h], pk[1][h], false, false);
+                            o[jp][h] = r[0];      // columns 8*(lq/2) + 2h, + 1 of tile 2jp + (lq & 1)
+                            o[jp][2 + h] = r[1];  // columns 8*(lq/2) + 4 + 2h, + 1
                         }
-                        if constexpr (BIAS) {
-#pragma unroll
-                            for (int e = 0; e < 8; e++) v[e] += cb[jp][e];
-                        }
-#pragma unroll
-                        for (int e = 0; e < 4; e++) o[jp][e] = Mma<T>::pack2(v[2 * e], v[2 * e + 1]);
                     }
                     if constexpr (TN == 4) {
                         u32x4 lo, hi;
@@ -566,10 +572,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
                 }
             };
             // beta = 1 on an interior tile without bias (every gradient product of whole tiles): all old values are
-            // requested before the first store goes out.  While loads and stores are outstanding together the
-            // compiler can only wait for everything (the two kinds may complete out of order), so the interleaved
-            // form of `rows` drains the stores of the tile sixteen times; here the loads overlap each other and
-            // are waited for in issue order.
+            // requested before the first store goes out.  The memory counter retires in issue order, so waiting for a
+            // load also waits for every store issued before it: the interleaved form of `rows` drains the stores of
+            // the tile sixteen times; here the loads overlap each other and are waited for in issue order.
             auto rows_accumulate = [&]() {
                 constexpr int IG = TM * (TN / 2) > 8 ? TM / 2 : TM;  // tile rows per batch: at most 8 vectors in flight
                 char *const base = tile_base;
