@@ -1,0 +1,355 @@
+// LayerNorm1D over the last (contiguous) axis of a (rows, cols) matrix and its backward:
+//   xhat = (x - mean) / sqrt(var + eps),  var = mean((x - mean)^2),  out = gamma * xhat + beta.
+// The reference composes it from mean / sub / square / mean / add / sqrt / div / mul / add tensor ops
+// (dfdx-core/src/tensor_ops/normalize.rs:35-49, dfdx/src/nn/layers/layer_norm1d.rs:87-91); here one wave owns a row,
+// evaluates the formula in f32 and rounds once.  HBM-bound: the forward reads x and writes out; the backward reads x
+// and grad_out, reads and writes grad_x, and leaves per-slice column sums for grad_gamma / grad_beta that a second
+// launch adds up in slice order.
+#include "ctx_internal.h"
+#include "elem.h"
+
+#include <algorithm>
+
+namespace dfdx_rocm {
+namespace {
+
+constexpr int WAVES = 4;  // rows in flight per workgroup
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// Lane l owns the N-element groups l, l + 64, ... of the row (CH of them; groups past the row end are skipped).
+template <typename T, int N, int CH>
+__global__ __launch_bounds__(WAVES * 64) void layer_norm_forward_kernel(const T *x, const T *gamma, const T *beta, T *out,
+                                                                        int64_t rows, int cols, float eps) {
+    const int lane = threadIdx.x % 64;
+    const float inv_n = 1.0f / (float)cols;
+    float gm[CH][N], bt[CH][N];
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int col = (c * 64 + lane) * N;
+        if (col < cols) {
+            load_elems<T, N>(gamma + col, gm[c]);
+            load_elems<T, N>(beta + col, bt[c]);
+        }
+    }
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const T *src = x + row * cols;
+        float v[CH][N];
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+                load_elems<T, N>(src + col, v[c]);
+#pragma unroll
+                for (int i = 0; i < N; i++) s += v[c][i];
+            }
+        }
+        const float mean = wave_sum(s) * inv_n;
+        float q = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) {
+                    v[c][i] -= mean;
+                    q += v[c][i] * v[c][i];
+                }
+            }
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_n + eps);
+        T *dst = out + row * cols;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) v[c][i] = v[c][i] * rstd * gm[c][i] + bt[c][i];
+                store_elems<T, N>(dst + col, v[c]);
+            }
+        }
+    }
+}
+
+// grad_x += rstd * (gh - mean(gh) - xhat * mean(gh * xhat)),  gh = grad_out * gamma;
+// partial[slice][0][col] = sum over the slice's rows of grad_out * xhat, partial[slice][1][col] = of grad_out.
+template <typename T, int N, int CH>
+__global__ __launch_bounds__(WAVES * 64) void layer_norm_backward_kernel(const T *x, const T *gamma, const T *go, T *gx,
+                                                                         float *partial, int64_t rows, int cols, float eps) {
+    __shared__ float red[WAVES][2][64 * N];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const float inv_n = 1.0f / (float)cols;
+    float gm[CH][N], dg[CH][N], db[CH][N];
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int col = (c * 64 + lane) * N;
+        if (col < cols) load_elems<T, N>(gamma + col, gm[c]);
+#pragma unroll
+        for (int i = 0; i < N; i++) dg[c][i] = db[c][i] = 0.0f;
+    }
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const T *src = x + row * cols, *gs = go + row * cols;
+        float v[CH][N], g[CH][N];
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+                load_elems<T, N>(src + col, v[c]);
+                load_elems<T, N>(gs + col, g[c]);
+#pragma unroll
+                for (int i = 0; i < N; i++) s += v[c][i];
+            }
+        }
+        const float mean = wave_sum(s) * inv_n;
+        float q = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) {
+                    v[c][i] -= mean;
+                    q += v[c][i] * v[c][i];
+                }
+            }
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_n + eps);
+        float s1 = 0.0f, s2 = 0.0f;  // sum gh, sum gh * xhat
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) {
+                    v[c][i] *= rstd;  // xhat
+                    dg[c][i] += g[c][i] * v[c][i];
+                    db[c][i] += g[c][i];
+                    g[c][i] *= gm[c][i];  // gh
+                    s1 += g[c][i];
+                    s2 += g[c][i] * v[c][i];
+                }
+            }
+        }
+        const float m1 = wave_sum(s1) * inv_n, m2 = wave_sum(s2) * inv_n;
+        T *dst = gx + row * cols;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * N;
+            if (col < cols) {
+                float old[N];
+                load_elems<T, N>(dst + col, old);
+#pragma unroll
+                for (int i = 0; i < N; i++) old[i] += rstd * (g[c][i] - m1 - v[c][i] * m2);
+                store_elems<T, N>(dst + col, old);
+            }
+        }
+    }
+    // column sums of the workgroup's rows: the four waves through LDS, one chunk of 64 * N columns at a time
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            red[wave][0][lane * N + i] = dg[c][i];
+            red[wave][1][lane * N + i] = db[c][i];
+        }
+        __syncthreads();
+        for (int t = threadIdx.x; t < 2 * 64 * N; t += WAVES * 64) {
+            const int which = t / (64 * N), j = t % (64 * N), col = c * 64 * N + j;
+            if (col < cols) {
+                float sum = 0.0f;
+#pragma unroll
+                for (int w = 0; w < WAVES; w++) sum += red[w][which][j];
+                partial[((int64_t)blockIdx.x * 2 + which) * cols + col] = sum;
+            }
+        }
+    }
+}
+
+// Long or unaligned rows: the same formulas with the row walked from memory once per pass.
+template <typename T>
+__global__ __launch_bounds__(WAVES * 64) void layer_norm_forward_loop_kernel(const T *x, const T *gamma, const T *beta, T *out,
+                                                                             int64_t rows, int cols, float eps) {
+    const int lane = threadIdx.x % 64;
+    const float inv_n = 1.0f / (float)cols;
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const T *src = x + row * cols;
+        float s = 0.0f;
+        for (int c = lane; c < cols; c += 64) s += Elem<T>::load(src + c);
+        const float mean = wave_sum(s) * inv_n;
+        float q = 0.0f;
+        for (int c = lane; c < cols; c += 64) {
+            const float d = Elem<T>::load(src + c) - mean;
+            q += d * d;
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_n + eps);
+        T *dst = out + row * cols;
+        for (int c = lane; c < cols; c += 64)
+            Elem<T>::store(dst + c, (Elem<T>::load(src + c) - mean) * rstd * Elem<T>::load(gamma + c) + Elem<T>::load(beta + c));
+    }
+}
+
+// One workgroup per slice of rows; the column sums go through atomics-free per-wave accumulation in memory order:
+// wave w adds its rows into partial[slice * WAVES + w], so `slices` counts waves here.
+template <typename T>
+__global__ __launch_bounds__(WAVES * 64) void layer_norm_backward_loop_kernel(const T *x, const T *gamma, const T *go, T *gx,
+                                                                              float *partial, int64_t rows, int cols, float eps) {
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const float inv_n = 1.0f / (float)cols;
+    float *pg = partial + ((int64_t)(blockIdx.x * WAVES + wave) * 2) * cols, *pb = pg + cols;
+    for (int c = lane; c < cols; c += 64) pg[c] = pb[c] = 0.0f;
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const T *src = x + row * cols, *gs = go + row * cols;
+        float s = 0.0f;
+        for (int c = lane; c < cols; c += 64) s += Elem<T>::load(src + c);
+        const float mean = wave_sum(s) * inv_n;
+        float q = 0.0f;
+        for (int c = lane; c < cols; c += 64) {
+            const float d = Elem<T>::load(src + c) - mean;
+            q += d * d;
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_n + eps);
+        float s1 = 0.0f, s2 = 0.0f;
+        for (int c = lane; c < cols; c += 64) {
+            const float xh = (Elem<T>::load(src + c) - mean) * rstd, g = Elem<T>::load(gs + c), gh = g * Elem<T>::load(gamma + c);
+            pg[c] += g * xh;  // column c of this wave's partial belongs to this lane alone
+            pb[c] += g;
+            s1 += gh;
+            s2 += gh * xh;
+        }
+        const float m1 = wave_sum(s1) * inv_n, m2 = wave_sum(s2) * inv_n;
+        T *dst = gx + row * cols;
+        for (int c = lane; c < cols; c += 64) {
+            const float xh = (Elem<T>::load(src + c) - mean) * rstd, gh = Elem<T>::load(gs + c) * Elem<T>::load(gamma + c);
+            Elem<T>::store(dst + c, Elem<T>::load(dst + c) + rstd * (gh - m1 - xh * m2));
+        }
+    }
+}
+
+// grad_gamma[c] += sum_s partial[s][0][c], grad_beta[c] += sum_s partial[s][1][c], slices in ascending order
+template <typename T>
+__global__ __launch_bounds__(64) void layer_norm_combine_kernel(const float *partial, int slices, int cols, T *grad_gamma, T *grad_beta) {
+    const int c = blockIdx.x * 64 + threadIdx.x;
+    if (c >= cols) return;
+    float sg = 0.0f, sb = 0.0f;
+    int j = 0;
+    for (; j + 4 <= slices; j += 4) {  // loads of four slices in flight, added in slice order
+        float a[4], b[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            a[u] = partial[((int64_t)(j + u) * 2) * cols + c];
+            b[u] = partial[((int64_t)(j + u) * 2 + 1) * cols + c];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            sg += a[u];
+            sb += b[u];
+        }
+    }
+    for (; j < slices; j++) {
+        sg += partial[((int64_t)j * 2) * cols + c];
+        sb += partial[((int64_t)j * 2 + 1) * cols + c];
+    }
+    Elem<T>::store(grad_gamma + c, Elem<T>::load(grad_gamma + c) + sg);
+    Elem<T>::store(grad_beta + c, Elem<T>::load(grad_beta + c) + sb);
+}
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+template <typename T>
+int forward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, const void *gamma, const void *beta, float eps,
+              void *out) {
+    constexpr int V = Elem<T>::VEC;
+    const bool vec = cols % V == 0 && aligned16(x) && aligned16(gamma) && aligned16(beta) && aligned16(out);
+    const unsigned grid = (unsigned)std::min<int64_t>((rows + WAVES - 1) / WAVES, (int64_t)ctx->compute_units * 16);
+    const dim3 block(WAVES * 64);
+    hipStream_t s = ctx->stream;
+#define DFDX_LN_FWD(CH)                                                                                                           \
+    do {                                                                                                                          \
+        layer_norm_forward_kernel<T, V, CH><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)beta, (T *)out, rows, \
+                                                                   (int)cols, eps);                                               \
+        return (int)hipGetLastError();                                                                                            \
+    } while (0)
+    if (vec) {
+        const int64_t groups = cols / V;
+        if (groups <= 64) DFDX_LN_FWD(1);
+        if (groups <= 128) DFDX_LN_FWD(2);
+        if (groups <= 256) DFDX_LN_FWD(4);
+    }
+#undef DFDX_LN_FWD
+    layer_norm_forward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)beta, (T *)out, rows, (int)cols, eps);
+    return (int)hipGetLastError();
+}
+
+template <typename T>
+int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, const void *gamma, float eps, const void *go,
+               void *gx, void *ggamma, void *gbeta) {
+    constexpr int V = Elem<T>::VEC;
+    const bool vec = cols % V == 0 && aligned16(x) && aligned16(gamma) && aligned16(go) && aligned16(gx);
+    const int64_t groups = cols / V;
+    const bool reg = vec && groups <= 256;
+    // at least 8 rows per wave so that the column sums amortise; at most four workgroups per compute unit
+    const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>((rows + 8 * WAVES - 1) / (8 * WAVES), (int64_t)ctx->compute_units * 4));
+    const int slices = (int)grid * (reg ? 1 : WAVES);
+    const dim3 block(WAVES * 64);
+    hipStream_t s = ctx->stream;
+    CtxLock lock(ctx->mu);  // two launches around the shared workspace
+    if (int rc = ensure_workspace(ctx, (size_t)slices * 2 * cols * sizeof(float))) return rc;
+    float *partial = (float *)ctx->workspace;
+#define DFDX_LN_BWD(CH)                                                                                                         \
+    layer_norm_backward_kernel<T, V, CH><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, \
+                                                                rows, (int)cols, eps)
+    if (reg && groups <= 64) DFDX_LN_BWD(1);
+    else if (reg && groups <= 128) DFDX_LN_BWD(2);
+    else if (reg) DFDX_LN_BWD(4);
+    else layer_norm_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, rows, (int)cols, eps);
+#undef DFDX_LN_BWD
+    HIP_TRY(hipGetLastError());
+    layer_norm_combine_kernel<T><<<(unsigned)((cols + 63) / 64), 64, 0, s>>>(partial, slices, (int)cols, (T *)ggamma, (T *)gbeta);
+    return (int)hipGetLastError();
+}
+
+bool dims_ok(int64_t rows, int64_t cols) { return rows >= 0 && cols >= 0 && rows < (1ll << 40) && cols < (1ll << 24); }
+
+}  // namespace
+}  // namespace dfdx_rocm
+
+using namespace dfdx_rocm;
+
+extern "C" {
+
+int dfdx_rocm_layer_norm_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *x, const void *gamma,
+                                 const void *beta, double epsilon, void *out) {
+    if (int e = bind(ctx)) return e;
+    if (!dims_ok(rows, cols)) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
+    if (!x || !gamma || !beta || !out) return DFDX_ROCM_ERR_INVALID_ARG;
+    switch (dtype) {
+    case DFDX_ROCM_F32: return forward_t<float>(ctx, rows, cols, x, gamma, beta, (float)epsilon, out);
+    case DFDX_ROCM_F16: return forward_t<_Float16>(ctx, rows, cols, x, gamma, beta, (float)epsilon, out);
+    case DFDX_ROCM_BF16: return forward_t<__bf16>(ctx, rows, cols, x, gamma, beta, (float)epsilon, out);
+    default: return DFDX_ROCM_ERR_UNSUPPORTED;
+    }
+}
+
+int dfdx_rocm_layer_norm_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *x, const void *gamma,
+                                  double epsilon, void *grad_x, void *grad_gamma, void *grad_beta, const void *grad_out) {
+    if (int e = bind(ctx)) return e;
+    if (!dims_ok(rows, cols)) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
+    if (!x || !gamma || !grad_x || !grad_gamma || !grad_beta || !grad_out) return DFDX_ROCM_ERR_INVALID_ARG;
+    switch (dtype) {
+    case DFDX_ROCM_F32: return backward_t<float>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta);
+    case DFDX_ROCM_F16: return backward_t<_Float16>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta);
+    case DFDX_ROCM_BF16: return backward_t<__bf16>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta);
+    default: return DFDX_ROCM_ERR_UNSUPPORTED;
+    }
+}
+
+}  // extern "C"

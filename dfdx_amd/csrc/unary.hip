@@ -1,6 +1,8 @@
-// Multiplication by a scalar (`t * s`, a unary op in dfdx): forward over the physical storage of the tensor,
-// backward grad_inp += s * grad_out.  The scalar is rounded to the element type first, as the reference holds it
-// in that type.
+// Elementwise ops over the physical storage of a tensor, forward and backward (gradients accumulate):
+//   * multiplication by a scalar (`t * s`, a unary op in dfdx); the scalar is rounded to the element type first, as
+//     the reference holds it in that type;
+//   * ReLU;
+//   * the binary add of two tensors of one shape (ResidualAdd).
 #include "ctx_internal.h"
 #include "elem.h"
 
@@ -23,6 +25,60 @@ __global__ __launch_bounds__(256) void scalar_mul_kernel(const T *x, T *out, int
             for (int i = 0; i < N; i++) v[i] *= s;
         }
         store_elems<T, N>(out + g * N, v);
+    }
+}
+
+// out = max(x, 0)
+template <typename T, int N> __global__ __launch_bounds__(256) void relu_forward_kernel(const T *x, T *out, int64_t groups) {
+    for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
+        float v[N];
+        load_elems<T, N>(x + g * N, v);
+#pragma unroll
+        for (int i = 0; i < N; i++) v[i] = fmaxf(v[i], 0.0f);
+        store_elems<T, N>(out + g * N, v);
+    }
+}
+
+// grad_x += (x > 0 ? 1 : 0) * grad_out
+template <typename T, int N>
+__global__ __launch_bounds__(256) void relu_backward_kernel(const T *x, const T *go, T *gx, int64_t groups) {
+    for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
+        float v[N], d[N], o[N];
+        load_elems<T, N>(x + g * N, v);
+        load_elems<T, N>(go + g * N, d);
+        load_elems<T, N>(gx + g * N, o);
+#pragma unroll
+        for (int i = 0; i < N; i++) o[i] += v[i] > 0.0f ? d[i] : 0.0f;
+        store_elems<T, N>(gx + g * N, o);
+    }
+}
+
+// out = a + b
+template <typename T, int N> __global__ __launch_bounds__(256) void add_forward_kernel(const T *a, const T *b, T *out, int64_t groups) {
+    for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
+        float v[N], w[N];
+        load_elems<T, N>(a + g * N, v);
+        load_elems<T, N>(b + g * N, w);
+#pragma unroll
+        for (int i = 0; i < N; i++) v[i] += w[i];
+        store_elems<T, N>(out + g * N, v);
+    }
+}
+
+// grad_lhs += grad_out, grad_rhs += grad_out (two distinct buffers)
+template <typename T, int N> __global__ __launch_bounds__(256) void add_backward_kernel(const T *go, T *gl, T *gr, int64_t groups) {
+    for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
+        float d[N], l[N], r[N];
+        load_elems<T, N>(go + g * N, d);
+        load_elems<T, N>(gl + g * N, l);
+        load_elems<T, N>(gr + g * N, r);
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            l[i] += d[i];
+            r[i] += d[i];
+        }
+        store_elems<T, N>(gl + g * N, l);
+        store_elems<T, N>(gr + g * N, r);
     }
 }
 
@@ -66,6 +122,41 @@ template <bool ACC> int dispatch(dfdx_rocm_ctx *ctx, int dtype, int64_t len, con
     }
 }
 
+enum { OP_RELU_FWD, OP_RELU_BWD, OP_ADD_FWD, OP_ADD_BWD };
+
+// a, b: read-only inputs (b unused by OP_RELU_FWD); c, d: written (d only by OP_ADD_BWD)
+template <typename T, int OP> int launch_op(dfdx_rocm_ctx *ctx, int64_t len, const void *a, const void *b, void *c, void *d) {
+    constexpr int V = Elem<T>::VEC;
+    const bool vec = len % V == 0 && (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) & 15u) == 0;
+    const int64_t groups = vec ? len / V : len;
+    const unsigned grid = (unsigned)std::min<int64_t>((groups + 255) / 256, (int64_t)ctx->compute_units * 16);
+    hipStream_t s = ctx->stream;
+#define DFDX_OP(N)                                                                                                       \
+    do {                                                                                                                 \
+        if constexpr (OP == OP_RELU_FWD) relu_forward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (T *)c, groups);    \
+        else if constexpr (OP == OP_RELU_BWD) relu_backward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (const T *)b, (T *)c, groups); \
+        else if constexpr (OP == OP_ADD_FWD) add_forward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (const T *)b, (T *)c, groups);    \
+        else add_backward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (T *)c, (T *)d, groups);                        \
+    } while (0)
+    if (vec) DFDX_OP(V);
+    else DFDX_OP(1);
+#undef DFDX_OP
+    return (int)hipGetLastError();
+}
+
+template <int OP> int dispatch_op(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const void *a, const void *b, void *c, void *d) {
+    if (int e = bind(ctx)) return e;
+    if (len < 0) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (len == 0) return DFDX_ROCM_OK;
+    if (!a || !c || (OP != OP_RELU_FWD && OP != OP_ADD_BWD && !b) || (OP == OP_ADD_BWD && !d)) return DFDX_ROCM_ERR_INVALID_ARG;
+    switch (dtype) {
+    case DFDX_ROCM_F32: return launch_op<float, OP>(ctx, len, a, b, c, d);
+    case DFDX_ROCM_F16: return launch_op<_Float16, OP>(ctx, len, a, b, c, d);
+    case DFDX_ROCM_BF16: return launch_op<__bf16, OP>(ctx, len, a, b, c, d);
+    default: return DFDX_ROCM_ERR_UNSUPPORTED;
+    }
+}
+
 }  // namespace
 }  // namespace dfdx_rocm
 
@@ -78,6 +169,26 @@ int dfdx_rocm_scalar_mul_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, con
 int dfdx_rocm_scalar_mul_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, double scalar, void *grad_inp,
                                   const void *grad_out) {
     return dfdx_rocm::dispatch<true>(ctx, dtype, len, grad_out, scalar, grad_inp);
+}
+
+int dfdx_rocm_relu_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const void *x, void *out) {
+    return dfdx_rocm::dispatch_op<dfdx_rocm::OP_RELU_FWD>(ctx, dtype, len, x, nullptr, out, nullptr);
+}
+
+int dfdx_rocm_relu_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const void *x, void *grad_x, const void *grad_out) {
+    return dfdx_rocm::dispatch_op<dfdx_rocm::OP_RELU_BWD>(ctx, dtype, len, x, grad_out, grad_x, nullptr);
+}
+
+int dfdx_rocm_add_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const void *lhs, const void *rhs, void *out) {
+    return dfdx_rocm::dispatch_op<dfdx_rocm::OP_ADD_FWD>(ctx, dtype, len, lhs, rhs, out, nullptr);
+}
+
+int dfdx_rocm_add_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, void *grad_lhs, void *grad_rhs, const void *grad_out) {
+    if (grad_lhs && grad_lhs == grad_rhs) {  // t + t: the one buffer receives grad_out twice, one add after the other
+        if (int e = dfdx_rocm::dispatch<true>(ctx, dtype, len, grad_out, 1.0, grad_lhs)) return e;
+        return dfdx_rocm::dispatch<true>(ctx, dtype, len, grad_out, 1.0, grad_lhs);
+    }
+    return dfdx_rocm::dispatch_op<dfdx_rocm::OP_ADD_BWD>(ctx, dtype, len, grad_out, nullptr, grad_lhs, grad_rhs);
 }
 
 }  // extern "C"

@@ -81,6 +81,9 @@ EXPORTS = [
     "dfdx_rocm_scalar_mul_forward", "dfdx_rocm_scalar_mul_backward",
     "dfdx_rocm_softmax_forward", "dfdx_rocm_softmax_backward",
     "dfdx_rocm_reshape_forward", "dfdx_rocm_reshape_backward",
+    "dfdx_rocm_layer_norm_forward", "dfdx_rocm_layer_norm_backward",
+    "dfdx_rocm_relu_forward", "dfdx_rocm_relu_backward",
+    "dfdx_rocm_add_forward", "dfdx_rocm_add_backward",
     "dfdx_rocm_conv2d_forward", "dfdx_rocm_conv2d_backward",
 ]
 
@@ -466,6 +469,60 @@ class Rocm:
         vp = ctypes.c_void_p
         self._check(self.lib.dfdx_rocm_reshape_backward(self.ctx, DTYPES[x.dtype], len(x.shape), _i64arr(x.shape),
                                                         _i64arr(x.strides), vp(grad_inp.ptr), vp(grad_out.ptr)))
+
+    # ------------------------------------------- ops between an encoder block's GEMMs --
+    def layer_norm_forward(self, x: View, gamma: View, beta: View, epsilon: float = 1e-5) -> View:
+        """``LayerNorm1D::try_forward`` over the last axis of a contiguous tensor (layer_norm1d.rs:87-91)."""
+        assert x.strides == _row_major(x.shape), "layer norm input must be contiguous"
+        cols = x.shape[-1]
+        assert gamma.shape == (cols,) and beta.shape == (cols,), f"left: {gamma.shape}\n right: {(cols,)}"
+        rows = int(np.prod(x.shape[:-1], dtype=np.int64))
+        out = View(self._torch.empty_like(x.storage), x.dtype, x.shape, x.strides)
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_layer_norm_forward(self.ctx, DTYPES[x.dtype], _c(rows), _c(cols), vp(x.ptr), vp(gamma.ptr),
+                                                          vp(beta.ptr), ctypes.c_double(epsilon), vp(out.ptr)))
+        return out
+
+    def layer_norm_backward(self, x: View, gamma: View, grad_x: View, grad_gamma: View, grad_beta: View, grad_out: View,
+                            epsilon: float = 1e-5):
+        assert x.strides == _row_major(x.shape) and grad_out.shape == x.shape and grad_x.shape == x.shape
+        cols = x.shape[-1]
+        rows = int(np.prod(x.shape[:-1], dtype=np.int64))
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_layer_norm_backward(self.ctx, DTYPES[x.dtype], _c(rows), _c(cols), vp(x.ptr), vp(gamma.ptr),
+                                                           ctypes.c_double(epsilon), vp(grad_x.ptr), vp(grad_gamma.ptr),
+                                                           vp(grad_beta.ptr), vp(grad_out.ptr)))
+
+    def relu_forward(self, x: View) -> View:
+        """``t.relu()`` over the physical storage (relu/cpu_kernel.rs:3-18); same strides."""
+        out = View(self._torch.empty_like(x.storage), x.dtype, x.shape, x.strides, x.offset)
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_relu_forward(self.ctx, DTYPES[x.dtype], _c(x.numel_storage()), vp(x.storage.data_ptr()),
+                                                    vp(out.storage.data_ptr())))
+        return out
+
+    def relu_backward(self, x: View, grad_x: View, grad_out: View):
+        assert grad_x.numel_storage() == grad_out.numel_storage() == x.numel_storage()
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_relu_backward(self.ctx, DTYPES[x.dtype], _c(x.numel_storage()), vp(x.storage.data_ptr()),
+                                                     vp(grad_x.storage.data_ptr()), vp(grad_out.storage.data_ptr())))
+
+    def add_forward(self, lhs: View, rhs: View) -> View:
+        """``lhs + rhs`` for two tensors of one shape and layout (add/cpu_kernel.rs:4-26)."""
+        assert lhs.shape == rhs.shape, f"left: {lhs.shape}\n right: {rhs.shape}"
+        assert lhs.strides == rhs.strides and lhs.numel_storage() == rhs.numel_storage()
+        out = View(self._torch.empty_like(lhs.storage), lhs.dtype, lhs.shape, lhs.strides, lhs.offset)
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_add_forward(self.ctx, DTYPES[lhs.dtype], _c(lhs.numel_storage()), vp(lhs.storage.data_ptr()),
+                                                   vp(rhs.storage.data_ptr()), vp(out.storage.data_ptr())))
+        return out
+
+    def add_backward(self, grad_lhs: View, grad_rhs: View, grad_out: View):
+        assert grad_lhs.numel_storage() == grad_rhs.numel_storage() == grad_out.numel_storage()
+        vp = ctypes.c_void_p
+        self._check(self.lib.dfdx_rocm_add_backward(self.ctx, DTYPES[grad_out.dtype], _c(grad_out.numel_storage()),
+                                                    vp(grad_lhs.storage.data_ptr()), vp(grad_rhs.storage.data_ptr()),
+                                                    vp(grad_out.storage.data_ptr())))
 
     # ---------------------------------------------------------------- conv2d --
     def _conv2d_op(self, img: View, filters: View, stride, padding, dilation, groups) -> Conv2DOp:

@@ -259,6 +259,44 @@ int dfdx_rocm_reshape_forward(dfdx_rocm_ctx *ctx, int dtype, int rank, const int
 int dfdx_rocm_reshape_backward(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, const int64_t *inp_strides,
                                void *grad_inp, const void *grad_out);
 
+/* ---- The ops between a transformer encoder block's GEMMs ----------------------
+ * TransformerEncoderBlock (dfdx/src/nn/layers/transformer.rs:24-48) is
+ * ResidualAdd<MultiHeadAttention>, LayerNorm1D, ResidualAdd<(Linear, ReLU,
+ * Linear)>, LayerNorm1D.  These entry points keep the three ops that are not
+ * matmuls on the device. */
+
+/* LayerNorm1D over the last axis of a contiguous (rows, cols) matrix
+ * (dfdx/src/nn/layers/layer_norm1d.rs:87-91: normalize, multiply by gamma, add
+ * beta; normalize = (t - mean) / sqrt(mean((t - mean)^2) + epsilon),
+ * dfdx-core/src/tensor_ops/normalize.rs:35-49).  The reference composes it from
+ * mean / sub / square / mean / add / sqrt / div / mul / add tensor ops, each
+ * rounding to the element type; here a row is processed in f32 and rounded
+ * once.  gamma and beta have `cols` elements.  Backward of the composition,
+ * from the saved input, with xhat the normalized row and gh = grad_out * gamma:
+ *   grad_x     += (gh - mean(gh) - xhat * mean(gh * xhat)) / sqrt(var + epsilon)
+ *   grad_gamma += sum over rows of grad_out * xhat
+ *   grad_beta  += sum over rows of grad_out. */
+int dfdx_rocm_layer_norm_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *x, const void *gamma,
+                                 const void *beta, double epsilon, void *out);
+int dfdx_rocm_layer_norm_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *x, const void *gamma,
+                                  double epsilon, void *grad_x, void *grad_gamma, void *grad_beta, const void *grad_out);
+
+/* ReLU (ReLUKernelOp, dfdx-core/src/tensor_ops/relu/cpu_kernel.rs:3-18, run by
+ * the unary kernel over the tensor's physical storage): out[i] = max(x[i], 0);
+ * out may be x.  Backward, from the saved input:
+ * grad_x[i] += (x[i] > 0 ? 1 : 0) * grad_out[i]. */
+int dfdx_rocm_relu_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const void *x, void *out);
+int dfdx_rocm_relu_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const void *x, void *grad_x, const void *grad_out);
+
+/* The binary add of two tensors with the same layout (BinaryAddKernelOp,
+ * dfdx-core/src/tensor_ops/add/cpu_kernel.rs:4-26; ResidualAdd::try_forward,
+ * dfdx/src/nn/layers/residual_add.rs:38-45): out[i] = lhs[i] + rhs[i]; out may
+ * be either operand.  Backward: grad_lhs[i] += grad_out[i] and
+ * grad_rhs[i] += grad_out[i] (grad_lhs == grad_rhs, the gradient of t + t,
+ * receives grad_out twice). */
+int dfdx_rocm_add_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const void *lhs, const void *rhs, void *out);
+int dfdx_rocm_add_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, void *grad_lhs, void *grad_rhs, const void *grad_out);
+
 /* ---- conv2d as unfold + batched GEMM ---------------------------------------
  * Conv2DKernel (dfdx-core/src/tensor_ops/conv2d/mod.rs:31-55; Cpu impl
  * cpu_kernel.rs:40-278, Cuda impl cuda_kernel.rs:62-281).  The op struct has

@@ -149,3 +149,77 @@ def reshape_backward(shape, strides, grad_inp: np.ndarray, grad_out: np.ndarray,
     for o, i in enumerate(idx):
         out[i] = round_to(out[i] + go[o], dtype)
     return out
+
+
+# ------------------------------------------------------------------------------- LayerNorm1D, ReLU, add --
+
+def normalize_forward(x: np.ndarray, epsilon: float, dtype: str, faithful: bool = True) -> np.ndarray:
+    """``try_normalize`` over the last axis (tensor_ops/normalize.rs:35-49): mean = sum * (1/n) (mean_to.rs:38-44),
+    centered = t - mean, std = sqrt(mean(centered^2) + epsilon), out = centered / std -- every step a kernel that
+    rounds to the element type, the sums running in index order.  ``faithful=False`` evaluates the same formula in
+    float64 and rounds once."""
+    x = np.asarray(x, np.float64)
+    n = x.shape[-1]
+    if not faithful:
+        c = x - x.mean(axis=-1, keepdims=True)
+        return round_to(c / np.sqrt((c * c).mean(axis=-1, keepdims=True) + epsilon), dtype)
+    inv_n = round_to(np.float64(1.0 / n), dtype)
+    mean = round_to(_seq_sum_last(x, dtype) * inv_n, dtype)[..., None]
+    centered = round_to(x - mean, dtype)
+    var = round_to(_seq_sum_last(round_to(centered * centered, dtype), dtype) * inv_n, dtype)[..., None]
+    std = round_to(np.sqrt(round_to(var + round_to(np.float64(epsilon), dtype), dtype)), dtype)
+    return round_to(centered / std, dtype)
+
+
+def layer_norm_forward(x, gamma, beta, epsilon: float, dtype: str, faithful: bool = True) -> np.ndarray:
+    """``LayerNorm1D::try_forward`` (dfdx/src/nn/layers/layer_norm1d.rs:87-91): normalize over the last axis, times
+    gamma, plus beta (one rounding per op when ``faithful``)."""
+    gamma, beta = np.asarray(gamma, np.float64), np.asarray(beta, np.float64)
+    if not faithful:
+        x = np.asarray(x, np.float64)
+        c = x - x.mean(axis=-1, keepdims=True)
+        return round_to(c / np.sqrt((c * c).mean(axis=-1, keepdims=True) + epsilon) * gamma + beta, dtype)
+    xhat = normalize_forward(x, epsilon, dtype, True)
+    return round_to(round_to(gamma * xhat, dtype) + beta, dtype)
+
+
+def layer_norm_backward(x, gamma, grad_out, epsilon: float, dtype: str, grad_x, grad_gamma, grad_beta):
+    """Gradients of that composition, accumulated into the given buffers and rounded once (the closed form of what the
+    tape replays through div / sqrt / mean / square / sub / mul / add backward ops; its rounding at every op is not
+    restated).  With xhat the normalized rows, rstd = 1 / sqrt(var + epsilon) and gh = grad_out * gamma:
+        grad_x += rstd * (gh - mean(gh) - xhat * mean(gh * xhat)),
+        grad_gamma += sum_rows grad_out * xhat,   grad_beta += sum_rows grad_out."""
+    x, g = np.asarray(x, np.float64), np.asarray(grad_out, np.float64)
+    gamma = np.asarray(gamma, np.float64)
+    c = x - x.mean(axis=-1, keepdims=True)
+    rstd = 1.0 / np.sqrt((c * c).mean(axis=-1, keepdims=True) + epsilon)
+    xhat = c * rstd
+    gh = g * gamma
+    gx = rstd * (gh - gh.mean(axis=-1, keepdims=True) - xhat * (gh * xhat).mean(axis=-1, keepdims=True))
+    cols = x.shape[-1]
+    return (round_to(np.asarray(grad_x, np.float64) + gx, dtype),
+            round_to(np.asarray(grad_gamma, np.float64) + (g * xhat).reshape(-1, cols).sum(axis=0), dtype),
+            round_to(np.asarray(grad_beta, np.float64) + g.reshape(-1, cols).sum(axis=0), dtype))
+
+
+def relu_forward(x: np.ndarray, dtype: str) -> np.ndarray:
+    """``ReLUKernelOp::f`` (tensor_ops/relu/cpu_kernel.rs:7-9): max(x, 0) on every element of the storage."""
+    return round_to(np.maximum(np.asarray(x, np.float64), 0.0), dtype)
+
+
+def relu_backward(x: np.ndarray, grad_x: np.ndarray, grad_out: np.ndarray, dtype: str) -> np.ndarray:
+    """``*g += df(x) * grad_out`` with df = 1 for x > 0, else 0 (relu/cpu_kernel.rs:11-17, utilities/cpu_kernels.rs:
+    95-104)."""
+    x = np.asarray(x, np.float64)
+    return round_to(np.asarray(grad_x, np.float64) + np.where(x > 0.0, np.asarray(grad_out, np.float64), 0.0), dtype)
+
+
+def add_forward(lhs: np.ndarray, rhs: np.ndarray, dtype: str) -> np.ndarray:
+    """``BinaryAddKernelOp::f`` (tensor_ops/add/cpu_kernel.rs:7-9) on two tensors of one layout."""
+    return round_to(np.asarray(lhs, np.float64) + np.asarray(rhs, np.float64), dtype)
+
+
+def add_backward(grad_lhs: np.ndarray, grad_rhs: np.ndarray, grad_out: np.ndarray, dtype: str):
+    """Both operands receive grad_out (const derivatives 1, add/cpu_kernel.rs:11-26)."""
+    go = np.asarray(grad_out, np.float64)
+    return round_to(np.asarray(grad_lhs, np.float64) + go, dtype), round_to(np.asarray(grad_rhs, np.float64) + go, dtype)
