@@ -3,8 +3,8 @@
 
 `bench.py` reports the headline metric (4096^3); this companion times every GEMM shape the configurations contain
 (Linear forward / dX / dW at small f32 size, broadcast-rhs f16, attention-shaped batched f16, the encoder block's
-bf16 Linears, vec.mat / mat.vec), the HBM-bound ops between them (softmax, bias, reshape) and a few conv2d
-layers.  GEMMs are timed with HIP events on the library's stream (dfdx_rocm_gemm_time), the other ops with
+bf16 Linears, vec.mat / mat.vec), the HBM-bound ops between them (softmax, bias, reshape, layer norm, ReLU, add), one
+whole encoder block with every op on the device, and a few conv2d layers.  GEMMs are timed with HIP events on the library's stream (dfdx_rocm_gemm_time), the other ops with
 events around a loop of calls.  One line per case on stdout; `--json FILE` also writes them as JSON.
 
 Synthetic inputs, resident in HBM before timing.  Nothing here touches the CPU oracle.
@@ -21,7 +21,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
-    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,gemv,glue,conv")
+    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,gemv,glue,block,conv")
     args = ap.parse_args()
     import torch
     from dfdx_amd import Rocm
@@ -201,6 +201,39 @@ def main():
                 gemm("gemv", f"vec.mat {dt}, Linear weight view", dev.gemm_desc(dt, 1, n_, n_, P(xv), (n_, 1), P(W), (1, n_), P(yv), (n_, 1)), 2 * n_ * n_, es * n_ * n_, 100)
                 gemm("gemv", f"mat.vec {dt} ({n_},{n_})x({n_},)", dev.gemm_desc(dt, n_, n_, 1, P(W), (n_, 1), P(xv), (1, 1), P(yv), (1, 1)), 2 * n_ * n_, es * n_ * n_, 100)
                 del W
+
+    # ---- config 5 end to end: one encoder block, every op on the device -----------------------------------------
+    if want("block"):
+        from dfdx_amd.encoder import EncoderBlock
+        dt, (B, S, d, H, ff) = "bf16", (16, 512, 1024, 16, 4096)
+        T = B * S
+        shapes = {"wq": (d, d), "wk": (d, d), "wv": (d, d), "wo": (d, d), "w1": (ff, d), "w2": (d, ff),
+                  "bq": (d,), "bk": (d,), "bv": (d,), "bo": (d,), "b1": (ff,), "b2": (d,)}
+        params = {n: view(rnd(sh, dt, 0.02), dt) for n, sh in shapes.items()}
+        for n in ("g1", "g2"):
+            params[n] = view(torch.ones(d, device="cuda", dtype=tdt[dt]), dt)
+        for n in ("be1", "be2"):
+            params[n] = view(zeros((d,), dt), dt)
+        blk = EncoderBlock(dev, dt, d, H, ff, params)
+        xv, gv = view(rnd((B, S, d), dt), dt), view(rnd((B, S, d), dt, 1.0 / T), dt)
+        D = d // H
+        fwd_flop = 2.0 * T * d * d * 4 + 2 * 2.0 * T * d * ff + 2 * 2.0 * B * H * S * S * D
+        ln_bytes = 2 * (2 * T * d * 2)
+        timed("block", "encoder block forward (20 calls)", lambda: blk.forward(xv), fwd_flop, 0, "EncoderBlock.forward")
+        _, saved = blk.forward(xv)
+        timed("block", "encoder block backward (37 calls, grads zero-filled)", lambda: blk.backward(saved, gv), 2 * fwd_flop, 0, "EncoderBlock.backward")
+
+        def step():
+            _, sv = blk.forward(xv)
+            blk.backward(sv, gv)
+        timed("block", "encoder block forward + backward", step, 3 * fwd_flop, 0, "EncoderBlock")
+        h = blk.dev.add_forward(xv, xv)
+        timed("glue", f"layer norm fwd ({T},{d}) {dt}", lambda: dev.layer_norm_forward(h, params["g1"], params["be1"]), 0, ln_bytes, "layer_norm_forward")
+        gx, gg, gb = view(zeros((B, S, d), dt), dt), view(zeros((d,), dt), dt), view(zeros((d,), dt), dt)
+        timed("glue", f"layer norm bwd ({T},{d}) {dt}", lambda: dev.layer_norm_backward(h, params["g1"], gx, gg, gb, gv), 0, 2 * ln_bytes, "layer_norm_backward")
+        f1 = view(rnd((B, S, ff), dt), dt)
+        timed("glue", f"relu fwd ({T},{ff}) {dt}", lambda: dev.relu_forward(f1), 0, 2 * T * ff * 2, "relu_forward")
+        timed("glue", f"residual add fwd ({T},{d}) {dt}", lambda: dev.add_forward(xv, h), 0, 3 * T * d * 2, "add_forward")
 
     # ---- conv2d (unfold + batched GEMM) -------------------------------------------------------------------------
     if want("conv"):

@@ -7,3 +7,4 @@ that tests and the benchmark read like the reference's own tests.  There is no
 CPU fallback: if the library is missing or no gfx950 GPU is present, calls fail.
 """
 from .rocm import DTYPES, Rocm, RocmError, View, lib_path, load_library  # noqa: F401
+from .encoder import EncoderBlock  # noqa: F401

@@ -13,7 +13,8 @@
 namespace dfdx_rocm {
 namespace {
 
-constexpr int WAVES = 4;  // rows in flight per workgroup
+constexpr int WAVES = 4;      // rows in flight per workgroup (forward)
+constexpr int WAVES_BWD = 8;  // backward: more rows per workgroup, so fewer slices of column sums to combine
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -79,9 +80,9 @@ __global__ __launch_bounds__(WAVES * 64) void layer_norm_forward_kernel(const T 
 // grad_x += rstd * (gh - mean(gh) - xhat * mean(gh * xhat)),  gh = grad_out * gamma;
 // partial[slice][0][col] = sum over the slice's rows of grad_out * xhat, partial[slice][1][col] = of grad_out.
 template <typename T, int N, int CH>
-__global__ __launch_bounds__(WAVES * 64) void layer_norm_backward_kernel(const T *x, const T *gamma, const T *go, T *gx,
+__global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_kernel(const T *x, const T *gamma, const T *go, T *gx,
                                                                          float *partial, int64_t rows, int cols, float eps) {
-    __shared__ float red[WAVES][2][64 * N];
+    __shared__ float red[WAVES_BWD][2][64 * N];
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const float inv_n = 1.0f / (float)cols;
     float gm[CH][N], dg[CH][N], db[CH][N];
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(WAVES * 64) void layer_norm_backward_kernel(const T
 #pragma unroll
         for (int i = 0; i < N; i++) dg[c][i] = db[c][i] = 0.0f;
     }
-    for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < rows; row += (int64_t)gridDim.x * WAVES) {
+    for (int64_t row = (int64_t)blockIdx.x * WAVES_BWD + wave; row < rows; row += (int64_t)gridDim.x * WAVES_BWD) {
         const T *src = x + row * cols, *gs = go + row * cols;
         float v[CH][N], g[CH][N];
         float s = 0.0f;
@@ -150,7 +151,7 @@ __global__ __launch_bounds__(WAVES * 64) void layer_norm_backward_kernel(const T
             }
         }
     }
-    // column sums of the workgroup's rows: the four waves through LDS, one chunk of 64 * N columns at a time
+    // column sums of the workgroup's rows: the waves through LDS, one chunk of 64 * N columns at a time
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         __syncthreads();
@@ -160,12 +161,12 @@ __global__ __launch_bounds__(WAVES * 64) void layer_norm_backward_kernel(const T
             red[wave][1][lane * N + i] = db[c][i];
         }
         __syncthreads();
-        for (int t = threadIdx.x; t < 2 * 64 * N; t += WAVES * 64) {
+        for (int t = threadIdx.x; t < 2 * 64 * N; t += WAVES_BWD * 64) {
             const int which = t / (64 * N), j = t % (64 * N), col = c * 64 * N + j;
             if (col < cols) {
                 float sum = 0.0f;
 #pragma unroll
-                for (int w = 0; w < WAVES; w++) sum += red[w][which][j];
+                for (int w = 0; w < WAVES_BWD; w++) sum += red[w][which][j];
                 partial[((int64_t)blockIdx.x * 2 + which) * cols + col] = sum;
             }
         }
@@ -196,15 +197,15 @@ __global__ __launch_bounds__(WAVES * 64) void layer_norm_forward_loop_kernel(con
 }
 
 // One workgroup per slice of rows; the column sums go through atomics-free per-wave accumulation in memory order:
-// wave w adds its rows into partial[slice * WAVES + w], so `slices` counts waves here.
+// wave w adds its rows into partial[slice * WAVES_BWD + w], so `slices` counts waves here.
 template <typename T>
-__global__ __launch_bounds__(WAVES * 64) void layer_norm_backward_loop_kernel(const T *x, const T *gamma, const T *go, T *gx,
+__global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_loop_kernel(const T *x, const T *gamma, const T *go, T *gx,
                                                                               float *partial, int64_t rows, int cols, float eps) {
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const float inv_n = 1.0f / (float)cols;
-    float *pg = partial + ((int64_t)(blockIdx.x * WAVES + wave) * 2) * cols, *pb = pg + cols;
+    float *pg = partial + ((int64_t)(blockIdx.x * WAVES_BWD + wave) * 2) * cols, *pb = pg + cols;
     for (int c = lane; c < cols; c += 64) pg[c] = pb[c] = 0.0f;
-    for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < rows; row += (int64_t)gridDim.x * WAVES) {
+    for (int64_t row = (int64_t)blockIdx.x * WAVES_BWD + wave; row < rows; row += (int64_t)gridDim.x * WAVES_BWD) {
         const T *src = x + row * cols, *gs = go + row * cols;
         float s = 0.0f;
         for (int c = lane; c < cols; c += 64) s += Elem<T>::load(src + c);
@@ -232,32 +233,52 @@ __global__ __launch_bounds__(WAVES * 64) void layer_norm_backward_loop_kernel(co
     }
 }
 
-// grad_gamma[c] += sum_s partial[s][0][c], grad_beta[c] += sum_s partial[s][1][c], slices in ascending order
+// grad_gamma[c] += sum_s partial[s][0][c], grad_beta[c] += sum_s partial[s][1][c].  A workgroup owns 64 columns; its
+// 16 lane rows each add up a contiguous sixteenth of the slices (four loads in flight), then lane row 0 adds the 16
+// sums in order: the result does not depend on timing.
+constexpr int COMBINE_GROUPS = 16;
 template <typename T>
-__global__ __launch_bounds__(64) void layer_norm_combine_kernel(const float *partial, int slices, int cols, T *grad_gamma, T *grad_beta) {
-    const int c = blockIdx.x * 64 + threadIdx.x;
-    if (c >= cols) return;
+__global__ __launch_bounds__(64 * COMBINE_GROUPS) void layer_norm_combine_kernel(const float *partial, int slices, int cols, T *grad_gamma,
+                                                                                 T *grad_beta) {
+    __shared__ float red[COMBINE_GROUPS][2][64];
+    const int lane = threadIdx.x % 64, grp = threadIdx.x / 64;
+    const int c = blockIdx.x * 64 + lane;
+    const int per = (slices + COMBINE_GROUPS - 1) / COMBINE_GROUPS;
+    const int j0 = grp * per, j1 = min(slices, j0 + per);
     float sg = 0.0f, sb = 0.0f;
-    int j = 0;
-    for (; j + 4 <= slices; j += 4) {  // loads of four slices in flight, added in slice order
-        float a[4], b[4];
+    if (c < cols) {
+        int j = j0;
+        for (; j + 4 <= j1; j += 4) {
+            float a[4], b[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            a[u] = partial[((int64_t)(j + u) * 2) * cols + c];
-            b[u] = partial[((int64_t)(j + u) * 2 + 1) * cols + c];
+            for (int u = 0; u < 4; u++) {
+                a[u] = partial[((int64_t)(j + u) * 2) * cols + c];
+                b[u] = partial[((int64_t)(j + u) * 2 + 1) * cols + c];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                sg += a[u];
+                sb += b[u];
+            }
         }
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            sg += a[u];
-            sb += b[u];
+        for (; j < j1; j++) {
+            sg += partial[((int64_t)j * 2) * cols + c];
+            sb += partial[((int64_t)j * 2 + 1) * cols + c];
         }
     }
-    for (; j < slices; j++) {
-        sg += partial[((int64_t)j * 2) * cols + c];
-        sb += partial[((int64_t)j * 2 + 1) * cols + c];
+    red[grp][0][lane] = sg;
+    red[grp][1][lane] = sb;
+    __syncthreads();
+    if (grp == 0 && c < cols) {
+        float tg = 0.0f, tb = 0.0f;
+#pragma unroll
+        for (int g = 0; g < COMBINE_GROUPS; g++) {
+            tg += red[g][0][lane];
+            tb += red[g][1][lane];
+        }
+        Elem<T>::store(grad_gamma + c, Elem<T>::load(grad_gamma + c) + tg);
+        Elem<T>::store(grad_beta + c, Elem<T>::load(grad_beta + c) + tb);
     }
-    Elem<T>::store(grad_gamma + c, Elem<T>::load(grad_gamma + c) + sg);
-    Elem<T>::store(grad_beta + c, Elem<T>::load(grad_beta + c) + sb);
 }
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
@@ -294,10 +315,10 @@ int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, co
     const bool vec = cols % V == 0 && aligned16(x) && aligned16(gamma) && aligned16(go) && aligned16(gx);
     const int64_t groups = cols / V;
     const bool reg = vec && groups <= 256;
-    // at least 8 rows per wave so that the column sums amortise; at most four workgroups per compute unit
-    const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>((rows + 8 * WAVES - 1) / (8 * WAVES), (int64_t)ctx->compute_units * 4));
-    const int slices = (int)grid * (reg ? 1 : WAVES);
-    const dim3 block(WAVES * 64);
+    // at least 2 rows per wave so that the column sums amortise; two workgroups (16 waves) per compute unit
+    const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>((rows + 2 * WAVES_BWD - 1) / (2 * WAVES_BWD), (int64_t)ctx->compute_units * 2));
+    const int slices = (int)grid * (reg ? 1 : WAVES_BWD);
+    const dim3 block(WAVES_BWD * 64);
     hipStream_t s = ctx->stream;
     CtxLock lock(ctx->mu);  // two launches around the shared workspace
     if (int rc = ensure_workspace(ctx, (size_t)slices * 2 * cols * sizeof(float))) return rc;
@@ -311,7 +332,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, co
     else layer_norm_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, rows, (int)cols, eps);
 #undef DFDX_LN_BWD
     HIP_TRY(hipGetLastError());
-    layer_norm_combine_kernel<T><<<(unsigned)((cols + 63) / 64), 64, 0, s>>>(partial, slices, (int)cols, (T *)ggamma, (T *)gbeta);
+    layer_norm_combine_kernel<T><<<(unsigned)((cols + 63) / 64), 64 * COMBINE_GROUPS, 0, s>>>(partial, slices, (int)cols, (T *)ggamma, (T *)gbeta);
     return (int)hipGetLastError();
 }
 

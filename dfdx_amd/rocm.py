@@ -205,6 +205,14 @@ class Rocm:
         raw = torch.zeros(max(n * ITEMSIZE[dtype], 16), dtype=torch.uint8, device=self.device)
         return View(raw, dtype, shape, _row_major(shape) if strides is None else tuple(strides))
 
+    def empty(self, dtype: str, shape) -> View:
+        """Uninitialised storage for an output that a forward kernel overwrites (``alloc_empty``,
+        tensor_ops/matmul/cuda_kernel.rs:253)."""
+        shape = tuple(shape)
+        n = int(np.prod(shape, dtype=np.int64))
+        raw = self._torch.empty(max(n * ITEMSIZE[dtype], 16), dtype=self._torch.uint8, device=self.device)
+        return View(raw, dtype, shape, _row_major(shape))
+
     def zeros_like_storage(self, v: View) -> View:
         """A gradient buffer for ``v``: zero-filled, same physical length, same strides (gradients.rs:53-58)."""
         raw = self._torch.zeros_like(v.storage)
@@ -259,7 +267,7 @@ class Rocm:
         vp = ctypes.c_void_p
         if L == 1 and R == 1:      # outer product: (M,1) x (1,N)
             m, n = lhs.shape[0], rhs.shape[0]
-            out = self.zeros(dt, (m, n))
+            out = self.empty(dt, (m, n))
             self._check(self.lib.dfdx_rocm_matmat_forward(
                 self.ctx, DTYPES[dt], _c(m), _c(1), _c(n), vp(lhs.ptr), _i64arr((lhs.strides[0], 1)),
                 vp(rhs.ptr), _i64arr((n * rhs.strides[0], rhs.strides[0])), vp(out.ptr)))
@@ -267,7 +275,7 @@ class Rocm:
         if L == 1 and R == 2:      # (1,K) x (K,N) -> (N,)
             assert lhs.shape[0] == rhs.shape[0], f"left: {lhs.shape[0]}\n right: {rhs.shape[0]}"
             k, n = rhs.shape
-            out = self.zeros(dt, (n,))
+            out = self.empty(dt, (n,))
             self._check(self.lib.dfdx_rocm_matmat_forward(
                 self.ctx, DTYPES[dt], _c(1), _c(k), _c(n), vp(lhs.ptr), _i64arr((k * lhs.strides[0], lhs.strides[0])),
                 vp(rhs.ptr), _i64arr(rhs.strides), vp(out.ptr)))
@@ -275,7 +283,7 @@ class Rocm:
         if L == 2 and R == 1:      # (M,K) x (K,1) -> (M,)
             assert lhs.shape[1] == rhs.shape[0], f"left: {lhs.shape[1]}\n right: {rhs.shape[0]}"
             m, k = lhs.shape
-            out = self.zeros(dt, (m,))
+            out = self.empty(dt, (m,))
             self._check(self.lib.dfdx_rocm_matmat_forward(
                 self.ctx, DTYPES[dt], _c(m), _c(k), _c(1), vp(lhs.ptr), _i64arr(lhs.strides),
                 vp(rhs.ptr), _i64arr((rhs.strides[0], 1)), vp(out.ptr)))
@@ -283,7 +291,7 @@ class Rocm:
         if L == 2 and R == 2:
             assert lhs.shape[1] == rhs.shape[0], f"left: {lhs.shape[1]}\n right: {rhs.shape[0]}"
             (m, k), n = lhs.shape, rhs.shape[1]
-            out = self.zeros(dt, (m, n))
+            out = self.empty(dt, (m, n))
             self._check(self.lib.dfdx_rocm_matmat_forward(
                 self.ctx, DTYPES[dt], _c(m), _c(k), _c(n), vp(lhs.ptr), _i64arr(lhs.strides),
                 vp(rhs.ptr), _i64arr(rhs.strides), vp(out.ptr)))
@@ -291,7 +299,7 @@ class Rocm:
         if L == 3 and R == 2:
             assert lhs.shape[2] == rhs.shape[0], f"left: {lhs.shape[2]}\n right: {rhs.shape[0]}"
             (b, m, k), n = lhs.shape, rhs.shape[1]
-            out = self.zeros(dt, (b, m, n))
+            out = self.empty(dt, (b, m, n))
             self._check(self.lib.dfdx_rocm_matmat_br_forward(
                 self.ctx, DTYPES[dt], _c(b), _c(m), _c(k), _c(n), vp(lhs.ptr), _i64arr(lhs.strides),
                 vp(rhs.ptr), _i64arr(rhs.strides), vp(out.ptr)))
@@ -300,7 +308,7 @@ class Rocm:
             assert lhs.shape[0] == rhs.shape[0], f"left: {lhs.shape[0]}\n right: {rhs.shape[0]}"
             assert lhs.shape[2] == rhs.shape[1], f"left: {lhs.shape[2]}\n right: {rhs.shape[1]}"
             (b, m, k), n = lhs.shape, rhs.shape[2]
-            out = self.zeros(dt, (b, m, n))
+            out = self.empty(dt, (b, m, n))
             self._check(self.lib.dfdx_rocm_matmat_batch3_forward(
                 self.ctx, DTYPES[dt], _c(b), _c(m), _c(k), _c(n), vp(lhs.ptr), _i64arr(lhs.strides),
                 vp(rhs.ptr), _i64arr(rhs.strides), vp(out.ptr)))
@@ -310,7 +318,7 @@ class Rocm:
             assert lhs.shape[1] == rhs.shape[1], f"left: {lhs.shape[1]}\n right: {rhs.shape[1]}"
             assert lhs.shape[3] == rhs.shape[2], f"left: {lhs.shape[3]}\n right: {rhs.shape[2]}"
             (b, s, m, k), n = lhs.shape, rhs.shape[3]
-            out = self.zeros(dt, (b, s, m, n))
+            out = self.empty(dt, (b, s, m, n))
             self._check(self.lib.dfdx_rocm_matmat_batch4_forward(
                 self.ctx, DTYPES[dt], _c(b), _c(s), _c(m), _c(k), _c(n), vp(lhs.ptr), _i64arr(lhs.strides),
                 vp(rhs.ptr), _i64arr(rhs.strides), vp(out.ptr)))
@@ -365,7 +373,7 @@ class Rocm:
         else:
             assert x.strides == _row_major(x.shape), "batched Linear input must be contiguous to fold its rows"
             rows, xs = int(np.prod(x.shape[:-1])), (i, 1)
-        out = self.zeros(x.dtype, tuple(x.shape[:-1]) + (o,))
+        out = self.empty(x.dtype, tuple(x.shape[:-1]) + (o,))
         self._check(self.lib.dfdx_rocm_linear_forward(
             self.ctx, DTYPES[x.dtype], _c(rows), _c(i), _c(o), ctypes.c_void_p(x.ptr), _i64arr(xs),
             ctypes.c_void_p(weight.ptr), ctypes.c_void_p(bias.ptr if bias is not None else None),
@@ -400,7 +408,7 @@ class Rocm:
         assert x.shape[-1] == cols, f"left: {x.shape[-1]}\n right: {cols}"
         assert x.strides == _row_major(x.shape) and bias.strides == (1,)
         rows = int(np.prod(x.shape[:-1], dtype=np.int64))
-        out = self.zeros(x.dtype, x.shape)
+        out = self.empty(x.dtype, x.shape)
         vp = ctypes.c_void_p
         self._check(self.lib.dfdx_rocm_bias_forward(self.ctx, DTYPES[x.dtype], _c(rows), _c(cols), vp(x.ptr),
                                                     vp(bias.ptr), vp(out.ptr)))
@@ -458,7 +466,7 @@ class Rocm:
             f"left: {int(np.prod(x.shape))}\n right: {int(np.prod(new_shape))}"
         if x.strides == _row_major(x.shape):
             return View(x.storage, x.dtype, new_shape, _row_major(new_shape), x.offset)
-        out = self.zeros(x.dtype, new_shape)
+        out = self.empty(x.dtype, new_shape)
         vp = ctypes.c_void_p
         self._check(self.lib.dfdx_rocm_reshape_forward(self.ctx, DTYPES[x.dtype], len(x.shape), _i64arr(x.shape),
                                                        _i64arr(x.strides), vp(x.ptr), vp(out.ptr)))
@@ -543,7 +551,7 @@ class Rocm:
         """``(img, filters).conv2d(stride, padding, dilation, groups)``; img (B, C, H, W) or (C, H, W)."""
         op = self._conv2d_op(img, filters, stride, padding, dilation, groups)
         lead = (op.batch,) if len(img.shape) == 4 else ()
-        out = self.zeros(img.dtype, lead + (op.chan_out, op.h_out, op.w_out))
+        out = self.empty(img.dtype, lead + (op.chan_out, op.h_out, op.w_out))
         vp = ctypes.c_void_p
         self._check(self.lib.dfdx_rocm_conv2d_forward(self.ctx, DTYPES[img.dtype], ctypes.byref(op), vp(img.ptr),
                                                       vp(filters.ptr), vp(out.ptr)))

@@ -101,3 +101,68 @@ def test_config5_encoder_block_bf16_full_size():
     np.testing.assert_allclose(val(grads["be2"], dtype), gout.sum(axis=0), atol=2 ** -7 * np.abs(gout.sum(axis=0)).max())
     for name in ("wq", "wk", "wv", "wo", "w1", "w2"):
         assert np.abs(val(grads[name], dtype)).max() > 0
+
+
+def _device_block(dev, dtype, p, d, H, ff):
+    from dfdx_amd.encoder import EncoderBlock
+    shapes = {"wq": (d, d), "wk": (d, d), "wv": (d, d), "wo": (d, d), "w1": (ff, d), "w2": (d, ff)}
+    params = {n: dev.tensor(v, dtype, shapes.get(n, (v.size,))) for n, v in p.items()}
+    return EncoderBlock(dev, dtype, d, H, ff, params)
+
+
+def test_small_encoder_block_entirely_on_the_device():
+    """The same block with EVERY op on the device (dfdx_amd/encoder.py: Linear with fused bias, the attention
+    matmuls, softmax with the scale folded in, the copying reshape, residual adds, LayerNorm, ReLU and all their
+    backward ops), against the host-glue + CPU-oracle path.  The device ops evaluate each formula in f32 and round
+    once where the host path rounds after every numpy op, so results agree to a few ulp of the largest value."""
+    dev, g = device(), rng(5005)
+    dtype, (B, S, d, H, ff) = "bf16", (2, 64, 128, 4, 256)
+    p = init_params(g, d, ff, dtype)
+    for name in ("g1", "g2", "be1", "be2"):                       # non-trivial LayerNorm parameters
+        p[name] = oracle.to_storage((val(p[name], dtype) + 0.1 * g.standard_normal(d)).astype(np.float32), dtype)
+    x = g.standard_normal((B * S, d)).astype(np.float32)
+    gout = g.standard_normal((B * S, d)).astype(np.float32) / (B * S)
+    out_o, grads_o, dx_o = encoder_block(OracleBackend(dtype), dtype, p, x, B, S, d, H, ff, gout)
+    announce("config5 on-device block", (B, S, d, H, ff))
+    blk = _device_block(dev, dtype, p, d, H, ff)
+    xd = dev.tensor(oracle.to_storage(x.reshape(-1), dtype), dtype, (B, S, d))
+    out_v, saved = blk.forward(xd)
+    grads_v, gx_v = blk.backward(saved, dev.tensor(oracle.to_storage(gout.reshape(-1), dtype), dtype, (B, S, d)))
+    out_g = val(dev.to_host(out_v), dtype).reshape(B * S, d)
+    assert np.abs(out_g - out_o).max() <= 16 * ULP[dtype] * np.abs(out_o).max()
+    dx_g = val(dev.to_host(gx_v), dtype).reshape(B * S, d)
+    assert np.abs(dx_g - dx_o).max() <= 24 * ULP[dtype] * np.abs(dx_o).max() + 1e-12
+    for name in grads_o:
+        go, gg = val(grads_o[name], dtype), val(dev.to_host(grads_v[name]), dtype)
+        if name == "bk":   # a bias on the keys shifts every score of a row alike: its gradient is 0 up to rounding noise
+            assert max(np.abs(go).max(), np.abs(gg).max()) <= 1e-2 * np.abs(val(grads_o["bq"], dtype)).max()
+            continue
+        # A pre-activation that rounds to the other side of 0 flips one ReLU derivative (the fused Linear bias rounds
+        # once, the host path twice): about 0.3 % of the entries of the gradient behind the ReLU are then off by
+        # their whole value, which is a few percent of its norm; everything else differs by rounding only.
+        assert np.abs(gg - go).max() <= 48 * ULP[dtype] * np.abs(go).max() + 1e-12, name
+        assert np.linalg.norm(gg - go) <= 6e-2 * np.linalg.norm(go) + 1e-12, name
+
+
+def test_config5_encoder_block_on_the_device_full_size():
+    """Full-size config 5 with every op on the device: invariants of the output and of the gradients that have
+    closed forms (the host path at this size is covered GEMM by GEMM above)."""
+    dev, g = device(), rng(5007)
+    dtype, (B, S, d, H, ff) = "bf16", (16, 512, 1024, 16, 4096)
+    p = init_params(g, d, ff, dtype)
+    blk = _device_block(dev, dtype, p, d, H, ff)
+    x = g.standard_normal((B * S, d)).astype(np.float32)
+    gout = g.standard_normal((B * S, d)).astype(np.float32) / (B * S)
+    announce("config5 on-device block, full size")
+    out_v, saved = blk.forward(dev.tensor(oracle.to_storage(x.reshape(-1), dtype), dtype, (B, S, d)))
+    gout_st = oracle.to_storage(gout.reshape(-1), dtype)
+    grads, gx = blk.backward(saved, dev.tensor(gout_st, dtype, (B, S, d)))
+    out = val(dev.to_host(out_v), dtype).reshape(B * S, d)
+    assert np.all(np.isfinite(out)) and np.all(np.isfinite(val(dev.to_host(gx), dtype)))
+    assert np.abs(out.mean(axis=-1)).max() < 2e-2 and np.abs(out.var(axis=-1) - 1).max() < 5e-2
+    gsum = val(gout_st, dtype).reshape(B * S, d).sum(axis=0)
+    np.testing.assert_allclose(val(dev.to_host(grads["be2"]), dtype), gsum, atol=2 ** -7 * np.abs(gsum).max())
+    probs = val(dev.to_host(saved["probs"]), dtype).reshape(-1, S)
+    assert np.abs(probs.sum(axis=-1) - 1).max() < 2e-2
+    for name in ("wq", "wk", "wv", "wo", "w1", "w2", "g1", "b1"):
+        assert np.abs(val(dev.to_host(grads[name]), dtype)).max() > 0, name
