@@ -338,11 +338,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
     // swapped operands: the lane ends up with m = l16 and 4 consecutive n = 4*lq + 0..3 per 16x16 tile
     auto mma = [&](const u32x4(&bf)[TN], int i0, int i1) {
 #pragma unroll
-        for (int i = 0; i < TM; i++)
-            if (i >= i0 && i < i1) {
+        for (int j = 0; j < TN; j++) {
 #pragma unroll
-                for (int j = 0; j < TN; j++) acc[i][j] = Mma<T>::mfma(bf[j], fa[i], acc[i][j]);
-            }
+            for (int i = 0; i < TM; i++)
+                if (i >= i0 && i < i1) acc[i][j] = Mma<T>::mfma(bf[j], fa[i], acc[i][j]);
+        }
     };
     // Make the oldest requested tile visible to every wave, then request the next one into the stage that the
     // previously computed tile occupied.  Callers guarantee that this wave has issued all its LDS reads of

@@ -89,3 +89,29 @@ def test_linear_backward_without_bias_gradient():
     gx, gw = dev.zeros("f32", (4, 8)), dev.zeros("f32", (3, 8))
     dev.linear_backward(x, gx, w, gw, None, go)
     dev.synchronize()
+
+
+def test_layer_norm_relu_add_argument_checks():
+    dev = device()
+    lib, ctx = dev.lib, dev.ctx
+    announce("layer norm / relu / add argument checks")
+    buf = dev.zeros("f32", (64,))
+    p = VP(buf.ptr)
+    assert lib.dfdx_rocm_layer_norm_forward(ctx, 0, I64(-1), I64(4), p, p, p, F64(1e-5), p) == INVALID
+    assert lib.dfdx_rocm_layer_norm_forward(ctx, 0, I64(2), I64(1 << 24), p, p, p, F64(1e-5), p) == INVALID
+    assert lib.dfdx_rocm_layer_norm_forward(ctx, 0, I64(2), I64(4), p, VP(), p, F64(1e-5), p) == INVALID
+    assert lib.dfdx_rocm_layer_norm_forward(ctx, 3, I64(2), I64(4), p, p, p, F64(1e-5), p) == UNSUPPORTED
+    assert lib.dfdx_rocm_layer_norm_forward(ctx, 0, I64(0), I64(4), VP(), VP(), VP(), F64(1e-5), VP()) == 0
+    assert lib.dfdx_rocm_layer_norm_backward(ctx, 0, I64(2), I64(4), p, p, F64(1e-5), p, p, VP(), p) == INVALID
+    assert lib.dfdx_rocm_layer_norm_backward(ctx, 0, I64(2), I64(0), VP(), VP(), F64(1e-5), VP(), VP(), VP(), VP()) == 0
+    assert lib.dfdx_rocm_relu_forward(ctx, 0, I64(-1), p, p) == INVALID
+    assert lib.dfdx_rocm_relu_forward(ctx, 0, I64(4), VP(), p) == INVALID
+    assert lib.dfdx_rocm_relu_forward(ctx, 3, I64(4), p, p) == UNSUPPORTED
+    assert lib.dfdx_rocm_relu_backward(ctx, 0, I64(4), p, p, VP()) == INVALID
+    assert lib.dfdx_rocm_relu_forward(ctx, 0, I64(0), VP(), VP()) == 0
+    assert lib.dfdx_rocm_add_forward(ctx, 0, I64(4), p, VP(), p) == INVALID
+    assert lib.dfdx_rocm_add_backward(ctx, 0, I64(4), p, VP(), p) == INVALID
+    assert lib.dfdx_rocm_add_backward(ctx, 0, I64(4), VP(), VP(), p) == INVALID
+    assert lib.dfdx_rocm_add_forward(ctx, 0, I64(0), VP(), VP(), VP()) == 0
+    dev.synchronize()
+    assert np.all(dev.to_host(buf) == 0)
