@@ -109,7 +109,11 @@ template <int ROWS, int NWAVES, bool KC> struct DmaTile {
     static constexpr int IPW = INSTRS / NWAVES;
     static_assert(INSTRS % NWAVES == 0 && IPW >= 1, "tile does not divide over the waves");
     static constexpr int CPR = KC ? BK / 8 : ROWS / 8;  // 16 B chunks per LDS row
-    uint32_t goff[IPW];                                 // byte offset from the tile origin in global memory
+    // Byte offset from the tile origin in global memory, plus 1024 * (IPW - 1 - i): the wave's IPW instructions share
+    // ONE LDS base, that of the last 1 KB piece (one M0 write instead of IPW), and reach their own piece through the
+    // instruction offset -1024 * (IPW - 1 - i), which the hardware adds to the global address as well.
+    static_assert((IPW - 1) * 1024 <= 4096, "instruction offsets are 13-bit signed");
+    uint32_t goff[IPW];
 
     __device__ __forceinline__ void init(int ld, int rows_left, int wave, int lane) {
 #pragma unroll
@@ -118,18 +122,21 @@ template <int ROWS, int NWAVES, bool KC> struct DmaTile {
             const int r = slot / CPR, cp = slot % CPR;
             if constexpr (KC) {
                 const int c = cp ^ ((r >> 1) & 7);
-                goff[i] = (uint32_t)(min(r, rows_left - 1) * ld + c * 8) * 2u;
+                goff[i] = (uint32_t)(min(r, rows_left - 1) * ld + c * 8) * 2u + (uint32_t)(1024 * (IPW - 1 - i));
             } else {
                 const int c = cp ^ mc_swizzle<ROWS>(r);
-                goff[i] = (uint32_t)(r * ld + min(c * 8, rows_left - 8)) * 2u;
+                goff[i] = (uint32_t)(r * ld + min(c * 8, rows_left - 8)) * 2u + (uint32_t)(1024 * (IPW - 1 - i));
             }
         }
     }
+    template <int I> __device__ __forceinline__ void issue_one(const char *origin, DFDX_LDS void *lds) const {
+        if constexpr (I < IPW) {
+            __builtin_amdgcn_global_load_lds((const DFDX_GLB void *)(origin + goff[I]), lds, 16, -1024 * (IPW - 1 - I), 0);
+            issue_one<I + 1>(origin, lds);
+        }
+    }
     __device__ __forceinline__ void issue(const uint16_t *g, uint8_t *lds_tile, int wave) const {
-#pragma unroll
-        for (int i = 0; i < IPW; i++)
-            __builtin_amdgcn_global_load_lds((const DFDX_GLB void *)((const char *)g + goff[i]),
-                                             (DFDX_LDS void *)(lds_tile + (wave * IPW + i) * 1024), 16, 0, 0);
+        issue_one<0>((const char *)g, (DFDX_LDS void *)(lds_tile + (wave * IPW + IPW - 1) * 1024));
     }
 };
 
