@@ -135,8 +135,11 @@ template <int ROWS, int NWAVES, bool KC> struct DmaTile {
             issue_one<I + 1>(origin, lds);
         }
     }
-    __device__ __forceinline__ void issue(const uint16_t *g, uint8_t *lds_tile, int wave) const {
-        issue_one<0>((const char *)g, (DFDX_LDS void *)(lds_tile + (wave * IPW + IPW - 1) * 1024));
+    // LDS byte address of the wave's last 1 KB piece inside a tile that starts at byte `tile` of the LDS allocation
+    static __device__ __forceinline__ uint32_t wave_base(uint32_t tile, int wave) { return tile + (uint32_t)(wave * IPW + IPW - 1) * 1024u; }
+    // `lds_last`: wave_base of the destination tile, wave-uniform (a scalar register: it goes to M0 as it is)
+    __device__ __forceinline__ void issue(const uint16_t *g, uint32_t lds_last) const {
+        issue_one<0>((const char *)g, (DFDX_LDS void *)(uintptr_t)lds_last);
     }
 };
 
@@ -221,11 +224,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
     };
     begin_fetch();
     bool fetching = true;
+    const uint32_t smem_addr = (uint32_t)(uintptr_t)(DFDX_LDS const uint8_t *)smem;
+    const uint32_t lds_last_a = __builtin_amdgcn_readfirstlane(TA::wave_base(smem_addr, wave));
+    const uint32_t lds_last_b = __builtin_amdgcn_readfirstlane(TB::wave_base(smem_addr + TA::BYTES, wave));
     auto issue = [&]() {
-        uint8_t *st = smem + f_stage * STAGE_BYTES;
+        const uint32_t st = (uint32_t)f_stage * STAGE_BYTES;
         f_stage ^= 1;
-        ta.issue(a_next, st, wave);
-        tb.issue(b_next, st + TA::BYTES, wave);
+        ta.issue(a_next, lds_last_a + st);
+        tb.issue(b_next, lds_last_b + st);
         if (--f_left == 0) {  // next request belongs to the next work item (if any)
             f_index += gridDim.x;
             fetching = f_index < p.total_blocks;
