@@ -152,7 +152,11 @@ constexpr int dma_waves_per_simd(int bm, int bn, int waves) {
     return w < 2 ? 2 : (w > 6 ? 6 : w);
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
+// EDGE = false is the instance for problems made of whole tiles (no per-row bias, no bias together with beta = 1): its
+// epilogue has only the two interior forms.  With the general form compiled in as well, the compiler guards the
+// fragment registers against a load of that form it cannot prove complete, with a wait for ALL memory traffic in the
+// middle of the k loop -- where every wave then stalls on the tile prefetched for the step after.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool EDGE>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, WAVES_M *WAVES_N)) void gemm_mfma16_dma_kernel(const Params p) {
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
@@ -634,12 +638,23 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
                     }
                 }
             };
-            const bool interior = bm0 + BM <= p.m && bn0 + BN <= p.n && p.bias_mode != BIAS_PER_ROW && p.ldc < (1 << 26);
+            // Every form ends by telling the compiler, with a wait that costs nothing, that the loads it issued are
+            // complete: "at most as many memory instructions outstanding as the stores issued after the last load" (the
+            // counter retires in issue order, and every loaded value has been consumed by then).  The general form
+            // cannot count its stores and waits for them (edge tiles).
+            constexpr auto vmcnt_only = [](int vm) { return (vm & 15) | ((vm >> 4) << 14) | 0x0F70; };
+            const bool interior = !EDGE || (bm0 + BM <= p.m && bn0 + BN <= p.n && p.bias_mode != BIAS_PER_ROW && p.ldc < (1 << 26));
             if (interior && !p.accumulate) {
                 if (p.bias_mode == BIAS_PER_COL) rows_plain(std::true_type{});
                 else rows_plain(std::false_type{});
-            } else if (interior && p.bias_mode == BIAS_NONE) rows_accumulate();
-            else rows();
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(TM * TN / 2));
+            } else if (!EDGE || (interior && p.bias_mode == BIAS_NONE)) {
+                rows_accumulate();
+                __builtin_amdgcn_s_waitcnt(vmcnt_only((TM * (TN / 2) > 8 ? TM / 2 : TM) * TN / 2));
+            } else if constexpr (EDGE) {
+                rows();
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+            }
             return;
         }
     }
@@ -744,9 +759,9 @@ template <typename T, int BM, int BN, int WM, int WN>
 hipError_t launch_layout(Params p, int compute_units, bool a_kc, bool b_kc, hipStream_t stream) {
     constexpr int NT = WM * WN * 64;
     constexpr size_t lds = (size_t)STAGES * (BM + BN) * BK * 2;
-#define DFDX_LAUNCH(AKC, BKC)                                                                                  \
+#define DFDX_LAUNCH(AKC, BKC, EDGE)                                                                            \
     do {                                                                                                       \
-        auto kern = gemm_mfma16_dma_kernel<T, BM, BN, WM, WN, AKC, BKC>;                                       \
+        auto kern = gemm_mfma16_dma_kernel<T, BM, BN, WM, WN, AKC, BKC, EDGE>;                                 \
         static int per_cu = 0;                                                                                 \
         if (per_cu == 0) {                                                                                     \
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,  \
@@ -761,10 +776,20 @@ hipError_t launch_layout(Params p, int compute_units, bool a_kc, bool b_kc, hipS
         p.grid = p.total_blocks <= resident ? p.total_blocks : resident;                                       \
         kern<<<dim3((unsigned)p.grid), dim3(NT), lds, stream>>>(p);                                            \
     } while (0)
-    if (a_kc && b_kc) DFDX_LAUNCH(true, true);
-    else if (a_kc && !b_kc) DFDX_LAUNCH(true, false);
-    else if (!a_kc && b_kc) DFDX_LAUNCH(false, true);
-    else DFDX_LAUNCH(false, false);
+    // whole tiles only, and nothing but the two interior epilogue forms: the instance without the general form
+    const bool edge = p.m % BM != 0 || p.n % BN != 0 || p.bias_mode == BIAS_PER_ROW || p.ldc >= (1 << 26) ||
+                      (p.accumulate && p.bias_mode != BIAS_NONE);
+    if (edge) {
+        if (a_kc && b_kc) DFDX_LAUNCH(true, true, true);
+        else if (a_kc && !b_kc) DFDX_LAUNCH(true, false, true);
+        else if (!a_kc && b_kc) DFDX_LAUNCH(false, true, true);
+        else DFDX_LAUNCH(false, false, true);
+    } else {
+        if (a_kc && b_kc) DFDX_LAUNCH(true, true, false);
+        else if (a_kc && !b_kc) DFDX_LAUNCH(true, false, false);
+        else if (!a_kc && b_kc) DFDX_LAUNCH(false, true, false);
+        else DFDX_LAUNCH(false, false, false);
+    }
 #undef DFDX_LAUNCH
     return hipGetLastError();
 }
