@@ -418,19 +418,36 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
         fence_a(DFDX_LEFT(RB + RA), Q, 2 * Q);
         mma(fb[1], Q, 2 * Q);
         __builtin_amdgcn_sched_barrier(0);
-        fence_a(DFDX_LEFT(RA / 2), 2 * Q, 3 * Q);
-        mma(fb[1], 2 * Q, 3 * Q);
-        __builtin_amdgcn_sched_barrier(0);
         if constexpr (HAS_NEXT) {
-            sync_tile();
+            // Every LDS read of this tile has been issued: wait for them and hand the stage over TWO MFMA groups before
+            // the end of the tile, so that the requests for the tile after next and the first fragment reads of the
+            // next one are issued under MFMAs instead of in front of an idle matrix core.  The two waves that share a
+            // SIMD (w and w + NW/2) take opposite orders: one issues its MFMA group while the other issues requests.
+            __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) & lgkmcnt(0)
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            fence_a(DFDX_LEFT(0), 2 * Q, TM);
+            const bool mfma_first = __builtin_amdgcn_readfirstlane(wave) >= NW / 2;
+            if (mfma_first) mma(fb[1], 2 * Q, 3 * Q);
+            __builtin_amdgcn_sched_barrier(0);
+            if (fetching) issue();
+            __builtin_amdgcn_sched_barrier(0);
+            if (!mfma_first) mma(fb[1], 2 * Q, 3 * Q);
+            __builtin_amdgcn_sched_barrier(0);
             read_a(sn, K0, 0, 2 * Q);
             read_b(sn, K0, fb[0]);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(fb[1], 3 * Q, TM);
+            __builtin_amdgcn_sched_barrier(0);
+            read_a(sn, K0, 2 * Q, TM);
+        } else {
+            fence_a(DFDX_LEFT(RA / 2), 2 * Q, 3 * Q);
+            mma(fb[1], 2 * Q, 3 * Q);
+            __builtin_amdgcn_sched_barrier(0);
+            fence_a(DFDX_LEFT(0), 3 * Q, TM);
+            mma(fb[1], 3 * Q, TM);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        fence_a(DFDX_LEFT(HAS_NEXT ? RA + RB : 0), 3 * Q, TM);
-        mma(fb[1], 3 * Q, TM);
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (HAS_NEXT) read_a(sn, K0, 2 * Q, TM);
         __builtin_amdgcn_sched_barrier(0);
     };
 
