@@ -429,16 +429,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
             asm volatile("" ::: "memory");
             fence_a(DFDX_LEFT(0), 2 * Q, TM);
             const bool mfma_first = __builtin_amdgcn_readfirstlane(wave) >= NW / 2;
-            if (mfma_first) mma(fb[1], 2 * Q, 3 * Q);
+            if (mfma_first) {
+                mma(fb[1], 2 * Q, 3 * Q);
+                mma(fb[1], 3 * Q, TM);
+            }
             __builtin_amdgcn_sched_barrier(0);
             if (fetching) issue();
-            __builtin_amdgcn_sched_barrier(0);
-            if (!mfma_first) mma(fb[1], 2 * Q, 3 * Q);
             __builtin_amdgcn_sched_barrier(0);
             read_a(sn, K0, 0, 2 * Q);
             read_b(sn, K0, fb[0]);
             __builtin_amdgcn_sched_barrier(0);
-            mma(fb[1], 3 * Q, TM);
+            if (!mfma_first) {
+                mma(fb[1], 2 * Q, 3 * Q);
+                mma(fb[1], 3 * Q, TM);
+            }
             __builtin_amdgcn_sched_barrier(0);
             read_a(sn, K0, 2 * Q, TM);
         } else {
