@@ -912,13 +912,13 @@ struct VariantModel {
     double rate1, rate2;  // flop/s of a compute unit with 1 / with >= 2 resident workgroups
 };
 constexpr VariantModel kModel[] = {
-    {1, 4.64e12, 4.64e12},  // 256x256
-    {1, 3.81e12, 3.81e12},  // 256x128
+    {1, 5.50e12, 5.50e12},  // 256x256
+    {1, 4.40e12, 4.40e12},  // 256x128
     {2, 3.00e12, 4.25e12},  // 128x128
     {1, 3.60e12, 3.60e12},  // 256x64
     {2, 2.20e12, 2.90e12},  // 128x64
 };
-constexpr double kItemOverhead = 3.1e-6, kLaunchLatency = 2e-6, kCuBandwidth = 24e9, kOperandWeight = 0.32;
+constexpr double kItemOverhead = 2.0e-6, kLaunchLatency = 2e-6, kCuBandwidth = 24e9, kOperandWeight = 0.32;
 constexpr double kIdleBoost = 0.146, kWsBandwidthCached = 9.5e12, kWsBandwidthHbm = 6.1e12, kWsCached = 128e6;
 constexpr double kSplitLaunch = 7e-6, kSplitPerPiece = 0.25e-6;  // 1024^3: 12.4 us unsplit, 15.9 / 18.0 us in 2 / 4 pieces
 }  // namespace
