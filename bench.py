@@ -34,9 +34,19 @@ def main():
                     help="counter-collection aid: 3 plain 256 MiB device copies, then 5 headline GEMM launches, nothing else")
     ap.add_argument("--probe-variants", action="store_true",
                     help="counter-collection aid: 3 launches of the headline GEMM with every f16 MFMA tile variant forced in turn")
+    ap.add_argument("--probe-mfma-power", action="store_true",
+                    help="run the stand-alone MFMA-only program (the matrix-core work of the headline GEMM on "
+                         "register-resident zero and U(-1,1) operands) and print its table")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+    if args.probe_mfma_power:   # a child process, started before this one touches the GPU
+        import subprocess
+
+        exe = os.path.join(ROOT, "dfdx_amd", "lib", "probe_mfma_power")
+        if not os.path.exists(exe):
+            sys.exit("bench.py: %s is not built (python __graft_entry__.py build)" % exe)
+        sys.exit(subprocess.call([exe]))
 
     import numpy as np
     import torch
