@@ -303,6 +303,30 @@ def test_split_k_many_ways_for_filter_gradient_shapes(dtype):
         assert_within(dtype, nb * k, oracle.to_f64(outs[0], dtype).reshape(m, n), want, A, B, extra=ulp * np.abs(want).max())
 
 
+# ------------------------------------------------------- planner's choices --
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+def test_auto_dispatch_seeded_shape_sweep(dtype):
+    """Whatever kernel, tile and split count the planner picks for a shape, the result is the oracle's: 48 seeded
+    shapes per dtype through KERNEL_AUTO -- extents from 1 to ~700 (aligned to the MFMA kernels' 8 / 64 granules or
+    not), contractions up to 4096, every operand layout, row- and column-major C, padded leading dimensions, with
+    and without accumulation, with and without the fused bias."""
+    g = rng(20240 + len(dtype))
+    for i in range(48):
+        kind = i % 4
+        if kind == 0:      # everything aligned: the LDS-DMA family (16-bit) / the f32 MFMA kernel
+            m, n, k = int(g.integers(1, 88)) * 8, int(g.integers(1, 88)) * 8, int(g.integers(1, 17)) * 64
+        elif kind == 1:    # aligned rows / columns, k not a multiple of 64: the register-staged family
+            m, n, k = int(g.integers(1, 88)) * 8, int(g.integers(1, 88)) * 8, int(g.integers(1, 130)) * 8
+        elif kind == 2:    # few output tiles, long contraction: split-k candidates
+            m, n, k = int(g.integers(4, 40)) * 8, int(g.integers(4, 40)) * 8, int(g.integers(16, 65)) * 64
+        else:              # nothing aligned: the generic kernel (or GEMV when an extent is 1)
+            m, n, k = int(g.integers(1, 300)), int(g.integers(1, 300)), int(g.integers(1, 500))
+        layout = list(LAYOUTS)[int(g.integers(0, 4))]
+        pads = tuple(int(g.integers(0, 3)) * 8 for _ in range(3)) if kind != 3 else tuple(int(g.integers(0, 5)) for _ in range(3))
+        accumulate, ccol, bias = bool(g.integers(0, 2)), bool(g.integers(0, 4) == 0), bool(g.integers(0, 3) == 0)
+        run_case(dtype, m, k, n, layout, accumulate, KERNEL_AUTO, 0, c_colmajor=ccol, bias=bias, seed=500 + i, pads=pads)
+
+
 # ------------------------------------------------------------------ batched --
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("kernel", [KERNEL_GENERIC, KERNEL_MFMA])
