@@ -21,7 +21,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
-    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,gemv,glue,block,conv")
+    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv")
     args = ap.parse_args()
     import torch
     from dfdx_amd import Rocm
@@ -190,6 +190,19 @@ def main():
         gemm("c5", "attn dV P^T.dO acc, interleaved rows", d5(S, S, D, p_, (1, S), sSS, d_o, (D, 1), sSD, gv, (H * D, 1), tok, True),
              fl, es * nb * (S * S + 3 * S * D))
         del sc, p_, gp
+
+    # ---- zero fill of gradient storage (Storage::try_alloc_len): HBM write roofline -----------------------------
+    if want("fill"):
+        import ctypes
+
+        for mb in (2, 16, 64, 256):   # config 5's weight, activation, ff activation and probability gradients
+            nbytes = mb << 20
+            buf = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+            ptr = ctypes.c_void_p(buf.data_ptr())
+            timed("fill", f"zero fill {mb} MiB (dfdx_rocm_memset_zero)",
+                  lambda: dev._check(dev.lib.dfdx_rocm_memset_zero(dev.ctx, ptr, ctypes.c_size_t(nbytes))), 0, nbytes, "zero_fill_kernel")
+            timed("fill", f"zero fill {mb} MiB (torch zero_, for comparison)", lambda: buf.zero_(), 0, nbytes, "torch fill")
+            del buf
 
     # ---- vec.mat / mat.vec: HBM roofline ------------------------------------------------------------------------
     if want("gemv"):

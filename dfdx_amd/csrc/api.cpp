@@ -229,7 +229,7 @@ int dfdx_rocm_alloc(dfdx_rocm_ctx *ctx, size_t bytes, int zeroed, void **out) {
     void *p = nullptr;
     HIP_TRY(hipMalloc(&p, bytes));
     if (zeroed) {
-        hipError_t e = hipMemsetAsync(p, 0, bytes, ctx->stream);
+        hipError_t e = launch_zero_fill(p, bytes, ctx->compute_units, ctx->stream);
         if (e != hipSuccess) {
             (void)hipFree(p);
             return (int)e;
@@ -250,7 +250,7 @@ int dfdx_rocm_free(dfdx_rocm_ctx *ctx, void *ptr) {
 int dfdx_rocm_memset_zero(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes) {
     if (int e = bind(ctx)) return e;
     if (!ptr && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
-    if (bytes) HIP_TRY(hipMemsetAsync(ptr, 0, bytes, ctx->stream));
+    if (bytes) HIP_TRY(launch_zero_fill(ptr, bytes, ctx->compute_units, ctx->stream));
     return DFDX_ROCM_OK;
 }
 

@@ -36,5 +36,7 @@ int bind(dfdx_rocm_ctx *ctx);
 int ensure_workspace(dfdx_rocm_ctx *ctx, size_t bytes);
 // Same for the conv2d patch buffer.
 int ensure_patches(dfdx_rocm_ctx *ctx, size_t bytes);
+// Clears `bytes` bytes at `ptr` (any alignment) with a fill kernel on `stream`.
+hipError_t launch_zero_fill(void *ptr, size_t bytes, int compute_units, hipStream_t stream);
 
 }  // namespace dfdx_rocm

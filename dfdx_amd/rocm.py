@@ -202,8 +202,14 @@ class Rocm:
         torch = self._torch
         shape = tuple(shape)
         n = int(np.prod(shape, dtype=np.int64)) if numel_storage is None else numel_storage
-        raw = torch.zeros(max(n * ITEMSIZE[dtype], 16), dtype=torch.uint8, device=self.device)
+        raw = self._zeroed_bytes(max(n * ITEMSIZE[dtype], 16))
         return View(raw, dtype, shape, _row_major(shape) if strides is None else tuple(strides))
+
+    def _zeroed_bytes(self, nbytes: int):
+        """Device memory from torch's allocator, cleared by the library's own fill kernel (``dfdx_rocm_memset_zero``)."""
+        raw = self._torch.empty(nbytes, dtype=self._torch.uint8, device=self.device)
+        self._check(self.lib.dfdx_rocm_memset_zero(self.ctx, ctypes.c_void_p(raw.data_ptr()), ctypes.c_size_t(nbytes)))
+        return raw
 
     def empty(self, dtype: str, shape) -> View:
         """Uninitialised storage for an output that a forward kernel overwrites (``alloc_empty``,
@@ -215,7 +221,7 @@ class Rocm:
 
     def zeros_like_storage(self, v: View) -> View:
         """A gradient buffer for ``v``: zero-filled, same physical length, same strides (gradients.rs:53-58)."""
-        raw = self._torch.zeros_like(v.storage)
+        raw = self._zeroed_bytes(v.storage.numel())
         return View(raw, v.dtype, v.shape, v.strides, v.offset)
 
     def to_host(self, v: View) -> np.ndarray:
