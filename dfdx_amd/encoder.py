@@ -6,8 +6,9 @@
     Linear / LayerNorm1D / ResidualAdd   linear.rs:82-89, layer_norm1d.rs:87-91, residual_add.rs:38-45
 
 The forward keeps what the reference's tape would keep (the inputs of every op); the backward walks the ops in
-reverse, each gradient buffer zero-filled when it is first needed and accumulated into after that, as
-``Gradients::get_or_alloc_mut`` does (dfdx-core/src/tensor/gradients.rs:53-58).  The multiplication by 1/sqrt(head
+reverse; every gradient buffer starts zero-filled and is accumulated into, as with
+``Gradients::get_or_alloc_mut`` (dfdx-core/src/tensor/gradients.rs:53-58) -- here all of a pass's buffers are carved
+from one allocation that a single fill launch clears.  The multiplication by 1/sqrt(head
 dim) between q.k^T and the softmax (multi_head_attention.rs:133-134) is folded into the softmax kernel.
 """
 from __future__ import annotations
@@ -63,34 +64,28 @@ class EncoderBlock:
     def backward(self, saved: dict, grad_out: View) -> Tuple[Dict[str, View], View]:
         """grad_out: d(loss)/d(out), contiguous like the output.  Returns ({parameter: gradient}, d(loss)/d(x))."""
         dev, p, s = self.dev, self.p, saved
-        z = lambda like: dev.zeros(like.dtype, like.shape)
-        grads = {n: z(p[n]) for n in PARAMS}
-        x, n1, tok = s["x"], s["n1"], s["tok"]
-        gh2 = z(s["h2"])
+        x, n1, tok, tokens, probs = s["x"], s["n1"], s["tok"], s["tokens"], s["probs"]
+        qv, kv, vv = s["qv"], s["kv"], s["vv"]
+        # every gradient buffer of the pass, zero-filled by one launch (one allocation, pieces aligned to 256 B)
+        acts = dict(gh2=s["h2"], gf2=s["h2"], gn1=n1, gr1=s["r1"], gf1=s["f1"], gh1=s["h1"], gattn=s["h1"], gx=x, gtok=tok,
+                    gtokens=tokens, gp=probs, gscores=probs, gq=x, gk=x, gv=x)   # gq, gk, gv: laid out like the q, k, v storages
+        bufs = dev.zeros_many([p[n] for n in PARAMS] + list(acts.values()))
+        grads = dict(zip(PARAMS, bufs[:len(PARAMS)]))
+        g = dict(zip(acts, bufs[len(PARAMS):]))
+        gh2, gf2, gn1, gr1, gf1, gh1, gattn, gx = (g[k] for k in ("gh2", "gf2", "gn1", "gr1", "gf1", "gh1", "gattn", "gx"))
+        gtok, gtokens, gp, gscores, gq, gk, gv = (g[k] for k in ("gtok", "gtokens", "gp", "gscores", "gq", "gk", "gv"))
         dev.layer_norm_backward(s["h2"], p["g2"], gh2, grads["g2"], grads["be2"], grad_out)
-        gf2, gn1 = z(s["h2"]), z(n1)
         dev.add_backward(gf2, gn1, gh2)            # h2 = f2 + n1
-        gr1 = z(s["r1"])
         dev.linear_backward(s["r1"], gr1, p["w2"], grads["w2"], grads["b2"], gf2)
-        gf1 = z(s["f1"])
         dev.relu_backward(s["f1"], gf1, gr1)
         dev.linear_backward(n1, gn1, p["w1"], grads["w1"], grads["b1"], gf1)
-        gh1 = z(s["h1"])
         dev.layer_norm_backward(s["h1"], p["g1"], gh1, grads["g1"], grads["be1"], gn1)
-        gattn, gx = z(s["h1"]), z(x)
         dev.add_backward(gattn, gx, gh1)           # h1 = attn + x
-        gtok = z(tok)
         dev.linear_backward(tok, gtok, p["wo"], grads["wo"], grads["bo"], gattn)
-        tokens = s["tokens"]
-        gtokens = z(tokens)
         dev.reshape_backward(tokens.permute(0, 2, 1, 3), gtokens, gtok)
-        probs, qv, kv, vv = s["probs"], s["qv"], s["kv"], s["vv"]
-        gp = z(probs)
-        gq, gk, gv = (dev.zeros(x.dtype, x.shape) for _ in range(3))     # laid out like the q, k, v storages
         dev.backward(probs, gp, vv, gv, gtokens)
-        gscores = z(probs)
         dev.softmax_backward(probs, gscores, gp, s["scale"])
         dev.backward(qv, gq, kv, gk, gscores)
-        for w, b, g in (("wq", "bq", gq), ("wk", "bk", gk), ("wv", "bv", gv)):   # x feeds three Linears: one buffer
-            dev.linear_backward(x, gx, p[w], grads[w], grads[b], g)
+        for w, b, gg in (("wq", "bq", gq), ("wk", "bk", gk), ("wv", "bv", gv)):   # x feeds three Linears: one buffer
+            dev.linear_backward(x, gx, p[w], grads[w], grads[b], gg)
         return grads, gx

@@ -205,6 +205,19 @@ class Rocm:
         raw = self._zeroed_bytes(max(n * ITEMSIZE[dtype], 16))
         return View(raw, dtype, shape, _row_major(shape) if strides is None else tuple(strides))
 
+    def zeros_many(self, likes) -> list:
+        """Zero-filled storages for several tensors at once: one allocation, ONE fill launch, each view on its own
+        256 B-aligned piece.  ``likes`` are Views whose dtype / shape give the sizes (contiguous row-major results).
+        What a pooling allocator behind ``try_alloc_grad`` would do for the gradient buffers of one backward pass:
+        small fills are launch-bound (3.5 us for 2 MiB), one large fill runs at the HBM write rate."""
+        sizes = [max(int(np.prod(v.shape, dtype=np.int64)) * ITEMSIZE[v.dtype], 16) for v in likes]
+        offs, total = [], 0
+        for n in sizes:
+            offs.append(total)
+            total += (n + 255) // 256 * 256
+        arena = self._zeroed_bytes(max(total, 16))
+        return [View(arena[o:o + n], v.dtype, tuple(v.shape), _row_major(tuple(v.shape))) for v, o, n in zip(likes, offs, sizes)]
+
     def _zeroed_bytes(self, nbytes: int):
         """Device memory from torch's allocator, cleared by the library's own fill kernel (``dfdx_rocm_memset_zero``)."""
         raw = self._torch.empty(nbytes, dtype=self._torch.uint8, device=self.device)
