@@ -49,6 +49,68 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, int
     }
 }
 
+// 16-bit outputs whose rows are 16 B-aligned: one thread owns 8 consecutive columns of one row -- two 16 B loads per
+// split, requested four splits at a time, the old C values (beta = 1) requested before the first partial arrives, one
+// 16 B store.  Same order of additions per element as the general kernel: splits ascending, row bias, column bias, old C.
+template <typename T> struct Bits16;
+template <> struct Bits16<_Float16> {
+    static __device__ __forceinline__ float widen(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+    static __device__ __forceinline__ uint16_t narrow(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+};
+template <> struct Bits16<__bf16> {
+    static __device__ __forceinline__ float widen(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+    static __device__ __forceinline__ uint16_t narrow(float v) {
+        uint32_t x = __float_as_uint(v);
+        return ((x & 0x7fffffffu) > 0x7f800000u) ? (uint16_t)((x >> 16) | 0x40u) : (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
+    }
+};
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T>
+__global__ __launch_bounds__(256) void splitk_reduce16_kernel(const float *ws, int splits, int64_t ws_ld, int64_t ws_split_stride,
+                                                              uint16_t *c, int64_t c_rs, int m, int n, int accumulate,
+                                                              int bias_mode, const uint16_t *bias) {
+    const int col = (blockIdx.x * 64 + threadIdx.x % 64) * 8;
+    const int row = blockIdx.y * 4 + threadIdx.x / 64;
+    if (row >= m || col >= n) return;   // n is a multiple of 8: a thread's 8 columns are all inside or all outside
+    const float *src = ws + (int64_t)row * ws_ld + col;
+    uint16_t *dst = c + (int64_t)row * c_rs + col;
+    u32x4 old = {0u, 0u, 0u, 0u}, cb = {0u, 0u, 0u, 0u};
+    if (accumulate) old = *(const u32x4 *)dst;
+    if (bias_mode == BIAS_PER_COL) cb = *(const u32x4 *)(bias + col);
+    f32x4 lo = *(const f32x4 *)src, hi = *(const f32x4 *)(src + 4);
+    int s = 1;
+    for (; s + 3 < splits; s += 4) {
+        f32x4 a[4], b[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            a[u] = *(const f32x4 *)(src + (s + u) * ws_split_stride);
+            b[u] = *(const f32x4 *)(src + (s + u) * ws_split_stride + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            lo += a[u];
+            hi += b[u];
+        }
+    }
+    for (; s < splits; s++) {
+        lo += *(const f32x4 *)(src + s * ws_split_stride);
+        hi += *(const f32x4 *)(src + s * ws_split_stride + 4);
+    }
+    const float rb = (bias_mode == BIAS_PER_ROW) ? Bits16<T>::widen(bias[row]) : 0.0f;
+    u32x4 out;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        float x = (e < 4 ? lo[e] : hi[e - 4]) + rb;
+        const int sh = (e & 1) * 16;
+        if (bias_mode == BIAS_PER_COL) x += Bits16<T>::widen((uint16_t)(cb[e / 2] >> sh));
+        if (accumulate) x += Bits16<T>::widen((uint16_t)(old[e / 2] >> sh));
+        const uint32_t bits = Bits16<T>::narrow(x);
+        out[e / 2] = (e & 1) ? (out[e / 2] | (bits << 16)) : bits;
+    }
+    *(u32x4 *)dst = out;
+}
+
 }  // namespace
 
 // C of `p` must have unit column stride and no batch (the planner only splits such problems).
@@ -56,6 +118,20 @@ hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_
     dim3 grid((unsigned)((p.n + 255) / 256), (unsigned)((p.m + 3) / 4)), block(256);
     const int64_t c_rs = p.m == 1 ? p.n : p.c_rs;
     const int bias_mode = p.bias ? p.bias_mode : BIAS_NONE;
+    const bool is16 = p.dtype == DT_F16 || p.dtype == DT_BF16;
+    if (is16 && p.n % 8 == 0 && c_rs % 8 == 0 && ws_ld % 4 == 0 && ws_split_stride % 4 == 0 && ((uintptr_t)p.c & 15u) == 0 &&
+        ((uintptr_t)p.workspace & 15u) == 0 && (bias_mode != BIAS_PER_COL || ((uintptr_t)p.bias & 15u) == 0)) {
+        dim3 grid16((unsigned)((p.n + 511) / 512), (unsigned)((p.m + 3) / 4));
+        if (p.dtype == DT_F16)
+            splitk_reduce16_kernel<_Float16><<<grid16, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (uint16_t *)p.c,
+                                                                            c_rs, (int)p.m, (int)p.n, p.accumulate, bias_mode,
+                                                                            (const uint16_t *)p.bias);
+        else
+            splitk_reduce16_kernel<__bf16><<<grid16, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (uint16_t *)p.c,
+                                                                          c_rs, (int)p.m, (int)p.n, p.accumulate, bias_mode,
+                                                                          (const uint16_t *)p.bias);
+        return hipGetLastError();
+    }
     switch (p.dtype) {
     case DT_F32:
         splitk_reduce_kernel<float><<<grid, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (float *)p.c, c_rs,
