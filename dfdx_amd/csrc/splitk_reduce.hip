@@ -30,7 +30,7 @@ template <> struct Cvt<__bf16> {
 template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, int splits, int64_t ws_ld, int64_t ws_split_stride,
                                                             T *c, int64_t c_rs, int m, int n, int accumulate, int bias_mode,
-                                                            const T *bias) {
+                                                            const T *bias, int vec4) {
     const int col = (blockIdx.x * 64 + threadIdx.x % 64) * 4;
     const int row = blockIdx.y * 4 + threadIdx.x / 64;
     if (row >= m || col >= n) return;
@@ -39,6 +39,15 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, int
     for (int s = 1; s < splits; s++) v += *(const f32x4 *)(src + s * ws_split_stride);
     T *dst = c + (int64_t)row * c_rs + col;
     const float rb = (bias_mode == BIAS_PER_ROW) ? Cvt<T>::load(bias + row) : 0.0f;
+    if constexpr (sizeof(T) == 4) {
+        if (vec4 && col + 3 < n) {   // f32 rows aligned to 16 B: one load of the old values, one store
+            f32x4 x = v + rb;
+            if (bias_mode == BIAS_PER_COL) x += *(const f32x4 *)(bias + col);
+            if (accumulate) x += *(const f32x4 *)dst;
+            *(f32x4 *)dst = x;
+            return;
+        }
+    }
 #pragma unroll
     for (int e = 0; e < 4; e++) {
         if (col + e >= n) break;
@@ -132,19 +141,21 @@ hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_
                                                                           (const uint16_t *)p.bias);
         return hipGetLastError();
     }
+    const int vec4 = p.dtype == DT_F32 && c_rs % 4 == 0 && ((uintptr_t)p.c & 15u) == 0 && ws_ld % 4 == 0 && ws_split_stride % 4 == 0 &&
+                     ((uintptr_t)p.workspace & 15u) == 0 && (bias_mode != BIAS_PER_COL || ((uintptr_t)p.bias & 15u) == 0);
     switch (p.dtype) {
     case DT_F32:
         splitk_reduce_kernel<float><<<grid, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (float *)p.c, c_rs,
-                                                                 (int)p.m, (int)p.n, p.accumulate, bias_mode, (const float *)p.bias);
+                                                                 (int)p.m, (int)p.n, p.accumulate, bias_mode, (const float *)p.bias, vec4);
         break;
     case DT_F16:
         splitk_reduce_kernel<_Float16><<<grid, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (_Float16 *)p.c,
                                                                     c_rs, (int)p.m, (int)p.n, p.accumulate, bias_mode,
-                                                                    (const _Float16 *)p.bias);
+                                                                    (const _Float16 *)p.bias, 0);
         break;
     case DT_BF16:
         splitk_reduce_kernel<__bf16><<<grid, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (__bf16 *)p.c, c_rs,
-                                                                  (int)p.m, (int)p.n, p.accumulate, bias_mode, (const __bf16 *)p.bias);
+                                                                  (int)p.m, (int)p.n, p.accumulate, bias_mode, (const __bf16 *)p.bias, 0);
         break;
     default: return hipErrorInvalidValue;
     }
