@@ -76,7 +76,9 @@ int dfdx_rocm_device_info(dfdx_rocm_ctx *ctx, char *name, size_t name_len, int *
  * What `Storage::try_alloc_len` (zero-filled; cuda/device.rs:259-266),
  * `alloc_empty` (cuda/device.rs:97-106), `CopySlice` / `tensor_to_vec`
  * (tensor/storage_traits.rs:93-96) and `Synchronize` (storage_traits.rs:31-39)
- * need from the device. */
+ * need from the device.  The zero fill (`zeroed` != 0, `dfdx_rocm_memset_zero`) is a
+ * kernel launch on the context's stream, not a memset node: stream-ordered like every
+ * other call, any alignment and length, and safe to record into a captured graph. */
 int dfdx_rocm_alloc(dfdx_rocm_ctx *ctx, size_t bytes, int zeroed, void **out);
 int dfdx_rocm_free(dfdx_rocm_ctx *ctx, void *ptr);
 int dfdx_rocm_memset_zero(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes);
