@@ -21,7 +21,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
-    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv")
+    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (and torch: vendor-library cross-check, only on request)")
     args = ap.parse_args()
     import torch
     from dfdx_amd import Rocm
@@ -203,6 +203,43 @@ def main():
                   lambda: dev._check(dev.lib.dfdx_rocm_memset_zero(dev.ctx, ptr, ctypes.c_size_t(nbytes))), 0, nbytes, "zero_fill_kernel")
             timed("fill", f"zero fill {mb} MiB (torch zero_, for comparison)", lambda: buf.zero_(), 0, nbytes, "torch fill")
             del buf
+
+    # ---- the vendor library on the same shapes (torch.matmul = hipBLASLt / rocBLAS), for orientation only ---------
+    if "torch" in only:   # not part of the default run: a cross-check, never a code path of the library
+        def pair(name, dt, fn_ours_desc, fn_torch, flop):
+            gemm("torch", name + " (this library)", fn_ours_desc, flop, 0)
+            timed("torch", name + " (torch.matmul)", fn_torch, flop, 0, "vendor library")
+
+        n = 4096
+        for dt in ("f16", "bf16", "f32"):
+            a, b, c = rnd((n, n), dt), rnd((n, n), dt), zeros((n, n), dt)
+            pair(f"4096^3 {dt} A.B", dt, dev.gemm_desc(dt, n, n, n, P(a), (n, 1), P(b), (n, 1), P(c), (n, 1)),
+                 lambda: torch.matmul(a, b, out=c), 2 * n ** 3)
+        dt = "f16"
+        x, w, go = rnd((16384, 1024), dt), rnd((1024, 1024), dt, 0.03), rnd((16384, 1024), dt)
+        y, gw = zeros((16384, 1024), dt), zeros((1024, 1024), dt)
+        pair("c3 fwd 16384x1024x1024 NN f16", dt, dev.gemm_desc(dt, 16384, 1024, 1024, P(x), (1024, 1), P(w), (1024, 1), P(y), (1024, 1)),
+             lambda: torch.matmul(x, w, out=y), 2 * 16384 * 1024 * 1024)
+        pair("c3 dW 1024x16384x1024 TN f16 (beta = 1 here, overwrite in torch)", dt,
+             dev.gemm_desc(dt, 1024, 16384, 1024, P(x), (1, 1024), P(go), (1024, 1), P(gw), (1024, 1), accumulate=True),
+             lambda: torch.matmul(x.t(), go, out=gw), 2 * 16384 * 1024 * 1024)
+        dt, T = "bf16", 8192
+        x, w, go = rnd((T, 1024), dt), rnd((4096, 1024), dt, 0.02), rnd((T, 4096), dt)
+        y, gw = zeros((T, 4096), dt), zeros((4096, 1024), dt)
+        pair("c5 ff1 fwd 8192x1024x4096 NT bf16", dt, dev.gemm_desc(dt, T, 1024, 4096, P(x), (1024, 1), P(w), (1, 1024), P(y), (4096, 1)),
+             lambda: torch.matmul(x, w.t(), out=y), 2 * T * 1024 * 4096)
+        pair("c5 ff1 dW TN col-major C bf16 (beta = 1 here, overwrite in torch)", dt,
+             dev.gemm_desc(dt, 1024, T, 4096, P(x), (1, 1024), P(go), (4096, 1), P(gw), (1, 1024), accumulate=True),
+             lambda: torch.matmul(go.t(), x, out=gw), 2 * T * 1024 * 4096)
+        dt, nb, S, D = "f16", 128, 1024, 64
+        q, k_, pm = rnd((nb, S, D), dt), rnd((nb, S, D), dt), rnd((nb, S, S), dt, 0.03)
+        sc, o = zeros((nb, S, S), dt), zeros((nb, S, D), dt)
+        pair("c4 scores Q.K^T 128 x 1024x64x1024 f16", dt,
+             dev.gemm_desc(dt, S, D, S, P(q), (D, 1), P(k_), (1, D), P(sc), (S, 1), batch=(nb, 1), a_batch=(S * D, 0), b_batch=(S * D, 0), c_batch=(S * S, 0)),
+             lambda: torch.bmm(q, k_.transpose(1, 2), out=sc), 2 * nb * S * S * D)
+        pair("c4 out P.V 128 x 1024x1024x64 f16", dt,
+             dev.gemm_desc(dt, S, S, D, P(pm), (S, 1), P(q), (D, 1), P(o), (D, 1), batch=(nb, 1), a_batch=(S * S, 0), b_batch=(S * D, 0), c_batch=(S * D, 0)),
+             lambda: torch.bmm(pm, q, out=o), 2 * nb * S * S * D)
 
     # ---- vec.mat / mat.vec: HBM roofline ------------------------------------------------------------------------
     if want("gemv"):

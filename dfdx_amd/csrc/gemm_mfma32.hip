@@ -61,6 +61,11 @@ template <int ROWS, int BK, int NT, bool KC> struct Loader {
             else regs[i] = ldg4(g + r * ld + ch * 4, ch * 4 < rows_left && r < k_left);
         }
     }
+    __device__ __forceinline__ void store_piece(float *lds, int tid, int i) const {
+        const int cid = i * NT + tid;
+        const int r = cid / CPR, ch = cid % CPR;
+        *(f32x4 *)(lds + r * LDS_ROW + ch * 4) = regs[i];
+    }
     __device__ __forceinline__ void store(float *lds, int tid) const {
 #pragma unroll
         for (int i = 0; i < LOADS; i++) {
@@ -147,53 +152,103 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
     const float *a_frag0 = A_KC ? As + (wm0 + l32) * LA::LDS_ROW + lh * 4 : As + (lh * 4) * LA::LDS_ROW + wm0 + l32;
     const float *b_frag0 = B_KC ? Bs + (wn0 + l32) * LB::LDS_ROW + lh * 4 : Bs + (lh * 4) * LB::LDS_ROW + wn0 + l32;
 
+    // One k step of 8 = 4 MFMA k pairs per tile; a lane's fragment values of a k step: 4 floats per 32-row tile.
+    constexpr int KS = BK / 8;
+    static_assert(KS >= 2, "the loop below keeps the first and the last k step of a tile in registers");
+    auto read_frags = [&](const float *af_base, const float *bf_base, int ks, float(&af)[TM][4], float(&bf)[TN][4]) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            if constexpr (A_KC) {
+                const f32x4 v = *(const f32x4 *)(af_base + i * 32 * LA::LDS_ROW + ks * 8);
+#pragma unroll
+                for (int e = 0; e < 4; e++) af[i][e] = v[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) af[i][e] = af_base[(ks * 8 + e) * LA::LDS_ROW + i * 32];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            if constexpr (B_KC) {
+                const f32x4 v = *(const f32x4 *)(bf_base + j * 32 * LB::LDS_ROW + ks * 8);
+#pragma unroll
+                for (int e = 0; e < 4; e++) bf[j][e] = v[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) bf[j][e] = bf_base[(ks * 8 + e) * LB::LDS_ROW + j * 32];
+            }
+        }
+    };
+    auto mma = [&](const float(&af)[TM][4], const float(&bf)[TN][4]) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j][e], af[i][e], acc[i][j], 0, 0, 0);
+    };
+
+    // The barrier that hands a stage over sits in FRONT of the tile's last k step: its fragments are already in
+    // registers, so every wave crosses the barrier with a full group of MFMAs still to issue, and the first fragments
+    // of the next tile are requested from LDS before that group -- neither the barrier skew nor the LDS latency
+    // leaves the matrix core idle.
+    float af_first[TM][4], bf_first[TN][4];
+    if (iters > 0) read_frags(a_frag0, b_frag0, 0, af_first, bf_first);
+    if (iters > 1) {   // the second tile waits in registers while the first is computed
+        la.load(a_tile(it0 + 1), p.lda, rows_left, k_left(it0 + 1), tid);
+        lb.load(b_tile(it0 + 1), p.ldb, cols_left, k_left(it0 + 1), tid);
+    }
     for (int it = 0; it < iters; it++) {
         const int cur = it & 1;
         const bool more = it + 1 < iters;
-        if (more) {
-            la.load(a_tile(it0 + it + 1), p.lda, rows_left, k_left(it0 + it + 1), tid);
-            lb.load(b_tile(it0 + it + 1), p.ldb, cols_left, k_left(it0 + it + 1), tid);
-        }
         const float *af_base = a_frag0 + cur * LA::LDS_SIZE;
         const float *bf_base = b_frag0 + cur * LB::LDS_SIZE;
-#pragma unroll
-        for (int ks = 0; ks < BK / 8; ks++) {
-            float af[TM][4], bf[TN][4];
-#pragma unroll
-            for (int i = 0; i < TM; i++) {
-                if constexpr (A_KC) {
-                    const f32x4 v = *(const f32x4 *)(af_base + i * 32 * LA::LDS_ROW + ks * 8);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) af[i][e] = v[e];
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) af[i][e] = af_base[(ks * 8 + e) * LA::LDS_ROW + i * 32];
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                if constexpr (B_KC) {
-                    const f32x4 v = *(const f32x4 *)(bf_base + j * 32 * LB::LDS_ROW + ks * 8);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) bf[j][e] = v[e];
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) bf[j][e] = bf_base[(ks * 8 + e) * LB::LDS_ROW + j * 32];
-                }
-            }
+        float af_last[TM][4], bf_last[TN][4];
+        {
+            // The next tile's registers (requested during the previous tile) go to LDS one 16 B piece at a time
+            // BETWEEN the MFMAs of the first k step: every store issues in the shadow of an MFMA instead of in a
+            // block in front of the barrier, where the matrix core would sit idle; the registers are then free for the
+            // tile after next, which has the rest of this tile to arrive.  Only the stores are conditional: accumulators
+            // written under a branch make the register allocator copy them.
+            float *an = As + (cur ^ 1) * LA::LDS_SIZE, *bn = Bs + (cur ^ 1) * LB::LDS_SIZE;
+            constexpr int M = 4 * TM * TN, S = LA::LOADS + LB::LOADS;
 #pragma unroll
             for (int e = 0; e < 4; e++)
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
-                    for (int j = 0; j < TN; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j][e], af[i][e], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < TN; j++) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf_first[j][e], af_first[i][e], acc[i][j], 0, 0, 0);
+                        const int n = (e * TM + i) * TN + j;
+                        const int before = n * S / M, after = (n + 1) * S / M;
+#pragma unroll
+                        for (int q = 0; q < S; q++)
+                            if (q >= before && q < after && more) {
+                                if (q < LA::LOADS) la.store_piece(an, tid, q);
+                                else lb.store_piece(bn, tid, q - LA::LOADS);
+                            }
+                    }
         }
-        if (more) {
-            la.store(As + (cur ^ 1) * LA::LDS_SIZE, tid);
-            lb.store(Bs + (cur ^ 1) * LB::LDS_SIZE, tid);
+        if (it + 2 < iters) {
+            la.load(a_tile(it0 + it + 2), p.lda, rows_left, k_left(it0 + it + 2), tid);
+            lb.load(b_tile(it0 + it + 2), p.ldb, cols_left, k_left(it0 + it + 2), tid);
+        }
+#pragma unroll
+        for (int ks = 1; ks < KS; ks++) {
+            if (ks < KS - 1) {
+                float af[TM][4], bf[TN][4];
+                read_frags(af_base, bf_base, ks, af, bf);
+                mma(af, bf);
+            } else {
+                read_frags(af_base, bf_base, ks, af_last, bf_last);
+            }
         }
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) read_frags(a_frag0 + (cur ^ 1) * LA::LDS_SIZE, b_frag0 + (cur ^ 1) * LB::LDS_SIZE, 0, af_first, bf_first);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(af_last, bf_last);
     }
 
     // ---- epilogue: lane holds m = l32 (per tile), n = 8g + 4*lh + 0..3 --------
