@@ -37,6 +37,29 @@ int ensure_patches(dfdx_rocm_ctx *ctx, size_t bytes) { return grow(ctx, &ctx->pa
 
 namespace {
 
+// Scratch of dfdx_rocm_gemm_noalloc: partial sums of split reductions for callers that may not allocate.  Every device
+// the library runs on holds its own copy of this array, at its own address, until the process ends.  In host code the
+// array's NAME is only a handle for hipGetSymbolAddress: the address a kernel may use is looked up once per device in
+// dfdx_rocm_create (with that device current) and kept in `scratch_of_device` / the context.
+__device__ __align__(256) __attribute__((used)) static unsigned char scratch[DFDX_ROCM_NOALLOC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mu;
+void *scratch_of_device[kMaxDevices];  // guarded by scratch_mu
+
+// The calling thread's current device must be `ordinal`.
+int scratch_address(int ordinal, void **out) {
+    if (ordinal < 0 || ordinal >= kMaxDevices) return DFDX_ROCM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lock(scratch_mu);
+    if (!scratch_of_device[ordinal]) {
+        void *ptr = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return (int)hipErrorInvalidSymbol;
+        scratch_of_device[ordinal] = ptr;
+    }
+    *out = scratch_of_device[ordinal];
+    return DFDX_ROCM_OK;
+}
+
 // Validates `d` and produces the canonical problem (row-major C whenever the view allows it).
 int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
     if (!d) return DFDX_ROCM_ERR_INVALID_ARG;
@@ -133,7 +156,21 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
     return DFDX_ROCM_OK;
 }
 
-int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan) {
+// Where the partial sums of a split plan go: the context's own buffer (grown on demand), or -- `static_scratch` --
+// the device's fixed scratch array, in which case nothing is allocated and a plan that needs more is refused.
+int partials_buffer(dfdx_rocm_ctx *ctx, size_t need, bool static_scratch, float **out) {
+    if (static_scratch) {
+        if (need > (size_t)DFDX_ROCM_NOALLOC_SCRATCH_BYTES) return DFDX_ROCM_ERR_SCRATCH_TOO_SMALL;
+        if (!ctx->static_scratch) return DFDX_ROCM_ERR_INVALID_ARG;
+        *out = (float *)ctx->static_scratch;
+        return DFDX_ROCM_OK;
+    }
+    if (int rc = ensure_workspace(ctx, need)) return rc;
+    *out = (float *)ctx->workspace;
+    return DFDX_ROCM_OK;
+}
+
+int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan, bool static_scratch = false) {
     CtxLock lock(ctx->mu);  // a split plan is two launches around the shared workspace
     GemmProblem p = problem;
     p.splits = 1;
@@ -142,14 +179,12 @@ int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan) {
     if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1) {
         const size_t need = p.dtype == DT_F32 ? mfma32_workspace_bytes(p, plan.variant, plan.splits)
                                               : mfma16dma_workspace_bytes(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
-        if (int rc = ensure_workspace(ctx, need)) return rc;
+        if (int rc = partials_buffer(ctx, need, static_scratch, &p.workspace)) return rc;
         p.splits = plan.splits;
-        p.workspace = (float *)ctx->workspace;
     }
     if (plan.kernel == DFDX_ROCM_KERNEL_GEMV) {
         if (const size_t need = gemv_workspace_bytes(p)) {
-            if (int rc = ensure_workspace(ctx, need)) return rc;
-            p.workspace = (float *)ctx->workspace;
+            if (int rc = partials_buffer(ctx, need, static_scratch, &p.workspace)) return rc;
         }
     }
     hipError_t e;
@@ -177,8 +212,11 @@ int dfdx_rocm_create(int ordinal, void *stream, dfdx_rocm_ctx **out) {
     HIP_TRY(hipGetDeviceProperties(&prop, ordinal));
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) return DFDX_ROCM_ERR_NO_DEVICE;  // code objects are gfx950 only
     HIP_TRY(hipSetDevice(ordinal));
+    void *static_scratch = nullptr;
+    if (int e = scratch_address(ordinal, &static_scratch)) return e;
     dfdx_rocm_ctx *ctx = new (std::nothrow) dfdx_rocm_ctx();
     if (!ctx) return (int)hipErrorOutOfMemory;
+    ctx->static_scratch = static_scratch;
     ctx->device = ordinal;
     ctx->stream = (hipStream_t)stream;
     ctx->compute_units = prop.multiProcessorCount;
@@ -207,6 +245,8 @@ const char *dfdx_rocm_strerror(int code) {
     case DFDX_ROCM_ERR_UNSUPPORTED: return "dfdx_rocm: no kernel for this request";
     case DFDX_ROCM_ERR_NO_DEVICE: return "dfdx_rocm: no usable gfx950 device";
     case DFDX_ROCM_ERR_ALIASED_OUTPUT: return "dfdx_rocm: output view aliases itself (zero stride)";
+    case DFDX_ROCM_ERR_SCRATCH_TOO_SMALL:
+        return "dfdx_rocm: the split reduction of this product needs more than the fixed scratch of the no-allocation entry";
     default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -295,6 +335,16 @@ int dfdx_rocm_gemm(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc) {
     Plan plan;
     if (int e = make_plan(ctx, desc, p, &plan)) return e;
     return run_plan(ctx, p, plan);
+}
+
+int dfdx_rocm_gemm_noalloc(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc) {
+    if (int e = bind(ctx)) return e;
+    GemmProblem p;
+    if (int e = make_problem(desc, &p)) return e;
+    if (p.m == 0) return DFDX_ROCM_OK;
+    Plan plan;
+    if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    return run_plan(ctx, p, plan, /*static_scratch=*/true);
 }
 
 int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int *kernel, int *variant, char *name,

@@ -16,6 +16,7 @@ struct dfdx_rocm_ctx {
     std::recursive_mutex mu;
     void *workspace = nullptr;  // partial sums of split reductions; grown on demand, owned by the context
     size_t workspace_bytes = 0;
+    void *static_scratch = nullptr;  // this device's copy of the fixed scratch array of dfdx_rocm_gemm_noalloc (never freed)
     void *patches = nullptr;  // unfolded images of conv2d (alive across the GEMMs that may regrow `workspace`)
     size_t patches_bytes = 0;
 };

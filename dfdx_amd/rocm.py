@@ -28,6 +28,8 @@ ITEMSIZE = {"f32": 4, "f16": 2, "bf16": 2, "f64": 8}
 NP_DTYPES = {"f32": np.float32, "f16": np.float16, "bf16": np.uint16, "f64": np.float64}
 
 KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_GEMV = 0, 1, 2, 3
+NOALLOC_SCRATCH_BYTES = 32 << 20   # DFDX_ROCM_NOALLOC_SCRATCH_BYTES
+ERR_SCRATCH_TOO_SMALL = -5
 
 
 class RocmError(RuntimeError):
@@ -70,7 +72,7 @@ _lib = None
 EXPORTS = [
     "dfdx_rocm_create", "dfdx_rocm_destroy", "dfdx_rocm_strerror", "dfdx_rocm_device_info",
     "dfdx_rocm_alloc", "dfdx_rocm_free", "dfdx_rocm_memset_zero", "dfdx_rocm_copy_h2d", "dfdx_rocm_copy_d2h",
-    "dfdx_rocm_copy_d2d", "dfdx_rocm_synchronize", "dfdx_rocm_gemm", "dfdx_rocm_gemm_plan",
+    "dfdx_rocm_copy_d2d", "dfdx_rocm_synchronize", "dfdx_rocm_gemm", "dfdx_rocm_gemm_noalloc", "dfdx_rocm_gemm_plan",
     "dfdx_rocm_mfma_variant_count", "dfdx_rocm_gemm_time",
     "dfdx_rocm_matmat_forward", "dfdx_rocm_matmat_backward",
     "dfdx_rocm_matmat_br_forward", "dfdx_rocm_matmat_br_backward",
@@ -261,6 +263,11 @@ class Rocm:
     def gemm(self, desc: GemmDesc):
         """``MatMulImpl::matmul`` / ``Cuda::gemm[_batch]`` (cpu_kernel.rs:38-50, cuda_kernel.rs:153-237)."""
         self._check(self.lib.dfdx_rocm_gemm(self.ctx, ctypes.byref(desc)))
+
+    def gemm_noalloc(self, desc: GemmDesc):
+        """The same product with the partial sums of a split reduction in the library's fixed scratch array: allocates
+        nothing; ``RocmError`` (code -5) when the plan needs more than ``NOALLOC_SCRATCH_BYTES``."""
+        self._check(self.lib.dfdx_rocm_gemm_noalloc(self.ctx, ctypes.byref(desc)))
 
     def gemm_plan(self, desc: GemmDesc):
         kernel, variant = ctypes.c_int(), ctypes.c_int()

@@ -51,7 +51,8 @@ enum {
     DFDX_ROCM_ERR_INVALID_ARG = -1,   /* null pointer, negative size, unknown dtype ...          */
     DFDX_ROCM_ERR_UNSUPPORTED = -2,   /* valid request this build has no kernel for              */
     DFDX_ROCM_ERR_NO_DEVICE = -3,     /* no usable gfx950 device                                 */
-    DFDX_ROCM_ERR_ALIASED_OUTPUT = -4 /* output view maps several logical elements to one address */
+    DFDX_ROCM_ERR_ALIASED_OUTPUT = -4, /* output view maps several logical elements to one address */
+    DFDX_ROCM_ERR_SCRATCH_TOO_SMALL = -5 /* dfdx_rocm_gemm_noalloc: the plan needs more scratch than the fixed array holds */
 };
 
 /* Kernel families, for dfdx_rocm_gemm_desc.kernel (0 lets the library choose). */
@@ -130,6 +131,25 @@ typedef struct dfdx_rocm_gemm_desc {
 #define DFDX_ROCM_GEMM_SPLIT_K(n) (((n) & 0xff) << 8)
 
 int dfdx_rocm_gemm(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc);
+
+/* The same product for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * No counterpart in the reference (its devices allocate freely).
+ * dfdx_rocm_gemm grows a context-owned buffer on demand for the f32 partial
+ * sums of a split reduction (split-k weight gradients, k-sliced vector
+ * products); this entry point plans exactly as dfdx_rocm_gemm does -- same
+ * kernels, same bits -- but keeps those partial sums in a fixed array of
+ * DFDX_ROCM_NOALLOC_SCRATCH_BYTES that lives in the library's device image
+ * (one copy per GPU, held until the process ends) and calls no hipMalloc /
+ * hipFree or any other allocating routine.  A plan whose partial sums do not
+ * fit is refused with DFDX_ROCM_ERR_SCRATCH_TOO_SMALL before anything is
+ * launched (the caller may then lower or forbid the split through `flags`).
+ * Nothing in the array has to start at zero: every partial sum that is read
+ * has been written by the same call.  All calls on one GPU share the array,
+ * so calls that overlap on one GPU (two contexts, two streams, two threads)
+ * race; calls on one context are ordered by its stream. */
+#define DFDX_ROCM_NOALLOC_SCRATCH_BYTES (32u << 20)
+int dfdx_rocm_gemm_noalloc(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc);
 
 /* Which kernel dfdx_rocm_gemm would run for `desc`: writes the family, the
  * variant and a short name ("mfma16_256x256x64_kc_kc" ...).  No launch. */
