@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 import oracle
+from oracle import nn_ops
 from helpers import assert_within, logical, rng, row_major_strides, tolerance
 from gpu_util import announce, device
 
@@ -44,15 +45,29 @@ def test_config1_linear_512_256_f32():
     assert_within(dtype, i, host(dev, y), want.astype(np.float64), X, W, extra=ULP[dtype] * 8, what="y")
     announce("config1 backward")
     dy = upload(dev, np.ones((rows, o)), dtype)
-    gx, gw = dev.zeros_like_storage(x), dev.zeros_like_storage(wt)
-    dev.backward(x, gx, wt, gw, dy)
+    gx, gw, gb = dev.zeros_like_storage(x), dev.zeros_like_storage(w), dev.zeros_like_storage(b)
+    dev.linear_backward(x, gx, w, gw, gb, dy)   # dx, dW and db all come from the device
     wgx, wgw = np.zeros_like(x_h), np.zeros_like(w_h)
     oracle.matmat_backward(dtype, rows, i, o, x_h, x.strides, wgx, w_h, wt.strides, wgw, dev.to_host(dy))
     ones = np.ones((rows, o))
     assert_within(dtype, o, oracle.to_f64(dev.to_host(gx), dtype), wgx.astype(np.float64), ones, W, what="dx")
     assert_within(dtype, rows, oracle.to_f64(dev.to_host(gw), dtype), wgw.astype(np.float64), X, ones, what="dW")
-    # db = column sum of dy = 64 for every output feature (utilities/cpu_kernels.rs:188-200)
-    assert np.array_equal(host(dev, dy).sum(axis=0), np.full(o, float(rows)))
+    # db: the broadcast add's backward sums dy down the rows (utilities/cpu_kernels.rs:188-200); with dy = 1 every
+    # partial sum is a small integer, so the reference's row-after-row f32 order and any other order agree exactly: 64
+    want_db = nn_ops.bias_backward(dev.to_host(dy).reshape(rows, o), np.zeros(o), dtype, faithful=True)
+    got_db = oracle.to_f64(dev.to_host(gb), dtype)
+    assert np.array_equal(want_db, np.full(o, float(rows)))
+    assert np.array_equal(got_db, want_db), np.max(np.abs(got_db - want_db))
+    # a second backward with a random dy accumulates into all three (beta = 1 everywhere, db included)
+    announce("config1 backward, random dy, accumulating")
+    dy2 = upload(dev, g.standard_normal((rows, o)), dtype)
+    dev.linear_backward(x, gx, w, gw, gb, dy2)
+    oracle.matmat_backward(dtype, rows, i, o, x_h, x.strides, wgx, w_h, wt.strides, wgw, dev.to_host(dy2))
+    DY2 = host(dev, dy2)
+    assert_within(dtype, o, oracle.to_f64(dev.to_host(gx), dtype), wgx.astype(np.float64), DY2, W, extra=ULP[dtype] * 64, what="dx (2)")
+    assert_within(dtype, rows, oracle.to_f64(dev.to_host(gw), dtype), wgw.astype(np.float64), X, DY2, extra=ULP[dtype] * 256, what="dW (2)")
+    want_db = nn_ops.bias_backward(dev.to_host(dy2).reshape(rows, o), want_db, dtype, faithful=True)
+    assert_within(dtype, rows, oracle.to_f64(dev.to_host(gb), dtype), want_db, DY2, np.ones(1), extra=ULP[dtype] * 128, what="db (2)")
 
 
 # ---- config 2: 4096^3, f32 and f16, A.B / A^T.B / A.B^T ------------------------------------------
@@ -135,53 +150,56 @@ def test_config3_batched_broadcast_rhs_f16():
 
 # ---- config 4: attention-shaped Rank4, f16 ---------------------------------------------------------
 def test_config4_attention_rank4_f16():
-    """Q,K,V [8,16,1024,64]; scores = Q.K^T / 8 -> softmax (host, float64, CPU-equivalent glue:
-    softmax.rs:70-83) -> out = P.V; backward through both matmuls with dO ~ N(0,1)."""
+    """Q,K,V [8,16,1024,64]; scores = Q.K^T, P = softmax(scores / 8) (the scale folded into the device softmax:
+    multi_head_attention.rs:129-134 over softmax.rs:70-83), out = P.V; backward through both matmuls AND the softmax
+    with dO ~ N(0,1), everything on the device.  Each GEMM is compared with the oracle's MatMat driver run on that
+    GEMM's own device-produced operands for sampled (batch, head) slices -- the Batch4 driver is a loop of exactly
+    these calls (cpu_kernel.rs:432-447,461-484) --, each softmax step with the numpy restatement."""
     dev, g = device(), rng(4004)
     dtype, (B, H, S, D) = "f16", (8, 16, 1024, 64)
+    scale = 0.125
     q, k, v, d_o = (upload(dev, g.standard_normal((B, H, S, D)).astype(np.float32), dtype) for _ in range(4))
     kt = k.permute(0, 1, 3, 2)
-    announce("config4 scores")
+    announce("config4 forward: scores, softmax, P.V")
     scores = dev.forward(q, kt)
-    s_h = dev.to_host(scores)
-    q_h, k_h, v_h, do_h = (dev.to_host(t) for t in (q, k, v, d_o))
-    sample = [(0, 0), (3, 7), (7, 15)]
-    sl = lambda arr, b, h, per: arr[(b * H + h) * per:(b * H + h + 1) * per]
-    Q, K = oracle.to_f64(q_h, dtype).reshape(B, H, S, D), oracle.to_f64(k_h, dtype).reshape(B, H, S, D)
-    for b, h in sample:
-        want = oracle.matmat_forward(dtype, S, D, S, sl(q_h, b, h, S * D), (D, 1), sl(k_h, b, h, S * D), (1, D))
-        assert_within(dtype, D, oracle.to_f64(sl(s_h, b, h, S * S), dtype), oracle.to_f64(want, dtype), Q[b, h], K[b, h],
-                      extra=2 * ULP[dtype] * 64, what=f"scores[{b},{h}]")
-    # glue on the host in float64, stored back as f16 (the reference's softmax is elementwise + reductions)
-    sc = oracle.to_f64(s_h, dtype).reshape(B, H, S, S) / 8.0
-    sc -= sc.max(axis=-1, keepdims=True)
-    p64 = np.exp(sc)
-    p64 /= p64.sum(axis=-1, keepdims=True)
-    p = upload(dev, p64.astype(np.float32), dtype)
-    del sc, p64
-    announce("config4 out")
+    p = dev.softmax_forward(scores, scale)
     out = dev.forward(p, v)
-    p_h, o_h = dev.to_host(p), dev.to_host(out)
-    P, V = oracle.to_f64(p_h, dtype).reshape(B, H, S, S), oracle.to_f64(v_h, dtype).reshape(B, H, S, D)
-    for b, h in sample:
-        want = oracle.matmat_forward(dtype, S, S, D, sl(p_h, b, h, S * S), (S, 1), sl(v_h, b, h, S * D), (D, 1))
-        assert_within(dtype, S, oracle.to_f64(sl(o_h, b, h, S * D), dtype), oracle.to_f64(want, dtype), P[b, h], V[b, h],
-                      extra=2 * ULP[dtype] * 4, what=f"out[{b},{h}]")
-    announce("config4 backward of P.V")
+    announce("config4 backward: P.V, softmax, Q.K^T")
     gp, gv = dev.zeros_like_storage(p), dev.zeros_like_storage(v)
     dev.backward(p, gp, v, gv, d_o)
-    announce("config4 backward of Q.K^T")
+    gs = dev.zeros_like_storage(scores)
+    dev.softmax_backward(p, gs, gp, scale)
     gq, gk = dev.zeros_like_storage(q), dev.zeros_like_storage(kt)
-    dev.backward(q, gq, kt, gk, gp)   # dS := dP as a stand-in for the softmax backward glue
-    gp_h, gv_h, gq_h, gk_h = (dev.to_host(t) for t in (gp, gv, gq, gk))
-    DO = oracle.to_f64(do_h, dtype).reshape(B, H, S, D)
-    DS = oracle.to_f64(gp_h, dtype).reshape(B, H, S, S)
+    dev.backward(q, gq, kt, gk, gs)
+    dev.synchronize()
+    announce("config4 checks")
+    q_h, k_h, v_h, do_h, s_h, p_h, o_h, gp_h, gv_h, gs_h, gq_h, gk_h = (
+        dev.to_host(t) for t in (q, k, v, d_o, scores, p, out, gp, gv, gs, gq, gk))
+    sample = [(0, 0), (3, 7), (7, 15)]
+    sl = lambda arr, b, h, per: arr[(b * H + h) * per:(b * H + h + 1) * per]
+    f = lambda arr, b, h, r, c: oracle.to_f64(sl(arr, b, h, r * c), dtype).reshape(r, c)
+    e = ULP[dtype]
     for b, h in sample:
+        Q, K, V, DO = (f(t, b, h, S, D) for t in (q_h, k_h, v_h, do_h))
+        SC, P, GP, GS = (f(t, b, h, S, S) for t in (s_h, p_h, gp_h, gs_h))
+        want = oracle.matmat_forward(dtype, S, D, S, sl(q_h, b, h, S * D), (D, 1), sl(k_h, b, h, S * D), (1, D))
+        assert_within(dtype, D, SC, oracle.to_f64(want, dtype).reshape(S, S), Q, K, extra=2 * e * 64, what=f"scores[{b},{h}]")
+        # softmax of the device's own scores: the exact formula rounded once, +-1 ulp of the largest probability
+        once = nn_ops.softmax_forward(SC * scale, dtype, faithful=False)
+        np.testing.assert_allclose(P, once, rtol=0, atol=2 * e * float(once.max()) + 1e-7)
+        want = oracle.matmat_forward(dtype, S, S, D, sl(p_h, b, h, S * S), (S, 1), sl(v_h, b, h, S * D), (D, 1))
+        assert_within(dtype, S, f(o_h, b, h, S, D), oracle.to_f64(want, dtype).reshape(S, D), P, V, extra=2 * e * 4, what=f"out[{b},{h}]")
         wgp, wgv = np.zeros(S * S, np.float16), np.zeros(S * D, np.float16)
         oracle.matmat_backward(dtype, S, S, D, sl(p_h, b, h, S * S), (S, 1), wgp, sl(v_h, b, h, S * D), (D, 1), wgv, sl(do_h, b, h, S * D))
-        assert_within(dtype, D, oracle.to_f64(sl(gp_h, b, h, S * S), dtype), oracle.to_f64(wgp, dtype), DO[b, h], V[b, h], extra=2 * ULP[dtype] * 64, what="dP")
-        assert_within(dtype, S, oracle.to_f64(sl(gv_h, b, h, S * D), dtype), oracle.to_f64(wgv, dtype), P[b, h], DO[b, h], extra=2 * ULP[dtype] * 8, what="dV")
+        assert_within(dtype, D, GP, oracle.to_f64(wgp, dtype).reshape(S, S), DO, V, extra=2 * e * 64, what="dP")
+        assert_within(dtype, S, f(gv_h, b, h, S, D), oracle.to_f64(wgv, dtype).reshape(S, D), P, DO, extra=2 * e * 8, what="dV")
+        # softmax backward from the saved output, on the device's own dP: scale * p * (g - sum g p)
+        want = scale * P * (GP - (GP * P).sum(axis=-1, keepdims=True))
+        np.testing.assert_allclose(GS, want, rtol=0, atol=2 * e * float(np.abs(want).max()) + 1e-6)
         wgq, wgk = np.zeros(S * D, np.float16), np.zeros(S * D, np.float16)
-        oracle.matmat_backward(dtype, S, D, S, sl(q_h, b, h, S * D), (D, 1), wgq, sl(k_h, b, h, S * D), (1, D), wgk, sl(gp_h, b, h, S * S))
-        assert_within(dtype, S, oracle.to_f64(sl(gq_h, b, h, S * D), dtype), oracle.to_f64(wgq, dtype), DS[b, h], K[b, h], extra=2 * ULP[dtype] * 2048, what="dQ")
-        assert_within(dtype, S, oracle.to_f64(sl(gk_h, b, h, S * D), dtype), oracle.to_f64(wgk, dtype), Q[b, h], DS[b, h], extra=2 * ULP[dtype] * 2048, what="dK")
+        oracle.matmat_backward(dtype, S, D, S, sl(q_h, b, h, S * D), (D, 1), wgq, sl(k_h, b, h, S * D), (1, D), wgk, sl(gs_h, b, h, S * S))
+        assert_within(dtype, S, f(gq_h, b, h, S, D), oracle.to_f64(wgq, dtype).reshape(S, D), GS, K, extra=2 * e * 16, what="dQ")
+        assert_within(dtype, S, f(gk_h, b, h, S, D), oracle.to_f64(wgk, dtype).reshape(S, D), Q, GS, extra=2 * e * 16, what="dK")
+    # the softmax backward's row identity over the WHOLE tensor: every row of dS sums to 0 (up to rounding of 1024 terms)
+    GS_all = oracle.to_f64(gs_h, dtype).reshape(-1, S)
+    assert float(np.max(np.abs(GS_all.sum(axis=-1)))) <= 1024 * e * float(np.max(np.abs(GS_all))) + 1e-6
