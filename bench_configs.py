@@ -22,7 +22,20 @@ def main():
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
     ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (and torch: vendor-library cross-check, only on request)")
+    ap.add_argument("--probe", default="", choices=["", "traffic", "variants", "mfma-power"],
+                    help="counter-collection aids for rocprofv3, nothing is timed: traffic = 3 plain 256 MiB device copies (a kernel "
+                         "of known size that calibrates FETCH_SIZE / WRITE_SIZE) then 5 launches of the 4096^3 f16 GEMM; variants = 3 "
+                         "launches of that GEMM with every f16 MFMA tile variant forced in turn; mfma-power = the stand-alone "
+                         "MFMA-only program (built by `make -C dfdx_amd/csrc probe`)")
     args = ap.parse_args()
+    if args.probe == "mfma-power":   # a child process, started before this one touches the GPU
+        import os
+        import subprocess
+
+        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "dfdx_amd", "lib", "probe_mfma_power")
+        if not os.path.exists(exe):
+            sys.exit("bench_configs.py: %s is not built (make -C dfdx_amd/csrc probe)" % exe)
+        sys.exit(subprocess.call([exe]))
     import torch
     from dfdx_amd import Rocm
     from dfdx_amd.rocm import View
@@ -30,6 +43,36 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench_configs.py needs a GPU")
     dev = Rocm(0)
+    if args.probe:
+        from dfdx_amd.rocm import KERNEL_MFMA
+
+        n = 4096
+        a = (torch.rand(n, n, device="cuda") * 2 - 1).half()
+        b = (torch.rand(n, n, device="cuda") * 2 - 1).half()
+        c = torch.zeros(n, n, device="cuda", dtype=torch.float16)
+        if args.probe == "traffic":
+            src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+            dst = torch.empty_like(src)
+            desc = dev.gemm_desc("f16", n, n, n, a.data_ptr(), (n, 1), b.data_ptr(), (n, 1), c.data_ptr(), (n, 1))
+            torch.cuda.synchronize()
+            for _ in range(3):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+            for _ in range(5):
+                dev.gemm(desc)
+            torch.cuda.synchronize()
+            print(json.dumps({"probe": "3 x 256 MiB copy, 5 x " + dev.gemm_plan(desc)[2]}))
+        else:
+            names = []
+            for v in range(1, dev.mfma_variant_count("f16") + 1):
+                desc = dev.gemm_desc("f16", n, n, n, a.data_ptr(), (n, 1), b.data_ptr(), (n, 1), c.data_ptr(), (n, 1),
+                                     kernel=KERNEL_MFMA, variant=v, no_split_k=True)
+                names.append(dev.gemm_plan(desc)[2])
+                for _ in range(3):
+                    dev.gemm(desc)
+                torch.cuda.synchronize()
+            print(json.dumps({"probe": names}))
+        return
     tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
     esz = {"f16": 2, "bf16": 2, "f32": 4}
     only = set(filter(None, args.only.split(",")))

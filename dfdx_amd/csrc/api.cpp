@@ -71,10 +71,36 @@ int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
     }
     if (!d->c || (d->k > 0 && (!d->a || !d->b))) return DFDX_ROCM_ERR_INVALID_ARG;
     if (d->c_rs < 0 || d->c_cs < 0 || d->c_b1 < 0 || d->c_b2 < 0) return DFDX_ROCM_ERR_INVALID_ARG;
-    // An output view that maps two logical elements to one address cannot be written without a reduction.
-    if ((d->m > 1 && d->c_rs == 0) || (d->n > 1 && d->c_cs == 0)) return DFDX_ROCM_ERR_ALIASED_OUTPUT;
     if (!d->reduce_batch && ((d->batch1 > 1 && d->c_b1 == 0) || (d->batch2 > 1 && d->c_b2 == 0)))
         return DFDX_ROCM_ERR_ALIASED_OUTPUT;
+    // An output view with a zero stride along a matrix axis maps a whole row (or column) of logical elements to one
+    // address: the gradient of an operand that was broadcast along that axis (matmul/mod.rs:318-320 lets such views
+    // in).  The elements that share an address are SUMMED, which is the gradient of a broadcast (the reference's Cpu
+    // path lets them overwrite each other, its Cuda path reads past the buffer).  The aliased axis becomes a batch axis
+    // of a product with one row (or column), reduced over the batch.
+    const bool rows_alias = d->m > 1 && d->c_rs == 0, cols_alias = d->n > 1 && d->c_cs == 0;
+    if (rows_alias || cols_alias) {
+        if (d->batch1 * d->batch2 != 1 || d->reduce_batch || d->bias) return DFDX_ROCM_ERR_ALIASED_OUTPUT;
+        dfdx_rocm_gemm_desc r = *d;
+        r.reduce_batch = 1;
+        r.c_b1 = r.c_b2 = 0;
+        if (rows_alias) {  // C[j] += sum_i sum_k A[i,k] B[k,j]: the rows become batch 1
+            r.m = 1;
+            r.batch1 = d->m;
+            r.a_b1 = d->a_rs;
+            r.b_b1 = 0;
+            r.c_rs = cols_alias ? 1 : d->n * (d->c_cs > 0 ? d->c_cs : 1);
+        }
+        if (cols_alias) {  // C[i] += sum_j sum_k A[i,k] B[k,j]: the columns become batch 2
+            r.n = 1;
+            r.batch2 = d->n;
+            r.a_b2 = 0;
+            r.b_b2 = d->b_cs;
+            r.c_cs = 1;
+        }
+        r.flags |= DFDX_ROCM_GEMM_NO_SPLIT_K;
+        return make_problem(&r, out);
+    }
     GemmProblem p;
     p.dtype = d->dtype;
     p.accumulate = d->accumulate != 0;

@@ -90,6 +90,20 @@ __global__ __launch_bounds__(64) void bias_backward_combine_kernel(const float *
     Elem<T>::store(grad_bias + c, Elem<T>::load(grad_bias + c) + s);
 }
 
+// ---- f64 (the reference runs its whole test suite in f64 as well): plain kernels, f64 arithmetic -----------------
+__global__ __launch_bounds__(256) void bias_forward_f64_kernel(const double *x, const double *bias, double *out, int64_t total, int64_t cols) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) out[i] = x[i] + bias[i % cols];
+}
+// One thread per column walks the rows in order (the order of the reference's row-after-row adds), neighbouring
+// threads read neighbouring columns.
+__global__ __launch_bounds__(256) void bias_backward_f64_kernel(const double *go, int64_t rows, int64_t cols, double *grad_bias) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= cols) return;
+    double s = grad_bias[c];
+    for (int64_t r = 0; r < rows; r++) s += go[r * cols + c];
+    grad_bias[c] = s;
+}
+
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 template <typename T>
@@ -157,6 +171,12 @@ int dfdx_rocm_bias_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t 
     case DFDX_ROCM_F32: return bias_forward_t<float>(ctx, rows, cols, x, bias, out);
     case DFDX_ROCM_F16: return bias_forward_t<_Float16>(ctx, rows, cols, x, bias, out);
     case DFDX_ROCM_BF16: return bias_forward_t<__bf16>(ctx, rows, cols, x, bias, out);
+    case DFDX_ROCM_F64: {
+        const int64_t total = rows * cols;
+        const unsigned grid = (unsigned)std::min<int64_t>((total + 255) / 256, (int64_t)ctx->compute_units * 8);
+        bias_forward_f64_kernel<<<grid, 256, 0, ctx->stream>>>((const double *)x, (const double *)bias, (double *)out, total, cols);
+        return (int)hipGetLastError();
+    }
     default: return DFDX_ROCM_ERR_UNSUPPORTED;
     }
 }
@@ -171,6 +191,9 @@ int dfdx_rocm_bias_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t
     case DFDX_ROCM_F32: return bias_backward_t<float>(ctx, rows, cols, grad_out, grad_bias);
     case DFDX_ROCM_F16: return bias_backward_t<_Float16>(ctx, rows, cols, grad_out, grad_bias);
     case DFDX_ROCM_BF16: return bias_backward_t<__bf16>(ctx, rows, cols, grad_out, grad_bias);
+    case DFDX_ROCM_F64:
+        bias_backward_f64_kernel<<<(unsigned)((cols + 255) / 256), 256, 0, ctx->stream>>>((const double *)grad_out, rows, cols, (double *)grad_bias);
+        return (int)hipGetLastError();
     default: return DFDX_ROCM_ERR_UNSUPPORTED;
     }
 }

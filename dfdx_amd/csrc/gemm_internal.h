@@ -1,6 +1,7 @@
 // Internal interfaces between the C ABI (api.cpp) and the kernel translation units.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdint.h>
 
 namespace dfdx_rocm {
@@ -39,6 +40,17 @@ struct ConvPatches {
     int h_src, w_src;    // the planes the windows come from (w_src >= 8)
     int off_y, off_x, step_y, step_x;
     int64_t plane;       // elements between channels
+};
+
+// What a launcher learns once per kernel instance AND device (the dynamic-LDS attribute is set, the occupancy is known):
+// one word per device, 0 = not yet.  Two host threads that arrive together both do the set-up and store the same value.
+struct PerDevice {
+    std::atomic<int> word[64];
+    std::atomic<int> &here() {
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        return word[dev & 63];
+    }
 };
 
 static inline size_t dtype_size(int dt) { return dt == DT_F32 ? 4 : (dt == DT_F64 ? 8 : 2); }

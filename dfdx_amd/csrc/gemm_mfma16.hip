@@ -422,12 +422,13 @@ hipError_t launch_layout(const Params &p, bool a_kc, bool b_kc, hipStream_t stre
 #define DFDX_LAUNCH(AKC, BKC)                                                                                   \
     do {                                                                                                        \
         auto kern = gemm_mfma16_kernel<T, BM, BN, BK, WM, WN, AKC, BKC>;                                        \
-        static bool configured = false;                                                                         \
-        if (!configured) {                                                                                      \
+        static PerDevice configured_on;                                                                         \
+        std::atomic<int> &configured = configured_on.here();                                                    \
+        if (!configured.load(std::memory_order_acquire)) {                                                      \
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,   \
                                                (int)lds);                                                       \
             if (e != hipSuccess) return e;                                                                      \
-            configured = true;                                                                                  \
+            configured.store(1, std::memory_order_release);                                                     \
         }                                                                                                       \
         kern<<<grid, block, lds, stream>>>(p);                                                                  \
     } while (0)
@@ -444,11 +445,12 @@ template <typename T, int BM, int BN, int BK, int WM, int WN> hipError_t launch_
     constexpr int NT = WM * WN * 64;
     constexpr size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * 2;
     auto kern = gemm_mfma16_kernel<T, BM, BN, BK, WM, WN, true, false, true>;
-    static bool configured = false;
-    if (!configured) {
+    static PerDevice configured_on;
+    std::atomic<int> &configured = configured_on.here();
+    if (!configured.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        configured = true;
+        configured.store(1, std::memory_order_release);
     }
     kern<<<dim3((unsigned)p.total_blocks), dim3(NT), lds, stream>>>(p);
     return hipGetLastError();

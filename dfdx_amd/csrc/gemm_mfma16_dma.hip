@@ -783,7 +783,9 @@ hipError_t launch_layout(Params p, int compute_units, bool a_kc, bool b_kc, hipS
 #define DFDX_LAUNCH(AKC, BKC, EDGE)                                                                            \
     do {                                                                                                       \
         auto kern = gemm_mfma16_dma_kernel<T, BM, BN, WM, WN, AKC, BKC, EDGE>;                                 \
-        static int per_cu = 0;                                                                                 \
+        static PerDevice occupancy_on;                                                                         \
+        std::atomic<int> &known = occupancy_on.here();                                                         \
+        int per_cu = known.load(std::memory_order_acquire);                                                    \
         if (per_cu == 0) {                                                                                     \
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,  \
                                                (int)lds);                                                      \
@@ -792,6 +794,7 @@ hipError_t launch_layout(Params p, int compute_units, bool a_kc, bool b_kc, hipS
             e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void *)kern, NT, lds);               \
             if (e != hipSuccess) return e;                                                                     \
             per_cu = occ < 1 ? 1 : occ;                                                                        \
+            known.store(per_cu, std::memory_order_release);                                                    \
         }                                                                                                      \
         const int resident = (compute_units < 8 ? 8 : compute_units) * per_cu / 8 * 8;                         \
         p.grid = p.total_blocks <= resident ? p.total_blocks : resident;                                       \

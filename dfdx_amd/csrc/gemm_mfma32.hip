@@ -336,12 +336,13 @@ hipError_t launch_layout(const Params &p, bool a_kc, bool b_kc, hipStream_t stre
     do {                                                                                                        \
         constexpr size_t lds = (size_t)2 * 4 * (Loader<BM, BK, NT, AKC>::LDS_SIZE + Loader<BN, BK, NT, BKC>::LDS_SIZE); \
         auto kern = gemm_mfma32_kernel<BM, BN, BK, WM, WN, AKC, BKC>;                                           \
-        static bool configured = false;                                                                         \
-        if (!configured) {                                                                                      \
+        static PerDevice configured_on;                                                                         \
+        std::atomic<int> &configured = configured_on.here();                                                    \
+        if (!configured.load(std::memory_order_acquire)) {                                                      \
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,   \
                                                (int)lds);                                                       \
             if (e != hipSuccess) return e;                                                                      \
-            configured = true;                                                                                  \
+            configured.store(1, std::memory_order_release);                                                     \
         }                                                                                                       \
         kern<<<grid, block, lds, stream>>>(p);                                                                  \
     } while (0)

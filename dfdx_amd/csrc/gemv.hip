@@ -246,7 +246,12 @@ template <typename T> hipError_t launch_t(const Shape &s, hipStream_t stream) {
 
 }  // namespace
 
-bool gemv_supported(const GemmProblem &g) { return classify(g).ok; }
+bool gemv_supported(const GemmProblem &g) {
+    Shape s = classify(g);
+    if (!s.ok) return false;
+    plan_slices(s, g.dtype);
+    return s.p.kslices <= 65535;  // the k slices are grid.y; beyond its limit the product goes to another kernel
+}
 
 size_t gemv_workspace_bytes(const GemmProblem &g) {
     Shape s = classify(g);

@@ -52,6 +52,68 @@ __global__ __launch_bounds__(256) void reshape_backward_kernel(T *grad_inp, cons
     }
 }
 
+// Backward through a view with broadcast axes (stride 0, extent > 1): every grad_inp element receives the SUM of the
+// grad_out elements that the view maps onto it (reshape_to/cpu_kernel.rs:28-32 adds them one after the other).  A thread
+// owns one grad_inp element -- an index over the kept axes -- and walks the broadcast axes itself: no atomics, a fixed
+// order, f32 accumulation with one rounding.
+struct ReduceDims {
+    int nkeep, nbro;
+    uint32_t keep_shape[MAX_RANK], bro_shape[MAX_RANK];
+    int64_t keep_dst[MAX_RANK];                       // stride in grad_inp (elements)
+    int64_t keep_src[MAX_RANK], bro_src[MAX_RANK];    // stride in the contiguous grad_out (elements)
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void reshape_backward_reduce_kernel(T *grad_inp, const T *grad_out, ReduceDims d, int64_t kept,
+                                                                      int64_t folded) {
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < kept; e += (int64_t)gridDim.x * 256) {
+        int64_t dst = 0, src0 = 0, q = e;
+        for (int a = d.nkeep - 1; a >= 0; a--) {
+            const int64_t i = q % d.keep_shape[a];
+            q /= d.keep_shape[a];
+            dst += i * d.keep_dst[a];
+            src0 += i * d.keep_src[a];
+        }
+        float sum = 0.0f;
+        for (int64_t r = 0; r < folded; r++) {
+            int64_t src = src0, t = r;
+            for (int a = d.nbro - 1; a >= 0; a--) {
+                src += (t % d.bro_shape[a]) * d.bro_src[a];
+                t /= d.bro_shape[a];
+            }
+            sum += Elem<T>::load(grad_out + src);
+        }
+        Elem<T>::store(grad_inp + dst, Elem<T>::load(grad_inp + dst) + sum);
+    }
+}
+
+template <typename T>
+int launch_reduce(dfdx_rocm_ctx *ctx, int rank, const int64_t *shape, const int64_t *strides, const void *grad_out, void *grad_inp) {
+    ReduceDims d = {};
+    int64_t kept = 1, folded = 1, logical = 1;
+    int64_t ls[MAX_RANK];  // row-major stride of each axis in grad_out
+    for (int a = rank - 1; a >= 0; a--) {
+        ls[a] = logical;
+        logical *= shape[a];
+        if (shape[a] > 1 && strides[a] == 0) folded *= shape[a];
+        else if (shape[a] > 1) kept *= shape[a];
+    }
+    for (int a = 0; a < rank; a++) {
+        if (shape[a] <= 1) continue;
+        if (strides[a] == 0) {
+            d.bro_shape[d.nbro] = (uint32_t)shape[a];
+            d.bro_src[d.nbro++] = ls[a];
+        } else {
+            d.keep_shape[d.nkeep] = (uint32_t)shape[a];
+            d.keep_dst[d.nkeep] = strides[a];
+            d.keep_src[d.nkeep++] = ls[a];
+        }
+    }
+    const unsigned grid = (unsigned)std::min<int64_t>((kept + 255) / 256, (int64_t)ctx->compute_units * 16);
+    reshape_backward_reduce_kernel<T><<<grid, 256, 0, ctx->stream>>>((T *)grad_inp, (const T *)grad_out, d, kept, folded);
+    return (int)hipGetLastError();
+}
+
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 // Drops size-1 axes and merges neighbours that are contiguous with respect to each other.
@@ -117,14 +179,23 @@ int dispatch(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, cons
     if (int e = bind(ctx)) return e;
     if (rank < 0 || rank > MAX_RANK || (rank > 0 && (!shape || !strides))) return DFDX_ROCM_ERR_INVALID_ARG;
     int64_t total = 1;
+    bool broadcast = false;
     for (int a = 0; a < rank; a++) {
         if (shape[a] < 0 || strides[a] < 0 || shape[a] >= (1ll << 32)) return DFDX_ROCM_ERR_INVALID_ARG;
         // a broadcast axis maps several grad_out elements to one grad_inp element: a reduction, not a scatter
-        if (!FWD && shape[a] > 1 && strides[a] == 0) return DFDX_ROCM_ERR_ALIASED_OUTPUT;
+        if (!FWD && shape[a] > 1 && strides[a] == 0) broadcast = true;
         total *= shape[a];
     }
     if (total == 0) return DFDX_ROCM_OK;
     if (!src || !dst) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (broadcast) {
+        switch (dtype) {
+        case DFDX_ROCM_F32: return launch_reduce<float>(ctx, rank, shape, strides, src, dst);
+        case DFDX_ROCM_F16: return launch_reduce<_Float16>(ctx, rank, shape, strides, src, dst);
+        case DFDX_ROCM_BF16: return launch_reduce<__bf16>(ctx, rank, shape, strides, src, dst);
+        default: return DFDX_ROCM_ERR_UNSUPPORTED;
+        }
+    }
     switch (dtype) {
     case DFDX_ROCM_F32: return launch_t<float, FWD>(ctx, rank, shape, strides, src, dst);
     case DFDX_ROCM_F16: return launch_t<_Float16, FWD>(ctx, rank, shape, strides, src, dst);

@@ -209,6 +209,8 @@ int dfdx_rocm_linear_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64
                               const void *x, const int64_t xs[2], void *grad_x, const void *weight, void *grad_weight,
                               void *grad_bias, const void *grad_out) {
     if (!xs) return DFDX_ROCM_ERR_INVALID_ARG;
+    // every step below supports all four element types; an unknown one is refused before any gradient is touched
+    if (dtype < DFDX_ROCM_F32 || dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_INVALID_ARG;
     const int64_t ws[2] = {1, in_dim};  // the (I,O) view of the (O,I) storage; its gradient lands in (O,I) row-major
     if (int e = dfdx_rocm_matmat_backward(ctx, dtype, rows, in_dim, out_dim, x, xs, grad_x, weight, ws, grad_weight, grad_out))
         return e;

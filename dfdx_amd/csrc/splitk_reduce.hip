@@ -31,8 +31,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, int splits, int64_t ws_ld, int64_t ws_split_stride,
                                                             T *c, int64_t c_rs, int m, int n, int accumulate, int bias_mode,
                                                             const T *bias, int vec4) {
-    const int col = (blockIdx.x * 64 + threadIdx.x % 64) * 4;
-    const int row = blockIdx.y * 4 + threadIdx.x / 64;
+    const int col = (blockIdx.y * 64 + threadIdx.x % 64) * 4;   // rows along grid.x: its limit is 2^31, grid.y's 65535
+    const int row = blockIdx.x * 4 + threadIdx.x / 64;
     if (row >= m || col >= n) return;
     const float *src = ws + (int64_t)row * ws_ld + col;
     f32x4 v = *(const f32x4 *)src;
@@ -79,8 +79,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce16_kernel(const float *ws, int splits, int64_t ws_ld, int64_t ws_split_stride,
                                                               uint16_t *c, int64_t c_rs, int m, int n, int accumulate,
                                                               int bias_mode, const uint16_t *bias) {
-    const int col = (blockIdx.x * 64 + threadIdx.x % 64) * 8;
-    const int row = blockIdx.y * 4 + threadIdx.x / 64;
+    const int col = (blockIdx.y * 64 + threadIdx.x % 64) * 8;
+    const int row = blockIdx.x * 4 + threadIdx.x / 64;
     if (row >= m || col >= n) return;   // n is a multiple of 8: a thread's 8 columns are all inside or all outside
     const float *src = ws + (int64_t)row * ws_ld + col;
     uint16_t *dst = c + (int64_t)row * c_rs + col;
@@ -124,13 +124,14 @@ __global__ __launch_bounds__(256) void splitk_reduce16_kernel(const float *ws, i
 
 // C of `p` must have unit column stride and no batch (the planner only splits such problems).
 hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_split_stride, hipStream_t stream) {
-    dim3 grid((unsigned)((p.n + 255) / 256), (unsigned)((p.m + 3) / 4)), block(256);
+    dim3 grid((unsigned)((p.m + 3) / 4), (unsigned)((p.n + 255) / 256)), block(256);
+    if ((p.n + 255) / 256 > 65535) return hipErrorInvalidValue;  // 16.7 M columns: no planner splits such a product
     const int64_t c_rs = p.m == 1 ? p.n : p.c_rs;
     const int bias_mode = p.bias ? p.bias_mode : BIAS_NONE;
     const bool is16 = p.dtype == DT_F16 || p.dtype == DT_BF16;
     if (is16 && p.n % 8 == 0 && c_rs % 8 == 0 && ws_ld % 4 == 0 && ws_split_stride % 4 == 0 && ((uintptr_t)p.c & 15u) == 0 &&
         ((uintptr_t)p.workspace & 15u) == 0 && (bias_mode != BIAS_PER_COL || ((uintptr_t)p.bias & 15u) == 0)) {
-        dim3 grid16((unsigned)((p.n + 511) / 512), (unsigned)((p.m + 3) / 4));
+        dim3 grid16((unsigned)((p.m + 3) / 4), (unsigned)((p.n + 511) / 512));
         if (p.dtype == DT_F16)
             splitk_reduce16_kernel<_Float16><<<grid16, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (uint16_t *)p.c,
                                                                             c_rs, (int)p.m, (int)p.n, p.accumulate, bias_mode,

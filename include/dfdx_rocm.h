@@ -274,8 +274,10 @@ int dfdx_rocm_softmax_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int6
  * view's elements, in logical row-major order, into the contiguous `out`;
  * backward adds grad_out (contiguous) into grad_inp through the view's
  * strides.  rank <= 6, strides in elements.  A zero stride on an axis longer
- * than 1 is accepted by forward and answered with
- * DFDX_ROCM_ERR_ALIASED_OUTPUT by backward. */
+ * than 1 (a broadcast view) is read repeatedly by forward; backward sums the
+ * grad_out elements that the view maps onto one grad_inp element
+ * (cpu_kernel.rs:28-32 adds them one after the other; here in f32, rounded
+ * once). */
 int dfdx_rocm_reshape_forward(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, const int64_t *inp_strides,
                               const void *inp, void *out);
 int dfdx_rocm_reshape_backward(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, const int64_t *inp_strides,

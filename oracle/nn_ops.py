@@ -147,7 +147,7 @@ def reshape_backward(shape, strides, grad_inp: np.ndarray, grad_out: np.ndarray,
         out[idx] = round_to(out[idx] + go, dtype)
         return out
     for o, i in enumerate(idx):
-        out[i] = round_to(out[i] + go[o], dtype)
+        out[i] = np.reshape(round_to(out[i] + go[o], dtype), -1)[0]
     return out
 
 

@@ -56,10 +56,11 @@ def test_reshape_literals(case):
     if "grad_storage" in case:
         dev.reshape_backward(x, gi, go)
         np.testing.assert_allclose(oracle.to_f64(dev.to_host(gi), "f32"), case["grad_storage"], rtol=0, atol=1e-6)
-    else:  # broadcast view: a scatter would race, the entry point says so
-        with pytest.raises(RocmError) as e:
-            dev.reshape_backward(x, gi, go)
-        assert e.value.code == -4
+    else:  # broadcast view (the reference's test holds no gradient literal for it): elements that share an address are
+        # summed, which is what reshape_to/cpu_kernel.rs:28-32 does one element after the other
+        dev.reshape_backward(x, gi, go)
+        want = nn_ops.reshape_backward(case["shape"], case["strides"], np.zeros(len(case["storage"])), host(dev, go), "f32")
+        np.testing.assert_allclose(oracle.to_f64(dev.to_host(gi), "f32"), want, rtol=0, atol=1e-6)
 
 
 @pytest.mark.parametrize("case", GLUE["scalar_mul"], ids=lambda c: c["name"])
@@ -248,3 +249,31 @@ def test_config4_attention_chain_on_device():
         np.testing.assert_allclose(GS[b, h], want, rtol=0, atol=2 * e * float(np.abs(want).max()) + 1e-6)
         assert_within(dtype, S, GQ[b, h], GS[b, h] @ K[b, h], GS[b, h], K[b, h], extra=2 * e * 16, what="dQ")
         assert_within(dtype, S, GK[b, h], GS[b, h].T @ Q[b, h], GS[b, h], Q[b, h], extra=2 * e * 16, what="dK")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_reshape_backward_through_broadcast_axes(dtype):
+    """Views with one or several broadcast axes (stride 0) between real ones: backward sums grad_out over them."""
+    from dfdx_amd.rocm import View
+    dev, g = device(), rng(5151)
+    for shape, strides, nstore in (((4, 6, 5), (5, 0, 1), 20), ((3, 4, 8, 16), (0, 16, 0, 1), 64), ((7, 9), (0, 0), 1),
+                                   ((2, 3, 4), (4, 0, 1), 8), ((64, 33, 8), (8, 0, 1), 512)):
+        announce("reshape backward, broadcast axes", dtype, shape, strides)
+        st = upload(dev, g.standard_normal(nstore), dtype)
+        x = View(st.storage, dtype, shape, strides)
+        total = int(np.prod(shape))
+        go = upload(dev, g.standard_normal(total), dtype)
+        gi0 = g.standard_normal(nstore)
+        gi = upload(dev, gi0, dtype)
+        dev.reshape_backward(x, gi, go)
+        want = nn_ops.reshape_backward(shape, strides, oracle.to_f64(dev.to_host(upload(dev, gi0, dtype)), dtype), host(dev, go), dtype)
+        exact = oracle.to_f64(dev.to_host(upload(dev, gi0, dtype)), dtype).copy()
+        np.add.at(exact, nn_ops._view_indices(shape, strides).reshape(-1), host(dev, go).reshape(-1))
+        got = oracle.to_f64(dev.to_host(gi), dtype)
+        folded = total // max(1, len(set(nn_ops._view_indices(shape, strides).reshape(-1).tolist())))
+        # one rounding of the exact sum; the reference rounds after every add, which the loose bound covers
+        np.testing.assert_allclose(got, exact, rtol=0, atol=EPS[dtype] * 2 * np.abs(exact).max() + 1e-6)
+        np.testing.assert_allclose(got, want, rtol=0, atol=EPS[dtype] * 2 * folded * np.abs(exact).max() + 1e-6)
+        # forward of the same view repeats the stored elements
+        out = dev.reshape_forward(x, (total,))
+        np.testing.assert_array_equal(host(dev, out), host(dev, x).reshape(-1))

@@ -105,13 +105,29 @@ def test_doubly_strided_operand_takes_generic_path():
     assert_within("f32", k, dev.to_host(dc).astype(np.float64).reshape(m, n), A @ B, A, B, extra=1e-6)
 
 
-def test_aliased_output_is_rejected():
+def test_aliased_output_sums_or_is_rejected():
+    """A zero stride on a matrix axis of C (the gradient view of a broadcast operand) sums the elements that share an
+    address; a zero BATCH stride without `reduce_batch`, or a bias on such a view, is refused."""
     from dfdx_amd import RocmError
 
     dev = device()
-    a = dev.tensor(np.zeros(64, np.float32), "f32")
-    with pytest.raises(RocmError) as e:
-        dev.gemm(dev.gemm_desc("f32", 4, 4, 4, a.ptr, (4, 1), a.ptr, (4, 1), a.ptr, (0, 1)))
+    g = rng(77)
+    A, B = g.integers(-3, 4, (4, 5)).astype(np.float32), g.integers(-3, 4, (5, 6)).astype(np.float32)
+    a, b = dev.tensor(A.reshape(-1), "f32"), dev.tensor(B.reshape(-1), "f32")
+    P = (A @ B).astype(np.float64)
+    for c_strides, want, size in (((0, 1), P.sum(axis=0), 6), ((1, 0), P.sum(axis=1), 4), ((0, 0), P.sum(keepdims=True).reshape(-1), 1)):
+        c = dev.tensor(np.full(size, 2.0, np.float32), "f32")
+        announce("gemm into an aliased view", c_strides)
+        dev.gemm(dev.gemm_desc("f32", 4, 5, 6, a.ptr, (5, 1), b.ptr, (6, 1), c.ptr, c_strides, accumulate=True))
+        assert np.array_equal(dev.to_host(c).astype(np.float64), want + 2.0)   # small integers: exact in any order
+        dev.gemm(dev.gemm_desc("f32", 4, 5, 6, a.ptr, (5, 1), b.ptr, (6, 1), c.ptr, c_strides, accumulate=False))
+        assert np.array_equal(dev.to_host(c).astype(np.float64), want)
+    c = dev.tensor(np.zeros(64, np.float32), "f32")
+    with pytest.raises(RocmError) as e:   # two batches into one matrix without reduce_batch
+        dev.gemm(dev.gemm_desc("f32", 4, 5, 6, a.ptr, (5, 1), b.ptr, (6, 1), c.ptr, (6, 1), batch=(2, 1)))
+    assert e.value.code == -4
+    with pytest.raises(RocmError) as e:   # a bias on a view whose columns share an address
+        dev.gemm(dev.gemm_desc("f32", 4, 5, 6, a.ptr, (5, 1), b.ptr, (6, 1), c.ptr, (1, 0), bias=b.ptr))
     assert e.value.code == -4
     with pytest.raises(RocmError):
         dev.gemm(dev.gemm_desc("f32", -1, 4, 4, a.ptr, (4, 1), a.ptr, (4, 1), a.ptr, (4, 1)))

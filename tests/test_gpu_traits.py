@@ -71,10 +71,16 @@ def test_linear_literals(case, dtype, fused):
         y = host(dev, dev.forward(x, wt)) + np.asarray(LINEAR["bias"])
     np.testing.assert_allclose(y, case["y"], rtol=0, atol=1e-6)
     gy = loss_grad("square_mean", y)
-    gx, gw = dev.zeros_like_storage(x), dev.zeros_like_storage(wt)
-    dev.backward(x, gx, wt, gw, upload(dev, gy, dtype))
+    if fused:   # the whole backward through the Linear entry point, grad_bias included (f64 too: the reference's CI runs in f64)
+        gx, gw, gb = dev.zeros_like_storage(x), dev.zeros_like_storage(w), dev.zeros_like_storage(bias)
+        dev.linear_backward(x, gx, w, gw, gb, upload(dev, gy, dtype))
+    else:       # MatMat backward on the permuted view + Bias1D's backward
+        gx, gw, gb = dev.zeros_like_storage(x), dev.zeros_like_storage(wt), dev.zeros_like_storage(bias)
+        gyv = upload(dev, gy, dtype)
+        dev.backward(x, gx, wt, gw, gyv)
+        dev.bias_backward(gyv, gb)
     np.testing.assert_allclose(oracle.to_f64(dev.to_host(gw), dtype).reshape(2, 5), case["grad_weight"], rtol=0, atol=1e-6)
-    np.testing.assert_allclose(gy.reshape(-1, 2).sum(axis=0), case["grad_bias"], rtol=0, atol=1e-6)
+    np.testing.assert_allclose(oracle.to_f64(dev.to_host(gb), dtype), case["grad_bias"], rtol=0, atol=1e-6)
 
 
 # ------------------------------------------------------------------ identities --
@@ -217,3 +223,60 @@ def test_shape_mismatch_panics_before_the_kernel(shapes, msg):
     with pytest.raises(AssertionError) as e:
         dev.forward(x, y)
     assert msg in str(e.value)
+
+
+# -------------------------------------------- broadcast views: a zero stride on a MATRIX axis --
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("shape", [(48, 40, 72), (200, 136, 264), (5, 3, 7)])
+@pytest.mark.parametrize("which", ["lhs_k", "lhs_m", "rhs_k", "rhs_n", "lhs_both", "ones"])
+def test_matmul_broadcast_matrix_axes(dtype, shape, which):
+    """`matrix_strides` lets views through whose matrix strides are [1,0], [0,1] or [1,1] (matmul/mod.rs:316-325): a
+    vector broadcast along one matrix axis (`broadcast_to.rs:68-75` shares the tensor id, so the gradient buffer has
+    the VECTOR's length and is written through the zero stride), or a size-1 tensor broadcast along both.  Forward is an
+    ordinary product of the logical matrices; backward must SUM the logical gradient over the broadcast axis (the
+    gradient of a broadcast).  Checked against float64 on the logical matrices; forward also against the oracle."""
+    dev, g = device(), rng(907)
+    m, k, n = shape
+    announce("broadcast matrix axis", dtype, shape, which)
+    vec = lambda length: upload(dev, g.standard_normal(length), dtype)
+    full = lambda r, c: upload(dev, g.standard_normal((r, c)), dtype)
+    from dfdx_amd.rocm import View
+    if which == "lhs_k":      # lhs[i, kk] = v[i]: strides [1, 0]
+        v = vec(m); lhs = View(v.storage, dtype, (m, k), (1, 0)); rhs = full(k, n)
+    elif which == "lhs_m":    # lhs[i, kk] = v[kk]: strides [0, 1]
+        v = vec(k); lhs = View(v.storage, dtype, (m, k), (0, 1)); rhs = full(k, n)
+    elif which == "rhs_k":    # rhs[kk, j] = v[kk]: strides [1, 0]
+        v = vec(k); rhs = View(v.storage, dtype, (k, n), (1, 0)); lhs = full(m, k)
+    elif which == "rhs_n":    # rhs[kk, j] = v[j]: strides [0, 1]
+        v = vec(n); rhs = View(v.storage, dtype, (k, n), (0, 1)); lhs = full(m, k)
+    elif which == "lhs_both":  # a one-element tensor broadcast along both axes: strides [0, 0]
+        v = vec(1); lhs = View(v.storage, dtype, (m, k), (0, 0)); rhs = full(k, n)
+    else:                      # strides [1, 1]: a (1, 1) matrix -- the arm exists for size-1 axes
+        m, k = 1, 1
+        v = vec(1); lhs = View(v.storage, dtype, (1, 1), (1, 1)); rhs = full(1, n)
+    out = dev.forward(lhs, rhs)
+    go = upload(dev, g.standard_normal((m, n)), dtype)
+    gl, gr = dev.zeros_like_storage(lhs), dev.zeros_like_storage(rhs)
+    dev.backward(lhs, gl, rhs, gr, go)
+    dev.synchronize()
+    L, R, G = host(dev, lhs), host(dev, rhs), host(dev, go)
+    ulp = {"f32": 2.0 ** -24, "f16": 2.0 ** -11}[dtype]
+    want = L @ R
+    assert_within(dtype, k, host(dev, out), want, L, R, extra=ulp * np.abs(want).max(), what="forward vs f64")
+    want_or = oracle.matmat_forward(dtype, m, k, n, dev.to_host(lhs), lhs.strides, dev.to_host(rhs), rhs.strides)
+    assert_within(dtype, k, host(dev, out), oracle.to_f64(want_or, dtype).reshape(m, n), L, R,
+                  extra=2 * ulp * np.abs(want).max(), what="forward vs oracle")
+    # logical gradients, then summed over the axes the storage does not have
+    GL, GR = G @ R.T, L.T @ G
+
+    def fold(grad, view):
+        for ax, st in enumerate(view.strides):
+            if st == 0 and view.shape[ax] > 1:
+                grad = grad.sum(axis=ax, keepdims=True)
+        return grad.reshape(-1)
+
+    # a sum over up to max(m, k, n) products of sums over up to max(m, k, n) terms
+    terms = max(m, k, n) ** 2
+    for name, got, want_g, a_, b_ in (("grad_lhs", gl, fold(GL, lhs), G, R), ("grad_rhs", gr, fold(GR, rhs), L, G)):
+        got64 = oracle.to_f64(dev.to_host(got), dtype)[: want_g.size]
+        assert_within(dtype, terms, got64, want_g, a_, b_, extra=ulp * np.abs(want_g).max(), what=name)
