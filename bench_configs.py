@@ -15,6 +15,7 @@ import argparse
 import json
 import sys
 
+ROTATE_BYTES = 320 << 20   # bytes in flight across the rotating buffer sets: more than the 256 MB last-level cache
 
 
 def main():
@@ -27,6 +28,7 @@ def main():
                          "of known size that calibrates FETCH_SIZE / WRITE_SIZE) then 5 launches of the 4096^3 f16 GEMM; variants = 3 "
                          "launches of that GEMM with every f16 MFMA tile variant forced in turn; mfma-power = the stand-alone "
                          "MFMA-only program (built by `make -C dfdx_amd/csrc probe`)")
+    ap.add_argument("--no-rotate", action="store_true", help="skip the second timing of the HBM-bound cases over rotating buffer sets")
     args = ap.parse_args()
     if args.probe == "mfma-power":   # a child process, started before this one touches the GPU
         import os
@@ -38,7 +40,7 @@ def main():
         sys.exit(subprocess.call([exe]))
     import torch
     from dfdx_amd import Rocm
-    from dfdx_amd.rocm import View
+    from dfdx_amd.rocm import GemmDesc, View
 
     if not torch.cuda.is_available():
         sys.exit("bench_configs.py needs a GPU")
@@ -90,30 +92,79 @@ def main():
     def view(t, dtype):
         return View(t.view(torch.uint8).reshape(-1), dtype, tuple(t.shape), tuple(t.stride()))
 
-    def report(group, name, flop, nbytes, ms, kernel):
+    def report(group, name, flop, nbytes, ms, kernel, rot_ms=None, sets=0):
         row = {"group": group, "case": name, "kernel": kernel, "us": round(ms * 1e3, 2),
                "tflops": round(flop / ms / 1e9, 1) if flop else None,
                "gbps": round(nbytes / ms / 1e6, 1) if nbytes else None}
+        tail = ""
+        if rot_ms:   # the same case over `sets` disjoint buffer sets taken in turn: no launch finds its operands cached
+            row.update({"sets": sets, "us_rotating": round(rot_ms * 1e3, 2),
+                        "tflops_rotating": round(flop / rot_ms / 1e9, 1) if flop else None,
+                        "gbps_rotating": round(nbytes / rot_ms / 1e6, 1) if nbytes else None})
+            tail = f"  | {sets:3d} sets {row['us_rotating']:9.1f} us " + (
+                f"{row['gbps_rotating']} GB/s" if nbytes else f"{row['tflops_rotating']} TFLOP/s")
         rows.append(row)
         print(f"{group:5s} {name:44s} {kernel:40s} {row['us']:9.1f} us "
-              f"{(str(row['tflops']) + ' TFLOP/s') if flop else '':>16s} {(str(row['gbps']) + ' GB/s') if nbytes else '':>14s}",
+              f"{(str(row['tflops']) + ' TFLOP/s') if flop else '':>16s} {(str(row['gbps']) + ' GB/s') if nbytes else '':>14s}{tail}",
               flush=True)
 
-    def gemm(group, name, desc, flop, nbytes, iters=None):
-        ms = dev.gemm_time(desc, 5, iters or args.iters)
-        report(group, name, flop, nbytes, ms, dev.gemm_plan(desc)[2])
+    def nsets(bufs):
+        """Buffer sets that put more than the last-level cache (256 MB) in flight: at least 4, at most 512."""
+        foot = sum(t.numel() * t.element_size() for t in bufs)
+        return int(min(512, max(4, -(-ROTATE_BYTES // max(foot, 1)))))
 
-    def timed(group, name, fn, flop, nbytes, kernel):
-        for _ in range(5):
-            fn()
+    def gemm(group, name, desc, flop, nbytes, iters=None, bufs=None):
+        """`bufs`: the tensors the descriptor points into; given, the case is also timed over rotating copies of them."""
+        iters = iters or args.iters
+        ms = dev.gemm_time(desc, 5, iters)
+        rot_ms, n = None, 0
+        if bufs and not args.no_rotate:
+            n = nsets(bufs)
+            descs, keep = [desc], []
+            for _ in range(n - 1):
+                d = GemmDesc.from_buffer_copy(desc)
+                copies = [t.clone() for t in bufs]
+                keep.append(copies)
+                for field in ("a", "b", "c", "bias"):
+                    ptr = getattr(desc, field)
+                    for t, cp in zip(bufs, copies):
+                        if ptr is not None and t.data_ptr() <= ptr < t.data_ptr() + t.numel() * t.element_size():
+                            setattr(d, field, cp.data_ptr() + (ptr - t.data_ptr()))
+                descs.append(d)
+            rot_ms = dev.gemm_time_rotating(descs, n, max(iters, 2 * n))
+            del keep
+        report(group, name, flop, nbytes, ms, dev.gemm_plan(desc)[2], rot_ms, n)
+
+    def loop_ms(call, iters):
+        for i in range(5):
+            call(i)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(args.iters):
-            fn()
+        for i in range(iters):
+            call(i)
         e1.record()
         torch.cuda.synchronize()
-        report(group, name, flop, nbytes, e0.elapsed_time(e1) / args.iters, kernel)
+        return e0.elapsed_time(e1) / iters
+
+    def timed(group, name, fn, flop, nbytes, kernel, sets=None):
+        """`sets`: the same call on disjoint buffers, one callable per set; results are held for one turn of the
+        rotation so that the outputs an op allocates are disjoint too."""
+        ms = loop_ms(lambda i: fn(), args.iters)
+        rot_ms, n = None, 0
+        if sets and not args.no_rotate:
+            n = len(sets)
+            hold = [None] * n
+
+            def call(i):
+                hold[i % n] = sets[i % n]()
+            rot_ms = loop_ms(call, max(args.iters, 2 * n))
+            del hold
+        report(group, name, flop, nbytes, ms, kernel, rot_ms, n)
+
+    def copies(n, *tensors):
+        """n sets of the given tensors: the originals first, then n - 1 clones of each."""
+        return [tensors] + [tuple(t.clone() for t in tensors) for _ in range(n - 1)]
 
     P = lambda t: t.data_ptr()
 
@@ -124,12 +175,12 @@ def main():
         y, gx, gw = zeros((r, o), dt), zeros((r, i), dt), zeros((o, i), dt)
         fl = 2 * r * i * o
         gemm("c1", "Linear fwd 64x512x256 NT", dev.gemm_desc(dt, r, i, o, P(x), (i, 1), P(w), (1, i), P(y), (o, 1)),
-             fl, es * (r * i + i * o + r * o), 200)
+             fl, es * (r * i + i * o + r * o), 200, bufs=(x, w, y))
         gemm("c1", "dX 64x256x512 NN acc", dev.gemm_desc(dt, r, o, i, P(go), (o, 1), P(w), (i, 1), P(gx), (i, 1), accumulate=True),
-             fl, es * (r * o + i * o + 2 * r * i), 200)
+             fl, es * (r * o + i * o + 2 * r * i), 200, bufs=(go, w, gx))
         gemm("c1", "dW 512x64x256 TN col-major C acc",
              dev.gemm_desc(dt, i, r, o, P(x), (1, i), P(go), (o, 1), P(gw), (1, i), accumulate=True),
-             fl, es * (r * o + r * i + 2 * i * o), 200)
+             fl, es * (r * o + r * i + 2 * i * o), 200, bufs=(x, go, gw))
 
     # ---- config 3: [32,512,1024] x [1024,1024], f16, broadcast rhs ---------------------------------------------
     if want("c3"):
@@ -168,28 +219,35 @@ def main():
                                  a_batch=ab, b_batch=bb, c_batch=cb)
 
         gemm("c4", "scores Q.K^T 1024x64x1024 NT", d4(S, D, S, q, (D, 1), sSD, k, (1, D), sSD, sc, (S, 1), sSS, False),
-             fl, es * nb * (2 * S * D + S * S))
+             fl, es * nb * (2 * S * D + S * S), bufs=(q, k, sc))
         gemm("c4", "out P.V 1024x1024x64 NN", d4(S, S, D, p, (S, 1), sSS, v, (D, 1), sSD, o, (D, 1), sSD, False),
-             fl, es * nb * (S * S + 2 * S * D))
+             fl, es * nb * (S * S + 2 * S * D), bufs=(p, v, o))
         gemm("c4", "dP dO.V^T NT acc", d4(S, D, S, d_o, (D, 1), sSD, v, (1, D), sSD, gp, (S, 1), sSS, True),
-             fl, es * nb * (2 * S * D + 2 * S * S))
+             fl, es * nb * (2 * S * D + 2 * S * S), bufs=(d_o, v, gp))
         gemm("c4", "dV P^T.dO TN acc", d4(S, S, D, p, (1, S), sSS, d_o, (D, 1), sSD, gv, (D, 1), sSD, True),
-             fl, es * nb * (S * S + 3 * S * D))
+             fl, es * nb * (S * S + 3 * S * D), bufs=(p, d_o, gv))
         gemm("c4", "dQ dS.K NN acc", d4(S, S, D, gp, (S, 1), sSS, k, (D, 1), sSD, gq, (D, 1), sSD, True),
-             fl, es * nb * (S * S + 3 * S * D))
+             fl, es * nb * (S * S + 3 * S * D), bufs=(gp, k, gq))
         gemm("c4", "dK^T Q^T.dS col-major C acc", d4(D, S, S, q, (1, D), sSD, gp, (S, 1), sSS, gk, (1, D), sSD, True),
-             fl, es * nb * (S * S + 3 * S * D))
+             fl, es * nb * (S * S + 3 * S * D), bufs=(q, gp, gk))
         if want("glue"):
             scv, pv, gpv, ov = view(sc, dt), view(p, dt), view(gp, dt), view(o, dt)
             mat = nb * S * S * es
-            timed("glue", "softmax fwd (8,16,1024,1024) f16, scale folded", lambda: dev.softmax_forward(scv, 0.125), 0, 2 * mat, "softmax_forward")
-            gsv = view(zeros((Bq, H, S, S), dt), dt)
-            timed("glue", "softmax bwd (8,16,1024,1024) f16", lambda: dev.softmax_backward(pv, gsv, gpv, 0.125), 0, 4 * mat, "softmax_backward")
+            vw = lambda t: view(t, dt)
+            timed("glue", "softmax fwd (8,16,1024,1024) f16, scale folded", lambda: dev.softmax_forward(scv, 0.125), 0, 2 * mat, "softmax_forward",
+                  sets=[(lambda a=vw(t): dev.softmax_forward(a, 0.125)) for (t,) in copies(4, sc)])
+            gs = zeros((Bq, H, S, S), dt)
+            gsv = view(gs, dt)
+            timed("glue", "softmax bwd (8,16,1024,1024) f16", lambda: dev.softmax_backward(pv, gsv, gpv, 0.125), 0, 4 * mat, "softmax_backward",
+                  sets=[(lambda a=vw(t0), b=vw(t1), c=vw(t2): dev.softmax_backward(a, b, c, 0.125)) for t0, t1, t2 in copies(4, p, gs, gp)])
             tok = nb * S * D * es
-            timed("glue", "reshape copy (B,H,S,D)->(B,S,H*D) f16", lambda: dev.reshape_forward(ov.permute(0, 2, 1, 3), (Bq, S, H * D)), 0, 2 * tok, "reshape_forward")
-            gt = view(rnd((Bq, S, H * D), dt), dt)
-            gov = view(zeros((Bq, H, S, D), dt), dt)
-            timed("glue", "reshape backward (scatter-add) f16", lambda: dev.reshape_backward(ov.permute(0, 2, 1, 3), gov, gt), 0, 3 * tok, "reshape_backward")
+            timed("glue", "reshape copy (B,H,S,D)->(B,S,H*D) f16", lambda: dev.reshape_forward(ov.permute(0, 2, 1, 3), (Bq, S, H * D)), 0, 2 * tok, "reshape_forward",
+                  sets=[(lambda a=vw(t): dev.reshape_forward(a.permute(0, 2, 1, 3), (Bq, S, H * D))) for (t,) in copies(12, o)])
+            g_t, g_o = rnd((Bq, S, H * D), dt), zeros((Bq, H, S, D), dt)
+            gt, gov = view(g_t, dt), view(g_o, dt)
+            timed("glue", "reshape backward (scatter-add) f16", lambda: dev.reshape_backward(ov.permute(0, 2, 1, 3), gov, gt), 0, 3 * tok, "reshape_backward",
+                  sets=[(lambda a=vw(t0), b=vw(t1), c=vw(t2): dev.reshape_backward(a.permute(0, 2, 1, 3), b, c)) for t0, t1, t2 in copies(8, o, g_o, g_t)])
+            del gs, g_t, g_o
         del sc, p, gp
 
     # ---- config 5: the encoder block's Linears, bf16, 8192 tokens ----------------------------------------------
@@ -207,8 +265,10 @@ def main():
             gemm("c5", f"{name} dW TN col-major C acc",
                  dev.gemm_desc(dt, kin, T, nout, P(x), (1, kin), P(go), (nout, 1), P(gw), (1, kin), accumulate=True), fl, 0)
             if want("glue"):
-                gov, gbv, bv = view(go, dt), view(zeros((nout,), dt), dt), view(rnd((nout,), dt), dt)
-                timed("glue", f"bias backward {T}x{nout} bf16", lambda: dev.bias_backward(gov, gbv), 0, T * nout * 2, "bias_backward")
+                gb = zeros((nout,), dt)
+                gov, gbv = view(go, dt), view(gb, dt)
+                timed("glue", f"bias backward {T}x{nout} bf16", lambda: dev.bias_backward(gov, gbv), 0, T * nout * 2, "bias_backward",
+                      sets=[(lambda a=view(t0, dt), b=view(t1, dt): dev.bias_backward(a, b)) for t0, t1 in copies(nsets((go,)), go, gb)])
 
         # the block's attention products: heads interleaved in the token rows (batch-2 stride 64 < row stride 1024),
         # as MultiHeadAttention's reshape + permute hands them over (multi_head_attention.rs:105-146)
@@ -225,13 +285,13 @@ def main():
                                  a_batch=ab, b_batch=bb, c_batch=cb)
 
         gemm("c5", "attn scores Q.K^T 512x64x512 interleaved", d5(S, D, S, q, (H * D, 1), tok, k, (1, H * D), tok, sc, (S, 1), sSS, False),
-             fl, es * nb * (2 * S * D + S * S))
+             fl, es * nb * (2 * S * D + S * S), bufs=(q, k, sc))
         gemm("c5", "attn out P.V 512x512x64 interleaved V", d5(S, S, D, p_, (S, 1), sSS, v, (H * D, 1), tok, o, (D, 1), sSD, False),
-             fl, es * nb * (S * S + 2 * S * D))
+             fl, es * nb * (S * S + 2 * S * D), bufs=(p_, v, o))
         gemm("c5", "attn dP dO.V^T acc", d5(S, D, S, d_o, (D, 1), sSD, v, (1, H * D), tok, gp, (S, 1), sSS, True),
-             fl, es * nb * (2 * S * D + 2 * S * S))
+             fl, es * nb * (2 * S * D + 2 * S * S), bufs=(d_o, v, gp))
         gemm("c5", "attn dV P^T.dO acc, interleaved rows", d5(S, S, D, p_, (1, S), sSS, d_o, (D, 1), sSD, gv, (H * D, 1), tok, True),
-             fl, es * nb * (S * S + 3 * S * D))
+             fl, es * nb * (S * S + 3 * S * D), bufs=(p_, d_o, gv))
         del sc, p_, gp
 
     # ---- zero fill of gradient storage (Storage::try_alloc_len): HBM write roofline -----------------------------
@@ -242,9 +302,15 @@ def main():
             nbytes = mb << 20
             buf = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
             ptr = ctypes.c_void_p(buf.data_ptr())
+            n = nsets((buf,))
+            more = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(n - 1)]
+            ptrs = [ptr] + [ctypes.c_void_p(t.data_ptr()) for t in more]
             timed("fill", f"zero fill {mb} MiB (dfdx_rocm_memset_zero)",
-                  lambda: dev._check(dev.lib.dfdx_rocm_memset_zero(dev.ctx, ptr, ctypes.c_size_t(nbytes))), 0, nbytes, "zero_fill_kernel")
-            timed("fill", f"zero fill {mb} MiB (torch zero_, for comparison)", lambda: buf.zero_(), 0, nbytes, "torch fill")
+                  lambda: dev._check(dev.lib.dfdx_rocm_memset_zero(dev.ctx, ptr, ctypes.c_size_t(nbytes))), 0, nbytes, "zero_fill_kernel",
+                  sets=[(lambda q=q: dev._check(dev.lib.dfdx_rocm_memset_zero(dev.ctx, q, ctypes.c_size_t(nbytes)))) for q in ptrs])
+            timed("fill", f"zero fill {mb} MiB (torch zero_, for comparison)", lambda: buf.zero_(), 0, nbytes, "torch fill",
+                  sets=[(lambda t=t: t.zero_()) for t in [buf] + more])
+            del more
             del buf
 
     # ---- the vendor library on the same shapes (torch.matmul = hipBLASLt / rocBLAS), for orientation only ---------
@@ -290,9 +356,9 @@ def main():
             es = esz[dt]
             for n_ in (4096, 16384):
                 W, xv, yv = rnd((n_, n_), dt), rnd((n_,), dt), zeros((n_,), dt)
-                gemm("gemv", f"vec.mat {dt} (1,{n_})x({n_},{n_})", dev.gemm_desc(dt, 1, n_, n_, P(xv), (n_, 1), P(W), (n_, 1), P(yv), (n_, 1)), 2 * n_ * n_, es * n_ * n_, 100)
-                gemm("gemv", f"vec.mat {dt}, Linear weight view", dev.gemm_desc(dt, 1, n_, n_, P(xv), (n_, 1), P(W), (1, n_), P(yv), (n_, 1)), 2 * n_ * n_, es * n_ * n_, 100)
-                gemm("gemv", f"mat.vec {dt} ({n_},{n_})x({n_},)", dev.gemm_desc(dt, n_, n_, 1, P(W), (n_, 1), P(xv), (1, 1), P(yv), (1, 1)), 2 * n_ * n_, es * n_ * n_, 100)
+                gemm("gemv", f"vec.mat {dt} (1,{n_})x({n_},{n_})", dev.gemm_desc(dt, 1, n_, n_, P(xv), (n_, 1), P(W), (n_, 1), P(yv), (n_, 1)), 2 * n_ * n_, es * n_ * n_, 100, bufs=(W, xv, yv))
+                gemm("gemv", f"vec.mat {dt}, Linear weight view", dev.gemm_desc(dt, 1, n_, n_, P(xv), (n_, 1), P(W), (1, n_), P(yv), (n_, 1)), 2 * n_ * n_, es * n_ * n_, 100, bufs=(W, xv, yv))
+                gemm("gemv", f"mat.vec {dt} ({n_},{n_})x({n_},)", dev.gemm_desc(dt, n_, n_, 1, P(W), (n_, 1), P(xv), (1, 1), P(yv), (1, 1)), 2 * n_ * n_, es * n_ * n_, 100, bufs=(W, xv, yv))
                 del W
 
     # ---- config 5 end to end: one encoder block, every op on the device -----------------------------------------
@@ -320,13 +386,23 @@ def main():
             _, sv = blk.forward(xv)
             blk.backward(sv, gv)
         timed("block", "encoder block forward + backward", step, 3 * fwd_flop, 0, "EncoderBlock")
-        h = blk.dev.add_forward(xv, xv)
-        timed("glue", f"layer norm fwd ({T},{d}) {dt}", lambda: dev.layer_norm_forward(h, params["g1"], params["be1"]), 0, ln_bytes, "layer_norm_forward")
-        gx, gg, gb = view(zeros((B, S, d), dt), dt), view(zeros((d,), dt), dt), view(zeros((d,), dt), dt)
-        timed("glue", f"layer norm bwd ({T},{d}) {dt}", lambda: dev.layer_norm_backward(h, params["g1"], gx, gg, gb, gv), 0, 2 * ln_bytes, "layer_norm_backward")
-        f1 = view(rnd((B, S, ff), dt), dt)
-        timed("glue", f"relu fwd ({T},{ff}) {dt}", lambda: dev.relu_forward(f1), 0, 2 * T * ff * 2, "relu_forward")
-        timed("glue", f"residual add fwd ({T},{d}) {dt}", lambda: dev.add_forward(xv, h), 0, 3 * T * d * 2, "add_forward")
+        x_t, g_t = rnd((B, S, d), dt), rnd((B, S, d), dt, 1.0 / T)
+        xs, gs_ = view(x_t, dt), view(g_t, dt)
+        vw = lambda t: view(t, dt)
+        g1, be1 = params["g1"], params["be1"]
+        timed("glue", f"layer norm fwd ({T},{d}) {dt}", lambda: dev.layer_norm_forward(xs, g1, be1), 0, ln_bytes, "layer_norm_forward",
+              sets=[(lambda a=vw(t): dev.layer_norm_forward(a, g1, be1)) for (t,) in copies(20, x_t)])
+        gx_t, gg, gb = zeros((B, S, d), dt), view(zeros((d,), dt), dt), view(zeros((d,), dt), dt)
+        gx = view(gx_t, dt)
+        timed("glue", f"layer norm bwd ({T},{d}) {dt}", lambda: dev.layer_norm_backward(xs, g1, gx, gg, gb, gs_), 0, 2 * ln_bytes, "layer_norm_backward",
+              sets=[(lambda a=vw(t0), b=vw(t1), c=vw(t2): dev.layer_norm_backward(a, g1, b, gg, gb, c)) for t0, t1, t2 in copies(8, x_t, gx_t, g_t)])
+        f_t = rnd((B, S, ff), dt)
+        f1 = view(f_t, dt)
+        timed("glue", f"relu fwd ({T},{ff}) {dt}", lambda: dev.relu_forward(f1), 0, 2 * T * ff * 2, "relu_forward",
+              sets=[(lambda a=vw(t): dev.relu_forward(a)) for (t,) in copies(6, f_t)])
+        timed("glue", f"residual add fwd ({T},{d}) {dt}", lambda: dev.add_forward(xs, gs_), 0, 3 * T * d * 2, "add_forward",
+              sets=[(lambda a=vw(t0), b=vw(t1): dev.add_forward(a, b)) for t0, t1 in copies(12, x_t, g_t)])
+        del x_t, g_t, gx_t, f_t
 
     # ---- conv2d (unfold + batched GEMM) -------------------------------------------------------------------------
     if want("conv"):

@@ -122,6 +122,22 @@ int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
     return DFDX_ROCM_OK;
 }
 
+// Frees every buffer the cache holds.  Work that may still use them is drained first.
+int drop_cache(dfdx_rocm_ctx *ctx) {
+    CtxLock lock(ctx->mu);
+    if (ctx->cache.empty()) return DFDX_ROCM_OK;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    hipError_t first = hipSuccess;
+    for (auto &kv : ctx->cache)
+        for (void *p : kv.second) {
+            const hipError_t e = hipFree(p);
+            if (first == hipSuccess) first = e;
+        }
+    ctx->cache.clear();
+    ctx->cache_bytes = 0;
+    return (int)first;
+}
+
 struct Plan {
     int kernel, variant, splits;
 };
@@ -254,11 +270,12 @@ int dfdx_rocm_create(int ordinal, void *stream, dfdx_rocm_ctx **out) {
 
 int dfdx_rocm_destroy(dfdx_rocm_ctx *ctx) {
     if (!ctx) return DFDX_ROCM_OK;
-    if (ctx->workspace || ctx->patches) {
+    if (ctx->workspace || ctx->patches || !ctx->cache.empty()) {
         (void)hipSetDevice(ctx->device);
         (void)hipStreamSynchronize(ctx->stream);
         if (ctx->workspace) (void)hipFree(ctx->workspace);
         if (ctx->patches) (void)hipFree(ctx->patches);
+        (void)drop_cache(ctx);
     }
     delete ctx;
     return DFDX_ROCM_OK;
@@ -293,11 +310,35 @@ int dfdx_rocm_alloc(dfdx_rocm_ctx *ctx, size_t bytes, int zeroed, void **out) {
     if (int e = bind(ctx)) return e;
     if (bytes == 0) bytes = 16;
     void *p = nullptr;
-    HIP_TRY(hipMalloc(&p, bytes));
+    bool recycled = false;
+    {   // a cached buffer of exactly this size, if the cache is on and has one (cache.rs:105-149)
+        CtxLock lock(ctx->mu);
+        if (ctx->cache_enabled) {
+            auto it = ctx->cache.find(bytes);
+            if (it != ctx->cache.end()) {
+                p = it->second.back();
+                it->second.pop_back();
+                if (it->second.empty()) ctx->cache.erase(it);
+                ctx->cache_bytes -= bytes;
+                recycled = true;
+            }
+        }
+    }
+    if (!recycled) {
+        const hipError_t e = hipMalloc(&p, bytes);
+        if (e == hipErrorOutOfMemory && dfdx_rocm_empty_cache(ctx) == DFDX_ROCM_OK) {
+            (void)hipGetLastError();
+            HIP_TRY(hipMalloc(&p, bytes));  // once more with the cached buffers given back
+        } else if (e != hipSuccess) {
+            return (int)e;
+        }
+        CtxLock lock(ctx->mu);
+        ctx->sizes[p] = bytes;
+    }
     if (zeroed) {
         hipError_t e = launch_zero_fill(p, bytes, ctx->compute_units, ctx->stream);
         if (e != hipSuccess) {
-            (void)hipFree(p);
+            (void)dfdx_rocm_free(ctx, p);
             return (int)e;
         }
     }
@@ -308,8 +349,54 @@ int dfdx_rocm_alloc(dfdx_rocm_ctx *ctx, size_t bytes, int zeroed, void **out) {
 int dfdx_rocm_free(dfdx_rocm_ctx *ctx, void *ptr) {
     if (int e = bind(ctx)) return e;
     if (!ptr) return DFDX_ROCM_OK;
+    {
+        CtxLock lock(ctx->mu);
+        auto it = ctx->sizes.find(ptr);
+        if (it != ctx->sizes.end() && ctx->cache_enabled) {
+            // Kept for the next allocation of this size.  No synchronisation: whoever gets the buffer next uses it
+            // through this context's stream, behind the work that still reads it.
+            ctx->cache[it->second].push_back(ptr);
+            ctx->cache_bytes += it->second;
+            return DFDX_ROCM_OK;
+        }
+        if (it != ctx->sizes.end()) ctx->sizes.erase(it);
+    }
     HIP_TRY(hipStreamSynchronize(ctx->stream));  // pending kernels may still use the buffer
     HIP_TRY(hipFree(ptr));
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_enable_cache(dfdx_rocm_ctx *ctx) {
+    if (!ctx) return DFDX_ROCM_ERR_INVALID_ARG;
+    CtxLock lock(ctx->mu);
+    ctx->cache_enabled = true;
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_disable_cache(dfdx_rocm_ctx *ctx) {
+    if (int e = bind(ctx)) return e;
+    {
+        CtxLock lock(ctx->mu);
+        ctx->cache_enabled = false;
+    }
+    return dfdx_rocm_empty_cache(ctx);
+}
+
+int dfdx_rocm_empty_cache(dfdx_rocm_ctx *ctx) {
+    if (int e = bind(ctx)) return e;
+    CtxLock lock(ctx->mu);
+    for (auto &kv : ctx->cache)
+        for (void *p : kv.second) ctx->sizes.erase(p);
+    return drop_cache(ctx);
+}
+
+int dfdx_rocm_cache_stats(dfdx_rocm_ctx *ctx, size_t *buffers, size_t *bytes) {
+    if (!ctx) return DFDX_ROCM_ERR_INVALID_ARG;
+    CtxLock lock(ctx->mu);
+    size_t n = 0;
+    for (auto &kv : ctx->cache) n += kv.second.size();
+    if (buffers) *buffers = n;
+    if (bytes) *bytes = ctx->cache_bytes;
     return DFDX_ROCM_OK;
 }
 
@@ -402,25 +489,29 @@ int dfdx_rocm_mfma_variant_count(int dtype) {
     return 0;
 }
 
-int dfdx_rocm_gemm_time(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int warmup, int iters, float *avg_ms) {
-    if (!avg_ms || iters < 1 || warmup < 0) return DFDX_ROCM_ERR_INVALID_ARG;
+int dfdx_rocm_gemm_time_rotating(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *descs, int count, int warmup, int iters,
+                                 float *avg_ms) {
+    if (!avg_ms || !descs || count < 1 || iters < 1 || warmup < 0) return DFDX_ROCM_ERR_INVALID_ARG;
     if (int e = bind(ctx)) return e;
-    GemmProblem p;
-    if (int e = make_problem(desc, &p)) return e;
-    if (p.m == 0) {
-        *avg_ms = 0.0f;
-        return DFDX_ROCM_OK;
+    std::vector<GemmProblem> problems((size_t)count);
+    std::vector<Plan> plans((size_t)count);
+    for (int i = 0; i < count; i++) {
+        if (int e = make_problem(&descs[i], &problems[(size_t)i])) return e;
+        if (problems[(size_t)i].m == 0) {   // an empty product launches nothing: there is no time to report
+            *avg_ms = 0.0f;
+            return DFDX_ROCM_OK;
+        }
+        if (int e = make_plan(ctx, &descs[i], problems[(size_t)i], &plans[(size_t)i])) return e;
     }
-    Plan plan;
-    if (int e = make_plan(ctx, desc, p, &plan)) return e;
     for (int i = 0; i < warmup; i++)
-        if (int e = run_plan(ctx, p, plan)) return e;
+        if (int e = run_plan(ctx, problems[(size_t)(i % count)], plans[(size_t)(i % count)])) return e;
     hipEvent_t t0, t1;
     HIP_TRY(hipEventCreate(&t0));
     HIP_TRY(hipEventCreate(&t1));
     int rc = DFDX_ROCM_OK;
     hipError_t he = hipEventRecord(t0, ctx->stream);
-    for (int i = 0; i < iters && rc == DFDX_ROCM_OK && he == hipSuccess; i++) rc = run_plan(ctx, p, plan);
+    for (int i = 0; i < iters && rc == DFDX_ROCM_OK && he == hipSuccess; i++)
+        rc = run_plan(ctx, problems[(size_t)(i % count)], plans[(size_t)(i % count)]);
     if (he == hipSuccess) he = hipEventRecord(t1, ctx->stream);
     if (he == hipSuccess) he = hipEventSynchronize(t1);
     float ms = 0.0f;
@@ -431,6 +522,10 @@ int dfdx_rocm_gemm_time(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int
     if (he != hipSuccess) return (int)he;
     *avg_ms = ms / (float)iters;
     return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_gemm_time(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int warmup, int iters, float *avg_ms) {
+    return dfdx_rocm_gemm_time_rotating(ctx, desc, desc ? 1 : 0, warmup, iters, avg_ms);
 }
 
 }  // extern "C"

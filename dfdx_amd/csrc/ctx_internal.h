@@ -3,7 +3,9 @@
 #include "../../include/dfdx_rocm.h"
 
 #include <hip/hip_runtime.h>
+#include <map>
 #include <mutex>
+#include <vector>
 
 struct dfdx_rocm_ctx {
     int device;
@@ -17,6 +19,14 @@ struct dfdx_rocm_ctx {
     void *workspace = nullptr;  // partial sums of split reductions; grown on demand, owned by the context
     size_t workspace_bytes = 0;
     void *static_scratch = nullptr;  // this device's copy of the fixed scratch array of dfdx_rocm_gemm_noalloc (never freed)
+    // The allocation cache (tensor/cache.rs:36-149): freed buffers kept by size for the next dfdx_rocm_alloc of that size.
+    // Off until dfdx_rocm_enable_cache.  The reference keys on (bytes, element size, alignment) because the Rust
+    // allocator wants a buffer back with the layout it was made with; device allocations are all 256 B-aligned raw
+    // bytes, so the key here is the byte count.
+    bool cache_enabled = false;
+    std::map<size_t, std::vector<void *>> cache;
+    size_t cache_bytes = 0;
+    std::map<void *, size_t> sizes;  // every live buffer of dfdx_rocm_alloc (free learns the size from here)
     void *patches = nullptr;  // unfolded images of conv2d (alive across the GEMMs that may regrow `workspace`)
     size_t patches_bytes = 0;
 };

@@ -72,8 +72,9 @@ _lib = None
 EXPORTS = [
     "dfdx_rocm_create", "dfdx_rocm_destroy", "dfdx_rocm_strerror", "dfdx_rocm_device_info",
     "dfdx_rocm_alloc", "dfdx_rocm_free", "dfdx_rocm_memset_zero", "dfdx_rocm_copy_h2d", "dfdx_rocm_copy_d2h",
-    "dfdx_rocm_copy_d2d", "dfdx_rocm_synchronize", "dfdx_rocm_gemm", "dfdx_rocm_gemm_noalloc", "dfdx_rocm_gemm_plan",
-    "dfdx_rocm_mfma_variant_count", "dfdx_rocm_gemm_time",
+    "dfdx_rocm_copy_d2d", "dfdx_rocm_synchronize", "dfdx_rocm_enable_cache", "dfdx_rocm_disable_cache",
+    "dfdx_rocm_empty_cache", "dfdx_rocm_cache_stats", "dfdx_rocm_gemm", "dfdx_rocm_gemm_noalloc", "dfdx_rocm_gemm_plan",
+    "dfdx_rocm_mfma_variant_count", "dfdx_rocm_gemm_time", "dfdx_rocm_gemm_time_rotating",
     "dfdx_rocm_matmat_forward", "dfdx_rocm_matmat_backward",
     "dfdx_rocm_matmat_br_forward", "dfdx_rocm_matmat_br_backward",
     "dfdx_rocm_matmat_batch3_forward", "dfdx_rocm_matmat_batch3_backward",
@@ -185,6 +186,31 @@ class Rocm:
         self._check(self.lib.dfdx_rocm_device_info(self.ctx, name, 128, ctypes.byref(cus), ctypes.byref(mhz)))
         return {"name": name.value.decode(), "compute_units": cus.value, "clock_mhz": mhz.value}
 
+    # ----------------------------------------------------------------- cache --
+    def enable_cache(self):
+        """``Cache::enable_cache`` (tensor/storage_traits.rs:41-77): freed buffers are kept for the next allocation of their size."""
+        self._check(self.lib.dfdx_rocm_enable_cache(self.ctx))
+
+    def disable_cache(self):
+        self._check(self.lib.dfdx_rocm_disable_cache(self.ctx))
+
+    def empty_cache(self):
+        self._check(self.lib.dfdx_rocm_empty_cache(self.ctx))
+
+    def cache_stats(self):
+        n, b = ctypes.c_size_t(), ctypes.c_size_t()
+        self._check(self.lib.dfdx_rocm_cache_stats(self.ctx, ctypes.byref(n), ctypes.byref(b)))
+        return n.value, b.value
+
+    def alloc(self, nbytes: int, zeroed: bool = True) -> int:
+        """``Storage::try_alloc_len`` / ``alloc_empty`` through the library's own allocator; returns the device address."""
+        p = ctypes.c_void_p()
+        self._check(self.lib.dfdx_rocm_alloc(self.ctx, ctypes.c_size_t(nbytes), int(zeroed), ctypes.byref(p)))
+        return p.value
+
+    def free(self, ptr: int):
+        self._check(self.lib.dfdx_rocm_free(self.ctx, ctypes.c_void_p(ptr)))
+
     # --------------------------------------------------------------- storage --
     def tensor(self, host: np.ndarray, dtype: str, shape=None, strides=None) -> View:
         """Upload ``host`` (storage order) and view it; bf16 storage is given as uint16 bit patterns."""
@@ -279,6 +305,13 @@ class Rocm:
     def gemm_time(self, desc: GemmDesc, warmup: int, iters: int) -> float:
         ms = ctypes.c_float()
         self._check(self.lib.dfdx_rocm_gemm_time(self.ctx, ctypes.byref(desc), warmup, iters, ctypes.byref(ms)))
+        return ms.value
+
+    def gemm_time_rotating(self, descs, warmup: int, iters: int) -> float:
+        """Average ms per launch with launch i running ``descs[i % len(descs)]`` (each on its own buffers)."""
+        arr = (GemmDesc * len(descs))(*descs)
+        ms = ctypes.c_float()
+        self._check(self.lib.dfdx_rocm_gemm_time_rotating(self.ctx, arr, len(descs), warmup, iters, ctypes.byref(ms)))
         return ms.value
 
     def mfma_variant_count(self, dtype: str) -> int:

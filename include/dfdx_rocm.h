@@ -88,6 +88,25 @@ int dfdx_rocm_copy_d2h(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t by
 int dfdx_rocm_copy_d2d(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes);
 int dfdx_rocm_synchronize(dfdx_rocm_ctx *ctx);
 
+/* The allocation cache of the device (`Cache::try_enable_cache`,
+ * `try_disable_cache`, `try_empty_cache`: dfdx-core/src/tensor/
+ * storage_traits.rs:41-77; `TensorCache`, tensor/cache.rs:36-149, which the
+ * Cuda device consults in `try_alloc_len` and feeds from `Drop`).  Off at
+ * first, as in the reference.  While it is on, dfdx_rocm_free keeps the
+ * buffer (no synchronisation, no hipFree) and the next dfdx_rocm_alloc of
+ * exactly that many bytes gets it back (zero-filled again when asked): a
+ * training step's gradient buffers then cost no hipMalloc / hipFree after
+ * the first step.  The reference keys on (bytes, element size, alignment)
+ * for the sake of the Rust allocator; device buffers are 256 B-aligned raw
+ * bytes, so the key is the byte count.  disable also empties; empty frees
+ * what is held (after draining the stream); an allocation that fails for
+ * lack of memory empties the cache and tries once more.
+ * dfdx_rocm_cache_stats reports what is held right now (tests, tooling). */
+int dfdx_rocm_enable_cache(dfdx_rocm_ctx *ctx);
+int dfdx_rocm_disable_cache(dfdx_rocm_ctx *ctx);
+int dfdx_rocm_empty_cache(dfdx_rocm_ctx *ctx);
+int dfdx_rocm_cache_stats(dfdx_rocm_ctx *ctx, size_t *buffers, size_t *bytes);
+
 /* ---- the strided (batched) GEMM -------------------------------------------
  * Stands in for `MatMulImpl::matmul` on Cpu
  * (dfdx-core/src/tensor_ops/matmul/cpu_kernel.rs:38-50) and for `Cuda::gemm` /
@@ -164,6 +183,12 @@ int dfdx_rocm_mfma_variant_count(int dtype);
  * (dfdx's benches time with `Instant` around `synchronize`,
  * dfdx/benches/conv2d.rs:25-45). */
 int dfdx_rocm_gemm_time(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int warmup, int iters, float *avg_ms);
+/* The same over `count` descriptors taken in turn (launch i runs descs[i % count]):
+ * with each descriptor on its own buffers and more bytes in flight than the
+ * 256 MB last-level cache holds, every launch reads HBM, not the previous
+ * launch's lines.  Benchmark aid; no reference counterpart. */
+int dfdx_rocm_gemm_time_rotating(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *descs, int count, int warmup, int iters,
+                                 float *avg_ms);
 
 /* ---- the four kernel traits -------------------------------------------------
  * One function per trait method.  `out` and `grad_out` are contiguous

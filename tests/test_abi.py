@@ -29,13 +29,27 @@ def test_header_symbols_are_all_exported():
     assert sorted(EXPORTS) == declared, "python binding list and header disagree"
 
 
+def test_integration_binding_lists_every_symbol():
+    """INTEGRATION.md's Rust `extern "C"` block declares every exported symbol except the four test / tooling aids it
+    names as left out."""
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    block = text[text.index('extern "C" {'):]
+    block = block[:block.index("```")]
+    bound = set(re.findall(r"pub fn (dfdx_rocm_[a-z0-9_]+)\(", block))
+    left_out = {"dfdx_rocm_gemm_plan", "dfdx_rocm_gemm_time", "dfdx_rocm_gemm_time_rotating", "dfdx_rocm_mfma_variant_count", "dfdx_rocm_cache_stats"}
+    assert bound == set(declared_symbols()) - left_out
+    for name in left_out:
+        assert name in text[:text.index('extern "C" {')]   # named where the binding says what it leaves out
+
+
 def test_every_declaration_cites_the_reference():
     """Each block of declarations names the reference interface it replaces (file:line)."""
     text = open(HEADER).read()
     for needle in ("cpu_kernel.rs:38-50", "cuda_kernel.rs:153-181", "matmul/mod.rs:116-131", "matmul/mod.rs:197-212",
                    "matmul/mod.rs:234-249", "matmul/mod.rs:273-288", "linear.rs:82-89", "cuda/device.rs:259-266",
                    "bias1d.rs:62-78", "utilities/cpu_kernels.rs:164-203", "softmax.rs:70-83", "mul/cpu_kernel.rs:\n * 5-17",
-                   "reshape_to/mod.rs:90-115", "conv2d/mod.rs:31-55", "multi_head_attention.rs:\n * 105-146"):
+                   "reshape_to/mod.rs:90-115", "conv2d/mod.rs:31-55", "multi_head_attention.rs:\n * 105-146",
+                   "storage_traits.rs:41-77", "tensor/cache.rs:36-149"):
         assert needle in text, needle
 
 

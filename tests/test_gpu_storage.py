@@ -48,3 +48,48 @@ def test_zeros_views_are_zero():
     assert not dev.to_host(v).any()
     w = dev.zeros_like_storage(dev.tensor(np.ones(1000, np.float32), "f32"))
     assert not dev.to_host(w).any()
+
+
+def test_allocation_cache_reuses_and_releases():
+    """`Cache` (tensor/storage_traits.rs:41-77) over `TensorCache` semantics (tensor/cache.rs:105-149, and its own unit
+    tests :192-260): off at first; while on, a freed buffer is handed to the next allocation of exactly its size (and to
+    no other size), zero-filled again when asked; `empty` and `disable` give everything back."""
+    dev = device()
+    announce("allocation cache")
+    assert dev.cache_stats() == (0, 0)
+    a = dev.alloc(1 << 20)
+    dev.free(a)
+    assert dev.cache_stats() == (0, 0)                 # disabled: freed for real
+    dev.enable_cache()
+    try:
+        a = dev.alloc(1 << 20, zeroed=False)
+        b = dev.alloc(1 << 20, zeroed=False)
+        c = dev.alloc(4096, zeroed=False)
+        ones = np.full(1 << 20, 0x77, np.uint8)
+        dev._check(dev.lib.dfdx_rocm_copy_h2d(dev.ctx, ctypes.c_void_p(a), ones.ctypes.data_as(ctypes.c_void_p), ctypes.c_size_t(ones.nbytes)))
+        dev.free(a)
+        dev.free(c)
+        assert dev.cache_stats() == (2, (1 << 20) + 4096)
+        d = dev.alloc(2 << 20, zeroed=False)           # another size: a fresh buffer, the cache keeps its two
+        assert d not in (a, c) and dev.cache_stats() == (2, (1 << 20) + 4096)
+        e = dev.alloc(1 << 20, zeroed=True)            # same size: the cached buffer, cleared again
+        assert e == a and dev.cache_stats() == (1, 4096)
+        host = np.full(1 << 20, 0x5A, np.uint8)
+        dev._check(dev.lib.dfdx_rocm_copy_d2h(dev.ctx, host.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(e), ctypes.c_size_t(host.nbytes)))
+        assert not host.any()
+        f = dev.alloc(4096, zeroed=False)
+        assert f == c and dev.cache_stats() == (0, 0)
+        for p in (b, d, e, f):
+            dev.free(p)
+        assert dev.cache_stats() == (4, (1 << 20) * 2 + (2 << 20) + 4096)
+        dev.empty_cache()
+        assert dev.cache_stats() == (0, 0)
+        g = dev.alloc(1 << 20)
+        dev.free(g)
+        assert dev.cache_stats()[0] == 1
+    finally:
+        dev.disable_cache()                            # also empties
+    assert dev.cache_stats() == (0, 0)
+    h = dev.alloc(64)
+    dev.free(h)
+    assert dev.cache_stats() == (0, 0)
