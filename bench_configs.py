@@ -23,9 +23,10 @@ def main():
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
     ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (and torch: vendor-library cross-check, only on request)")
-    ap.add_argument("--probe", default="", choices=["", "traffic", "variants", "mfma-power"],
+    ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "mfma-power"],
                     help="counter-collection aids for rocprofv3, nothing is timed: traffic = 3 plain 256 MiB device copies (a kernel "
-                         "of known size that calibrates FETCH_SIZE / WRITE_SIZE) then 5 launches of the 4096^3 f16 GEMM; variants = 3 "
+                         "of known size that calibrates FETCH_SIZE / WRITE_SIZE) then 5 launches of the 4096^3 f16 GEMM; rows = the same copies, then 3 launches each of "
+                         "the HBM-bound rows (config 4 scores and dP, softmax forward and backward on them, the 16384^2 f16 vec.mat); variants = 3 "
                          "launches of that GEMM with every f16 MFMA tile variant forced in turn; mfma-power = the stand-alone "
                          "MFMA-only program (built by `make -C dfdx_amd/csrc probe`)")
     ap.add_argument("--no-rotate", action="store_true", help="skip the second timing of the HBM-bound cases over rotating buffer sets")
@@ -64,6 +65,40 @@ def main():
                 dev.gemm(desc)
             torch.cuda.synchronize()
             print(json.dumps({"probe": "3 x 256 MiB copy, 5 x " + dev.gemm_plan(desc)[2]}))
+        elif args.probe == "rows":
+            del a, b, c
+            src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+            del src, dst
+            Bq, H, S, D = 8, 16, 1024, 64
+            sSD, sSS = (H * S * D, S * D), (H * S * S, S * S)
+            q, k, v, d_o = ((torch.randn(Bq, H, S, D, device="cuda")).half() for _ in range(4))
+            sc = torch.zeros(Bq, H, S, S, device="cuda", dtype=torch.float16)
+            gp, gs = torch.zeros_like(sc), torch.zeros_like(sc)
+            P = lambda t: t.data_ptr()
+            vw = lambda t: View(t.view(torch.uint8).reshape(-1), "f16", tuple(t.shape), tuple(t.stride()))
+            scores = dev.gemm_desc("f16", S, D, S, P(q), (D, 1), P(k), (1, D), P(sc), (S, 1), batch=(Bq, H), a_batch=sSD, b_batch=sSD, c_batch=sSS)
+            dp = dev.gemm_desc("f16", S, D, S, P(d_o), (D, 1), P(v), (1, D), P(gp), (S, 1), accumulate=True, batch=(Bq, H),
+                               a_batch=sSD, b_batch=sSD, c_batch=sSS)
+            n_ = 16384
+            W, xv, yv = torch.randn(n_, n_, device="cuda").half(), torch.randn(n_, device="cuda").half(), torch.zeros(n_, device="cuda").half()
+            gv = dev.gemm_desc("f16", 1, n_, n_, P(xv), (n_, 1), P(W), (n_, 1), P(yv), (n_, 1))
+            names = []
+            for desc in (scores, dp, gv):
+                names.append(dev.gemm_plan(desc)[2])
+                for _ in range(3):
+                    dev.gemm(desc)
+                torch.cuda.synchronize()
+            for _ in range(3):
+                prob = dev.softmax_forward(vw(sc), 0.125)
+                torch.cuda.synchronize()
+            for _ in range(3):
+                dev.softmax_backward(prob, vw(gs), vw(gp), 0.125)
+                torch.cuda.synchronize()
+            print(json.dumps({"probe": ["3 x 256 MiB copy"] + names + ["softmax_forward", "softmax_backward"]}))
         else:
             names = []
             for v in range(1, dev.mfma_variant_count("f16") + 1):
