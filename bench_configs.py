@@ -415,7 +415,7 @@ def main():
         ln_bytes = 2 * (2 * T * d * 2)
         timed("block", "encoder block forward (20 calls)", lambda: blk.forward(xv), fwd_flop, 0, "EncoderBlock.forward")
         _, saved = blk.forward(xv)
-        timed("block", "encoder block backward (37 calls + 1 zero fill of all grads)", lambda: blk.backward(saved, gv), 2 * fwd_flop, 0, "EncoderBlock.backward")
+        timed("block", "encoder block backward (37 calls, gradient zeros deferred)", lambda: blk.backward(saved, gv), 2 * fwd_flop, 0, "EncoderBlock.backward")
 
         def step():
             _, sv = blk.forward(xv)

@@ -30,6 +30,109 @@ static int grow(dfdx_rocm_ctx *ctx, void **buf, size_t *have, size_t bytes) {
     return DFDX_ROCM_OK;
 }
 
+static std::map<uintptr_t, size_t>::iterator pending_holding(dfdx_rocm_ctx *ctx, uintptr_t p) {
+    auto it = ctx->pending_zero.upper_bound(p);
+    if (it == ctx->pending_zero.begin()) return ctx->pending_zero.end();
+    --it;
+    return p < it->first + it->second ? it : ctx->pending_zero.end();
+}
+
+static int fill_and_drop(dfdx_rocm_ctx *ctx, std::map<uintptr_t, size_t>::iterator it) {
+    const hipError_t e = launch_zero_fill((void *)it->first, it->second, ctx->compute_units, ctx->stream);
+    if (e != hipSuccess) return (int)e;
+    ctx->pending_zero.erase(it);
+    ctx->pending_count.store((int)ctx->pending_zero.size(), std::memory_order_release);
+    return DFDX_ROCM_OK;
+}
+
+int settle(dfdx_rocm_ctx *ctx, const void *ptr) {
+    if (!ptr || ctx->pending_count.load(std::memory_order_acquire) == 0) return DFDX_ROCM_OK;
+    CtxLock lock(ctx->mu);
+    auto it = pending_holding(ctx, (uintptr_t)ptr);
+    return it == ctx->pending_zero.end() ? DFDX_ROCM_OK : fill_and_drop(ctx, it);
+}
+
+int settle_output(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes, bool accumulates, bool *fresh) {
+    if (fresh) *fresh = false;
+    if (!ptr || ctx->pending_count.load(std::memory_order_acquire) == 0) return DFDX_ROCM_OK;
+    CtxLock lock(ctx->mu);
+    auto it = pending_holding(ctx, (uintptr_t)ptr);
+    if (it == ctx->pending_zero.end()) return DFDX_ROCM_OK;
+    const bool covered = bytes && it->first == (uintptr_t)ptr && it->second == bytes;
+    if (covered && (!accumulates || fresh)) {  // every byte is stored without being read first: no fill needed
+        ctx->pending_zero.erase(it);
+        ctx->pending_count.store((int)ctx->pending_zero.size(), std::memory_order_release);
+        if (fresh) *fresh = accumulates;
+        return DFDX_ROCM_OK;
+    }
+    return fill_and_drop(ctx, it);
+}
+
+// Runs every deferred fill that overlaps [ptr, ptr + bytes) (a read of that range follows).
+static int settle_range(dfdx_rocm_ctx *ctx, const void *ptr, size_t bytes) {
+    if (!ptr || ctx->pending_count.load(std::memory_order_acquire) == 0) return DFDX_ROCM_OK;
+    CtxLock lock(ctx->mu);
+    const uintptr_t lo = (uintptr_t)ptr, hi = lo + bytes;
+    auto first = pending_holding(ctx, lo);
+    if (first != ctx->pending_zero.end())
+        if (int e = fill_and_drop(ctx, first)) return e;
+    for (auto it = ctx->pending_zero.lower_bound(lo); it != ctx->pending_zero.end() && it->first < hi;
+         it = ctx->pending_zero.lower_bound(lo))
+        if (int e = fill_and_drop(ctx, it)) return e;
+    return DFDX_ROCM_OK;
+}
+
+// Forgets (without filling) every deferred fill that lies wholly inside [ptr, ptr + bytes); one that straddles an end is run.
+static int drop_pending_inside(dfdx_rocm_ctx *ctx, const void *ptr, size_t bytes) {
+    if (!ptr || ctx->pending_count.load(std::memory_order_acquire) == 0) return DFDX_ROCM_OK;
+    CtxLock lock(ctx->mu);
+    const uintptr_t lo = (uintptr_t)ptr, hi = lo + bytes;
+    auto first = pending_holding(ctx, lo);
+    if (first != ctx->pending_zero.end() && first->first < lo)
+        if (int e = fill_and_drop(ctx, first)) return e;
+    for (auto it = ctx->pending_zero.lower_bound(lo); it != ctx->pending_zero.end() && it->first < hi;) {
+        if (it->first + it->second > hi) {
+            if (int e = fill_and_drop(ctx, it)) return e;
+            break;
+        }
+        it = ctx->pending_zero.erase(it);
+    }
+    ctx->pending_count.store((int)ctx->pending_zero.size(), std::memory_order_release);
+    return DFDX_ROCM_OK;
+}
+
+int settle_all(dfdx_rocm_ctx *ctx) {
+    if (ctx->pending_count.load(std::memory_order_acquire) == 0) return DFDX_ROCM_OK;
+    CtxLock lock(ctx->mu);
+    while (!ctx->pending_zero.empty())
+        if (int e = fill_and_drop(ctx, ctx->pending_zero.begin())) return e;
+    return DFDX_ROCM_OK;
+}
+
+size_t dense_bytes(int rank, const int64_t *extents, const int64_t *strides, size_t elem_bytes) {
+    int64_t ext[8], str[8];
+    int n = 0;
+    if (rank > 8) return 0;
+    for (int i = 0; i < rank; i++) {
+        if (extents[i] == 0) return 0;
+        if (extents[i] == 1) continue;
+        if (strides[i] <= 0) return 0;
+        int j = n++;
+        for (; j > 0 && str[j - 1] > strides[i]; j--) {  // insertion sort by stride
+            ext[j] = ext[j - 1];
+            str[j] = str[j - 1];
+        }
+        ext[j] = extents[i];
+        str[j] = strides[i];
+    }
+    int64_t run = 1;
+    for (int i = 0; i < n; i++) {
+        if (str[i] != run) return 0;
+        run *= ext[i];
+    }
+    return (size_t)run * elem_bytes;
+}
+
 int ensure_workspace(dfdx_rocm_ctx *ctx, size_t bytes) { return grow(ctx, &ctx->workspace, &ctx->workspace_bytes, bytes); }
 int ensure_patches(dfdx_rocm_ctx *ctx, size_t bytes) { return grow(ctx, &ctx->patches, &ctx->patches_bytes, bytes); }
 
@@ -241,6 +344,24 @@ int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan, b
     return (int)e;
 }
 
+// Deferred zero fills among the operands: inputs are filled now; an accumulation that covers the whole of a pending C
+// becomes a plain store (`may_overwrite`), which leaves the same bits as 0 + value.
+int settle_operands(dfdx_rocm_ctx *ctx, GemmProblem *p, bool may_overwrite) {
+    if (ctx->pending_count.load(std::memory_order_acquire) == 0) return DFDX_ROCM_OK;
+    if (p->k > 0) {
+        if (int e = settle(ctx, p->a)) return e;
+        if (int e = settle(ctx, p->b)) return e;
+    }
+    if (int e = settle(ctx, p->bias)) return e;
+    const int64_t ext[4] = {p->reduce ? 1 : p->nb1, p->reduce ? 1 : p->nb2, p->m, p->n};
+    const int64_t str[4] = {p->c_b1, p->c_b2, p->c_rs, p->c_cs};
+    const size_t es = p->dtype == DT_F64 ? 8 : p->dtype == DT_F32 ? 4 : 2;
+    bool fresh = false;
+    if (int e = settle_output(ctx, p->c, dense_bytes(4, ext, str, es), p->accumulate, may_overwrite ? &fresh : nullptr)) return e;
+    if (fresh) p->accumulate = false;
+    return DFDX_ROCM_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -270,8 +391,9 @@ int dfdx_rocm_create(int ordinal, void *stream, dfdx_rocm_ctx **out) {
 
 int dfdx_rocm_destroy(dfdx_rocm_ctx *ctx) {
     if (!ctx) return DFDX_ROCM_OK;
-    if (ctx->workspace || ctx->patches || !ctx->cache.empty()) {
+    if (ctx->workspace || ctx->patches || !ctx->cache.empty() || ctx->pending_count.load()) {
         (void)hipSetDevice(ctx->device);
+        (void)settle_all(ctx);  // the caller's buffers outlive the context: they must hold the zeros they were promised
         (void)hipStreamSynchronize(ctx->stream);
         if (ctx->workspace) (void)hipFree(ctx->workspace);
         if (ctx->patches) (void)hipFree(ctx->patches);
@@ -335,7 +457,11 @@ int dfdx_rocm_alloc(dfdx_rocm_ctx *ctx, size_t bytes, int zeroed, void **out) {
         CtxLock lock(ctx->mu);
         ctx->sizes[p] = bytes;
     }
-    if (zeroed) {
+    if (zeroed == DFDX_ROCM_ZERO_DEFERRED) {
+        CtxLock lock(ctx->mu);
+        ctx->pending_zero[(uintptr_t)p] = bytes;
+        ctx->pending_count.store((int)ctx->pending_zero.size(), std::memory_order_release);
+    } else if (zeroed) {
         hipError_t e = launch_zero_fill(p, bytes, ctx->compute_units, ctx->stream);
         if (e != hipSuccess) {
             (void)dfdx_rocm_free(ctx, p);
@@ -352,6 +478,13 @@ int dfdx_rocm_free(dfdx_rocm_ctx *ctx, void *ptr) {
     {
         CtxLock lock(ctx->mu);
         auto it = ctx->sizes.find(ptr);
+        if (ctx->pending_count.load(std::memory_order_acquire)) {  // a fill nobody waited for is not run
+            if (it != ctx->sizes.end()) {
+                if (int e = drop_pending_inside(ctx, ptr, it->second)) return e;
+            } else if (ctx->pending_zero.erase((uintptr_t)ptr)) {
+                ctx->pending_count.store((int)ctx->pending_zero.size(), std::memory_order_release);
+            }
+        }
         if (it != ctx->sizes.end() && ctx->cache_enabled) {
             // Kept for the next allocation of this size.  No synchronisation: whoever gets the buffer next uses it
             // through this context's stream, behind the work that still reads it.
@@ -403,14 +536,36 @@ int dfdx_rocm_cache_stats(dfdx_rocm_ctx *ctx, size_t *buffers, size_t *bytes) {
 int dfdx_rocm_memset_zero(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes) {
     if (int e = bind(ctx)) return e;
     if (!ptr && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
-    if (bytes) HIP_TRY(launch_zero_fill(ptr, bytes, ctx->compute_units, ctx->stream));
+    if (bytes) {
+        if (int e = drop_pending_inside(ctx, ptr, bytes)) return e;
+        HIP_TRY(launch_zero_fill(ptr, bytes, ctx->compute_units, ctx->stream));
+    }
     return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_zero_deferred(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes) {
+    if (int e = bind(ctx)) return e;
+    if (!ptr && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (!bytes) return DFDX_ROCM_OK;
+    if (int e = drop_pending_inside(ctx, ptr, bytes)) return e;  // earlier declarations inside the range are replaced
+    CtxLock lock(ctx->mu);
+    if (pending_holding(ctx, (uintptr_t)ptr) != ctx->pending_zero.end())  // still inside a larger pending buffer
+        return DFDX_ROCM_OK;                                             // which already stands for these zeros
+    ctx->pending_zero[(uintptr_t)ptr] = bytes;
+    ctx->pending_count.store((int)ctx->pending_zero.size(), std::memory_order_release);
+    return DFDX_ROCM_OK;
+}
+
+int dfdx_rocm_settle_zeros(dfdx_rocm_ctx *ctx) {
+    if (int e = bind(ctx)) return e;
+    return settle_all(ctx);
 }
 
 int dfdx_rocm_copy_h2d(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes) {
     if (int e = bind(ctx)) return e;
     if ((!dst || !src) && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
     if (bytes) {
+        if (int e = drop_pending_inside(ctx, dst, bytes)) return e;
         HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));  // the host buffer may be reused on return
     }
@@ -421,6 +576,7 @@ int dfdx_rocm_copy_d2h(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t by
     if (int e = bind(ctx)) return e;
     if ((!dst || !src) && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
     if (bytes) {
+        if (int e = settle_range(ctx, src, bytes)) return e;
         HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));
     }
@@ -430,12 +586,17 @@ int dfdx_rocm_copy_d2h(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t by
 int dfdx_rocm_copy_d2d(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes) {
     if (int e = bind(ctx)) return e;
     if ((!dst || !src) && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
-    if (bytes) HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    if (bytes) {
+        if (int e = settle_range(ctx, src, bytes)) return e;
+        if (int e = drop_pending_inside(ctx, dst, bytes)) return e;
+        HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    }
     return DFDX_ROCM_OK;
 }
 
 int dfdx_rocm_synchronize(dfdx_rocm_ctx *ctx) {
     if (int e = bind(ctx)) return e;
+    if (int e = settle_all(ctx)) return e;  // whoever reads the memory after this call must find the zeros
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     return DFDX_ROCM_OK;
 }
@@ -445,6 +606,7 @@ int dfdx_rocm_gemm(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc) {
     GemmProblem p;
     if (int e = make_problem(desc, &p)) return e;
     if (p.m == 0) return DFDX_ROCM_OK;
+    if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
     Plan plan;
     if (int e = make_plan(ctx, desc, p, &plan)) return e;
     return run_plan(ctx, p, plan);
@@ -455,6 +617,7 @@ int dfdx_rocm_gemm_noalloc(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc) 
     GemmProblem p;
     if (int e = make_problem(desc, &p)) return e;
     if (p.m == 0) return DFDX_ROCM_OK;
+    if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
     Plan plan;
     if (int e = make_plan(ctx, desc, p, &plan)) return e;
     return run_plan(ctx, p, plan, /*static_scratch=*/true);
@@ -501,6 +664,7 @@ int dfdx_rocm_gemm_time_rotating(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *
             *avg_ms = 0.0f;
             return DFDX_ROCM_OK;
         }
+        if (int e = settle_operands(ctx, &problems[(size_t)i], /*may_overwrite=*/false)) return e;
         if (int e = make_plan(ctx, &descs[i], problems[(size_t)i], &plans[(size_t)i])) return e;
     }
     for (int i = 0; i < warmup; i++)

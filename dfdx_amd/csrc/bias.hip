@@ -29,7 +29,7 @@ __global__ __launch_bounds__(256) void bias_forward_kernel(const T *x, const T *
 // [slices][cols] and a second kernel adds them, again in a fixed order, so the result does not depend on timing.
 template <typename T, int N, int LPR>
 __global__ __launch_bounds__(256) void bias_backward_kernel(const T *go, int rows, int cols, int rows_per_slice,
-                                                            float *partial, T *grad_bias) {
+                                                            float *partial, T *grad_bias, bool fresh) {
     constexpr int RL = 256 / LPR;  // row lanes
     __shared__ float red[RL][LPR * N + 1];
     const int c_lane = threadIdx.x % LPR, r_lane = threadIdx.x / LPR;
@@ -67,13 +67,13 @@ __global__ __launch_bounds__(256) void bias_backward_kernel(const T *go, int row
 #pragma unroll
             for (int j = 0; j < RL; j++) s += red[j][threadIdx.x];
             if (partial) partial[(int64_t)blockIdx.y * cols + c] = s;
-            else Elem<T>::store(grad_bias + c, Elem<T>::load(grad_bias + c) + s);
+            else Elem<T>::store(grad_bias + c, (fresh ? 0.0f : Elem<T>::load(grad_bias + c)) + s);
         }
     }
 }
 
 template <typename T>
-__global__ __launch_bounds__(64) void bias_backward_combine_kernel(const float *partial, int slices, int cols, T *grad_bias) {
+__global__ __launch_bounds__(64) void bias_backward_combine_kernel(const float *partial, int slices, int cols, T *grad_bias, bool fresh) {
     const int c = blockIdx.x * 64 + threadIdx.x;
     if (c >= cols) return;
     const float *src = partial + c;
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(64) void bias_backward_combine_kernel(const float *
         for (int u = 0; u < 8; u++) s += v[u];
     }
     for (; j < slices; j++) s += src[(int64_t)j * cols];
-    Elem<T>::store(grad_bias + c, Elem<T>::load(grad_bias + c) + s);
+    Elem<T>::store(grad_bias + c, (fresh ? 0.0f : Elem<T>::load(grad_bias + c)) + s);
 }
 
 // ---- f64 (the reference runs its whole test suite in f64 as well): plain kernels, f64 arithmetic -----------------
@@ -96,10 +96,10 @@ __global__ __launch_bounds__(256) void bias_forward_f64_kernel(const double *x, 
 }
 // One thread per column walks the rows in order (the order of the reference's row-after-row adds), neighbouring
 // threads read neighbouring columns.
-__global__ __launch_bounds__(256) void bias_backward_f64_kernel(const double *go, int64_t rows, int64_t cols, double *grad_bias) {
+__global__ __launch_bounds__(256) void bias_backward_f64_kernel(const double *go, int64_t rows, int64_t cols, double *grad_bias, bool fresh) {
     const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (c >= cols) return;
-    double s = grad_bias[c];
+    double s = fresh ? 0.0 : grad_bias[c];
     for (int64_t r = 0; r < rows; r++) s += go[r * cols + c];
     grad_bias[c] = s;
 }
@@ -120,7 +120,7 @@ int bias_forward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x
 }
 
 template <typename T>
-int bias_backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *go, void *gb) {
+int bias_backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *go, void *gb, bool fresh) {
     constexpr int V = Elem<T>::VEC;
     const bool vec = cols % V == 0 && aligned16(go);
     constexpr int LPR_VEC = 16, LPR_SCALAR = 64;
@@ -141,17 +141,18 @@ int bias_backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *
     }
     dim3 grid((unsigned)strips, (unsigned)slices);
     if (vec)
-        bias_backward_kernel<T, V, LPR_VEC><<<grid, 256, 0, ctx->stream>>>((const T *)go, (int)rows, (int)cols, (int)rows_per_slice, partial, (T *)gb);
+        bias_backward_kernel<T, V, LPR_VEC><<<grid, 256, 0, ctx->stream>>>((const T *)go, (int)rows, (int)cols, (int)rows_per_slice, partial, (T *)gb, fresh);
     else
-        bias_backward_kernel<T, 1, LPR_SCALAR><<<grid, 256, 0, ctx->stream>>>((const T *)go, (int)rows, (int)cols, (int)rows_per_slice, partial, (T *)gb);
+        bias_backward_kernel<T, 1, LPR_SCALAR><<<grid, 256, 0, ctx->stream>>>((const T *)go, (int)rows, (int)cols, (int)rows_per_slice, partial, (T *)gb, fresh);
     HIP_TRY(hipGetLastError());
     if (slices > 1) {
-        bias_backward_combine_kernel<T><<<(unsigned)((cols + 63) / 64), 64, 0, ctx->stream>>>(partial, (int)slices, (int)cols, (T *)gb);
+        bias_backward_combine_kernel<T><<<(unsigned)((cols + 63) / 64), 64, 0, ctx->stream>>>(partial, (int)slices, (int)cols, (T *)gb, fresh);
         HIP_TRY(hipGetLastError());
     }
     return DFDX_ROCM_OK;
 }
 
+size_t elem_bytes(int dtype) { return dtype == DFDX_ROCM_F64 ? 8 : dtype == DFDX_ROCM_F32 ? 4 : 2; }
 bool dims_ok(int64_t rows, int64_t cols) { return rows >= 0 && cols >= 0 && rows < (1ll << 31) && cols < (1ll << 31); }
 
 }  // namespace
@@ -167,6 +168,10 @@ int dfdx_rocm_bias_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t 
     if (!dims_ok(rows, cols)) return DFDX_ROCM_ERR_INVALID_ARG;
     if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
     if (!x || !bias || !out) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (dtype < DFDX_ROCM_F32 || dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_UNSUPPORTED;
+    if (int e = settle(ctx, x)) return e;
+    if (int e = settle(ctx, bias)) return e;
+    if (int e = settle_output(ctx, out, (size_t)(rows * cols) * elem_bytes(dtype), false, nullptr)) return e;
     switch (dtype) {
     case DFDX_ROCM_F32: return bias_forward_t<float>(ctx, rows, cols, x, bias, out);
     case DFDX_ROCM_F16: return bias_forward_t<_Float16>(ctx, rows, cols, x, bias, out);
@@ -187,12 +192,16 @@ int dfdx_rocm_bias_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t
     if (!dims_ok(rows, cols)) return DFDX_ROCM_ERR_INVALID_ARG;
     if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
     if (!grad_out || !grad_bias) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (dtype < DFDX_ROCM_F32 || dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_UNSUPPORTED;
+    bool fresh = false;  // a gradient whose zero fill is still deferred: stored without being read
+    if (int e = settle(ctx, grad_out)) return e;
+    if (int e = settle_output(ctx, grad_bias, (size_t)cols * elem_bytes(dtype), true, &fresh)) return e;
     switch (dtype) {
-    case DFDX_ROCM_F32: return bias_backward_t<float>(ctx, rows, cols, grad_out, grad_bias);
-    case DFDX_ROCM_F16: return bias_backward_t<_Float16>(ctx, rows, cols, grad_out, grad_bias);
-    case DFDX_ROCM_BF16: return bias_backward_t<__bf16>(ctx, rows, cols, grad_out, grad_bias);
+    case DFDX_ROCM_F32: return bias_backward_t<float>(ctx, rows, cols, grad_out, grad_bias, fresh);
+    case DFDX_ROCM_F16: return bias_backward_t<_Float16>(ctx, rows, cols, grad_out, grad_bias, fresh);
+    case DFDX_ROCM_BF16: return bias_backward_t<__bf16>(ctx, rows, cols, grad_out, grad_bias, fresh);
     case DFDX_ROCM_F64:
-        bias_backward_f64_kernel<<<(unsigned)((cols + 255) / 256), 256, 0, ctx->stream>>>((const double *)grad_out, rows, cols, (double *)grad_bias);
+        bias_backward_f64_kernel<<<(unsigned)((cols + 255) / 256), 256, 0, ctx->stream>>>((const double *)grad_out, rows, cols, (double *)grad_bias, fresh);
         return (int)hipGetLastError();
     default: return DFDX_ROCM_ERR_UNSUPPORTED;
     }

@@ -3,6 +3,8 @@
 // filters with batch stride 0 over the images, groups as the second batch axis, the filter gradient as a GEMM
 // that reduces over the batch.
 #include "ctx_internal.h"
+
+#include <initializer_list>
 #include "elem.h"
 #include "gemm_internal.h"
 
@@ -428,6 +430,8 @@ int dfdx_rocm_conv2d_forward(dfdx_rocm_ctx *ctx, int dtype, const dfdx_rocm_conv
     if (int e = narrow(op, &o)) return e;
     if (o.batch == 0 || o.chan_out == 0 || o.h_out == 0 || o.w_out == 0) return DFDX_ROCM_OK;
     if (!img || !filters || !out) return DFDX_ROCM_ERR_INVALID_ARG;
+    for (const void *p : {img, filters, (const void *)out})  // deferred zero fills among the operands run first
+        if (int e = settle(ctx, p)) return e;
     switch (dtype) {
     case DFDX_ROCM_F32: return forward_t<float>(ctx, dtype, o, img, filters, out);
     case DFDX_ROCM_F16: return forward_t<_Float16>(ctx, dtype, o, img, filters, out);
@@ -444,6 +448,9 @@ int dfdx_rocm_conv2d_backward(dfdx_rocm_ctx *ctx, int dtype, const dfdx_rocm_con
     if (int e = narrow(op, &o)) return e;
     if (o.batch == 0 || o.chan_out == 0 || o.chan_in == 0) return DFDX_ROCM_OK;
     if (!img || !grad_img || !filters || !grad_filters || !grad_out) return DFDX_ROCM_ERR_INVALID_ARG;
+    // deferred zero fills among the operands run first (the gradients are reached through several kernels here)
+    for (const void *p : {img, filters, grad_out, (const void *)grad_img, (const void *)grad_filters})
+        if (int e = settle(ctx, p)) return e;
     switch (dtype) {
     case DFDX_ROCM_F32: return backward_t<float>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out);
     case DFDX_ROCM_F16: return backward_t<_Float16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out);

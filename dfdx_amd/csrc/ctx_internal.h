@@ -3,6 +3,8 @@
 #include "../../include/dfdx_rocm.h"
 
 #include <hip/hip_runtime.h>
+#include <atomic>
+#include <cstdint>
 #include <map>
 #include <mutex>
 #include <vector>
@@ -27,6 +29,11 @@ struct dfdx_rocm_ctx {
     std::map<size_t, std::vector<void *>> cache;
     size_t cache_bytes = 0;
     std::map<void *, size_t> sizes;  // every live buffer of dfdx_rocm_alloc (free learns the size from here)
+    // Buffers declared zero whose fill has not run (start address -> bytes): dfdx_rocm_alloc with
+    // DFDX_ROCM_ZERO_DEFERRED and dfdx_rocm_zero_deferred put them here.  The first call that reads such a buffer, or
+    // writes part of it, runs the fill; a call that accumulates into ALL of it takes it out and stores 0 + value.
+    std::map<uintptr_t, size_t> pending_zero;
+    std::atomic<int> pending_count{0};  // pending_zero.size(), readable without the lock
     void *patches = nullptr;  // unfolded images of conv2d (alive across the GEMMs that may regrow `workspace`)
     size_t patches_bytes = 0;
 };
@@ -47,6 +54,19 @@ int bind(dfdx_rocm_ctx *ctx);
 int ensure_workspace(dfdx_rocm_ctx *ctx, size_t bytes);
 // Same for the conv2d patch buffer.
 int ensure_patches(dfdx_rocm_ctx *ctx, size_t bytes);
+// `ptr` is about to be read, or written in part: if it points into a buffer whose zero fill is deferred, the fill runs
+// now (on the context's stream, ahead of the caller's launch).
+int settle(dfdx_rocm_ctx *ctx, const void *ptr);
+// `ptr` is about to be written: `bytes` = the extent the call writes when it writes every byte of [ptr, ptr + bytes),
+// 0 when the written bytes have gaps.  If ptr points into a buffer with a deferred fill: a full cover takes the buffer
+// out of the pending set without filling it and reports *fresh = accumulates (the caller then stores 0 + value and
+// does not read the old contents); anything else runs the fill.  *fresh is false otherwise.
+int settle_output(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes, bool accumulates, bool *fresh);
+// Runs every deferred fill of the context.
+int settle_all(dfdx_rocm_ctx *ctx);
+// Bytes a dense view covers: extents/strides (elements) of up to `rank` axes; 0 if the view has gaps, overlaps or does
+// not start at its lowest address.  Any permutation of a contiguous layout is dense.
+size_t dense_bytes(int rank, const int64_t *extents, const int64_t *strides, size_t elem_bytes);
 // Clears `bytes` bytes at `ptr` (any alignment) with a fill kernel on `stream`.
 hipError_t launch_zero_fill(void *ptr, size_t bytes, int compute_units, hipStream_t stream);
 

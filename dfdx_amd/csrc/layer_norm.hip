@@ -81,7 +81,7 @@ __global__ __launch_bounds__(WAVES * 64) void layer_norm_forward_kernel(const T 
 // partial[slice][0][col] = sum over the slice's rows of grad_out * xhat, partial[slice][1][col] = of grad_out.
 template <typename T, int N, int CH>
 __global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_kernel(const T *x, const T *gamma, const T *go, T *gx,
-                                                                         float *partial, int64_t rows, int cols, float eps) {
+                                                                         float *partial, int64_t rows, int cols, float eps, bool fresh_x) {
     __shared__ float red[WAVES_BWD][2][64 * N];
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const float inv_n = 1.0f / (float)cols;
@@ -144,7 +144,12 @@ __global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_kernel(con
             const int col = (c * 64 + lane) * N;
             if (col < cols) {
                 float old[N];
-                load_elems<T, N>(dst + col, old);
+                if (fresh_x) {  // grad_x counts as zero and is not read
+#pragma unroll
+                    for (int i = 0; i < N; i++) old[i] = 0.0f;
+                } else {
+                    load_elems<T, N>(dst + col, old);
+                }
 #pragma unroll
                 for (int i = 0; i < N; i++) old[i] += rstd * (g[c][i] - m1 - v[c][i] * m2);
                 store_elems<T, N>(dst + col, old);
@@ -200,7 +205,7 @@ __global__ __launch_bounds__(WAVES * 64) void layer_norm_forward_loop_kernel(con
 // wave w adds its rows into partial[slice * WAVES_BWD + w], so `slices` counts waves here.
 template <typename T>
 __global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_loop_kernel(const T *x, const T *gamma, const T *go, T *gx,
-                                                                              float *partial, int64_t rows, int cols, float eps) {
+                                                                              float *partial, int64_t rows, int cols, float eps, bool fresh_x) {
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const float inv_n = 1.0f / (float)cols;
     float *pg = partial + ((int64_t)(blockIdx.x * WAVES_BWD + wave) * 2) * cols, *pb = pg + cols;
@@ -228,7 +233,7 @@ __global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_loop_kerne
         T *dst = gx + row * cols;
         for (int c = lane; c < cols; c += 64) {
             const float xh = (Elem<T>::load(src + c) - mean) * rstd, gh = Elem<T>::load(gs + c) * Elem<T>::load(gamma + c);
-            Elem<T>::store(dst + c, Elem<T>::load(dst + c) + rstd * (gh - m1 - xh * m2));
+            Elem<T>::store(dst + c, (fresh_x ? 0.0f : Elem<T>::load(dst + c)) + rstd * (gh - m1 - xh * m2));
         }
     }
 }
@@ -239,7 +244,7 @@ __global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_loop_kerne
 constexpr int COMBINE_GROUPS = 16;
 template <typename T>
 __global__ __launch_bounds__(64 * COMBINE_GROUPS) void layer_norm_combine_kernel(const float *partial, int slices, int cols, T *grad_gamma,
-                                                                                 T *grad_beta) {
+                                                                                 T *grad_beta, bool fresh_gamma, bool fresh_beta) {
     __shared__ float red[COMBINE_GROUPS][2][64];
     const int lane = threadIdx.x % 64, grp = threadIdx.x / 64;
     const int c = blockIdx.x * 64 + lane;
@@ -276,8 +281,8 @@ __global__ __launch_bounds__(64 * COMBINE_GROUPS) void layer_norm_combine_kernel
             tg += red[g][0][lane];
             tb += red[g][1][lane];
         }
-        Elem<T>::store(grad_gamma + c, Elem<T>::load(grad_gamma + c) + tg);
-        Elem<T>::store(grad_beta + c, Elem<T>::load(grad_beta + c) + tb);
+        Elem<T>::store(grad_gamma + c, (fresh_gamma ? 0.0f : Elem<T>::load(grad_gamma + c)) + tg);
+        Elem<T>::store(grad_beta + c, (fresh_beta ? 0.0f : Elem<T>::load(grad_beta + c)) + tb);
     }
 }
 
@@ -310,7 +315,7 @@ int forward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, con
 
 template <typename T>
 int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, const void *gamma, float eps, const void *go,
-               void *gx, void *ggamma, void *gbeta) {
+               void *gx, void *ggamma, void *gbeta, const bool fresh[3]) {
     constexpr int V = Elem<T>::VEC;
     const bool vec = cols % V == 0 && aligned16(x) && aligned16(gamma) && aligned16(go) && aligned16(gx);
     const int64_t groups = cols / V;
@@ -325,14 +330,14 @@ int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, co
     float *partial = (float *)ctx->workspace;
 #define DFDX_LN_BWD(CH)                                                                                                         \
     layer_norm_backward_kernel<T, V, CH><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, \
-                                                                rows, (int)cols, eps)
+                                                                rows, (int)cols, eps, fresh[0])
     if (reg && groups <= 64) DFDX_LN_BWD(1);
     else if (reg && groups <= 128) DFDX_LN_BWD(2);
     else if (reg) DFDX_LN_BWD(4);
-    else layer_norm_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, rows, (int)cols, eps);
+    else layer_norm_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, rows, (int)cols, eps, fresh[0]);
 #undef DFDX_LN_BWD
     HIP_TRY(hipGetLastError());
-    layer_norm_combine_kernel<T><<<(unsigned)((cols + 63) / 64), 64 * COMBINE_GROUPS, 0, s>>>(partial, slices, (int)cols, (T *)ggamma, (T *)gbeta);
+    layer_norm_combine_kernel<T><<<(unsigned)((cols + 63) / 64), 64 * COMBINE_GROUPS, 0, s>>>(partial, slices, (int)cols, (T *)ggamma, (T *)gbeta, fresh[1], fresh[2]);
     return (int)hipGetLastError();
 }
 
@@ -351,6 +356,11 @@ int dfdx_rocm_layer_norm_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, in
     if (!dims_ok(rows, cols)) return DFDX_ROCM_ERR_INVALID_ARG;
     if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
     if (!x || !gamma || !beta || !out) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    if (int e = settle(ctx, x)) return e;
+    if (int e = settle(ctx, gamma)) return e;
+    if (int e = settle(ctx, beta)) return e;
+    if (int e = settle_output(ctx, out, (size_t)(rows * cols) * (dtype == DFDX_ROCM_F32 ? 4 : 2), false, nullptr)) return e;
     switch (dtype) {
     case DFDX_ROCM_F32: return forward_t<float>(ctx, rows, cols, x, gamma, beta, (float)epsilon, out);
     case DFDX_ROCM_F16: return forward_t<_Float16>(ctx, rows, cols, x, gamma, beta, (float)epsilon, out);
@@ -365,10 +375,19 @@ int dfdx_rocm_layer_norm_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, i
     if (!dims_ok(rows, cols)) return DFDX_ROCM_ERR_INVALID_ARG;
     if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
     if (!x || !gamma || !grad_x || !grad_gamma || !grad_beta || !grad_out) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    const size_t es = dtype == DFDX_ROCM_F32 ? 4 : 2;
+    bool fresh[3] = {false, false, false};  // gradients whose zero fill is still deferred: stored without being read
+    if (int e = settle(ctx, x)) return e;
+    if (int e = settle(ctx, gamma)) return e;
+    if (int e = settle(ctx, grad_out)) return e;
+    if (int e = settle_output(ctx, grad_x, (size_t)(rows * cols) * es, true, &fresh[0])) return e;
+    if (int e = settle_output(ctx, grad_gamma, (size_t)cols * es, true, &fresh[1])) return e;
+    if (int e = settle_output(ctx, grad_beta, (size_t)cols * es, true, &fresh[2])) return e;
     switch (dtype) {
-    case DFDX_ROCM_F32: return backward_t<float>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta);
-    case DFDX_ROCM_F16: return backward_t<_Float16>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta);
-    case DFDX_ROCM_BF16: return backward_t<__bf16>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta);
+    case DFDX_ROCM_F32: return backward_t<float>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta, fresh);
+    case DFDX_ROCM_F16: return backward_t<_Float16>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta, fresh);
+    case DFDX_ROCM_BF16: return backward_t<__bf16>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta, fresh);
     default: return DFDX_ROCM_ERR_UNSUPPORTED;
     }
 }

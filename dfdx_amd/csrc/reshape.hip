@@ -40,12 +40,17 @@ __global__ __launch_bounds__(256) void reshape_forward_kernel(const T *inp, T *o
 }
 
 template <typename T, int N, typename Index>
-__global__ __launch_bounds__(256) void reshape_backward_kernel(T *grad_inp, const T *grad_out, ViewDims d, Index groups) {
+__global__ __launch_bounds__(256) void reshape_backward_kernel(T *grad_inp, const T *grad_out, ViewDims d, Index groups, bool fresh) {
     for (Index g = (Index)blockIdx.x * 256 + threadIdx.x; g < groups; g += (Index)gridDim.x * 256) {
         float v[N], old[N];
         load_elems<T, N>(grad_out + (int64_t)g * N, v);
         T *dst = grad_inp + view_offset<Index>(d, g);
-        load_elems<T, N>(dst, old);
+        if (fresh) {  // grad_inp counts as zero and is not read
+#pragma unroll
+            for (int i = 0; i < N; i++) old[i] = 0.0f;
+        } else {
+            load_elems<T, N>(dst, old);
+        }
 #pragma unroll
         for (int i = 0; i < N; i++) old[i] += v[i];
         store_elems<T, N>(dst, old);
@@ -139,7 +144,7 @@ int canonical(int rank, const int64_t *shape, const int64_t *strides, int64_t *c
 }
 
 template <typename T, bool FWD>
-int launch_t(dfdx_rocm_ctx *ctx, int rank, const int64_t *shape, const int64_t *strides, const void *src, void *dst) {
+int launch_t(dfdx_rocm_ctx *ctx, int rank, const int64_t *shape, const int64_t *strides, const void *src, void *dst, bool fresh) {
     // forward: src = inp (strided), dst = out (contiguous);  backward: src = grad_out (contiguous), dst = grad_inp (strided)
     int64_t cs[MAX_RANK], cst[MAX_RANK];
     const int n = canonical(rank, shape, strides, cs, cst);
@@ -164,7 +169,7 @@ int launch_t(dfdx_rocm_ctx *ctx, int rank, const int64_t *shape, const int64_t *
 #define DFDX_RESHAPE(N, IDX)                                                                                       \
     do {                                                                                                           \
         if constexpr (FWD) reshape_forward_kernel<T, N, IDX><<<grid, 256, 0, s>>>((const T *)src, (T *)dst, d, (IDX)groups); \
-        else reshape_backward_kernel<T, N, IDX><<<grid, 256, 0, s>>>((T *)dst, (const T *)src, d, (IDX)groups);   \
+        else reshape_backward_kernel<T, N, IDX><<<grid, 256, 0, s>>>((T *)dst, (const T *)src, d, (IDX)groups, fresh); \
     } while (0)
     if (vec && small) DFDX_RESHAPE(V, uint32_t);
     else if (vec) DFDX_RESHAPE(V, uint64_t);
@@ -188,6 +193,14 @@ int dispatch(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, cons
     }
     if (total == 0) return DFDX_ROCM_OK;
     if (!src || !dst) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    // Deferred zero fills: the contiguous side covers total elements; the strided side covers its buffer when the view
+    // is a permutation of a contiguous layout (a backward through such a view then stores 0 + value).
+    const size_t es = dtype == DFDX_ROCM_F32 ? 4 : 2;
+    bool fresh = false;
+    if (int e = settle(ctx, src)) return e;
+    if (int e = settle_output(ctx, dst, FWD ? (size_t)total * es : dense_bytes(rank, shape, strides, es), !FWD, broadcast ? nullptr : &fresh))
+        return e;
     if (broadcast) {
         switch (dtype) {
         case DFDX_ROCM_F32: return launch_reduce<float>(ctx, rank, shape, strides, src, dst);
@@ -197,9 +210,9 @@ int dispatch(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, cons
         }
     }
     switch (dtype) {
-    case DFDX_ROCM_F32: return launch_t<float, FWD>(ctx, rank, shape, strides, src, dst);
-    case DFDX_ROCM_F16: return launch_t<_Float16, FWD>(ctx, rank, shape, strides, src, dst);
-    case DFDX_ROCM_BF16: return launch_t<__bf16, FWD>(ctx, rank, shape, strides, src, dst);
+    case DFDX_ROCM_F32: return launch_t<float, FWD>(ctx, rank, shape, strides, src, dst, fresh);
+    case DFDX_ROCM_F16: return launch_t<_Float16, FWD>(ctx, rank, shape, strides, src, dst, fresh);
+    case DFDX_ROCM_BF16: return launch_t<__bf16, FWD>(ctx, rank, shape, strides, src, dst, fresh);
     default: return DFDX_ROCM_ERR_UNSUPPORTED;
     }
 }

@@ -74,10 +74,10 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_forward_reg_kernel(const T
     }
 }
 
-// grad_x += scale * p * (g - sum_j g_j p_j)
+// grad_x += scale * p * (g - sum_j g_j p_j); `fresh`: grad_x counts as zero and is not read
 template <typename T, int N, int CH>
 __global__ __launch_bounds__(WAVES * 64) void softmax_backward_reg_kernel(const T *p, const T *go, T *gx, int64_t rows, int cols,
-                                                                          float scale) {
+                                                                          float scale, bool fresh) {
     const int lane = threadIdx.x % 64;
     for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
         const T *ps = p + row * cols, *gs = go + row * cols;
@@ -100,7 +100,12 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_backward_reg_kernel(const 
             const int col = (c * 64 + lane) * N;
             if (col < cols) {
                 float old[N];
-                load_elems<T, N>(dst + col, old);
+                if (fresh) {
+#pragma unroll
+                    for (int i = 0; i < N; i++) old[i] = 0.0f;
+                } else {
+                    load_elems<T, N>(dst + col, old);
+                }
 #pragma unroll
                 for (int i = 0; i < N; i++) old[i] += scale * (pv[c][i] * (gv[c][i] - dot));
                 store_elems<T, N>(dst + col, old);
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_forward_loop_kernel(const 
 
 template <typename T>
 __global__ __launch_bounds__(WAVES * 64) void softmax_backward_loop_kernel(const T *p, const T *go, T *gx, int64_t rows, int cols,
-                                                                           float scale) {
+                                                                           float scale, bool fresh) {
     const int lane = threadIdx.x % 64;
     for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
         const T *ps = p + row * cols, *gs = go + row * cols;
@@ -138,14 +143,14 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_backward_loop_kernel(const
         dot = wave_sum(dot);
         T *dst = gx + row * cols;
         for (int c = lane; c < cols; c += 64)
-            Elem<T>::store(dst + c, Elem<T>::load(dst + c) + scale * (Elem<T>::load(ps + c) * (Elem<T>::load(gs + c) - dot)));
+            Elem<T>::store(dst + c, (fresh ? 0.0f : Elem<T>::load(dst + c)) + scale * (Elem<T>::load(ps + c) * (Elem<T>::load(gs + c) - dot)));
     }
 }
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 template <typename T, bool FWD>
-int launch_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *a, const void *b, void *c, float scale) {
+int launch_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *a, const void *b, void *c, float scale, bool fresh) {
     // forward: a = x, c = out;  backward: a = p, b = grad_out, c = grad_x
     constexpr int V = Elem<T>::VEC;
     const bool vec = cols % V == 0 && aligned16(a) && aligned16(c) && (FWD || aligned16(b));
@@ -156,7 +161,7 @@ int launch_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *a, cons
 #define DFDX_SOFTMAX_REG(N, CH)                                                                                        \
     do {                                                                                                               \
         if constexpr (FWD) softmax_forward_reg_kernel<T, N, CH><<<grid, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale); \
-        else softmax_backward_reg_kernel<T, N, CH><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale); \
+        else softmax_backward_reg_kernel<T, N, CH><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh); \
         return (int)hipGetLastError();                                                                                 \
     } while (0)
     if (vec) {
@@ -172,7 +177,7 @@ int launch_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *a, cons
     }
 #undef DFDX_SOFTMAX_REG
     if constexpr (FWD) softmax_forward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale);
-    else softmax_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale);
+    else softmax_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh);
     return (int)hipGetLastError();
 }
 
@@ -182,10 +187,15 @@ int dispatch(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const vo
     if (rows < 0 || cols < 0 || cols >= (1ll << 31)) return DFDX_ROCM_ERR_INVALID_ARG;
     if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
     if (!a || !c || (!FWD && !b)) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    bool fresh = false;  // a gradient whose zero fill is still deferred: stored without being read
+    if (int e = settle(ctx, a)) return e;
+    if (int e = settle(ctx, b)) return e;
+    if (int e = settle_output(ctx, c, (size_t)(rows * cols) * (dtype == DFDX_ROCM_F32 ? 4 : 2), !FWD, &fresh)) return e;
     switch (dtype) {
-    case DFDX_ROCM_F32: return launch_t<float, FWD>(ctx, rows, cols, a, b, c, scale);
-    case DFDX_ROCM_F16: return launch_t<_Float16, FWD>(ctx, rows, cols, a, b, c, scale);
-    case DFDX_ROCM_BF16: return launch_t<__bf16, FWD>(ctx, rows, cols, a, b, c, scale);
+    case DFDX_ROCM_F32: return launch_t<float, FWD>(ctx, rows, cols, a, b, c, scale, fresh);
+    case DFDX_ROCM_F16: return launch_t<_Float16, FWD>(ctx, rows, cols, a, b, c, scale, fresh);
+    case DFDX_ROCM_BF16: return launch_t<__bf16, FWD>(ctx, rows, cols, a, b, c, scale, fresh);
     default: return DFDX_ROCM_ERR_UNSUPPORTED;
     }
 }

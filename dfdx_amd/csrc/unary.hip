@@ -9,15 +9,20 @@
 namespace dfdx_rocm {
 namespace {
 
-// ACC: out[i] += s * x[i] (backward), else out[i] = s * x[i]
+// ACC: out[i] += s * x[i] (backward; `fresh`: out counts as zero and is not read), else out[i] = s * x[i]
 template <typename T, int N, bool ACC>
-__global__ __launch_bounds__(256) void scalar_mul_kernel(const T *x, T *out, int64_t groups, float s) {
+__global__ __launch_bounds__(256) void scalar_mul_kernel(const T *x, T *out, int64_t groups, float s, bool fresh) {
     for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
         float v[N];
         load_elems<T, N>(x + g * N, v);
         if constexpr (ACC) {
             float o[N];
-            load_elems<T, N>(out + g * N, o);
+            if (fresh) {
+#pragma unroll
+                for (int i = 0; i < N; i++) o[i] = 0.0f;
+            } else {
+                load_elems<T, N>(out + g * N, o);
+            }
 #pragma unroll
             for (int i = 0; i < N; i++) v[i] = o[i] + s * v[i];
         } else {
@@ -39,14 +44,19 @@ template <typename T, int N> __global__ __launch_bounds__(256) void relu_forward
     }
 }
 
-// grad_x += (x > 0 ? 1 : 0) * grad_out
+// grad_x += (x > 0 ? 1 : 0) * grad_out; `fresh`: grad_x counts as zero and is not read
 template <typename T, int N>
-__global__ __launch_bounds__(256) void relu_backward_kernel(const T *x, const T *go, T *gx, int64_t groups) {
+__global__ __launch_bounds__(256) void relu_backward_kernel(const T *x, const T *go, T *gx, int64_t groups, bool fresh) {
     for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
         float v[N], d[N], o[N];
         load_elems<T, N>(x + g * N, v);
         load_elems<T, N>(go + g * N, d);
-        load_elems<T, N>(gx + g * N, o);
+        if (fresh) {
+#pragma unroll
+            for (int i = 0; i < N; i++) o[i] = 0.0f;
+        } else {
+            load_elems<T, N>(gx + g * N, o);
+        }
 #pragma unroll
         for (int i = 0; i < N; i++) o[i] += v[i] > 0.0f ? d[i] : 0.0f;
         store_elems<T, N>(gx + g * N, o);
@@ -65,13 +75,16 @@ template <typename T, int N> __global__ __launch_bounds__(256) void add_forward_
     }
 }
 
-// grad_lhs += grad_out, grad_rhs += grad_out (two distinct buffers)
-template <typename T, int N> __global__ __launch_bounds__(256) void add_backward_kernel(const T *go, T *gl, T *gr, int64_t groups) {
+// grad_lhs += grad_out, grad_rhs += grad_out (two distinct buffers); fresh_l / fresh_r: that one counts as zero, not read
+template <typename T, int N>
+__global__ __launch_bounds__(256) void add_backward_kernel(const T *go, T *gl, T *gr, int64_t groups, bool fresh_l, bool fresh_r) {
     for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
         float d[N], l[N], r[N];
         load_elems<T, N>(go + g * N, d);
-        load_elems<T, N>(gl + g * N, l);
-        load_elems<T, N>(gr + g * N, r);
+#pragma unroll
+        for (int i = 0; i < N; i++) l[i] = r[i] = 0.0f;
+        if (!fresh_l) load_elems<T, N>(gl + g * N, l);
+        if (!fresh_r) load_elems<T, N>(gr + g * N, r);
 #pragma unroll
         for (int i = 0; i < N; i++) {
             l[i] += d[i];
@@ -98,14 +111,14 @@ template <typename T> float round_scalar(double s) {
     }
 }
 
-template <typename T, bool ACC> int launch_t(dfdx_rocm_ctx *ctx, int64_t len, const void *x, double scalar, void *out) {
+template <typename T, bool ACC> int launch_t(dfdx_rocm_ctx *ctx, int64_t len, const void *x, double scalar, void *out, bool fresh) {
     constexpr int V = Elem<T>::VEC;
     const bool vec = len % V == 0 && (((uintptr_t)x | (uintptr_t)out) & 15u) == 0;
     const int64_t groups = vec ? len / V : len;
     const unsigned grid = (unsigned)std::min<int64_t>((groups + 255) / 256, (int64_t)ctx->compute_units * 16);
     const float s = round_scalar<T>(scalar);
-    if (vec) scalar_mul_kernel<T, V, ACC><<<grid, 256, 0, ctx->stream>>>((const T *)x, (T *)out, groups, s);
-    else scalar_mul_kernel<T, 1, ACC><<<grid, 256, 0, ctx->stream>>>((const T *)x, (T *)out, groups, s);
+    if (vec) scalar_mul_kernel<T, V, ACC><<<grid, 256, 0, ctx->stream>>>((const T *)x, (T *)out, groups, s, fresh);
+    else scalar_mul_kernel<T, 1, ACC><<<grid, 256, 0, ctx->stream>>>((const T *)x, (T *)out, groups, s, fresh);
     return (int)hipGetLastError();
 }
 
@@ -114,10 +127,14 @@ template <bool ACC> int dispatch(dfdx_rocm_ctx *ctx, int dtype, int64_t len, con
     if (len < 0) return DFDX_ROCM_ERR_INVALID_ARG;
     if (len == 0) return DFDX_ROCM_OK;
     if (!x || !out) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    bool fresh = false;  // a gradient whose zero fill is still deferred: stored without being read
+    if (int e = settle(ctx, x)) return e;
+    if (int e = settle_output(ctx, out, (size_t)len * (dtype == DFDX_ROCM_F32 ? 4 : 2), ACC, &fresh)) return e;
     switch (dtype) {
-    case DFDX_ROCM_F32: return launch_t<float, ACC>(ctx, len, x, scalar, out);
-    case DFDX_ROCM_F16: return launch_t<_Float16, ACC>(ctx, len, x, scalar, out);
-    case DFDX_ROCM_BF16: return launch_t<__bf16, ACC>(ctx, len, x, scalar, out);
+    case DFDX_ROCM_F32: return launch_t<float, ACC>(ctx, len, x, scalar, out, fresh);
+    case DFDX_ROCM_F16: return launch_t<_Float16, ACC>(ctx, len, x, scalar, out, fresh);
+    case DFDX_ROCM_BF16: return launch_t<__bf16, ACC>(ctx, len, x, scalar, out, fresh);
     default: return DFDX_ROCM_ERR_UNSUPPORTED;
     }
 }
@@ -125,7 +142,8 @@ template <bool ACC> int dispatch(dfdx_rocm_ctx *ctx, int dtype, int64_t len, con
 enum { OP_RELU_FWD, OP_RELU_BWD, OP_ADD_FWD, OP_ADD_BWD };
 
 // a, b: read-only inputs (b unused by OP_RELU_FWD); c, d: written (d only by OP_ADD_BWD)
-template <typename T, int OP> int launch_op(dfdx_rocm_ctx *ctx, int64_t len, const void *a, const void *b, void *c, void *d) {
+template <typename T, int OP>
+int launch_op(dfdx_rocm_ctx *ctx, int64_t len, const void *a, const void *b, void *c, void *d, bool fresh_c, bool fresh_d) {
     constexpr int V = Elem<T>::VEC;
     const bool vec = len % V == 0 && (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) & 15u) == 0;
     const int64_t groups = vec ? len / V : len;
@@ -134,9 +152,9 @@ template <typename T, int OP> int launch_op(dfdx_rocm_ctx *ctx, int64_t len, con
 #define DFDX_OP(N)                                                                                                       \
     do {                                                                                                                 \
         if constexpr (OP == OP_RELU_FWD) relu_forward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (T *)c, groups);    \
-        else if constexpr (OP == OP_RELU_BWD) relu_backward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (const T *)b, (T *)c, groups); \
+        else if constexpr (OP == OP_RELU_BWD) relu_backward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (const T *)b, (T *)c, groups, fresh_c); \
         else if constexpr (OP == OP_ADD_FWD) add_forward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (const T *)b, (T *)c, groups);    \
-        else add_backward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (T *)c, (T *)d, groups);                        \
+        else add_backward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (T *)c, (T *)d, groups, fresh_c, fresh_d);      \
     } while (0)
     if (vec) DFDX_OP(V);
     else DFDX_OP(1);
@@ -149,10 +167,18 @@ template <int OP> int dispatch_op(dfdx_rocm_ctx *ctx, int dtype, int64_t len, co
     if (len < 0) return DFDX_ROCM_ERR_INVALID_ARG;
     if (len == 0) return DFDX_ROCM_OK;
     if (!a || !c || (OP != OP_RELU_FWD && OP != OP_ADD_BWD && !b) || (OP == OP_ADD_BWD && !d)) return DFDX_ROCM_ERR_INVALID_ARG;
+    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    bool fresh_c = false, fresh_d = false;  // gradients whose zero fill is still deferred: stored without being read
+    constexpr bool BWD = OP == OP_RELU_BWD || OP == OP_ADD_BWD;
+    const size_t bytes = (size_t)len * (dtype == DFDX_ROCM_F32 ? 4 : 2);
+    if (int e = settle(ctx, a)) return e;
+    if (int e = settle(ctx, b)) return e;
+    if (int e = settle_output(ctx, c, bytes, BWD, &fresh_c)) return e;
+    if (int e = settle_output(ctx, d, bytes, BWD, &fresh_d)) return e;
     switch (dtype) {
-    case DFDX_ROCM_F32: return launch_op<float, OP>(ctx, len, a, b, c, d);
-    case DFDX_ROCM_F16: return launch_op<_Float16, OP>(ctx, len, a, b, c, d);
-    case DFDX_ROCM_BF16: return launch_op<__bf16, OP>(ctx, len, a, b, c, d);
+    case DFDX_ROCM_F32: return launch_op<float, OP>(ctx, len, a, b, c, d, fresh_c, fresh_d);
+    case DFDX_ROCM_F16: return launch_op<_Float16, OP>(ctx, len, a, b, c, d, fresh_c, fresh_d);
+    case DFDX_ROCM_BF16: return launch_op<__bf16, OP>(ctx, len, a, b, c, d, fresh_c, fresh_d);
     default: return DFDX_ROCM_ERR_UNSUPPORTED;
     }
 }

@@ -6,10 +6,13 @@
     Linear / LayerNorm1D / ResidualAdd   linear.rs:82-89, layer_norm1d.rs:87-91, residual_add.rs:38-45
 
 The forward keeps what the reference's tape would keep (the inputs of every op); the backward walks the ops in
-reverse; every gradient buffer starts zero-filled and is accumulated into, as with
+reverse; every gradient buffer starts as zeros and is accumulated into, as with
 ``Gradients::get_or_alloc_mut`` (dfdx-core/src/tensor/gradients.rs:53-58) -- here all of a pass's buffers are carved
-from one allocation that a single fill launch clears.  The multiplication by 1/sqrt(head
-dim) between q.k^T and the softmax (multi_head_attention.rs:133-134) is folded into the softmax kernel.
+from one allocation and declared zero without a fill (``dfdx_rocm_zero_deferred``): the first op that accumulates
+into a whole buffer stores 0 + value, so the step pays neither the fill nor the read of the zeros; a buffer whose
+first use is anything else is filled then.  ``deferred_zeros=False`` restores the single eager fill.  The
+multiplication by 1/sqrt(head dim) between q.k^T and the softmax (multi_head_attention.rs:133-134) is folded into the
+softmax kernel.
 """
 from __future__ import annotations
 
@@ -25,11 +28,13 @@ class EncoderBlock:
     """Parameters are device ``View``s: w* are (out, in) row-major Linear weights, b* biases, g*/be* the LayerNorm
     gamma / beta."""
 
-    def __init__(self, dev: Rocm, dtype: str, d_model: int, heads: int, d_ff: int, params: Dict[str, View]):
+    def __init__(self, dev: Rocm, dtype: str, d_model: int, heads: int, d_ff: int, params: Dict[str, View],
+                 deferred_zeros: bool = True):
         assert d_model % heads == 0, f"left: {d_model % heads}\n right: 0"
         missing = [n for n in PARAMS if n not in params]
         assert not missing, f"missing parameters: {missing}"
         self.dev, self.dtype, self.d, self.h, self.ff, self.p = dev, dtype, d_model, heads, d_ff, params
+        self.deferred_zeros = deferred_zeros
 
     def forward(self, x: View) -> Tuple[View, dict]:
         """x: (batch, seq, d_model) contiguous.  Returns the block's output and the tensors the backward needs."""
@@ -66,10 +71,10 @@ class EncoderBlock:
         dev, p, s = self.dev, self.p, saved
         x, n1, tok, tokens, probs = s["x"], s["n1"], s["tok"], s["tokens"], s["probs"]
         qv, kv, vv = s["qv"], s["kv"], s["vv"]
-        # every gradient buffer of the pass, zero-filled by one launch (one allocation, pieces aligned to 256 B)
+        # every gradient buffer of the pass: one allocation, pieces aligned to 256 B, zero by declaration (or one fill)
         acts = dict(gh2=s["h2"], gf2=s["h2"], gn1=n1, gr1=s["r1"], gf1=s["f1"], gh1=s["h1"], gattn=s["h1"], gx=x, gtok=tok,
                     gtokens=tokens, gp=probs, gscores=probs, gq=x, gk=x, gv=x)   # gq, gk, gv: laid out like the q, k, v storages
-        bufs = dev.zeros_many([p[n] for n in PARAMS] + list(acts.values()))
+        bufs = dev.zeros_many([p[n] for n in PARAMS] + list(acts.values()), deferred=self.deferred_zeros)
         grads = dict(zip(PARAMS, bufs[:len(PARAMS)]))
         g = dict(zip(acts, bufs[len(PARAMS):]))
         gh2, gf2, gn1, gr1, gf1, gh1, gattn, gx = (g[k] for k in ("gh2", "gf2", "gn1", "gr1", "gf1", "gh1", "gattn", "gx"))
@@ -88,4 +93,5 @@ class EncoderBlock:
         dev.backward(qv, gq, kv, gk, gscores)
         for w, b, gg in (("wq", "bq", gq), ("wk", "bk", gk), ("wv", "bv", gv)):   # x feeds three Linears: one buffer
             dev.linear_backward(x, gx, p[w], grads[w], grads[b], gg)
+        dev.settle_zeros()   # nothing is left pending in this block; a gradient no op touched would be filled here
         return grads, gx

@@ -28,6 +28,7 @@ ITEMSIZE = {"f32": 4, "f16": 2, "bf16": 2, "f64": 8}
 NP_DTYPES = {"f32": np.float32, "f16": np.float16, "bf16": np.uint16, "f64": np.float64}
 
 KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_GEMV = 0, 1, 2, 3
+ZERO_DEFERRED = 2   # dfdx_rocm_alloc: zero as far as the library can tell, fill only if needed
 NOALLOC_SCRATCH_BYTES = 32 << 20   # DFDX_ROCM_NOALLOC_SCRATCH_BYTES
 ERR_SCRATCH_TOO_SMALL = -5
 
@@ -72,7 +73,7 @@ _lib = None
 EXPORTS = [
     "dfdx_rocm_create", "dfdx_rocm_destroy", "dfdx_rocm_strerror", "dfdx_rocm_device_info",
     "dfdx_rocm_alloc", "dfdx_rocm_free", "dfdx_rocm_memset_zero", "dfdx_rocm_copy_h2d", "dfdx_rocm_copy_d2h",
-    "dfdx_rocm_copy_d2d", "dfdx_rocm_synchronize", "dfdx_rocm_enable_cache", "dfdx_rocm_disable_cache",
+    "dfdx_rocm_copy_d2d", "dfdx_rocm_synchronize", "dfdx_rocm_zero_deferred", "dfdx_rocm_settle_zeros", "dfdx_rocm_enable_cache", "dfdx_rocm_disable_cache",
     "dfdx_rocm_empty_cache", "dfdx_rocm_cache_stats", "dfdx_rocm_gemm", "dfdx_rocm_gemm_noalloc", "dfdx_rocm_gemm_plan",
     "dfdx_rocm_mfma_variant_count", "dfdx_rocm_gemm_time", "dfdx_rocm_gemm_time_rotating",
     "dfdx_rocm_matmat_forward", "dfdx_rocm_matmat_backward",
@@ -202,14 +203,24 @@ class Rocm:
         self._check(self.lib.dfdx_rocm_cache_stats(self.ctx, ctypes.byref(n), ctypes.byref(b)))
         return n.value, b.value
 
-    def alloc(self, nbytes: int, zeroed: bool = True) -> int:
-        """``Storage::try_alloc_len`` / ``alloc_empty`` through the library's own allocator; returns the device address."""
+    def alloc(self, nbytes: int, zeroed=True) -> int:
+        """``Storage::try_alloc_len`` / ``alloc_empty`` through the library's own allocator; returns the device address.
+        ``zeroed`` = ``ZERO_DEFERRED``: zero as far as the library's calls can tell, the fill only runs if a call needs it."""
         p = ctypes.c_void_p()
         self._check(self.lib.dfdx_rocm_alloc(self.ctx, ctypes.c_size_t(nbytes), int(zeroed), ctypes.byref(p)))
         return p.value
 
     def free(self, ptr: int):
         self._check(self.lib.dfdx_rocm_free(self.ctx, ctypes.c_void_p(ptr)))
+
+    def zero_deferred(self, ptr: int, nbytes: int):
+        """Declares ``nbytes`` at ``ptr`` zero without filling them (``dfdx_rocm_zero_deferred``): the first call that
+        accumulates into the whole buffer stores 0 + value, any other first use runs the fill."""
+        self._check(self.lib.dfdx_rocm_zero_deferred(self.ctx, ctypes.c_void_p(ptr), ctypes.c_size_t(nbytes)))
+
+    def settle_zeros(self):
+        """Runs every deferred fill still pending: needed before code outside the library reads such a buffer."""
+        self._check(self.lib.dfdx_rocm_settle_zeros(self.ctx))
 
     # --------------------------------------------------------------- storage --
     def tensor(self, host: np.ndarray, dtype: str, shape=None, strides=None) -> View:
@@ -233,17 +244,25 @@ class Rocm:
         raw = self._zeroed_bytes(max(n * ITEMSIZE[dtype], 16))
         return View(raw, dtype, shape, _row_major(shape) if strides is None else tuple(strides))
 
-    def zeros_many(self, likes) -> list:
+    def zeros_many(self, likes, deferred: bool = False) -> list:
         """Zero-filled storages for several tensors at once: one allocation, ONE fill launch, each view on its own
         256 B-aligned piece.  ``likes`` are Views whose dtype / shape give the sizes (contiguous row-major results).
         What a pooling allocator behind ``try_alloc_grad`` would do for the gradient buffers of one backward pass:
-        small fills are launch-bound (3.5 us for 2 MiB), one large fill runs at the HBM write rate."""
+        small fills are launch-bound (3.5 us for 2 MiB), one large fill runs at the HBM write rate.
+        ``deferred``: no fill at all; every piece is declared zero (``zero_deferred``) and the first backward op that
+        accumulates into the whole of it stores instead -- read the results through this object (``to_host``) or
+        call ``settle_zeros`` first."""
         sizes = [max(int(np.prod(v.shape, dtype=np.int64)) * ITEMSIZE[v.dtype], 16) for v in likes]
         offs, total = [], 0
         for n in sizes:
             offs.append(total)
             total += (n + 255) // 256 * 256
-        arena = self._zeroed_bytes(max(total, 16))
+        if deferred:
+            arena = self._torch.empty(max(total, 16), dtype=self._torch.uint8, device=self.device)
+            for o, n in zip(offs, sizes):
+                self.zero_deferred(arena.data_ptr() + o, n)
+        else:
+            arena = self._zeroed_bytes(max(total, 16))
         return [View(arena[o:o + n], v.dtype, tuple(v.shape), _row_major(tuple(v.shape))) for v, o, n in zip(likes, offs, sizes)]
 
     def _zeroed_bytes(self, nbytes: int):
@@ -268,6 +287,7 @@ class Rocm:
     def to_host(self, v: View) -> np.ndarray:
         """The storage bytes as a flat numpy array of the storage dtype."""
         n = v.numel_storage()
+        self.settle_zeros()   # the storage may still wait for a deferred zero fill
         return v.storage.cpu().numpy().view(NP_DTYPES[v.dtype])[:n].copy()
 
     # ------------------------------------------------------------------ gemm --

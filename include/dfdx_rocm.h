@@ -88,6 +88,30 @@ int dfdx_rocm_copy_d2h(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t by
 int dfdx_rocm_copy_d2d(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes);
 int dfdx_rocm_synchronize(dfdx_rocm_ctx *ctx);
 
+/* Deferred zero fill, for gradient storage.  `Gradients::get_or_alloc_mut`
+ * (dfdx-core/src/tensor/gradients.rs:53-58) allocates every gradient
+ * zero-filled and the backward ops then accumulate into it: in a training
+ * step the fill and the first read of those zeros are pure HBM traffic.
+ * A buffer allocated with `zeroed` = DFDX_ROCM_ZERO_DEFERRED (or declared
+ * with dfdx_rocm_zero_deferred, for storage the caller owns) is zero as far as
+ * any call of this library can tell, but its fill has not run:
+ *   - the first call that accumulates into every byte of it (a backward
+ *     entry or an accumulating GEMM whose output view is a permutation of
+ *     the contiguous layout, starting at the buffer's first byte) stores
+ *     0 + value without reading it, and the fill never runs;
+ *   - any other first use through this library (an input operand, a partial
+ *     or strided write, a copy out of it) runs the fill first;
+ *   - dfdx_rocm_synchronize, dfdx_rocm_settle_zeros and dfdx_rocm_destroy run
+ *     every fill still pending; dfdx_rocm_free drops the buffer's.
+ * Results are bit-identical to the eager fill.  A deferred buffer is looked
+ * up by the pointer a call is given: hand views of it to the library by a
+ * pointer inside the buffer.  Code outside this library that reads the memory
+ * (another stream, a host copy not made by dfdx_rocm_copy_d2h) must call
+ * dfdx_rocm_settle_zeros or dfdx_rocm_synchronize first. */
+#define DFDX_ROCM_ZERO_DEFERRED 2
+int dfdx_rocm_zero_deferred(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes);
+int dfdx_rocm_settle_zeros(dfdx_rocm_ctx *ctx);
+
 /* The allocation cache of the device (`Cache::try_enable_cache`,
  * `try_disable_cache`, `try_empty_cache`: dfdx-core/src/tensor/
  * storage_traits.rs:41-77; `TensorCache`, tensor/cache.rs:36-149, which the
