@@ -327,6 +327,15 @@ def main():
              fl, es * nb * (2 * S * D + 2 * S * S), bufs=(d_o, v, gp))
         gemm("c5", "attn dV P^T.dO acc, interleaved rows", d5(S, S, D, p_, (1, S), sSS, d_o, (D, 1), sSD, gv, (H * D, 1), tok, True),
              fl, es * nb * (S * S + 3 * S * D), bufs=(p_, d_o, gv))
+        if want("glue"):
+            vw = lambda t: view(t, dt)
+            mat = nb * S * S * es
+            timed("glue", "softmax fwd (16,16,512,512) bf16, scale folded", lambda: dev.softmax_forward(vw(sc), 0.125), 0, 2 * mat, "softmax_forward",
+                  sets=[(lambda a=vw(t): dev.softmax_forward(a, 0.125)) for (t,) in copies(4, sc)])
+            gs = zeros((Bq, H, S, S), dt)
+            timed("glue", "softmax bwd (16,16,512,512) bf16", lambda: dev.softmax_backward(vw(p_), vw(gs), vw(gp), 0.125), 0, 4 * mat, "softmax_backward",
+                  sets=[(lambda a=vw(t0), b=vw(t1), c=vw(t2): dev.softmax_backward(a, b, c, 0.125)) for t0, t1, t2 in copies(4, p_, gs, gp)])
+            del gs
         del sc, p_, gp
 
     # ---- zero fill of gradient storage (Storage::try_alloc_len): HBM write roofline -----------------------------

@@ -365,8 +365,19 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
     // previously computed tile occupied.  Callers guarantee that this wave has issued all its LDS reads of
     // that previous tile; lgkmcnt(0) makes sure they are done.  (vmcnt(0) also covers the stores of a finished
     // C tile: they had a whole k step to drain.)
-    auto sync_tile = [&]() {
-        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) & lgkmcnt(0)
+    // `behind`: how many memory instructions this wave issued AFTER its last tile request -- the stores of the C tile
+    // finished before this one (one of the compile-time counts below, else 0).  The counter retires in issue order, so
+    // waiting until that many are left means: the requested tile has landed, the stores may still be draining.  With
+    // one k tile per work item (attention scores) a wait for everything would stop every workgroup until its previous
+    // C tile is in memory, and the chip would alternate between storing and computing.
+    constexpr int ST_PLAIN = TM * TN / 2, ST_ACC = (TM * (TN / 2) > 8 ? TM / 2 : TM) * TN / 2, ST_SPLIT = TM * TN;
+    static_assert(ST_SPLIT < 64, "vmcnt is a 6-bit count");
+    constexpr auto wait_vm_lgkm0 = [](int vm) { return (vm & 15) | ((vm >> 4) << 14) | 0x0070; };  // vmcnt(vm) & lgkmcnt(0)
+    auto sync_tile = [&](int behind = 0) {
+        if (behind == ST_PLAIN) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(ST_PLAIN));
+        else if (behind == ST_ACC) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(ST_ACC));
+        else if (behind == ST_SPLIT) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(ST_SPLIT));
+        else __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) & lgkmcnt(0)
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -456,7 +467,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
     };
 
     // ---- epilogue of one work item: lane holds m = l16 (per tile), n = 4*lq + 0..3 -------------
-    auto store_tile = [&](const Work &w) {
+    // Returns the number of stores it issued after its last load (see sync_tile), 0 when that is not a fixed count.
+    auto store_tile = [&](const Work &w) -> int {
         const int bm0 = w.bm0, bn0 = w.bn0, split = w.split, batch = w.batch;
     if (p.splits > 1) {  // f32 partial tile into the workspace (padded to whole tiles: no bounds checks)
         float *wbase = p.ws + split * p.ws_split_stride;
@@ -466,7 +478,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
 #pragma unroll
             for (int j = 0; j < TN; j++) *(f32x4 *)(wrow + j * 16) = acc[i][j];
         }
-        return;
+        return ST_SPLIT;
     }
     const int cb = p.kbatches > 1 ? 0 : batch;
     uint16_t *cbase = p.c + (int64_t)(cb / p.nb2) * p.c_b1 + (int64_t)(cb % p.nb2) * p.c_b2;
@@ -668,15 +680,17 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
             if (interior && !p.accumulate) {
                 if (p.bias_mode == BIAS_PER_COL) rows_plain(std::true_type{});
                 else rows_plain(std::false_type{});
-                __builtin_amdgcn_s_waitcnt(vmcnt_only(TM * TN / 2));
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(ST_PLAIN));
+                return ST_PLAIN;
             } else if (!EDGE || (interior && p.bias_mode == BIAS_NONE)) {
                 rows_accumulate();
-                __builtin_amdgcn_s_waitcnt(vmcnt_only((TM * (TN / 2) > 8 ? TM / 2 : TM) * TN / 2));
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(ST_ACC));
+                return ST_ACC;
             } else if constexpr (EDGE) {
                 rows();
                 __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
             }
-            return;
+            return 0;
         }
     }
     if constexpr (TN % 2 != 0) {  // a single 16-column tile per wave: 8 B per lane (the host guarantees n % 4 == 0 etc.)
@@ -711,18 +725,21 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
             }
         }
     }
+    return 0;
     };
 
     // ---- compute state ---------------------------------------------------------------------------------------
     int c_index = blockIdx.x;
     Work cw = decode(c_index);
     int c_left = cw.iters, c_stage = 0;
+    int behind = 0;  // stores of the previous work item that may still be in flight
     issue();
     sync_tile();
     read_first(smem);
     for (;;) {
         for (; c_left > 1; --c_left) {
-            tile_body(c_stage, std::true_type{});
+            tile_body(c_stage, std::true_type{});  // waits for everything outstanding and requests a tile
+            behind = 0;
             c_stage ^= 1;
         }
         tile_body(c_stage, std::false_type{});
@@ -732,8 +749,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
         // the next tile is computed.  (Converting the accumulators before that wait was tried: it costs registers
         // inside the k loop and lost.)
         const bool more = c_index + (int)gridDim.x < p.total_blocks;
-        if (more) sync_tile();
-        store_tile(cw);
+        if (more) sync_tile(behind);
+        behind = __builtin_amdgcn_readfirstlane(store_tile(cw));
         if (!more) break;
 #pragma unroll
         for (int i = 0; i < TM; i++)
