@@ -22,7 +22,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
-    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (and torch: vendor-library cross-check, only on request)")
+    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them)")
     ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "mfma-power"],
                     help="counter-collection aids for rocprofv3, nothing is timed: traffic = 3 plain 256 MiB device copies (a kernel "
                          "of known size that calibrates FETCH_SIZE / WRITE_SIZE) then 5 launches of the 4096^3 f16 GEMM; rows = the same copies, then 3 launches each of "
@@ -404,6 +404,29 @@ def main():
                 gemm("gemv", f"vec.mat {dt}, Linear weight view", dev.gemm_desc(dt, 1, n_, n_, P(xv), (n_, 1), P(W), (1, n_), P(yv), (n_, 1)), 2 * n_ * n_, es * n_ * n_, 100, bufs=(W, xv, yv))
                 gemm("gemv", f"mat.vec {dt} ({n_},{n_})x({n_},)", dev.gemm_desc(dt, n_, n_, 1, P(W), (n_, 1), P(xv), (1, 1), P(yv), (1, 1)), 2 * n_ * n_, es * n_ * n_, 100, bufs=(W, xv, yv))
                 del W
+
+    # ---- operands off the 16-byte grid: an LM head with 50257 outputs, a first-layer convolution -------------------
+    if "edge" in only:   # on request: the scalar kernel's rows take milliseconds each
+        from dfdx_amd.rocm import KERNEL_GENERIC
+        for dt in ("f16", "f32"):
+            M, K = 2048, 1024
+            for N in (50257, 50264):
+                x, W, y = rnd((M, K), dt), rnd((N, K), dt, 0.03), zeros((M, N), dt)
+                go, gx, gw = rnd((M, N), dt), zeros((M, K), dt), zeros((N, K), dt)
+                fl = 2.0 * M * K * N
+                cases = (("LM head fwd x.W^T", (M, K, N, P(x), (K, 1), P(W), (1, K), P(y), (N, 1)), False),
+                         ("LM head dX go.W", (M, N, K, P(go), (N, 1), P(W), (K, 1), P(gx), (K, 1)), True),
+                         ("LM head dW go^T.x", (N, M, K, P(go), (1, N), P(x), (K, 1), P(gw), (K, 1)), True))
+                for name, a, acc in cases:
+                    gemm("edge", f"{name} {dt} N={N}", dev.gemm_desc(dt, *a, accumulate=acc), fl, 0, 10)
+                    if N % 8:
+                        gemm("edge", f"{name} {dt} N={N}, scalar kernel forced", dev.gemm_desc(dt, *a, accumulate=acc, kernel=KERNEL_GENERIC), fl, 0, 3)
+                del x, W, y, go, gx, gw
+        for dt in ("f16", "f32"):
+            B, C, O, H, W_, K = 32, 3, 64, 224, 224, 3
+            xv, wv = view(rnd((B, C, H, W_), dt), dt), view(rnd((O, C, K, K), dt, 0.2), dt)
+            fl = 2.0 * B * O * C * K * K * H * W_
+            timed("edge", f"conv2d fwd {dt} B{B} 3->64 224x224 k3 (C*K*K = 27)", lambda: dev.conv2d_forward(xv, wv, stride=1, padding=1), fl, 0, "conv2d_forward")
 
     # ---- config 5 end to end: one encoder block, every op on the device -----------------------------------------
     if want("block"):

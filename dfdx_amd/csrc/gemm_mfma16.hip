@@ -45,6 +45,7 @@ struct Params {
     int kbatches;  // batches folded into the k loop (reduce mode), else 1
     int tiles_m, tiles_n, tiles_per_batch, total_blocks;
     int accumulate, bias_mode, c_vec;
+    int window;  // operands that 16 B-aligned vector loads cannot walk (odd leading dimension, extent or address): window loads
     int group_m;
     ConvPatches conv;  // CONV_B kernels: B is the patch matrix of a unit-stride convolution, formed on the fly
 };
@@ -114,7 +115,7 @@ template <int ROWS, int BK, int NT, bool KC> struct Loader {
                 soff[u] = (mb * 8) * LDS_ROW + kb * KR;
 #pragma unroll
                 for (int r = 0; r < KR; r++) {
-                    goff[u * KR + r] = (uint32_t)((kb * KR + r) * ld + min(mb * 8, rows_left - 8)) * 2u;
+                    goff[u * KR + r] = (uint32_t)((kb * KR + r) * ld + max(min(mb * 8, rows_left - 8), 0)) * 2u;
                     koff[u * KR + r] = kb * KR + r;
                 }
             }
@@ -173,6 +174,31 @@ template <int ROWS, int BK, int NT, bool KC> struct Loader {
     __device__ __forceinline__ void load_tail(const uint16_t *g, int k_left) {
 #pragma unroll
         for (int i = 0; i < LOADS; i++) regs[i] = ldg16((const uint16_t *)((const char *)g + goff[i]), koff[i] < k_left);
+    }
+
+    // The same tile for an operand whose rows do not start on 16 B boundaries, or whose contiguous extent is not a
+    // multiple of 8: every 8-element piece is one unaligned 16 B load from the nearest window inside the matrix,
+    // shifted into place, zeros beyond the extent (row_window_bytes).  `g` = tile origin (first row r0, first k k0);
+    // the contiguous extent (k_total if KC, else rows_total) is at least 8.
+    __device__ __forceinline__ void load_window(const uint16_t *g, int ld, int k0, int k_total, int r0, int rows_total, int tid) {
+        if constexpr (KC) {
+#pragma unroll
+            for (int i = 0; i < LOADS; i++) {
+                const char *row = (const char *)g + (goff[i] - (uint32_t)koff[i] * 2u) - (int64_t)k0 * 2;  // k = 0 of the (clamped) row
+                regs[i] = row_window_bytes<2>(row, true, k0 + koff[i], k_total);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) {
+                const int mb = (u * NT + tid) / NKB;
+#pragma unroll
+                for (int r = 0; r < KR; r++) {
+                    const int i = u * KR + r;
+                    const char *krow = (const char *)g + (int64_t)koff[i] * ld * 2 - (int64_t)r0 * 2;  // row 0 of this k
+                    regs[i] = row_window_bytes<2>(krow, k0 + koff[i] < k_total, r0 + mb * 8, rows_total);
+                }
+            }
+        }
     }
 
     __device__ __forceinline__ void store(uint16_t *lds) const {
@@ -287,10 +313,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
 
     // The k loop exists twice: K a multiple of BK runs with unpredicated loads only; any
     // other K runs with the k-tail predicate on every load.
-    auto k_loop = [&](auto tail_tag) {
-        constexpr bool TAIL = decltype(tail_tag)::value;
+    auto k_loop = [&](auto tail_tag, auto window_tag) {
+        constexpr bool TAIL = decltype(tail_tag)::value, WINDOW = decltype(window_tag)::value;
         auto fetch = [&]() {
-            if constexpr (TAIL) {
+            if constexpr (WINDOW) {
+                la.load_window(a_next, p.lda, f_kt * BK, p.k, bm0, p.m, tid);
+                if constexpr (!CONV_B) lb.load_window(b_next, p.ldb, f_kt * BK, p.k, bn0, p.n, tid);
+            } else if constexpr (TAIL) {
                 const int kl = p.k - f_kt * BK;
                 la.load_tail(a_next, kl);
                 if constexpr (!CONV_B) lb.load_tail(b_next, kl);
@@ -332,8 +361,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
             __syncthreads();
         }
     };
-    if (p.k % BK == 0) k_loop(std::false_type{});
-    else k_loop(std::true_type{});
+    if constexpr (!CONV_B) {
+        if (p.window) k_loop(std::true_type{}, std::true_type{});
+        else if (p.k % BK == 0) k_loop(std::false_type{}, std::false_type{});
+        else k_loop(std::true_type{}, std::false_type{});
+    } else {
+        if (p.k % BK == 0) k_loop(std::false_type{}, std::false_type{});
+        else k_loop(std::true_type{}, std::false_type{});
+    }
 
     // ---- epilogue: lane holds m = l32 (per tile), n = 8g + 4*lh + 0..3 --------
     const int cb = p.kbatches > 1 ? 0 : batch;
@@ -482,16 +517,26 @@ inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 // element and rows are 16 B apart), rows-contiguous when the row stride is 1.
 struct OperandLayout {
     bool ok, kc;
+    bool window;  // walkable, but not by 16 B-aligned loads: odd leading dimension or extent (the kernel's window loads)
     int64_t ld;
 };
 inline OperandLayout classify(int64_t rows, int64_t kdim, int64_t row_stride, int64_t k_stride) {
-    OperandLayout r{false, false, 0};
+    OperandLayout r{false, false, false, 0};
     if (k_stride == 1 && kdim % 8 == 0 && (rows == 1 || (row_stride % 8 == 0 && row_stride >= kdim))) {
         r.ok = true; r.kc = true; r.ld = rows == 1 ? kdim : row_stride;
     } else if (row_stride == 1 && rows % 8 == 0 && (kdim == 1 || (k_stride % 8 == 0 && k_stride >= rows))) {
         r.ok = true; r.kc = false; r.ld = kdim == 1 ? rows : k_stride;
+    } else if (k_stride == 1 && kdim >= 8 && (rows == 1 || row_stride >= kdim)) {
+        r.ok = true; r.kc = true; r.window = true; r.ld = rows == 1 ? kdim : row_stride;
+    } else if (row_stride == 1 && rows >= 8 && (kdim == 1 || k_stride >= rows)) {
+        r.ok = true; r.kc = false; r.window = true; r.ld = kdim == 1 ? rows : k_stride;
     }
     return r;
+}
+// Window loads for the whole launch when either operand needs them, or an address / batch stride is not 16 B-aligned.
+inline bool needs_window(const GemmProblem &p, const OperandLayout &la, const OperandLayout &lb) {
+    if (la.window || lb.window || !aligned16(p.a) || !aligned16(p.b)) return true;
+    return p.nb1 * p.nb2 > 1 && (p.a_b1 % 8 || p.a_b2 % 8 || p.b_b1 % 8 || p.b_b2 % 8);
 }
 
 }  // namespace
@@ -517,11 +562,8 @@ bool mfma16_supported(const GemmProblem &p, int variant) {
     const Variant &v = kVariants[variant - 1];
     // 32-bit offsets inside one tile
     if (la.ld * (la.kc ? v.bm : v.bk) >= (1ll << 30) || lb.ld * (lb.kc ? v.bn : v.bk) >= (1ll << 30)) return false;
-    if (!aligned16(p.a) || !aligned16(p.b)) return false;
-    if (p.nb1 * p.nb2 > 1) {
-        if (p.a_b1 % 8 || p.a_b2 % 8 || p.b_b1 % 8 || p.b_b2 % 8) return false;
-        if (p.a_b1 < 0 || p.a_b2 < 0 || p.b_b1 < 0 || p.b_b2 < 0) return false;
-    }
+    if (((uintptr_t)p.a | (uintptr_t)p.b) & 1u) return false;  // elements sit on 2 B boundaries at least
+    if (p.nb1 * p.nb2 > 1 && (p.a_b1 < 0 || p.a_b2 < 0 || p.b_b1 < 0 || p.b_b2 < 0)) return false;
     const int64_t tiles = ((p.m + v.bm - 1) / v.bm) * ((p.n + v.bn - 1) / v.bn);
     const int64_t blocks = tiles * (p.reduce ? 1 : p.nb1 * p.nb2);
     if (blocks >= (1ll << 31) || p.nb1 * p.nb2 >= (1ll << 31)) return false;
@@ -585,6 +627,7 @@ hipError_t launch_mfma16(const GemmProblem &g, int variant, hipStream_t stream) 
     p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
     p.c_vec = (g.n % 4 == 0) && (p.ldc % 4 == 0) && (((uintptr_t)g.c & 7u) == 0) &&
               (g.c_b1 % 4 == 0) && (g.c_b2 % 4 == 0) && (!g.bias || ((uintptr_t)g.bias & 7u) == 0);
+    p.window = needs_window(g, la, lb);
     p.group_m = 4;
     p.conv = ConvPatches{};
     if (g.dtype == DT_F16) return launch_variant<_Float16>(variant, p, la.kc, lb.kc, stream);
@@ -596,7 +639,7 @@ hipError_t launch_mfma16_conv(const GemmProblem &g, const ConvPatches &conv, int
     if (g.reduce || g.bias || g.m < 1 || g.n < 8 || g.k < 8) return hipErrorNotSupported;
     if (g.m >= (1 << 30) || g.n >= (1 << 30) || g.k >= (1 << 30) || g.nb1 * g.nb2 >= (1ll << 31)) return hipErrorNotSupported;
     const OperandLayout la = classify(g.m, g.k, g.a_rs, g.a_cs);
-    if (!la.ok || !la.kc || !aligned16(g.a) || g.a_b1 % 8 || g.a_b2 % 8 || g.a_b1 < 0 || g.a_b2 < 0) return hipErrorNotSupported;
+    if (!la.ok || !la.kc || la.window || !aligned16(g.a) || g.a_b1 % 8 || g.a_b2 % 8 || g.a_b1 < 0 || g.a_b2 < 0) return hipErrorNotSupported;
     if (g.c_cs != 1 || g.n % 4 || g.c_rs % 4 || g.c_rs < g.n || ((uintptr_t)g.c & 7u) || g.c_b1 % 4 || g.c_b2 % 4) return hipErrorNotSupported;
     if (conv.w_dst < 8 || g.n % conv.w_dst || conv.w_src < 8 || conv.taps != conv.ksize * conv.ksize ||
         g.k % conv.taps || g.b_b1 < 0 || g.b_b2 < 0 || ((uintptr_t)g.b & 1u))
@@ -621,6 +664,7 @@ hipError_t launch_mfma16_conv(const GemmProblem &g, const ConvPatches &conv, int
     p.total_blocks = (int)blocks;
     p.accumulate = g.accumulate; p.bias_mode = BIAS_NONE;
     p.c_vec = 1;
+    p.window = 0;
     p.group_m = 4;
     p.conv = conv;
     if (g.dtype == DT_F16) return launch_conv_variant<_Float16>(variant, p, stream);

@@ -13,6 +13,7 @@
 // stride; pointers, leading and batch strides multiples of 4 elements (16 B); the
 // contiguous extent a multiple of 4.
 #include "gemm_internal.h"
+#include "elem.h"
 
 namespace dfdx_rocm {
 namespace {
@@ -32,6 +33,7 @@ struct Params {
     int nb2, kbatches;
     int tiles_m, tiles_n, tiles_per_batch, total_blocks;
     int accumulate, bias_mode, c_vec;
+    int window;  // operands that 16 B-aligned vector loads cannot walk (odd leading dimension, extent or address): window loads
     int group_m;
     // split-k: k-loop steps [split * chunk, +chunk) per workgroup, f32 partial tiles to ws[split][row][col]
     int splits, chunk;
@@ -61,6 +63,21 @@ template <int ROWS, int BK, int NT, bool KC> struct Loader {
             else regs[i] = ldg4(g + r * ld + ch * 4, ch * 4 < rows_left && r < k_left);
         }
     }
+    // The same tile for an operand whose rows do not start on 16 B boundaries, or whose contiguous extent is not a
+    // multiple of 4: every 4-element piece is one unaligned 16 B load from the nearest window inside the matrix,
+    // shifted into place, zeros beyond the extent (row_window_bytes).  `g` = tile origin: first row r0 of rows_total,
+    // first k k0 of k_total; the contiguous extent is at least 4.
+    __device__ __forceinline__ void load_window(const float *g, int ld, int r0, int rows_total, int k0, int k_total, int tid) {
+#pragma unroll
+        for (int i = 0; i < LOADS; i++) {
+            const int cid = i * NT + tid;
+            const int r = cid / CPR, ch = cid % CPR;
+            u32x4 w;
+            if constexpr (KC) w = row_window_bytes<4>(g + (int64_t)min(r, rows_total - r0 - 1) * ld - k0, true, k0 + ch * 4, k_total);
+            else w = row_window_bytes<4>(g + (int64_t)r * ld - r0, k0 + r < k_total, r0 + ch * 4, rows_total);
+            regs[i] = __builtin_bit_cast(f32x4, w);
+        }
+    }
     __device__ __forceinline__ void store_piece(float *lds, int tid, int i) const {
         const int cid = i * NT + tid;
         const int r = cid / CPR, ch = cid % CPR;
@@ -76,7 +93,9 @@ template <int ROWS, int BK, int NT, bool KC> struct Loader {
     }
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC>
+// WINDOW: operands off the 16-byte grid, fetched with window loads (an instantiation of its own: the aligned kernels
+// keep their register allocation).
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool WINDOW>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(const Params p) {
     constexpr int NT = WAVES_M * WAVES_N * 64;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
@@ -127,10 +146,19 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
         const int kt = p.kbatches > 1 ? it % ktiles : it;
         return p.k - kt * BK;
     };
+    auto fetch = [&](LA &la_, LB &lb_, int it) {
+        if constexpr (WINDOW) {
+            const int k0 = p.k - k_left(it);
+            la_.load_window(a_tile(it), p.lda, bm0, p.m, k0, p.k, tid);
+            lb_.load_window(b_tile(it), p.ldb, bn0, p.n, k0, p.k, tid);
+        } else {
+            la_.load(a_tile(it), p.lda, p.m - bm0, k_left(it), tid);
+            lb_.load(b_tile(it), p.ldb, p.n - bn0, k_left(it), tid);
+        }
+    };
 
     LA la;
     LB lb;
-    const int rows_left = p.m - bm0, cols_left = p.n - bn0;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -141,8 +169,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     if (iters > 0) {
-        la.load(a_tile(it0), p.lda, rows_left, k_left(it0), tid);
-        lb.load(b_tile(it0), p.ldb, cols_left, k_left(it0), tid);
+        fetch(la, lb, it0);
         la.store(As, tid);
         lb.store(Bs, tid);
     }
@@ -196,8 +223,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
     float af_first[TM][4], bf_first[TN][4];
     if (iters > 0) read_frags(a_frag0, b_frag0, 0, af_first, bf_first);
     if (iters > 1) {   // the second tile waits in registers while the first is computed
-        la.load(a_tile(it0 + 1), p.lda, rows_left, k_left(it0 + 1), tid);
-        lb.load(b_tile(it0 + 1), p.ldb, cols_left, k_left(it0 + 1), tid);
+        fetch(la, lb, it0 + 1);
     }
     for (int it = 0; it < iters; it++) {
         const int cur = it & 1;
@@ -231,8 +257,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_kernel(cons
                     }
         }
         if (it + 2 < iters) {
-            la.load(a_tile(it0 + it + 2), p.lda, rows_left, k_left(it0 + it + 2), tid);
-            lb.load(b_tile(it0 + it + 2), p.ldb, cols_left, k_left(it0 + it + 2), tid);
+            fetch(la, lb, it0 + it + 2);
         }
 #pragma unroll
         for (int ks = 1; ks < KS; ks++) {
@@ -328,14 +353,14 @@ constexpr Variant kVariants[] = {
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
-template <int BM, int BN, int BK, int WM, int WN>
+template <int BM, int BN, int BK, int WM, int WN, bool WINDOW>
 hipError_t launch_layout(const Params &p, bool a_kc, bool b_kc, hipStream_t stream) {
     constexpr int NT = WM * WN * 64;
     dim3 grid((unsigned)p.total_blocks), block(NT);
 #define DFDX_LAUNCH(AKC, BKC)                                                                                   \
     do {                                                                                                        \
         constexpr size_t lds = (size_t)2 * 4 * (Loader<BM, BK, NT, AKC>::LDS_SIZE + Loader<BN, BK, NT, BKC>::LDS_SIZE); \
-        auto kern = gemm_mfma32_kernel<BM, BN, BK, WM, WN, AKC, BKC>;                                           \
+        auto kern = gemm_mfma32_kernel<BM, BN, BK, WM, WN, AKC, BKC, WINDOW>;                                   \
         static PerDevice configured_on;                                                                         \
         std::atomic<int> &configured = configured_on.here();                                                    \
         if (!configured.load(std::memory_order_acquire)) {                                                      \
@@ -358,16 +383,26 @@ inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 struct OperandLayout {
     bool ok, kc;
+    bool window;  // walkable, but not by 16 B-aligned loads: odd leading dimension or extent (the kernel's window loads)
     int64_t ld;
 };
 inline OperandLayout classify(int64_t rows, int64_t kdim, int64_t row_stride, int64_t k_stride) {
-    OperandLayout r{false, false, 0};
+    OperandLayout r{false, false, false, 0};
     if (k_stride == 1 && kdim % 4 == 0 && (rows == 1 || (row_stride % 4 == 0 && row_stride >= kdim))) {
         r.ok = true; r.kc = true; r.ld = rows == 1 ? kdim : row_stride;
     } else if (row_stride == 1 && rows % 4 == 0 && (kdim == 1 || (k_stride % 4 == 0 && k_stride >= rows))) {
         r.ok = true; r.kc = false; r.ld = kdim == 1 ? rows : k_stride;
+    } else if (k_stride == 1 && kdim >= 4 && (rows == 1 || row_stride >= kdim)) {
+        r.ok = true; r.kc = true; r.window = true; r.ld = rows == 1 ? kdim : row_stride;
+    } else if (row_stride == 1 && rows >= 4 && (kdim == 1 || k_stride >= rows)) {
+        r.ok = true; r.kc = false; r.window = true; r.ld = kdim == 1 ? rows : k_stride;
     }
     return r;
+}
+// Window loads for the whole launch when either operand needs them, or an address / batch stride is not 16 B-aligned.
+inline bool needs_window(const GemmProblem &p, const OperandLayout &la, const OperandLayout &lb) {
+    if (la.window || lb.window || !aligned16(p.a) || !aligned16(p.b)) return true;
+    return p.nb1 * p.nb2 > 1 && (p.a_b1 % 4 || p.a_b2 % 4 || p.b_b1 % 4 || p.b_b2 % 4);
 }
 
 }  // namespace
@@ -387,11 +422,8 @@ bool mfma32_supported(const GemmProblem &p, int variant) {
     if (!la.ok || !lb.ok) return false;
     const Variant &v = kVariants[variant - 1];
     if (la.ld * (la.kc ? v.bm : v.bk) >= (1ll << 31) || lb.ld * (lb.kc ? v.bn : v.bk) >= (1ll << 31)) return false;
-    if (!aligned16(p.a) || !aligned16(p.b)) return false;
-    if (p.nb1 * p.nb2 > 1) {
-        if (p.a_b1 % 4 || p.a_b2 % 4 || p.b_b1 % 4 || p.b_b2 % 4) return false;
-        if (p.a_b1 < 0 || p.a_b2 < 0 || p.b_b1 < 0 || p.b_b2 < 0) return false;
-    }
+    if (((uintptr_t)p.a | (uintptr_t)p.b) & 3u) return false;  // elements sit on 4 B boundaries at least
+    if (p.nb1 * p.nb2 > 1 && (p.a_b1 < 0 || p.a_b2 < 0 || p.b_b1 < 0 || p.b_b2 < 0)) return false;
     const int64_t tiles = ((p.m + v.bm - 1) / v.bm) * ((p.n + v.bn - 1) / v.bn);
     const int64_t blocks = tiles * (p.reduce ? 1 : p.nb1 * p.nb2);
     if (blocks >= (1ll << 31) || p.nb1 * p.nb2 >= (1ll << 31)) return false;
@@ -512,6 +544,7 @@ hipError_t launch_mfma32(const GemmProblem &g, int variant, hipStream_t stream) 
     p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
     p.c_vec = (g.n % 4 == 0) && (p.ldc % 4 == 0) && (((uintptr_t)g.c & 15u) == 0) &&
               (g.c_b1 % 4 == 0) && (g.c_b2 % 4 == 0) && (!g.bias || ((uintptr_t)g.bias & 15u) == 0);
+    p.window = needs_window(g, la, lb);
     p.group_m = 4;
     const int total_iters = (int)(((g.k + v.bk - 1) / v.bk) * p.kbatches);
     p.splits = 1; p.chunk = total_iters; p.ws = nullptr; p.ws_ld = 0; p.ws_split_stride = 0;
@@ -531,15 +564,19 @@ hipError_t launch_mfma32(const GemmProblem &g, int variant, hipStream_t stream) 
 
 static hipError_t launch_tiles(const Params &p, int variant, bool a_kc, bool b_kc, hipStream_t stream) {
     struct { bool kc; } la{a_kc}, lb{b_kc};
+#define DFDX_TILE(BM, BN, WM, WN)                                                                    \
+    return p.window ? launch_layout<BM, BN, 32, WM, WN, true>(p, la.kc, lb.kc, stream)               \
+                    : launch_layout<BM, BN, 32, WM, WN, false>(p, la.kc, lb.kc, stream)
     switch (variant) {
-    case 1: return launch_layout<256, 256, 32, 2, 4>(p, la.kc, lb.kc, stream);
-    case 2: return launch_layout<256, 256, 32, 2, 2>(p, la.kc, lb.kc, stream);
-    case 3: return launch_layout<256, 128, 32, 2, 2>(p, la.kc, lb.kc, stream);
-    case 4: return launch_layout<128, 128, 32, 2, 2>(p, la.kc, lb.kc, stream);
-    case 5: return launch_layout<128, 64, 32, 4, 1>(p, la.kc, lb.kc, stream);
-    case 6: return launch_layout<64, 64, 32, 2, 2>(p, la.kc, lb.kc, stream);
+    case 1: DFDX_TILE(256, 256, 2, 4);
+    case 2: DFDX_TILE(256, 256, 2, 2);
+    case 3: DFDX_TILE(256, 128, 2, 2);
+    case 4: DFDX_TILE(128, 128, 2, 2);
+    case 5: DFDX_TILE(128, 64, 4, 1);
+    case 6: DFDX_TILE(64, 64, 2, 2);
     default: return hipErrorInvalidValue;
     }
+#undef DFDX_TILE
 }
 
 }  // namespace dfdx_rocm

@@ -66,6 +66,8 @@ CONFIGS = [
     (2, 32, 48, 7, 7, 3, 1, 1, 1, 1),      # n = 49
     (2, 16, 32, 15, 13, 3, 2, 1, 1, 1),    # input 195 and output 56 positions: only the backward side is padded
     (3, 32, 64, 24, 40, 5, 1, 2, 2, 1),
+    (2, 3, 64, 32, 32, 3, 1, 1, 1, 1),     # a first layer: C*K*K = 27, a contraction no 16-byte load can walk (window loads)
+    (2, 3, 64, 30, 30, 3, 2, 1, 1, 1),     # the same through the patch matrix (stride 2), 15 x 15 = 225 output pixels
 ]
 
 

@@ -202,9 +202,61 @@ def test_auto_dispatch_prefers_mfma_when_aligned():
     d = dev.gemm_desc("f16", 256, 256, 256, a.ptr, (256, 1), a.ptr, (256, 1), a.ptr, (256, 1))
     assert dev.gemm_plan(d)[0] == KERNEL_MFMA
     d = dev.gemm_desc("f16", 255, 256, 256, a.ptr, (1, 256), a.ptr, (256, 1), a.ptr, (256, 1))
-    assert dev.gemm_plan(d)[0] == KERNEL_GENERIC  # M-contiguous A with M % 8 != 0
+    assert dev.gemm_plan(d)[0] == KERNEL_MFMA     # M-contiguous A with M % 8 != 0: the MFMA kernel's window loads
+    d = dev.gemm_desc("f16", 128, 64, 128, a.ptr, (128, 2), a.ptr, (256, 1), a.ptr, (256, 1))
+    assert dev.gemm_plan(d)[0] == KERNEL_GENERIC  # neither stride of A is 1
     d = dev.gemm_desc("f64", 256, 256, 256, a.ptr, (256, 1), a.ptr, (256, 1), a.ptr, (256, 1))
     assert dev.gemm_plan(d)[0] == KERNEL_GENERIC
+
+
+# ------------------------------------------- operands off the 16-byte grid --
+UNALIGNED_SHAPES = [
+    # (m, k, n): odd everything; a vocabulary-sized extent (GPT-2's 50257) as n, as k and as m; k below one MFMA step
+    (67, 45, 83), (33, 50257, 24), (16, 72, 50257), (50257, 40, 24), (130, 9, 70), (8, 8, 8), (257, 129, 255),
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("shape", UNALIGNED_SHAPES)
+def test_unaligned_operands_run_on_the_mfma_kernels(dtype, shape):
+    """Leading dimensions, extents and base addresses that are not multiples of 16 bytes (an LM head with 50257 outputs,
+    its two gradients, a first-layer convolution with C*K*K = 27): the register-staged MFMA kernels walk such operands
+    with window loads; only a view with no unit stride at all is left to the scalar kernel."""
+    m, k, n = shape
+    dev = device()
+    for i, layout in enumerate(LAYOUTS):
+        pads = ((1, 3, 5), (0, 0, 0), (7, 1, 0), (2, 2, 2))[i]
+        g = rng(900 + i)
+        at, bt = LAYOUTS[layout]
+        a, astr = make_operand(g, m, k, at, dtype, pads[0])
+        b, bstr = make_operand(g, k, n, bt, dtype, pads[1])
+        da, db = dev.tensor(a, dtype), dev.tensor(b, dtype)
+        dc = dev.zeros(dtype, (m, n + pads[2]))
+        desc = dev.gemm_desc(dtype, m, k, n, da.ptr, astr, db.ptr, bstr, dc.ptr, (n + pads[2], 1))
+        assert dev.gemm_plan(desc)[0] == KERNEL_MFMA, (shape, layout, dev.gemm_plan(desc))
+        run_case(dtype, m, k, n, layout, bool(i % 2), KERNEL_AUTO, 0, c_colmajor=(i == 3), seed=900 + i, pads=pads)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_unaligned_base_address_and_batch_strides(dtype):
+    """Operands that start one element into their allocation, batches an odd number of elements apart."""
+    dev, g = device(), rng(77)
+    nb, m, k, n = 3, 70, 52, 41
+    es = {"f16": 2, "f32": 4}[dtype]
+    a_st = oracle.to_storage(g.standard_normal(1 + nb * (m * k + 1)), dtype)
+    b_st = oracle.to_storage(g.standard_normal(1 + nb * (k * n + 3)), dtype)
+    da, db, dc = dev.tensor(a_st, dtype), dev.tensor(b_st, dtype), dev.zeros(dtype, (nb, m, n))
+    desc = dev.gemm_desc(dtype, m, k, n, da.ptr + es, (k, 1), db.ptr + es, (n, 1), dc.ptr, (n, 1), batch=(nb, 1),
+                         a_batch=(m * k + 1, 0), b_batch=(k * n + 3, 0), c_batch=(m * n, 0))
+    assert dev.gemm_plan(desc)[0] == KERNEL_MFMA
+    announce("gemm unaligned base / batch strides", dtype, dev.gemm_plan(desc)[2])
+    dev.gemm(desc)
+    got = oracle.to_f64(dev.to_host(dc), dtype).reshape(nb, m, n)
+    A64, B64 = oracle.to_f64(a_st, dtype), oracle.to_f64(b_st, dtype)
+    for i in range(nb):
+        A = A64[1 + i * (m * k + 1):][:m * k].reshape(m, k)
+        B = B64[1 + i * (k * n + 3):][:k * n].reshape(k, n)
+        assert_within(dtype, k, got[i], A @ B, A, B, extra=1e-6, what=f"batch {i}")
 
 
 # --------------------------------------------------------------------- gemv --
