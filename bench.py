@@ -2,7 +2,7 @@
 
 A step is one 4096^3 f16 GEMM (f32 accumulate), C = A.B with row-major operands ~U(-1,1) resident in
 HBM -- the configuration the headline metric is quoted on.  The same launch is also timed for the
-transposed-stride variants and for f32.  One JSON line is printed:
+transposed-stride variants, for f32, bf16 and f64.  One JSON line is printed:
 
   value       f16 A.B throughput in TFLOP/s: the LOWER of (a) the K timed steps by the wall clock, synchronised on both
               sides, and (b) HIP events around max(K, 200) launches on the launch stream -- K = 20 launches are 2 ms of
@@ -23,7 +23,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
+PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3, "f64": 78.6}   # MI355X dense MFMA peaks
 N = 4096
 
 
@@ -47,7 +47,7 @@ def main():
     dev = Rocm(0)
     info = dev.device_info()
     flop = 2.0 * N ** 3
-    tdt = {"f16": torch.float16, "f32": torch.float32, "bf16": torch.bfloat16}
+    tdt = {"f16": torch.float16, "f32": torch.float32, "bf16": torch.bfloat16, "f64": torch.float64}
     res = {}
     headline = None
     if args.spinup_ms > 0:
@@ -63,14 +63,14 @@ def main():
                 dev.gemm(sd)
             torch.cuda.synchronize()
         del sa, sc
-    for dtype in ("f16", "f32", "bf16"):
+    for dtype in ("f16", "f32", "bf16", "f64"):
         gen = torch.Generator(device="cuda").manual_seed(1234)
         a = (torch.rand(N, N, device="cuda", generator=gen) * 2 - 1).to(tdt[dtype])
         b = (torch.rand(N, N, device="cuda", generator=gen) * 2 - 1).to(tdt[dtype])
         c = torch.zeros(N, N, device="cuda", dtype=tdt[dtype])
         layouts = {"A.B": ((N, 1), (N, 1)), "At.B": ((1, N), (N, 1)), "A.Bt": ((N, 1), (1, N))}
-        if dtype == "bf16":
-            layouts = {"A.B": layouts["A.B"]}   # same kernel as f16; one layout as a cross-check
+        if dtype in ("bf16", "f64"):
+            layouts = {"A.B": layouts["A.B"]}   # bf16: same kernel as f16, one layout as a cross-check; f64: 2.7 ms a launch
         res[dtype] = {}
         for name, (astr, bstr) in layouts.items():
             desc = dev.gemm_desc(dtype, N, N, N, a.data_ptr(), astr, b.data_ptr(), bstr, c.data_ptr(), (N, 1))

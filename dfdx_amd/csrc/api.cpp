@@ -247,7 +247,7 @@ struct Plan {
 
 int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProblem &p, Plan *plan) {
     const bool is16 = p.dtype == DT_F16 || p.dtype == DT_BF16;
-    const bool is32 = p.dtype == DT_F32;
+    const bool is32 = p.dtype == DT_F32, is64 = p.dtype == DT_F64;
     // split-k: 1 = never (NO_SPLIT_K), n = forced by the caller, 0 = let the planner decide
     const int forced_splits = (d->flags & DFDX_ROCM_GEMM_NO_SPLIT_K) ? 1 : ((d->flags >> 8) & 0xff);
     switch (d->kernel) {
@@ -269,8 +269,10 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
             }
             if (v) return DFDX_ROCM_ERR_UNSUPPORTED;
         }
-        if (v == 0) v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units, forced_splits) : 0;
-        const bool ok = is16 ? mfma16_supported(p, v) : is32 ? mfma32_supported(p, v) : false;
+        if (v == 0)
+            v = is16 ? mfma16_pick_variant(p, ctx->compute_units)
+                     : is32 ? mfma32_pick_variant(p, ctx->compute_units, forced_splits) : is64 ? mfma64_pick_variant(p, ctx->compute_units) : 0;
+        const bool ok = is16 ? mfma16_supported(p, v) : is32 ? mfma32_supported(p, v) : is64 ? mfma64_supported(p, v) : false;
         if (!ok) return DFDX_ROCM_ERR_UNSUPPORTED;
         *plan = {DFDX_ROCM_KERNEL_MFMA, v, is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
         return DFDX_ROCM_OK;
@@ -292,7 +294,8 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
             return DFDX_ROCM_OK;
         }
     }
-    int v = is16 ? mfma16_pick_variant(p, ctx->compute_units) : is32 ? mfma32_pick_variant(p, ctx->compute_units, forced_splits) : 0;
+    int v = is16 ? mfma16_pick_variant(p, ctx->compute_units)
+                 : is32 ? mfma32_pick_variant(p, ctx->compute_units, forced_splits) : is64 ? mfma64_pick_variant(p, ctx->compute_units) : 0;
     if (v > 0) {
         *plan = {DFDX_ROCM_KERNEL_MFMA, v, is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
         return DFDX_ROCM_OK;
@@ -337,7 +340,8 @@ int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan, b
     case DFDX_ROCM_KERNEL_GENERIC: e = launch_generic(p, ctx->stream); break;
     case DFDX_ROCM_KERNEL_GEMV: e = launch_gemv(p, ctx->stream); break;
     case DFDX_ROCM_KERNEL_MFMA:
-        e = (p.dtype == DT_F32) ? launch_mfma32(p, plan.variant, ctx->stream) : launch_mfma16(p, plan.variant, ctx->stream);
+        e = (p.dtype == DT_F32) ? launch_mfma32(p, plan.variant, ctx->stream)
+                                : (p.dtype == DT_F64) ? launch_mfma64(p, plan.variant, ctx->stream) : launch_mfma16(p, plan.variant, ctx->stream);
         break;
     default: return DFDX_ROCM_ERR_INVALID_ARG;
     }
@@ -637,6 +641,8 @@ int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int
         if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1)
             std::snprintf(name, name_len, "%s_%s_splitk%d", p.dtype == DT_F32 ? "mfma32" : "mfma16",
                           p.dtype == DT_F32 ? mfma32_variant_name(plan.variant) : mfma16_variant_name(plan.variant), plan.splits);
+        else if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && p.dtype == DT_F64)
+            std::snprintf(name, name_len, "mfma64_%s", mfma64_variant_name(plan.variant));
         else if (plan.kernel == DFDX_ROCM_KERNEL_MFMA)
             std::snprintf(name, name_len, "%s_%s", p.dtype == DT_F32 ? "mfma32" : "mfma16",
                           p.dtype == DT_F32 ? mfma32_variant_name(plan.variant) : mfma16_variant_name(plan.variant));
@@ -649,6 +655,7 @@ int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int
 int dfdx_rocm_mfma_variant_count(int dtype) {
     if (dtype == DFDX_ROCM_F16 || dtype == DFDX_ROCM_BF16) return mfma16_variant_count();
     if (dtype == DFDX_ROCM_F32) return mfma32_variant_count();
+    if (dtype == DFDX_ROCM_F64) return mfma64_variant_count();
     return 0;
 }
 

@@ -108,6 +108,13 @@ int mfma32_plan_splits(const GemmProblem &p, int variant, int compute_units, int
 size_t mfma32_workspace_bytes(const GemmProblem &p, int variant, int splits);
 hipError_t launch_mfma32(const GemmProblem &p, int variant, hipStream_t stream);
 
+// ---- MFMA kernels for f64 (gemm_mfma64.hip) ----
+int mfma64_variant_count();
+const char *mfma64_variant_name(int variant);
+bool mfma64_supported(const GemmProblem &p, int variant);
+int mfma64_pick_variant(const GemmProblem &p, int compute_units);
+hipError_t launch_mfma64(const GemmProblem &p, int variant, hipStream_t stream);
+
 // ---- bandwidth-bound vector products (gemv.hip) ----
 bool gemv_supported(const GemmProblem &p);
 size_t gemv_workspace_bytes(const GemmProblem &p);  // f32 partial sums of the k slices (0 when not sliced)

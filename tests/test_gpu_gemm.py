@@ -206,7 +206,41 @@ def test_auto_dispatch_prefers_mfma_when_aligned():
     d = dev.gemm_desc("f16", 128, 64, 128, a.ptr, (128, 2), a.ptr, (256, 1), a.ptr, (256, 1))
     assert dev.gemm_plan(d)[0] == KERNEL_GENERIC  # neither stride of A is 1
     d = dev.gemm_desc("f64", 256, 256, 256, a.ptr, (256, 1), a.ptr, (256, 1), a.ptr, (256, 1))
-    assert dev.gemm_plan(d)[0] == KERNEL_GENERIC
+    assert dev.gemm_plan(d)[0] == KERNEL_MFMA and dev.gemm_plan(d)[2].startswith("mfma64")
+
+
+# ----------------------------------------------------------- f64 on MFMA --
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+def test_mfma_f64_variants(variant, layout):
+    """`MatMulImpl<f64>` (cpu_kernel.rs:189-229) on v_mfma_f64_16x16x4_f64: both tiles, every operand layout, extents that
+    are no multiple of anything, overwrite and accumulate, row- and column-major C, bias, a k of 1 and of one k tile."""
+    shapes = [(67, 45, 83), (130, 129, 200), (256, 16, 128), (16, 1, 16), (300, 64, 17)]
+    for i, (m, k, n) in enumerate(shapes):
+        run_case("f64", m, k, n, layout, bool(i % 2), KERNEL_MFMA, variant, c_colmajor=(i == 2), bias=(i == 1), seed=40 + i,
+                 pads=((0, 0, 0), (3, 1, 2))[i % 2])
+
+
+def test_mfma_f64_exact_on_integers_and_batched_reduce():
+    dev, g = device(), rng(41)
+    m, k, n, nb = 96, 80, 72, 5
+    A = g.integers(-3, 4, (nb, m, k)).astype(np.float64)
+    B = g.integers(-3, 4, (nb, k, n)).astype(np.float64)
+    da, db = dev.tensor(A.reshape(-1), "f64"), dev.tensor(B.reshape(-1), "f64")
+    dc = dev.zeros("f64", (nb, m, n))
+    desc = dev.gemm_desc("f64", m, k, n, da.ptr, (k, 1), db.ptr, (n, 1), dc.ptr, (n, 1), batch=(nb, 1),
+                         a_batch=(m * k, 0), b_batch=(k * n, 0), c_batch=(m * n, 0))
+    assert dev.gemm_plan(desc)[2].startswith("mfma64")
+    announce("gemm f64 batched", dev.gemm_plan(desc)[2])
+    dev.gemm(desc)
+    assert np.array_equal(dev.to_host(dc).reshape(nb, m, n), A @ B)
+    # all batches summed into one C, on top of what it holds (a broadcast operand's gradient)
+    dr = dev.tensor(np.ones(m * n), "f64")
+    desc = dev.gemm_desc("f64", m, k, n, da.ptr, (k, 1), db.ptr, (n, 1), dr.ptr, (n, 1), accumulate=True, batch=(nb, 1),
+                         a_batch=(m * k, 0), b_batch=(k * n, 0), reduce_batch=True)
+    announce("gemm f64 reduce", dev.gemm_plan(desc)[2])
+    dev.gemm(desc)
+    assert np.array_equal(dev.to_host(dr).reshape(m, n), (A @ B).sum(axis=0) + 1.0)
 
 
 # ------------------------------------------- operands off the 16-byte grid --
