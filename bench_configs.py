@@ -23,10 +23,11 @@ def main():
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
     ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them)")
-    ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "mfma-power"],
+    ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "f32-forms", "mfma-power"],
                     help="counter-collection aids for rocprofv3, nothing is timed: traffic = 3 plain 256 MiB device copies (a kernel "
                          "of known size that calibrates FETCH_SIZE / WRITE_SIZE) then 5 launches of the 4096^3 f16 GEMM; rows = the same copies, then 3 launches each of "
-                         "the HBM-bound rows (config 4 scores and dP, softmax forward and backward on them, the 16384^2 f16 vec.mat); variants = 3 "
+                         "the HBM-bound rows (config 4 scores and dP, softmax forward and backward on them, the 16384^2 f16 vec.mat); f32-forms = 3 "
+                         "launches each of the register-staged and the LDS-DMA f32 kernel (256x256 tile) on 4096^3 A.B^T and A.B; variants = 3 "
                          "launches of that GEMM with every f16 MFMA tile variant forced in turn; mfma-power = the stand-alone "
                          "MFMA-only program (built by `make -C dfdx_amd/csrc probe`)")
     ap.add_argument("--no-rotate", action="store_true", help="skip the second timing of the HBM-bound cases over rotating buffer sets")
@@ -65,6 +66,19 @@ def main():
                 dev.gemm(desc)
             torch.cuda.synchronize()
             print(json.dumps({"probe": "3 x 256 MiB copy, 5 x " + dev.gemm_plan(desc)[2]}))
+        elif args.probe == "f32-forms":
+            del a, b, c
+            a, b, c = (torch.randn(n, n, device="cuda", dtype=torch.float32) for _ in range(3))
+            names = []
+            for bstr in ((1, n), (n, 1)):
+                for v in (1, dev.mfma_variant_count("f32")):   # the register-staged 256x256 tile, the LDS-DMA form of it
+                    desc = dev.gemm_desc("f32", n, n, n, a.data_ptr(), (n, 1), b.data_ptr(), bstr, c.data_ptr(), (n, 1),
+                                         kernel=KERNEL_MFMA, variant=v, no_split_k=True)
+                    names.append(dev.gemm_plan(desc)[2])
+                    for _ in range(3):
+                        dev.gemm(desc)
+                    torch.cuda.synchronize()
+            print(json.dumps({"probe": names}))
         elif args.probe == "rows":
             del a, b, c
             src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
@@ -259,6 +273,12 @@ def main():
              fl, es * nb * (S * S + 2 * S * D), bufs=(p, v, o))
         gemm("c4", "dP dO.V^T NT acc", d4(S, D, S, d_o, (D, 1), sSD, v, (1, D), sSD, gp, (S, 1), sSS, True),
              fl, es * nb * (2 * S * D + 2 * S * S), bufs=(d_o, v, gp))
+        dp_desc = d4(S, D, S, d_o, (D, 1), sSD, v, (1, D), sSD, gp, (S, 1), sSS, True)
+
+        def dp_fresh():   # the same accumulation into a gradient that is only DECLARED zero: stored, not read
+            dev.zero_deferred(P(gp), gp.numel() * es)
+            dev.gemm(dp_desc)
+        timed("c4", "dP acc into a deferred-zero gradient", dp_fresh, fl, es * nb * (2 * S * D + S * S), "gemm, beta = 0 by declaration")
         gemm("c4", "dV P^T.dO TN acc", d4(S, S, D, p, (1, S), sSS, d_o, (D, 1), sSD, gv, (D, 1), sSD, True),
              fl, es * nb * (S * S + 3 * S * D), bufs=(p, d_o, gv))
         gemm("c4", "dQ dS.K NN acc", d4(S, S, D, gp, (S, 1), sSS, k, (D, 1), sSD, gq, (D, 1), sSD, True),
