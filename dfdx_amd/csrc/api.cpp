@@ -274,7 +274,9 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
                      : is32 ? mfma32_pick_variant(p, ctx->compute_units, forced_splits) : is64 ? mfma64_pick_variant(p, ctx->compute_units) : 0;
         const bool ok = is16 ? mfma16_supported(p, v) : is32 ? mfma32_supported(p, v) : is64 ? mfma64_supported(p, v) : false;
         if (!ok) return DFDX_ROCM_ERR_UNSUPPORTED;
-        *plan = {DFDX_ROCM_KERNEL_MFMA, v, is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
+        *plan = {DFDX_ROCM_KERNEL_MFMA, v,
+                 is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits)
+                      : is16 ? mfma16_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
         return DFDX_ROCM_OK;
     }
     case DFDX_ROCM_KERNEL_AUTO:
@@ -297,7 +299,9 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
     int v = is16 ? mfma16_pick_variant(p, ctx->compute_units)
                  : is32 ? mfma32_pick_variant(p, ctx->compute_units, forced_splits) : is64 ? mfma64_pick_variant(p, ctx->compute_units) : 0;
     if (v > 0) {
-        *plan = {DFDX_ROCM_KERNEL_MFMA, v, is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
+        *plan = {DFDX_ROCM_KERNEL_MFMA, v,
+                 is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits)
+                      : is16 ? mfma16_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
         return DFDX_ROCM_OK;
     }
     *plan = {DFDX_ROCM_KERNEL_GENERIC, 0, 1};
@@ -326,7 +330,9 @@ int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan, b
     p.compute_units = ctx->compute_units;
     if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1) {
         const size_t need = p.dtype == DT_F32 ? mfma32_workspace_bytes(p, plan.variant, plan.splits)
-                                              : mfma16dma_workspace_bytes(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
+                            : plan.variant < mfma16_dma_first_variant()
+                                ? mfma16_workspace_bytes(p, plan.variant, plan.splits)
+                                : mfma16dma_workspace_bytes(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
         if (int rc = partials_buffer(ctx, need, static_scratch, &p.workspace)) return rc;
         p.splits = plan.splits;
     }

@@ -77,6 +77,9 @@ const char *mfma16_variant_name(int variant);
 bool mfma16_supported(const GemmProblem &p, int variant);
 int mfma16_pick_variant(const GemmProblem &p, int compute_units);
 int mfma16_dma_first_variant();  // variant ids >= this are the LDS-DMA kernels
+// split-k of the register-staged variants (ids below mfma16_dma_first_variant)
+int mfma16_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits);
+size_t mfma16_workspace_bytes(const GemmProblem &p, int variant, int splits);
 hipError_t launch_mfma16(const GemmProblem &p, int variant, hipStream_t stream);
 // The same product with B given as a patch matrix (`p.b` = channel 0 of the first image, b_b1 / b_b2 = image and group
 // strides, b_rs / b_cs unused): register-staged kernels only, tile chosen inside.  Returns hipErrorNotSupported when

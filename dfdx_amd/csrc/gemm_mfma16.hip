@@ -47,6 +47,10 @@ struct Params {
     int accumulate, bias_mode, c_vec;
     int window;  // operands that 16 B-aligned vector loads cannot walk (odd leading dimension, extent or address): window loads
     int group_m;
+    // split-k: k-loop steps [split * chunk, +chunk) per workgroup, f32 partial tiles to ws[split][row][col]
+    int splits, chunk;
+    float *ws;
+    int64_t ws_ld, ws_split_stride;
     ConvPatches conv;  // CONV_B kernels: B is the patch matrix of a unit-stride convolution, formed on the fly
 };
 
@@ -252,7 +256,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
 
     // ---- which tile -------------------------------------------------------
     const int work = xcd_remap(blockIdx.x, p.total_blocks);
-    const int batch = work / p.tiles_per_batch;
+    const int bidx = work / p.tiles_per_batch;  // batch, or k split
+    const int batch = p.splits > 1 ? 0 : bidx;
+    const int split = p.splits > 1 ? bidx : 0;
     const int tile = work % p.tiles_per_batch;
     const int gsize = p.group_m * p.tiles_n;
     const int group = tile / gsize;
@@ -263,7 +269,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
     const int bm0 = tm_idx * BM, bn0 = tn_idx * BN;
 
     const int ktiles = (p.k + BK - 1) / BK;
-    const int iters = ktiles * p.kbatches;
+    const int it0 = split * p.chunk;  // this workgroup owns k-loop steps [it0, it0 + iters)
+    const int iters = min(ktiles * p.kbatches - it0, p.chunk);
 
     // Uniform pointers to the origin of the NEXT tile to fetch, advanced incrementally; the
     // divisions needed to locate a batch run once per batch, not once per k step.
@@ -278,10 +285,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
     };
     const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
     const int64_t b_step = B_KC ? BK : (int64_t)BK * p.ldb;
-    int f_kb = p.kbatches > 1 ? 0 : batch;  // batch of the next tile to fetch
-    int f_kt = 0;                            // its k-tile index
-    const uint16_t *a_next = a_origin(f_kb);
-    const uint16_t *b_next = b_origin(f_kb);
+    int f_kb = p.kbatches > 1 ? it0 / ktiles : batch;  // batch of the next tile to fetch
+    int f_kt = p.kbatches > 1 ? it0 % ktiles : it0;    // its k-tile index
+    const uint16_t *a_next = a_origin(f_kb) + f_kt * a_step;
+    const uint16_t *b_next = CONV_B ? b_origin(f_kb) : b_origin(f_kb) + f_kt * b_step;
 
     Loader<BM, BK, NT, A_KC> la;
     Loader<BN, BK, NT, B_KC> lb;
@@ -371,6 +378,24 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
     }
 
     // ---- epilogue: lane holds m = l32 (per tile), n = 8g + 4*lh + 0..3 --------
+    if (p.splits > 1) {  // f32 partial tile into the workspace (padded to whole tiles: no bounds checks)
+        float *wbase = p.ws + split * p.ws_split_stride;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            float *wrow = wbase + (int64_t)(bm0 + wm0 + i * 32 + l32) * p.ws_ld + bn0 + wn0 + lh * 4;
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    typedef float f32x4 __attribute__((ext_vector_type(4)));
+                    f32x4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = acc[i][j][g * 4 + e];
+                    *(f32x4 *)(wrow + j * 32 + g * 8) = v;
+                }
+        }
+        return;
+    }
     const int cb = p.kbatches > 1 ? 0 : batch;
     uint16_t *cbase = p.c + (int64_t)(cb / p.nb2) * p.c_b1 + (int64_t)(cb % p.nb2) * p.c_b2;
 #pragma unroll
@@ -595,14 +620,52 @@ static int pick_staged(const GemmProblem &p, int compute_units, bool check_suppo
         if (check_support && !mfma16_supported(p, v)) continue;
         const Variant &t = kVariants[v - 1];
         const double blocks = (double)((p.m + t.bm - 1) / t.bm) * (double)((p.n + t.bn - 1) / t.bn) * (double)nbatch;
-        const double fill = std::min(1.0, blocks / std::max(1, compute_units));
-        const double time = blocks * t.bm * t.bn / (rate[i] * fill);
+        const int s = mfma16_plan_splits(p, v, compute_units, 0);
+        const double fill = std::min(1.0, blocks * s / std::max(1, compute_units));
+        // a split adds the f32 round trip of its partial tiles: s * 8 bytes per padded C element against 2 * k flops
+        const double round_trip = s > 1 ? 1.0 + (double)s * 8.0 * 250.0 / (2.0 * (double)std::max<int64_t>(p.k, 1)) : 1.0;
+        const double time = blocks * t.bm * t.bn / (rate[i] * fill) * round_trip;
         if (time < best_time) {
             best_time = time;
             best = v;
         }
     }
     return best;
+}
+
+// Split-k of the register-staged family: for products whose tiles leave most of the chip idle while the contraction is
+// long (an LM head's dX off the 16-byte grid: 32 tiles of 256 x 256, k = 50257).  Pieces of at least 4 k tiles, at most
+// 16 of them, no more than fill the chip once; none may be empty.
+int mfma16_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits) {
+    if (variant < 1 || variant > kNumVariants) return 1;
+    const Variant &t = kVariants[variant - 1];
+    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+    const int64_t total_iters = ((p.k + t.bk - 1) / t.bk) * (p.reduce ? p.nb1 * p.nb2 : 1);
+    if (nbatch != 1 || p.c_cs != 1 || total_iters < 2) return 1;
+    auto valid = [&](int64_t s) { return s == 1 || (s - 1) * ((total_iters + s - 1) / s) < total_iters; };
+    int64_t s;
+    if (forced_splits > 0) {
+        s = std::min<int64_t>(forced_splits, total_iters);
+    } else {
+        const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn);
+        s = std::min<int64_t>({16, std::max<int64_t>(1, compute_units / blocks), total_iters / 4});
+        if (s < 2) return 1;
+    }
+    while (!valid(s)) s--;
+    return (int)s;
+}
+
+static void ws_layout16(const GemmProblem &p, int variant, int64_t *ld, int64_t *split_stride) {
+    const Variant &v = kVariants[variant - 1];
+    *ld = ((p.n + v.bn - 1) / v.bn) * v.bn;
+    *split_stride = *ld * (((p.m + v.bm - 1) / v.bm) * v.bm);
+}
+
+size_t mfma16_workspace_bytes(const GemmProblem &p, int variant, int splits) {
+    if (splits <= 1 || variant < 1 || variant > kNumVariants) return 0;
+    int64_t ld, stride;
+    ws_layout16(p, variant, &ld, &stride);
+    return (size_t)stride * splits * sizeof(float);
 }
 
 hipError_t launch_mfma16(const GemmProblem &g, int variant, hipStream_t stream) {
@@ -630,8 +693,21 @@ hipError_t launch_mfma16(const GemmProblem &g, int variant, hipStream_t stream) 
     p.window = needs_window(g, la, lb);
     p.group_m = 4;
     p.conv = ConvPatches{};
-    if (g.dtype == DT_F16) return launch_variant<_Float16>(variant, p, la.kc, lb.kc, stream);
-    return launch_variant<__bf16>(variant, p, la.kc, lb.kc, stream);
+    const int total_iters = (int)(((g.k + v.bk - 1) / v.bk) * p.kbatches);
+    p.splits = 1; p.chunk = total_iters; p.ws = nullptr; p.ws_ld = 0; p.ws_split_stride = 0;
+    if (g.splits > 1) {
+        if (!g.workspace || p.total_blocks != p.tiles_per_batch) return hipErrorInvalidValue;
+        p.splits = g.splits;
+        p.chunk = (total_iters + g.splits - 1) / g.splits;
+        if ((int64_t)(g.splits - 1) * p.chunk >= total_iters) return hipErrorInvalidValue;
+        p.ws = g.workspace;
+        ws_layout16(g, variant, &p.ws_ld, &p.ws_split_stride);
+        p.total_blocks = p.tiles_per_batch * g.splits;
+    }
+    const hipError_t e = (g.dtype == DT_F16) ? launch_variant<_Float16>(variant, p, la.kc, lb.kc, stream)
+                                             : launch_variant<__bf16>(variant, p, la.kc, lb.kc, stream);
+    if (e != hipSuccess || g.splits <= 1) return e;
+    return launch_splitk_reduce(g, p.ws_ld, p.ws_split_stride, stream);
 }
 
 hipError_t launch_mfma16_conv(const GemmProblem &g, const ConvPatches &conv, int compute_units, hipStream_t stream) {
@@ -666,6 +742,7 @@ hipError_t launch_mfma16_conv(const GemmProblem &g, const ConvPatches &conv, int
     p.c_vec = 1;
     p.window = 0;
     p.group_m = 4;
+    p.splits = 1; p.chunk = (int)((g.k + v.bk - 1) / v.bk); p.ws = nullptr; p.ws_ld = 0; p.ws_split_stride = 0;
     p.conv = conv;
     if (g.dtype == DT_F16) return launch_conv_variant<_Float16>(variant, p, stream);
     return launch_conv_variant<__bf16>(variant, p, stream);

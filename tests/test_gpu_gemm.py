@@ -323,6 +323,20 @@ def test_split_k_forced(dtype, layout, splits):
     run_case(dtype, 264, 576, 136, layout, True, KERNEL_MFMA, 0, split_k=splits, c_colmajor=True)
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("splits", [0, 2, 5])
+def test_split_k_register_staged_family(dtype, splits):
+    """k not a multiple of 64, or operands off the 16-byte grid, with few output tiles and a long contraction (an LM head's
+    dX): the register-staged kernels split the k loop as well; forced piece counts and the planner's own."""
+    dev = device()
+    for i, (m, k, n, layout, pads) in enumerate([(264, 1000, 200, "nn", (8, 8, 8)), (130, 2057, 72, "nt", (1, 3, 5)),
+                                                 (96, 4104, 256, "tn", (0, 8, 0))]):
+        run_case(dtype, m, k, n, layout, bool(i % 2), KERNEL_MFMA, 0, split_k=splits, seed=700 + i, pads=pads)
+    a = dev.zeros(dtype, (256, 4104))
+    d = dev.gemm_desc(dtype, 256, 4104, 256, a.ptr, (4104, 1), a.ptr, (1, 4104), a.ptr, (256, 1))
+    assert "splitk" in dev.gemm_plan(d)[2] and "dma" not in dev.gemm_plan(d)[2], dev.gemm_plan(d)
+
+
 def test_split_k_is_planned_for_weight_gradients_and_is_deterministic():
     dev = device()
     g = rng(77)
