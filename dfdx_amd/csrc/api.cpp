@@ -164,7 +164,9 @@ int scratch_address(int ordinal, void **out) {
 }
 
 // Validates `d` and produces the canonical problem (row-major C whenever the view allows it).
-int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
+// `colsum_b` (may be null): where the caller would like the sums of B over the contraction; it stays in the problem only
+// when the problem is the plain one (no aliased output axis).
+int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out, void *colsum_b = nullptr) {
     if (!d) return DFDX_ROCM_ERR_INVALID_ARG;
     if (d->dtype < DFDX_ROCM_F32 || d->dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_INVALID_ARG;
     if (d->m < 0 || d->n < 0 || d->k < 0 || d->batch1 < 1 || d->batch2 < 1) return DFDX_ROCM_ERR_INVALID_ARG;
@@ -216,6 +218,9 @@ int make_problem(const dfdx_rocm_gemm_desc *d, GemmProblem *out) {
     p.c = d->c; p.c_rs = d->c_rs; p.c_cs = d->c_cs;
     p.c_b1 = p.reduce ? 0 : d->c_b1; p.c_b2 = p.reduce ? 0 : d->c_b2;
     p.bias = d->bias;
+    p.ksum = colsum_b;
+    p.ksum_of = colsum_b ? KSUM_OF_B : KSUM_NONE;
+    p.ksum_accumulate = 1;
     p.splits = 1;
     p.workspace = nullptr;
     p.compute_units = 0;
@@ -373,6 +378,35 @@ int settle_operands(dfdx_rocm_ctx *ctx, GemmProblem *p, bool may_overwrite) {
 }
 
 }  // namespace
+
+namespace dfdx_rocm {
+
+int gemm_with_colsum(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, void *colsum_b, bool *fused) {
+    *fused = false;
+    if (int e = bind(ctx)) return e;
+    GemmProblem p;
+    if (int e = make_problem(desc, &p, colsum_b)) return e;
+    if (p.m == 0) return DFDX_ROCM_OK;
+    if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
+    Plan plan;
+    if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    const bool can = p.ksum && plan.kernel == DFDX_ROCM_KERNEL_MFMA && (p.dtype == DT_F16 || p.dtype == DT_BF16) &&
+                     plan.variant >= mfma16_dma_first_variant() &&
+                     mfma16dma_ksum_supported(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
+    if (can) {
+        bool fresh = false;
+        const int64_t len = p.ksum_of == KSUM_OF_A ? p.m : p.n;
+        if (int e = settle_output(ctx, p.ksum, (size_t)len * 2, true, &fresh)) return e;
+        p.ksum_accumulate = !fresh;
+        *fused = true;
+    } else {
+        p.ksum = nullptr;
+        p.ksum_of = KSUM_NONE;
+    }
+    return run_plan(ctx, p, plan);
+}
+
+}  // namespace dfdx_rocm
 
 extern "C" {
 

@@ -67,6 +67,10 @@ int settle_all(dfdx_rocm_ctx *ctx);
 // Bytes a dense view covers: extents/strides (elements) of up to `rank` axes; 0 if the view has gaps, overlaps or does
 // not start at its lowest address.  Any permutation of a contiguous layout is dense.
 size_t dense_bytes(int rank, const int64_t *extents, const int64_t *strides, size_t elem_bytes);
+// dfdx_rocm_gemm(ctx, desc) which, where the kernel it picks can, also adds the sums of B over the contraction (and over
+// the batches of a reduced product) to colsum_b[0 .. n) in the element type: colsum_b[j] += sum_k B[k][j].  *fused tells
+// whether it did; when not, colsum_b has not been touched and the caller runs that reduction itself.
+int gemm_with_colsum(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, void *colsum_b, bool *fused);
 // Clears `bytes` bytes at `ptr` (any alignment) with a fill kernel on `stream`.
 hipError_t launch_zero_fill(void *ptr, size_t bytes, int compute_units, hipStream_t stream);
 

@@ -8,6 +8,7 @@ namespace dfdx_rocm {
 
 enum { DT_F32 = 0, DT_F16 = 1, DT_BF16 = 2, DT_F64 = 3 };
 enum { BIAS_NONE = 0, BIAS_PER_COL = 1, BIAS_PER_ROW = 2 };
+enum { KSUM_NONE = 0, KSUM_OF_A = 1, KSUM_OF_B = 2 };
 
 // One strided, batched GEMM:  C[b][i,j] = (accumulate ? C : 0) + bias + sum_k A[b][i,k] * B[b][k,j].
 // Strides are in elements.  With `reduce` set, all nb1*nb2 batches are summed into one C.
@@ -25,6 +26,13 @@ struct GemmProblem {
     void *c;
     int64_t c_rs, c_cs, c_b1, c_b2;
     const void *bias;
+    // Optional second result, in the element type: the sums of one operand over the contraction (and over the batches
+    // of a reduced product), ksum[i] (+)= sum_k A[i,k] (KSUM_OF_A, length m) or ksum[j] (+)= sum_k B[k,j] (KSUM_OF_B,
+    // length n).  `Linear`'s bias gradient is the latter for the weight-gradient product x^T . grad_out.  Only some
+    // kernels produce it (mfma16dma_ksum_supported); the caller clears `ksum` and runs the reduction itself otherwise.
+    void *ksum = nullptr;
+    int ksum_of = KSUM_NONE;
+    int ksum_accumulate = 0;
     // split-k (filled in by the planner): `splits` workgroups share one C tile; f32 partials go to `workspace`
     int splits;
     float *workspace;
@@ -64,6 +72,8 @@ static inline GemmProblem transposed(const GemmProblem &p) {
     t.c_rs = p.c_cs; t.c_cs = p.c_rs;
     if (p.bias_mode == BIAS_PER_COL) t.bias_mode = BIAS_PER_ROW;
     else if (p.bias_mode == BIAS_PER_ROW) t.bias_mode = BIAS_PER_COL;
+    if (p.ksum_of == KSUM_OF_A) t.ksum_of = KSUM_OF_B;
+    else if (p.ksum_of == KSUM_OF_B) t.ksum_of = KSUM_OF_A;
     return t;
 }
 
@@ -98,9 +108,12 @@ hipError_t launch_mfma16dma(const GemmProblem &p, int variant, hipStream_t strea
 void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_variant, int forced_splits, int *variant,
                           int *splits);
 size_t mfma16dma_workspace_bytes(const GemmProblem &p, int variant, int splits);
+bool mfma16dma_ksum_supported(const GemmProblem &p, int variant, int splits);  // can this plan also produce p.ksum?
 
 // ---- split-k combine (splitk_reduce.hip): C = (accumulate ? C : 0) + bias + sum_s partial[s], s ascending ----
-hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_split_stride, hipStream_t stream);
+// `ws_ksum` (may be null): [ksum_slots][ws_ksum_stride] f32 partial sums of p.ksum, added up in slot order into p.ksum.
+hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_split_stride, hipStream_t stream,
+                                const float *ws_ksum = nullptr, int64_t ws_ksum_stride = 0, int ksum_slots = 0);
 
 // ---- MFMA kernels for f32 (gemm_mfma32.hip) ----
 int mfma32_variant_count();

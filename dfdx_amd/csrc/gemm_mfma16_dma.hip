@@ -58,6 +58,10 @@ struct Params {
     int grid;  // workgroups launched (<= total_blocks: each walks blockIdx.x, blockIdx.x + grid, ...)
     float *ws;
     int64_t ws_ld, ws_split_stride;
+    // sums of A's rows over the contraction as a second result (KSUM instances, split-k only): f32 partial sums in
+    // ws_ksum[(split * (BM / 64) + tile column) * 8 + wave][tiles_m * BM], combined by the reduce kernel
+    float *ws_ksum;
+    int ws_ksum_stride;
 };
 
 template <typename T> struct Mma;
@@ -67,6 +71,7 @@ template <> struct Mma<_Float16> {
     }
     static __device__ __forceinline__ float to_f32(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
     static __device__ __forceinline__ uint16_t from_f32(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+    static constexpr uint32_t ONE2 = 0x3C003C00u;  // two 1.0
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // v_cvt_pk_f16_f32: RNE, lo in bits 15:0
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, h2));
@@ -82,6 +87,7 @@ template <> struct Mma<__bf16> {
         if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
         return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);  // round to nearest even
     }
+    static constexpr uint32_t ONE2 = 0x3F803F80u;
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // v_cvt_pk_bf16_f32: RNE, quiet NaNs
         typedef __bf16 b2 __attribute__((ext_vector_type(2)));
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, b2));
@@ -156,7 +162,15 @@ constexpr int dma_waves_per_simd(int bm, int bn, int waves) {
 // epilogue has only the two interior forms.  With the general form compiled in as well, the compiler guards the
 // fragment registers against a load of that form it cannot prove complete, with a wait for ALL memory traffic in the
 // middle of the k loop -- where every wave then stalls on the tile prefetched for the step after.
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool EDGE>
+//
+// KSUM = true (A stored [k][m] only, split-k only) adds a second result: the sums of A's rows over the contraction --
+// the bias gradient of a Linear layer when A is grad_out^T and the product is the weight gradient.  The A tile sits in
+// LDS as 64 k-rows of BM values; its column sums need no MFMA and no fragment: every thread reads ONE 16-byte piece
+// (8 values of one k-row) per k tile and adds it to 8 f32 sums of its own.  The 512 threads cover 512 of the tile's
+// 64 * BM / 8 pieces; the workgroups of a tile row all hold the same A tiles, so tile column q < BM / 64 takes the q-th
+// 512 pieces and the others none.  At the end of a work item lanes that hold the same 8 columns are added up and each
+// wave leaves its sums in a workspace slot of its own; the split-k reduce kernel adds the slots.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool EDGE, bool KSUM = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, WAVES_M *WAVES_N)) void gemm_mfma16_dma_kernel(const Params p) {
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
@@ -313,6 +327,35 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
             for (int v = 0; v < 4; v++) acc[i][j][v] = 0.0f;
 
     u32x4 fa[TM], fb[2][TN];
+    // KSUM: the thread's piece of every A tile is chunk ks_chunk = tid % CH (8 columns) of one k-row, at byte ks_off of
+    // the tile (the swizzle depends on the k-row only, so the same place in every tile).
+    constexpr int CH = BM / 8, KS_SHARE = BM / 64;  // pieces per k-row; tile columns that share a tile's pieces
+    static_assert(!KSUM || (!A_KC && NW == 8 && (CH == 32 || CH == 16)), "row sums: [k][m] tiles of 8-wave workgroups");
+    [[maybe_unused]] float ks_sum[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    [[maybe_unused]] u32x4 ks_piece;
+    [[maybe_unused]] uint32_t ks_off = 0;
+    [[maybe_unused]] int ks_chunk = 0;
+    [[maybe_unused]] bool ks_on = false;
+    [[maybe_unused]] auto ks_begin = [&](int bn0) {
+        const int tn = bn0 / BN;
+        ks_on = tn < KS_SHARE;
+        const int cell = (ks_on ? tn : 0) * 512 + tid;
+        const int krow = cell / CH;
+        ks_chunk = cell % CH;  // lanes CH apart hold the same chunk of neighbouring k-rows
+        ks_off = (uint32_t)(krow * BM * 2 + (ks_chunk ^ mc_swizzle<BM>(krow)) * 16);
+    };
+    [[maybe_unused]] auto ks_read = [&](const uint8_t *sa) {  // asm: see the note on the transposing reads above
+        if constexpr (KSUM) asm volatile("ds_read_b128 %0, %1" : "=v"(ks_piece) : "v"(lds_addr(sa) + ks_off));
+    };
+    [[maybe_unused]] auto ks_add = [&]() {  // after a wait for every LDS read of the wave
+        if constexpr (KSUM) {
+            tie(ks_piece);
+            if (ks_on) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) ks_sum[e] += Mma<T>::to_f32((uint16_t)(ks_piece[e / 2] >> ((e & 1) * 16)));
+            }
+        }
+    };
     auto read_a = [&](const uint8_t *sa, auto ks_tag, int i0, int i1) {
         constexpr int ks = decltype(ks_tag)::value;
         [[maybe_unused]] const uint32_t base = lds_addr(sa);
@@ -387,7 +430,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
     // one 64-wide k tile from stage `cs`; HAS_NEXT: the next tile belongs to the same work item (hand the stage
     // over and prefetch its first fragments while the last MFMAs of this tile run)
     // LDS instructions per group of reads, as issued below: half of the A fragments, all B fragments of a k step
-    constexpr int RA = 2 * Q * OPS_A, RB = TN * OPS_B;
+    constexpr int RA = 2 * Q * OPS_A, RB = TN * OPS_B, KS_READS = KSUM ? 1 : 0;
     constexpr std::integral_constant<int, 0> K0{};
     constexpr std::integral_constant<int, 1> K1{};
 #define DFDX_LEFT(n) std::integral_constant<int, (n)> {}
@@ -425,8 +468,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
         mma(fb[1], 0, Q);
         __builtin_amdgcn_sched_barrier(0);
         read_a(sa, K1, 2 * Q, TM);
+        ks_read(sa);  // KSUM: the last (youngest) LDS read of this tile, consumed behind a wait for all of them
         __builtin_amdgcn_sched_barrier(0);
-        fence_a(DFDX_LEFT(RB + RA), Q, 2 * Q);
+        fence_a(DFDX_LEFT(RB + RA + KS_READS), Q, 2 * Q);
         mma(fb[1], Q, 2 * Q);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (HAS_NEXT) {
@@ -439,6 +483,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             fence_a(DFDX_LEFT(0), 2 * Q, TM);
+            ks_add();
             const bool mfma_first = __builtin_amdgcn_readfirstlane(wave) >= NW / 2;
             if (mfma_first) {
                 mma(fb[1], 2 * Q, 3 * Q);
@@ -457,11 +502,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
             __builtin_amdgcn_sched_barrier(0);
             read_a(sn, K0, 2 * Q, TM);
         } else {
-            fence_a(DFDX_LEFT(RA / 2), 2 * Q, 3 * Q);
+            fence_a(DFDX_LEFT(RA / 2 + KS_READS), 2 * Q, 3 * Q);
             mma(fb[1], 2 * Q, 3 * Q);
             __builtin_amdgcn_sched_barrier(0);
             fence_a(DFDX_LEFT(0), 3 * Q, TM);
             mma(fb[1], 3 * Q, TM);
+            ks_add();
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -470,6 +516,25 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
     // Returns the number of stores it issued after its last load (see sync_tile), 0 when that is not a fixed count.
     auto store_tile = [&](const Work &w) -> int {
         const int bm0 = w.bm0, bn0 = w.bn0, split = w.split, batch = w.batch;
+        if constexpr (KSUM) {
+            // Lanes that hold the same 8 columns (they differ in the k-row) are added up; the first CH lanes of each wave
+            // store.  These stores come before the C tile's: the count returned below stays a lower bound of what was
+            // issued after the last load.
+            if (ks_on) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+#pragma unroll
+                    for (int d = CH; d < 64; d *= 2) ks_sum[e] += __shfl_xor(ks_sum[e], d, 64);
+                }
+                if (lane < CH) {
+                    float *slot = p.ws_ksum + (int64_t)((split * KS_SHARE + bn0 / BN) * 8 + wave) * p.ws_ksum_stride + bm0 + ks_chunk * 8;
+                    *(f32x4 *)slot = f32x4{ks_sum[0], ks_sum[1], ks_sum[2], ks_sum[3]};  // rows padded to whole tiles
+                    *(f32x4 *)(slot + 4) = f32x4{ks_sum[4], ks_sum[5], ks_sum[6], ks_sum[7]};
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) ks_sum[e] = 0.0f;
+            }
+        }
     if (p.splits > 1) {  // f32 partial tile into the workspace (padded to whole tiles: no bounds checks)
         float *wbase = p.ws + split * p.ws_split_stride;
 #pragma unroll
@@ -733,6 +798,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
     Work cw = decode(c_index);
     int c_left = cw.iters, c_stage = 0;
     int behind = 0;  // stores of the previous work item that may still be in flight
+    if constexpr (KSUM) ks_begin(cw.bn0);
     issue();
     sync_tile();
     read_first(smem);
@@ -761,6 +827,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
         c_index += gridDim.x;
         cw = decode(c_index);
         c_left = cw.iters;
+        if constexpr (KSUM) ks_begin(cw.bn0);
         read_first(smem + c_stage * STAGE_BYTES);
     }
 }
@@ -797,9 +864,9 @@ template <typename T, int BM, int BN, int WM, int WN>
 hipError_t launch_layout(Params p, int compute_units, bool a_kc, bool b_kc, hipStream_t stream) {
     constexpr int NT = WM * WN * 64;
     constexpr size_t lds = (size_t)STAGES * (BM + BN) * BK * 2;
-#define DFDX_LAUNCH(AKC, BKC, EDGE)                                                                            \
+#define DFDX_LAUNCH(AKC, BKC, EDGE, ...)                                                                       \
     do {                                                                                                       \
-        auto kern = gemm_mfma16_dma_kernel<T, BM, BN, WM, WN, AKC, BKC, EDGE>;                                 \
+        auto kern = gemm_mfma16_dma_kernel<T, BM, BN, WM, WN, AKC, BKC, EDGE, ##__VA_ARGS__>;                  \
         static PerDevice occupancy_on;                                                                         \
         std::atomic<int> &known = occupancy_on.here();                                                         \
         int per_cu = known.load(std::memory_order_acquire);                                                    \
@@ -820,7 +887,11 @@ hipError_t launch_layout(Params p, int compute_units, bool a_kc, bool b_kc, hipS
     // whole tiles only, and nothing but the two interior epilogue forms: the instance without the general form
     const bool edge = p.m % BM != 0 || p.n % BN != 0 || p.bias_mode == BIAS_PER_ROW || p.ldc >= (1 << 26) ||
                       (p.accumulate && p.bias_mode != BIAS_NONE);
-    if (edge) {
+    if (p.ws_ksum) {  // row sums of A: compiled for the layout of weight gradients only (ksum_supported)
+        if (a_kc || b_kc) return hipErrorInvalidValue;
+        if (edge) DFDX_LAUNCH(false, false, true, true);
+        else DFDX_LAUNCH(false, false, false, true);
+    } else if (edge) {
         if (a_kc && b_kc) DFDX_LAUNCH(true, true, true);
         else if (a_kc && !b_kc) DFDX_LAUNCH(true, false, true);
         else if (!a_kc && b_kc) DFDX_LAUNCH(false, true, true);
@@ -996,18 +1067,35 @@ void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_va
     }
 }
 
-// layout of the split-k workspace: [splits][tiles_m * BM][tiles_n * BN] f32
-static void ws_layout(const GemmProblem &p, int variant, int64_t *ld, int64_t *split_stride) {
+// layout of the split-k workspace: [splits][tiles_m * BM][tiles_n * BN] f32, then -- row sums of A asked for --
+// [splits * (BM / 64) * 8][tiles_m * BM] f32
+static void ws_layout(const GemmProblem &p, int variant, int64_t *ld, int64_t *split_stride, int64_t *ksum_stride = nullptr) {
     const Variant &v = kVariants[variant - 1];
     *ld = ((p.n + v.bn - 1) / v.bn) * v.bn;
     *split_stride = *ld * (((p.m + v.bm - 1) / v.bm) * v.bm);
+    if (ksum_stride) *ksum_stride = ((p.m + v.bm - 1) / v.bm) * v.bm;
 }
+// Workspace slots of the row sums: one per split, sharing tile column and wave.
+static int ksum_slots(int variant, int splits) { return splits * (kVariants[variant - 1].bm / 64) * 8; }
 
 size_t mfma16dma_workspace_bytes(const GemmProblem &p, int variant, int splits) {
     if (splits <= 1) return 0;
-    int64_t ld, stride;
-    ws_layout(p, variant, &ld, &stride);
-    return (size_t)stride * splits * sizeof(float);
+    int64_t ld, stride, ks;
+    ws_layout(p, variant, &ld, &stride, &ks);
+    const int64_t slots = p.ksum ? ksum_slots(variant, splits) : 0;
+    return (size_t)(stride * splits + ks * slots) * sizeof(float);
+}
+
+// The sums of A's rows ride along only where A and B are both stored contraction-major (m- and n-contiguous: the
+// weight gradient grad_out^T . x after the output transposition) and the contraction is split (the partial sums are
+// combined by the reduce kernel that runs then anyway).
+bool mfma16dma_ksum_supported(const GemmProblem &p, int variant, int splits) {
+    if (!p.ksum || p.ksum_of != KSUM_OF_A || splits <= 1 || !mfma16dma_supported(p, variant)) return false;
+    if (!p.reduce && p.nb1 * p.nb2 != 1) return false;
+    if ((uintptr_t)p.ksum & 1u) return false;
+    const Variant &v = kVariants[variant - 1];
+    if ((p.n + v.bn - 1) / v.bn < v.bm / 64) return false;  // too few tile columns to share a tile's pieces
+    return !classify(p.m, p.k, p.a_rs, p.a_cs).kc && !classify(p.n, p.k, p.b_cs, p.b_rs).kc;
 }
 
 hipError_t launch_mfma16dma(const GemmProblem &g, int variant, hipStream_t stream) {
@@ -1032,20 +1120,27 @@ hipError_t launch_mfma16dma(const GemmProblem &g, int variant, hipStream_t strea
     p.group_m = 4;
     const int total_iters = (p.k / BK) * p.kbatches;
     p.splits = 1; p.chunk = total_iters; p.ws = nullptr; p.ws_ld = 0; p.ws_split_stride = 0;
+    p.ws_ksum = nullptr; p.ws_ksum_stride = 0;
+    if (g.ksum && !mfma16dma_ksum_supported(g, variant, g.splits)) return hipErrorInvalidValue;
     if (g.splits > 1) {
         if (!g.workspace || p.total_blocks != p.tiles_per_batch) return hipErrorInvalidValue;
         p.splits = g.splits;
         p.chunk = (total_iters + g.splits - 1) / g.splits;
         if ((int64_t)(g.splits - 1) * p.chunk >= total_iters) return hipErrorInvalidValue;
         p.ws = g.workspace;
-        ws_layout(g, variant, &p.ws_ld, &p.ws_split_stride);
+        int64_t ks_stride = 0;
+        ws_layout(g, variant, &p.ws_ld, &p.ws_split_stride, &ks_stride);
+        if (g.ksum) {
+            p.ws_ksum = g.workspace + p.ws_split_stride * g.splits;
+            p.ws_ksum_stride = (int)ks_stride;
+        }
         p.total_blocks = p.tiles_per_batch * g.splits;
     }
     p.grid = 0;  // set per kernel instantiation at launch
     hipError_t e = (g.dtype == DT_F16) ? launch_variant<_Float16>(variant, p, g.compute_units, la.kc, lb.kc, stream)
                                        : launch_variant<__bf16>(variant, p, g.compute_units, la.kc, lb.kc, stream);
     if (e != hipSuccess || g.splits <= 1) return e;
-    return launch_splitk_reduce(g, p.ws_ld, p.ws_split_stride, stream);
+    return launch_splitk_reduce(g, p.ws_ld, p.ws_split_stride, stream, p.ws_ksum, p.ws_ksum_stride, ksum_slots(variant, g.splits));
 }
 
 }  // namespace dfdx_rocm

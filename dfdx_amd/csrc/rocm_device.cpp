@@ -6,6 +6,7 @@
 // reference becomes ONE launch (batch in the grid, or folded into the k loop when
 // all batches share one gradient accumulator).
 #include "../../include/dfdx_rocm.h"
+#include "ctx_internal.h"
 
 #include <cstring>
 
@@ -212,10 +213,29 @@ int dfdx_rocm_linear_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64
     // every step below supports all four element types; an unknown one is refused before any gradient is touched
     if (dtype < DFDX_ROCM_F32 || dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_INVALID_ARG;
     const int64_t ws[2] = {1, in_dim};  // the (I,O) view of the (O,I) storage; its gradient lands in (O,I) row-major
-    if (int e = dfdx_rocm_matmat_backward(ctx, dtype, rows, in_dim, out_dim, x, xs, grad_x, weight, ws, grad_weight, grad_out))
-        return e;
-    if (!grad_bias) return DFDX_ROCM_OK;
-    return dfdx_rocm_bias_backward(ctx, dtype, rows, out_dim, grad_out, grad_bias);
+    if (!grad_bias || rows == 0 || in_dim == 0 || out_dim == 0) {
+        if (int e = dfdx_rocm_matmat_backward(ctx, dtype, rows, in_dim, out_dim, x, xs, grad_x, weight, ws, grad_weight, grad_out))
+            return e;
+        return grad_bias ? dfdx_rocm_bias_backward(ctx, dtype, rows, out_dim, grad_out, grad_bias) : DFDX_ROCM_OK;
+    }
+    // The two products of MatMatKernel::backward (cpu_kernel.rs:265-286), the second one asked to produce the bias
+    // gradient as well: grad_out is its B operand, and the column sums of B over the contraction (the rows) are
+    // exactly what Bias1D's backward adds to grad_bias.  Kernels that cannot do that leave it to the reduction kernel.
+    if (bad(x, weight, grad_out) || !grad_x || !grad_weight) return DFDX_ROCM_ERR_INVALID_ARG;
+    dfdx_rocm_gemm_desc d = blank(dtype, rows, out_dim, in_dim);
+    d.accumulate = 1;
+    d.a = grad_out; d.a_rs = out_dim; d.a_cs = 1;
+    d.b = weight; d.b_rs = ws[1]; d.b_cs = ws[0];
+    d.c = grad_x; d.c_rs = xs[0]; d.c_cs = xs[1];
+    if (int e = dfdx_rocm_gemm(ctx, &d)) return e;
+    d = blank(dtype, in_dim, rows, out_dim);
+    d.accumulate = 1;
+    d.a = x; d.a_rs = xs[1]; d.a_cs = xs[0];
+    d.b = grad_out; d.b_rs = out_dim; d.b_cs = 1;
+    d.c = grad_weight; d.c_rs = ws[0]; d.c_cs = ws[1];
+    bool fused = false;
+    if (int e = dfdx_rocm::gemm_with_colsum(ctx, &d, grad_bias, &fused)) return e;
+    return fused ? DFDX_ROCM_OK : dfdx_rocm_bias_backward(ctx, dtype, rows, out_dim, grad_out, grad_bias);
 }
 
 }  // extern "C"

@@ -26,13 +26,52 @@ template <> struct Cvt<__bf16> {
     }
 };
 
+// The row sums that ride along with a split product (`ksum`, one value per row of C, `slots` partial sums each, stored
+// [slot][row]).  The first `blocks` workgroups of grid row 0 do nothing else: each takes 16 rows; thread t adds the
+// slots t / 16, t / 16 + 16, ... of row t % 16 in ascending order, four loads in flight at a time; the 16 partial sums
+// of a row are added in a fixed order through LDS, then the old value unless the gradient is fresh.
+struct KsumParts {
+    const float *ws;   // null = none
+    int64_t stride;
+    void *out;
+    int accumulate, slots, blocks;
+};
+constexpr int KSUM_ROWS = 16, KSUM_GROUPS = 256 / KSUM_ROWS;
+template <typename T> __device__ __forceinline__ void combine_ksum(const KsumParts &ks, int m) {
+    __shared__ float part[KSUM_GROUPS][KSUM_ROWS];
+    const int r = threadIdx.x % KSUM_ROWS, g = threadIdx.x / KSUM_ROWS;
+    const int row = min((int)blockIdx.x * KSUM_ROWS + r, m - 1);  // rows past the end repeat the last one, unused
+    const float *src = ks.ws + row;
+    float v = 0.0f;
+    int s = g;
+    for (; s + 3 * KSUM_GROUPS < ks.slots; s += 4 * KSUM_GROUPS) {
+        const float a = src[(int64_t)s * ks.stride], b = src[(int64_t)(s + KSUM_GROUPS) * ks.stride];
+        const float c = src[(int64_t)(s + 2 * KSUM_GROUPS) * ks.stride], d = src[(int64_t)(s + 3 * KSUM_GROUPS) * ks.stride];
+        v = (((v + a) + b) + c) + d;
+    }
+    for (; s < ks.slots; s += KSUM_GROUPS) v += src[(int64_t)s * ks.stride];
+    part[g][r] = v;
+    __syncthreads();
+    if (g == 0 && (int)blockIdx.x * KSUM_ROWS + r < m) {
+#pragma unroll
+        for (int q = 1; q < KSUM_GROUPS; q++) v += part[q][r];
+        T *dst = (T *)ks.out + row;
+        const float old = ks.accumulate ? Cvt<T>::load(dst) : 0.0f;
+        Cvt<T>::store(dst, old + v);
+    }
+}
+
 // one thread: 4 consecutive columns of one row
 template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, int splits, int64_t ws_ld, int64_t ws_split_stride,
                                                             T *c, int64_t c_rs, int m, int n, int accumulate, int bias_mode,
-                                                            const T *bias, int vec4) {
+                                                            const T *bias, int vec4, KsumParts ks) {
+    if (ks.ws && (int)blockIdx.x < ks.blocks) {   // uniform over the workgroup
+        if (blockIdx.y == 0) combine_ksum<T>(ks, m);
+        return;   // the same block index in the other grid rows has no work
+    }
     const int col = (blockIdx.y * 64 + threadIdx.x % 64) * 4;   // rows along grid.x: its limit is 2^31, grid.y's 65535
-    const int row = blockIdx.x * 4 + threadIdx.x / 64;
+    const int row = ((int)blockIdx.x - (ks.ws ? ks.blocks : 0)) * 4 + threadIdx.x / 64;
     if (row >= m || col >= n) return;
     const float *src = ws + (int64_t)row * ws_ld + col;
     f32x4 v = *(const f32x4 *)src;
@@ -78,9 +117,13 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce16_kernel(const float *ws, int splits, int64_t ws_ld, int64_t ws_split_stride,
                                                               uint16_t *c, int64_t c_rs, int m, int n, int accumulate,
-                                                              int bias_mode, const uint16_t *bias) {
+                                                              int bias_mode, const uint16_t *bias, KsumParts ks) {
+    if (ks.ws && (int)blockIdx.x < ks.blocks) {   // uniform over the workgroup
+        if (blockIdx.y == 0) combine_ksum<T>(ks, m);
+        return;   // the same block index in the other grid rows has no work
+    }
     const int col = (blockIdx.y * 64 + threadIdx.x % 64) * 8;
-    const int row = blockIdx.x * 4 + threadIdx.x / 64;
+    const int row = ((int)blockIdx.x - (ks.ws ? ks.blocks : 0)) * 4 + threadIdx.x / 64;
     if (row >= m || col >= n) return;   // n is a multiple of 8: a thread's 8 columns are all inside or all outside
     const float *src = ws + (int64_t)row * ws_ld + col;
     uint16_t *dst = c + (int64_t)row * c_rs + col;
@@ -123,23 +166,27 @@ __global__ __launch_bounds__(256) void splitk_reduce16_kernel(const float *ws, i
 }  // namespace
 
 // C of `p` must have unit column stride and no batch (the planner only splits such problems).
-hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_split_stride, hipStream_t stream) {
-    dim3 grid((unsigned)((p.m + 3) / 4), (unsigned)((p.n + 255) / 256)), block(256);
+hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_split_stride, hipStream_t stream,
+                                const float *ws_ksum, int64_t ws_ksum_stride, int ksum_slots) {
+    const bool with_ksum = p.ksum && ws_ksum;
+    const KsumParts ks{with_ksum ? ws_ksum : nullptr, ws_ksum_stride, p.ksum, p.ksum_accumulate, ksum_slots,
+                       with_ksum ? (int)((p.m + KSUM_ROWS - 1) / KSUM_ROWS) : 0};
+    dim3 grid((unsigned)((p.m + 3) / 4 + ks.blocks), (unsigned)((p.n + 255) / 256)), block(256);
     if ((p.n + 255) / 256 > 65535) return hipErrorInvalidValue;  // 16.7 M columns: no planner splits such a product
     const int64_t c_rs = p.m == 1 ? p.n : p.c_rs;
     const int bias_mode = p.bias ? p.bias_mode : BIAS_NONE;
     const bool is16 = p.dtype == DT_F16 || p.dtype == DT_BF16;
     if (is16 && p.n % 8 == 0 && c_rs % 8 == 0 && ws_ld % 4 == 0 && ws_split_stride % 4 == 0 && ((uintptr_t)p.c & 15u) == 0 &&
         ((uintptr_t)p.workspace & 15u) == 0 && (bias_mode != BIAS_PER_COL || ((uintptr_t)p.bias & 15u) == 0)) {
-        dim3 grid16((unsigned)((p.m + 3) / 4), (unsigned)((p.n + 511) / 512));
+        dim3 grid16((unsigned)((p.m + 3) / 4 + ks.blocks), (unsigned)((p.n + 511) / 512));
         if (p.dtype == DT_F16)
             splitk_reduce16_kernel<_Float16><<<grid16, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (uint16_t *)p.c,
                                                                             c_rs, (int)p.m, (int)p.n, p.accumulate, bias_mode,
-                                                                            (const uint16_t *)p.bias);
+                                                                            (const uint16_t *)p.bias, ks);
         else
             splitk_reduce16_kernel<__bf16><<<grid16, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (uint16_t *)p.c,
                                                                           c_rs, (int)p.m, (int)p.n, p.accumulate, bias_mode,
-                                                                          (const uint16_t *)p.bias);
+                                                                          (const uint16_t *)p.bias, ks);
         return hipGetLastError();
     }
     const int vec4 = p.dtype == DT_F32 && c_rs % 4 == 0 && ((uintptr_t)p.c & 15u) == 0 && ws_ld % 4 == 0 && ws_split_stride % 4 == 0 &&
@@ -147,16 +194,16 @@ hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_
     switch (p.dtype) {
     case DT_F32:
         splitk_reduce_kernel<float><<<grid, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (float *)p.c, c_rs,
-                                                                 (int)p.m, (int)p.n, p.accumulate, bias_mode, (const float *)p.bias, vec4);
+                                                                 (int)p.m, (int)p.n, p.accumulate, bias_mode, (const float *)p.bias, vec4, ks);
         break;
     case DT_F16:
         splitk_reduce_kernel<_Float16><<<grid, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (_Float16 *)p.c,
                                                                     c_rs, (int)p.m, (int)p.n, p.accumulate, bias_mode,
-                                                                    (const _Float16 *)p.bias, 0);
+                                                                    (const _Float16 *)p.bias, 0, ks);
         break;
     case DT_BF16:
         splitk_reduce_kernel<__bf16><<<grid, block, 0, stream>>>(p.workspace, p.splits, ws_ld, ws_split_stride, (__bf16 *)p.c, c_rs,
-                                                                  (int)p.m, (int)p.n, p.accumulate, bias_mode, (const __bf16 *)p.bias, 0);
+                                                                  (int)p.m, (int)p.n, p.accumulate, bias_mode, (const __bf16 *)p.bias, 0, ks);
         break;
     default: return hipErrorInvalidValue;
     }

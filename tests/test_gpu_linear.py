@@ -118,3 +118,68 @@ def test_linear_backward_seeded(dtype, rows, i, o):
     assert_within(dtype, o, host(dev, gx), oracle.to_f64(ogx, dtype).reshape(rows, i), go64, w64, what="grad_x")
     assert_within(dtype, rows, host(dev, gw), oracle.to_f64(ogw, dtype).reshape(o, i), go64, x64, what="grad_weight")
     assert_within(dtype, rows, host(dev, gb), go64.sum(axis=0), go64, np.ones(1), what="grad_bias")
+
+
+# Shapes whose weight-gradient product x^T . grad_out runs on the LDS-DMA kernels (rows % 64 == 0, 16-bit): there the bias
+# gradient is produced by the same launch (one more MFMA per A fragment in the work items of tile column 0) instead of
+# by the reduction kernels.  Both tile families, split and unsplit contractions, edge tiles in either direction.
+FUSED_SHAPES = [(8192, 1024, 1024), (4096, 1024, 4096), (512, 256, 512), (640, 264, 1000), (128, 64, 8), (2048, 4096, 1024),
+                (64, 1024, 1024)]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("rows,i,o", FUSED_SHAPES)
+def test_linear_backward_bias_gradient_from_the_weight_gradient_launch(dtype, rows, i, o):
+    """grad_bias: exact on small integers (sums below 2^8 for bf16, 2^11 for f16 are representable), and twice the
+    value after a second call (the first call finds the gradient fresh when its zeros are deferred, the second adds)."""
+    from helpers import assert_within
+    dev, g = device(), rng(305)
+    announce("linear backward, fused bias gradient", dtype, rows, i, o)
+    x = upload(dev, g.standard_normal((rows, i)), dtype)
+    w = upload(dev, g.uniform(-1, 1, (o, i)) / np.sqrt(i), dtype)
+    # mostly zeros, a few +-1: column sums stay small integers whatever the number of rows
+    go_host = (g.random((rows, o)) < 4.0 / rows) * g.choice([-1.0, 1.0], size=(rows, o))
+    go_host[0, :] += np.arange(o) % 3
+    go = upload(dev, go_host, dtype)
+    start = (np.arange(o) % 4).astype(np.float64)
+    for deferred in (False, True):
+        gx, gw = dev.zeros_like_storage(x), dev.zeros_like_storage(w)
+        if deferred:   # NaN patterns that are only DECLARED zero: a read of the old contents would show
+            import torch
+            from dfdx_amd.rocm import View
+            raw = torch.full((o * 2,), 0xFF, dtype=torch.uint8, device="cuda")
+            dev.zero_deferred(raw.data_ptr(), o * 2)
+            gb, base = View(raw, dtype, (o,), (1,)), np.zeros(o)
+        else:
+            gb, base = upload(dev, start, dtype), start
+        dev.linear_backward(x, gx, w, gw, gb, go)
+        np.testing.assert_array_equal(host(dev, gb), base + go_host.sum(axis=0))
+        dev.linear_backward(x, gx, w, gw, gb, go)
+        np.testing.assert_array_equal(host(dev, gb), base + 2 * go_host.sum(axis=0))
+    # the products themselves are unchanged by the extra result
+    xs, ws_, gos = dev.to_host(x), dev.to_host(w), dev.to_host(go)
+    gx, gw, gb = dev.zeros_like_storage(x), dev.zeros_like_storage(w), dev.zeros(dtype, (o,))
+    dev.linear_backward(x, gx, w, gw, gb, go)
+    gx2, gw2 = dev.zeros_like_storage(x), dev.zeros_like_storage(w)
+    dev.linear_backward(x, gx2, w, gw2, None, go)
+    assert np.array_equal(dev.to_host(gw).view(np.uint8), dev.to_host(gw2).view(np.uint8))
+    assert np.array_equal(dev.to_host(gx).view(np.uint8), dev.to_host(gx2).view(np.uint8))
+    ogx, ogw = np.zeros_like(xs), np.zeros_like(ws_)
+    oracle.matmat_backward(dtype, rows, i, o, xs, (i, 1), ogx, ws_, (1, i), ogw, gos)
+    assert_within(dtype, rows, host(dev, gw), oracle.to_f64(ogw, dtype).reshape(o, i), host(dev, go), host(dev, x), what="grad_weight")
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_linear_backward_fused_bias_gradient_random(dtype):
+    """Random grad_out: against the f64 column sums within the tolerance of one f32-accumulated reduction."""
+    from helpers import assert_within
+    dev, g = device(), rng(306)
+    for rows, i, o in ((8192, 1024, 1024), (1024, 512, 2048), (640, 264, 1000)):
+        announce("linear backward, fused bias gradient, random", dtype, rows, i, o)
+        x = upload(dev, g.standard_normal((rows, i)), dtype)
+        w = upload(dev, g.uniform(-1, 1, (o, i)) / np.sqrt(i), dtype)
+        go = upload(dev, g.standard_normal((rows, o)), dtype)
+        gx, gw, gb = dev.zeros_like_storage(x), dev.zeros_like_storage(w), dev.zeros(dtype, (o,))
+        dev.linear_backward(x, gx, w, gw, gb, go)
+        go64 = host(dev, go)
+        assert_within(dtype, rows, host(dev, gb), go64.sum(axis=0), go64, np.ones(1), what="grad_bias")
