@@ -237,8 +237,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
         f_kt = p.kbatches > 1 ? fw.it0 % ktiles : fw.it0;
         a_next = a_origin(fw, f_kb) + f_kt * a_step;
         b_next = b_origin(fw, f_kb) + f_kt * b_step;
-        ta.init(p.lda, p.m - fw.bm0, wave, lane);
-        tb.init(p.ldb, p.n - fw.bn0, wave, lane);
+        // wave and lane as new values: the tile coordinates derived from them are needed once per work item only and
+        // are recomputed here instead of being carried through the k loop
+        int f_wave = wave, f_lane = lane;
+        asm volatile("" : "+v"(f_wave), "+v"(f_lane));
+        ta.init(p.lda, p.m - fw.bm0, f_wave, f_lane);
+        tb.init(p.ldb, p.n - fw.bn0, f_wave, f_lane);
     };
     begin_fetch();
     bool fetching = true;
