@@ -88,21 +88,26 @@ def test_generic_k_zero_and_empty():
 
 
 def test_doubly_strided_operand_takes_generic_path():
-    """Neither stride is 1 (reachable through user permutes/slices): Cuda panics there (mod.rs:323), Cpu does not."""
+    """Neither stride is 1 (reachable through user permutes/slices): Cuda panics there (mod.rs:323), Cpu does not.  16-bit
+    products take the generic kernel; a small f32 product takes the k-sliced 16 x 16 kernel, which reads its operands
+    element by element and accepts any strides; a large f32 one the generic kernel again."""
     dev = device()
     g = rng(5)
-    m, k, n = 40, 24, 16
-    a = oracle.to_storage(g.standard_normal(m * (2 * k + 3)), "f32")
-    astr = (2 * k + 3, 2)
-    b, bstr = make_operand(g, k, n, False, "f32")
-    c = np.zeros(m * n, np.float32)
-    da, db, dc = dev.tensor(a, "f32"), dev.tensor(b, "f32"), dev.tensor(c, "f32")
-    desc = dev.gemm_desc("f32", m, k, n, da.ptr, astr, db.ptr, bstr, dc.ptr, (n, 1))
-    assert dev.gemm_plan(desc)[0] == KERNEL_GENERIC
-    announce("gemm doubly strided")
-    dev.gemm(desc)
-    A, B = values(a, "f32", (m, k), astr), values(b, "f32", (k, n), bstr)
-    assert_within("f32", k, dev.to_host(dc).astype(np.float64).reshape(m, n), A @ B, A, B, extra=1e-6)
+    for dtype, (m, k, n), family, kernel_name in (("f16", (40, 24, 16), KERNEL_GENERIC, "generic"),
+                                                  ("f32", (40, 24, 16), KERNEL_MFMA, "mfma32_small_16x16_ksliced"),
+                                                  ("f32", (600, 520, 440), KERNEL_GENERIC, "generic")):
+        a = oracle.to_storage(g.standard_normal(m * (2 * k + 3)), dtype)
+        astr = (2 * k + 3, 2)
+        b, bstr = make_operand(g, k, n, False, dtype)
+        c = oracle.to_storage(np.zeros(m * n), dtype)
+        da, db, dc = dev.tensor(a, dtype), dev.tensor(b, dtype), dev.tensor(c, dtype)
+        desc = dev.gemm_desc(dtype, m, k, n, da.ptr, astr, db.ptr, bstr, dc.ptr, (n, 1))
+        plan = dev.gemm_plan(desc)
+        assert plan[0] == family and plan[2] == kernel_name, plan
+        announce("gemm doubly strided", dtype, (m, k, n), kernel_name)
+        dev.gemm(desc)
+        A, B = values(a, dtype, (m, k), astr), values(b, dtype, (k, n), bstr)
+        assert_within(dtype, k, oracle.to_f64(dev.to_host(dc), dtype).reshape(m, n), A @ B, A, B, extra=1e-6)
 
 
 def test_aliased_output_sums_or_is_rejected():
@@ -160,6 +165,27 @@ def test_mfma_variants(dtype, variant, layout):
 def test_mfma_column_major_c(dtype, layout):
     """A permuted operand's gradient is a column-major C (cpu_kernel.rs:283-284): solved as C^T = B^T A^T."""
     run_case(dtype, 264, 72, 136, layout, True, KERNEL_MFMA, 0, c_colmajor=True, pads=(0, 8, 8))
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+def test_small_f32_kernel_tails_bias_and_wave_counts(layout):
+    """The 16 x 16 kernel that cuts k over the waves of a workgroup: extents that are no multiple of 16 or 4 in any
+    direction, every wave count (k = 20 .. 600: 1, 2, 4, 8 slices), bias per column and (column-major C) per row, beta = 1,
+    padded rows (vector loads off / on).  Config 1's three products take it on their own."""
+    dev = device()
+    small = dev.mfma_variant_count("f32")
+    for i, (m, k, n) in enumerate([(64, 512, 256), (19, 20, 35), (33, 70, 17), (50, 131, 49), (16, 600, 16), (1, 77, 5), (130, 258, 3)]):
+        for pads in ((0, 0, 0), (3, 1, 5), (8, 4, 4)):
+            run_case("f32", m, k, n, layout, bool(i % 2), KERNEL_MFMA, small, bias=(i % 3 == 0), c_colmajor=(i % 3 == 1 and n > 1),
+                     seed=60 + i, pads=pads)
+    x, w, y = dev.tensor(np.zeros(64 * 512, np.float32), "f32"), dev.tensor(np.zeros(256 * 512, np.float32), "f32"), dev.tensor(np.zeros(64 * 256, np.float32), "f32")
+    for desc in (dev.gemm_desc("f32", 64, 512, 256, x.ptr, (512, 1), w.ptr, (1, 512), y.ptr, (256, 1)),
+                 dev.gemm_desc("f32", 64, 256, 512, y.ptr, (256, 1), w.ptr, (512, 1), x.ptr, (512, 1), accumulate=True),
+                 dev.gemm_desc("f32", 512, 64, 256, x.ptr, (1, 512), y.ptr, (256, 1), w.ptr, (1, 512), accumulate=True)):
+        assert dev.gemm_plan(desc)[2] == "mfma32_small_16x16_ksliced"
+    # the plain k order asked for (broadcast-rhs forward): not this kernel
+    from dfdx_amd.rocm import View
+    assert "small" not in dev.gemm_plan(dev.gemm_desc("f32", 64, 512, 256, x.ptr, (512, 1), w.ptr, (1, 512), y.ptr, (256, 1), no_split_k=True))[2]
 
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])

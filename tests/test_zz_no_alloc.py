@@ -63,7 +63,7 @@ def test_weight_gradient_shape_twice_second_smaller(dtype):
 
 def test_f32_split_twice_second_smaller():
     both_entries("f32", 256, 4096, 512, (True, False), True, seed=21)
-    both_entries("f32", 64, 2048, 256, (False, True), False, seed=22)
+    both_entries("f32", 128, 4096, 384, (False, True), False, seed=22)
 
 
 def test_forced_split_then_unsplit_then_sliced_vector_product():
