@@ -390,13 +390,18 @@ int gemm_with_colsum(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, void *
     if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
     Plan plan;
     if (int e = make_plan(ctx, desc, p, &plan)) return e;
-    const bool can = p.ksum && plan.kernel == DFDX_ROCM_KERNEL_MFMA && (p.dtype == DT_F16 || p.dtype == DT_BF16) &&
-                     plan.variant >= mfma16_dma_first_variant() &&
-                     mfma16dma_ksum_supported(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
+    bool can = p.ksum && plan.kernel == DFDX_ROCM_KERNEL_MFMA;
+    if (can && (p.dtype == DT_F16 || p.dtype == DT_BF16))
+        can = plan.variant >= mfma16_dma_first_variant() &&
+              mfma16dma_ksum_supported(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
+    else if (can && p.dtype == DT_F32)
+        can = plan.splits <= 1 && mfma32_ksum_supported(p, plan.variant);
+    else
+        can = false;
     if (can) {
         bool fresh = false;
         const int64_t len = p.ksum_of == KSUM_OF_A ? p.m : p.n;
-        if (int e = settle_output(ctx, p.ksum, (size_t)len * 2, true, &fresh)) return e;
+        if (int e = settle_output(ctx, p.ksum, (size_t)len * dtype_size(p.dtype), true, &fresh)) return e;
         p.ksum_accumulate = !fresh;
         *fused = true;
     } else {

@@ -123,6 +123,7 @@ int mfma32_pick_variant(const GemmProblem &p, int compute_units, int forced_spli
 int mfma32_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits);
 size_t mfma32_workspace_bytes(const GemmProblem &p, int variant, int splits);
 hipError_t launch_mfma32(const GemmProblem &p, int variant, hipStream_t stream);
+bool mfma32_ksum_supported(const GemmProblem &p, int variant);  // can this variant also produce p.ksum? (the small kernel)
 
 // ---- MFMA kernels for f64 (gemm_mfma64.hip) ----
 int mfma64_variant_count();

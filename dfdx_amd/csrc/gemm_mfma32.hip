@@ -558,6 +558,10 @@ struct SmallParams {
     int accumulate, bias_mode;
     int a_vec, b_vec;  // the operand is stored along k and every 4-k group of a row is one aligned 16-byte piece
     int slice;         // k per wave, a multiple of 16
+    // second result (may be null): ksum[i] (+)= sum_k A[i][k], produced by the workgroups of tile column 0 from the A
+    // values they hold anyway (Linear's bias gradient out of the weight-gradient launch)
+    float *ksum;
+    int ksum_accumulate;
 };
 
 template <int WAVES> __global__ __launch_bounds__(WAVES * 64) void gemm_small32_kernel(const SmallParams p) {
@@ -580,12 +584,18 @@ template <int WAVES> __global__ __launch_bounds__(WAVES * 64) void gemm_small32_
         return v;
     };
     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    const bool sums = p.ksum && tn == 0;
+    float rsum = 0.0f;  // of A[row r16][this lane's k values]
     for (int kb = k0; kb < k1; kb += 64) {  // four steps of 16 k per pass: 8 loads in flight per lane
         f32x4 av[4], bv[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             av[u] = fetch(ap, p.a_cs, row_ok, p.a_vec, kb + 16 * u + 4 * q);
             bv[u] = fetch(bp, p.b_rs, col_ok, p.b_vec, kb + 16 * u + 4 * q);
+        }
+        if (sums) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) rsum += (av[u][0] + av[u][1]) + (av[u][2] + av[u][3]);
         }
 #pragma unroll
         for (int u = 0; u < 4; u++)
@@ -597,6 +607,12 @@ template <int WAVES> __global__ __launch_bounds__(WAVES * 64) void gemm_small32_
     }
     // lane l, register r: C[tm * 16 + 4 * (l / 16) + r][tn * 16 + l % 16]
     f32x4 sum = acc0 + acc1;
+    __shared__ float part_rows[WAVES][16];
+    if (sums) {  // uniform over the workgroup
+        rsum += __shfl_xor(rsum, 16, 64);
+        rsum += __shfl_xor(rsum, 32, 64);
+        if (lane < 16) part_rows[wave][lane] = rsum;
+    }
     if constexpr (WAVES > 1) {
 #pragma unroll
         for (int r = 0; r < 4; r++) part[wave][r * 64 + lane] = sum[r];
@@ -607,6 +623,12 @@ template <int WAVES> __global__ __launch_bounds__(WAVES * 64) void gemm_small32_
         for (int w = 1; w < WAVES; w++)
 #pragma unroll
             for (int r = 0; r < 4; r++) sum[r] += part[w][r * 64 + lane];
+    }
+    if (sums && lane < 16 && row_ok) {  // slices in wave order, then the old value unless the gradient is fresh
+        float v = part_rows[0][lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) v += part_rows[w][lane];
+        p.ksum[row] = (p.ksum_accumulate ? p.ksum[row] : 0.0f) + v;
     }
     if (!col_ok) return;
     const float cb = p.bias_mode == BIAS_PER_COL ? p.bias[col] : 0.0f;
@@ -721,6 +743,10 @@ inline bool needs_window(const GemmProblem &p, const OperandLayout &la, const Op
 }  // namespace
 
 int mfma32_variant_count() { return kNumVariants; }
+bool mfma32_ksum_supported(const GemmProblem &p, int variant) {
+    return p.ksum && p.ksum_of == KSUM_OF_A && variant >= 1 && variant <= kNumVariants && kVariants[variant - 1].small &&
+           mfma32_supported(p, variant) && ((uintptr_t)p.ksum & 3u) == 0;
+}
 const char *mfma32_variant_name(int v) { return (v >= 1 && v <= kNumVariants) ? kVariants[v - 1].name : "?"; }
 
 bool mfma32_supported(const GemmProblem &p, int variant) {
@@ -867,6 +893,8 @@ static hipError_t launch_small(const GemmProblem &g, hipStream_t stream) {
     p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
     p.a_vec = g.a_cs == 1 && (g.m == 1 || g.a_rs % 4 == 0) && aligned16(g.a);
     p.b_vec = g.b_rs == 1 && (g.n == 1 || g.b_cs % 4 == 0) && aligned16(g.b);
+    p.ksum = (g.ksum && g.ksum_of == KSUM_OF_A) ? (float *)g.ksum : nullptr;
+    p.ksum_accumulate = g.ksum_accumulate;
     const int waves = small_waves(g.k);
     p.slice = (int)(((g.k + waves - 1) / waves + 15) / 16 * 16);
     const dim3 grid((unsigned)(((g.m + 15) / 16) * p.tiles_n));

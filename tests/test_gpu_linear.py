@@ -127,8 +127,11 @@ FUSED_SHAPES = [(8192, 1024, 1024), (4096, 1024, 4096), (512, 256, 512), (640, 2
                 (64, 1024, 1024)]
 
 
-@pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("rows,i,o", FUSED_SHAPES)
+# f32: the k-sliced small kernel produces the row sums (config 1's Linear and smaller)
+FUSED_F32 = [("f32", 64, 512, 256), ("f32", 100, 40, 24), ("f32", 17, 33, 9), ("f32", 300, 16, 130)]
+
+
+@pytest.mark.parametrize("dtype,rows,i,o", [(d, *shape) for d in ("f16", "bf16") for shape in FUSED_SHAPES] + FUSED_F32)
 def test_linear_backward_bias_gradient_from_the_weight_gradient_launch(dtype, rows, i, o):
     """grad_bias: exact on small integers (sums below 2^8 for bf16, 2^11 for f16 are representable), and twice the
     value after a second call (the first call finds the gradient fresh when its zeros are deferred, the second adds)."""
@@ -147,8 +150,9 @@ def test_linear_backward_bias_gradient_from_the_weight_gradient_launch(dtype, ro
         if deferred:   # NaN patterns that are only DECLARED zero: a read of the old contents would show
             import torch
             from dfdx_amd.rocm import View
-            raw = torch.full((o * 2,), 0xFF, dtype=torch.uint8, device="cuda")
-            dev.zero_deferred(raw.data_ptr(), o * 2)
+            es = 4 if dtype == "f32" else 2
+            raw = torch.full((o * es,), 0xFF, dtype=torch.uint8, device="cuda")
+            dev.zero_deferred(raw.data_ptr(), o * es)
             gb, base = View(raw, dtype, (o,), (1,)), np.zeros(o)
         else:
             gb, base = upload(dev, start, dtype), start
