@@ -71,7 +71,6 @@ template <> struct Mma<_Float16> {
     }
     static __device__ __forceinline__ float to_f32(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
     static __device__ __forceinline__ uint16_t from_f32(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
-    static constexpr uint32_t ONE2 = 0x3C003C00u;  // two 1.0
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // v_cvt_pk_f16_f32: RNE, lo in bits 15:0
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, h2));
@@ -87,7 +86,6 @@ template <> struct Mma<__bf16> {
         if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
         return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);  // round to nearest even
     }
-    static constexpr uint32_t ONE2 = 0x3F803F80u;
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // v_cvt_pk_bf16_f32: RNE, quiet NaNs
         typedef __bf16 b2 __attribute__((ext_vector_type(2)));
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, b2));
