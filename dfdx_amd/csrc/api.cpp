@@ -15,17 +15,39 @@ int bind(dfdx_rocm_ctx *ctx) {
     return DFDX_ROCM_OK;
 }
 
+// Frees the buffers that `grow` replaced.  The caller has drained the stream.
+static hipError_t free_retired(dfdx_rocm_ctx *ctx) {
+    hipError_t first = hipSuccess;
+    for (void *p : ctx->retired) {
+        const hipError_t e = hipFree(p);
+        if (first == hipSuccess) first = e;
+    }
+    ctx->retired.clear();
+    return first;
+}
+
+// The stream is not drained here: work already queued keeps the old buffer, which is retired, and the call in hand
+// gets a new one (only a failed allocation drains, frees what is retired and tries once more).
 static int grow(dfdx_rocm_ctx *ctx, void **buf, size_t *have, size_t bytes) {
     CtxLock lock(ctx->mu);
     if (bytes <= *have) return DFDX_ROCM_OK;
     if (*buf) {
-        HIP_TRY(hipStreamSynchronize(ctx->stream));
-        HIP_TRY(hipFree(*buf));
+        ctx->retired.push_back(*buf);
         *buf = nullptr;
         *have = 0;
     }
     bytes = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
-    HIP_TRY(hipMalloc(buf, bytes));
+    hipError_t e = hipMalloc(buf, bytes);
+    if (e == hipErrorOutOfMemory && !ctx->retired.empty()) {
+        (void)hipGetLastError();
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+        (void)free_retired(ctx);
+        e = hipMalloc(buf, bytes);
+    }
+    if (e != hipSuccess) {
+        *buf = nullptr;
+        return (int)e;
+    }
     *have = bytes;
     return DFDX_ROCM_OK;
 }
@@ -440,10 +462,11 @@ int dfdx_rocm_create(int ordinal, void *stream, dfdx_rocm_ctx **out) {
 
 int dfdx_rocm_destroy(dfdx_rocm_ctx *ctx) {
     if (!ctx) return DFDX_ROCM_OK;
-    if (ctx->workspace || ctx->patches || !ctx->cache.empty() || ctx->pending_count.load()) {
+    if (ctx->workspace || ctx->patches || !ctx->retired.empty() || !ctx->cache.empty() || ctx->pending_count.load()) {
         (void)hipSetDevice(ctx->device);
         (void)settle_all(ctx);  // the caller's buffers outlive the context: they must hold the zeros they were promised
         (void)hipStreamSynchronize(ctx->stream);
+        (void)free_retired(ctx);
         if (ctx->workspace) (void)hipFree(ctx->workspace);
         if (ctx->patches) (void)hipFree(ctx->patches);
         (void)drop_cache(ctx);
@@ -647,6 +670,8 @@ int dfdx_rocm_synchronize(dfdx_rocm_ctx *ctx) {
     if (int e = bind(ctx)) return e;
     if (int e = settle_all(ctx)) return e;  // whoever reads the memory after this call must find the zeros
     HIP_TRY(hipStreamSynchronize(ctx->stream));
+    CtxLock lock(ctx->mu);
+    HIP_TRY(free_retired(ctx));  // workspaces outgrown since the last call: nothing on the stream uses them any more
     return DFDX_ROCM_OK;
 }
 

@@ -20,6 +20,10 @@ struct dfdx_rocm_ctx {
     std::recursive_mutex mu;
     void *workspace = nullptr;  // partial sums of split reductions; grown on demand, owned by the context
     size_t workspace_bytes = 0;
+    // Outgrown workspace / patch buffers.  Launches already on the stream may still use them, so they are not freed where
+    // they are replaced (that would mean draining the stream in the middle of a GEMM call) but at the next
+    // dfdx_rocm_synchronize, at destroy, or when an allocation fails for lack of memory.
+    std::vector<void *> retired;
     void *static_scratch = nullptr;  // this device's copy of the fixed scratch array of dfdx_rocm_gemm_noalloc (never freed)
     // The allocation cache (tensor/cache.rs:36-149): freed buffers kept by size for the next dfdx_rocm_alloc of that size.
     // Off until dfdx_rocm_enable_cache.  The reference keys on (bytes, element size, alignment) because the Rust

@@ -93,3 +93,29 @@ def test_allocation_cache_reuses_and_releases():
     h = dev.alloc(64)
     dev.free(h)
     assert dev.cache_stats() == (0, 0)
+
+
+def test_workspace_growth_does_not_disturb_queued_work():
+    """A split product that needs a larger workspace than the context holds gets a new one while the launches queued
+    before it keep the old one (retired, freed at the next synchronize): both results are right, in either order."""
+    import oracle
+    from gpu_util import make_operand, values
+    from helpers import assert_within, rng
+    from dfdx_amd import Rocm
+
+    dev = Rocm(0)   # a context of its own: its workspace starts empty
+    g = rng(91)
+    outs = []
+    for (m, k, n, split) in ((64, 2048, 64, 4), (256, 4096, 512, 8), (128, 2048, 128, 4), (512, 4096, 1024, 8)):
+        a, astr = make_operand(g, m, k, True, "f32")
+        b, bstr = make_operand(g, k, n, False, "f32")
+        c = np.zeros(m * n, np.float32)
+        da, db, dc = dev.tensor(a, "f32"), dev.tensor(b, "f32"), dev.tensor(c, "f32")
+        desc = dev.gemm_desc("f32", m, k, n, da.ptr, astr, db.ptr, bstr, dc.ptr, (n, 1), split_k=split, kernel=2, variant=4)
+        announce("workspace growth", (m, k, n), dev.gemm_plan(desc)[2])
+        assert "splitk" in dev.gemm_plan(desc)[2]
+        dev.gemm(desc)   # no synchronize in between: the next, larger product is planned while this one may still run
+        outs.append((dc, values(a, "f32", (m, k), astr), values(b, "f32", (k, n), bstr), (m, k, n), (da, db)))
+    dev.synchronize()
+    for dc, A, B, (m, k, n), _keep in outs:
+        assert_within("f32", k, dev.to_host(dc).astype(np.float64).reshape(m, n), A @ B, A, B, extra=1e-5)
