@@ -114,6 +114,117 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_backward_reg_kernel(const 
     }
 }
 
+// ---- short rows: four rows per wave, 16 lanes each -------------------------------------------------------------
+// A row of up to 16 * N * CH elements (1024 16-bit values) is spread over the 16 lanes of one DPP row: lane j of the row
+// owns the N-element groups j, j + 16, ...  Its maximum and its sums then need four DPP steps that ride on the max / add
+// itself (two quad permutations, the half-row and the row mirror) instead of six cross-lane moves through the LDS
+// crossbar, and a wave keeps four rows' loads in flight.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_move<0x141>(v));  // row_half_mirror
+    return fmaxf(v, dpp_move<0x140>(v));  // row_mirror
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    return v + dpp_move<0x140>(v);
+}
+
+template <typename T, int N, int CH>
+__global__ __launch_bounds__(WAVES * 64) void softmax_forward_row16_kernel(const T *x, T *out, int64_t rows, int cols, float scale) {
+    const int lane = threadIdx.x % 64, j = lane % 16, sub = lane / 16;
+    for (int64_t row0 = ((int64_t)blockIdx.x * WAVES + threadIdx.x / 64) * 4; row0 < rows; row0 += (int64_t)gridDim.x * WAVES * 4) {
+        const bool live = row0 + sub < rows;
+        const int64_t row = live ? row0 + sub : rows - 1;  // lanes past the last row repeat it and store nothing
+        const T *src = x + row * cols;
+        float v[CH][N];
+        float m = -FLT_MAX;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 16 + j) * N;
+            if (col < cols) {
+                load_elems<T, N>(src + col, v[c]);
+#pragma unroll
+                for (int i = 0; i < N; i++) {
+                    v[c][i] *= scale;
+                    m = fmaxf(m, v[c][i]);
+                }
+            }
+        }
+        m = row16_max(m);
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 16 + j) * N;
+            if (col < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) {
+                    v[c][i] = expf(v[c][i] - m);
+                    s += v[c][i];
+                }
+            }
+        }
+        s = row16_sum(s);
+        const float inv = 1.0f / s;
+        T *dst = out + row * cols;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 16 + j) * N;
+            if (live && col < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) v[c][i] *= inv;
+                store_elems<T, N>(dst + col, v[c]);
+            }
+        }
+    }
+}
+
+template <typename T, int N, int CH>
+__global__ __launch_bounds__(WAVES * 64) void softmax_backward_row16_kernel(const T *p, const T *go, T *gx, int64_t rows, int cols,
+                                                                            float scale, bool fresh) {
+    const int lane = threadIdx.x % 64, j = lane % 16, sub = lane / 16;
+    for (int64_t row0 = ((int64_t)blockIdx.x * WAVES + threadIdx.x / 64) * 4; row0 < rows; row0 += (int64_t)gridDim.x * WAVES * 4) {
+        const bool live = row0 + sub < rows;
+        const int64_t row = live ? row0 + sub : rows - 1;
+        const T *ps = p + row * cols, *gs = go + row * cols;
+        float pv[CH][N], gv[CH][N];
+        float dot = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 16 + j) * N;
+            if (col < cols) {
+                load_elems<T, N>(ps + col, pv[c]);
+                load_elems<T, N>(gs + col, gv[c]);
+#pragma unroll
+                for (int i = 0; i < N; i++) dot += pv[c][i] * gv[c][i];
+            }
+        }
+        dot = row16_sum(dot);
+        T *dst = gx + row * cols;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 16 + j) * N;
+            if (live && col < cols) {
+                float old[N];
+                if (fresh) {
+#pragma unroll
+                    for (int i = 0; i < N; i++) old[i] = 0.0f;
+                } else {
+                    load_elems<T, N>(dst + col, old);
+                }
+#pragma unroll
+                for (int i = 0; i < N; i++) old[i] += scale * (pv[c][i] * (gv[c][i] - dot));
+                store_elems<T, N>(dst + col, old);
+            }
+        }
+    }
+}
+
 // ---- long rows: three passes over memory --------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(WAVES * 64) void softmax_forward_loop_kernel(const T *x, T *out, int64_t rows, int cols, float scale) {
@@ -164,8 +275,18 @@ int launch_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *a, cons
         else softmax_backward_reg_kernel<T, N, CH><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh); \
         return (int)hipGetLastError();                                                                                 \
     } while (0)
+#define DFDX_SOFTMAX_ROW16(N, CH)                                                                                      \
+    do {                                                                                                               \
+        const unsigned g16 = (unsigned)std::min<int64_t>((rows + WAVES * 4 - 1) / (WAVES * 4), (int64_t)ctx->compute_units * 16); \
+        if constexpr (FWD) softmax_forward_row16_kernel<T, N, CH><<<g16, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale); \
+        else softmax_backward_row16_kernel<T, N, CH><<<g16, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh); \
+        return (int)hipGetLastError();                                                                                 \
+    } while (0)
     if (vec) {
         const int64_t groups = cols / V;
+        if (groups <= 16) DFDX_SOFTMAX_ROW16(V, 1);
+        if (groups <= 32) DFDX_SOFTMAX_ROW16(V, 2);
+        if (FWD && groups <= 64) DFDX_SOFTMAX_ROW16(V, 4);  // the backward holds two rows of values per lane: no gain at 4 groups
         if (groups <= 64) DFDX_SOFTMAX_REG(V, 1);
         if (groups <= 128) DFDX_SOFTMAX_REG(V, 2);
         if (groups <= 256) DFDX_SOFTMAX_REG(V, 4);
@@ -176,6 +297,7 @@ int launch_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *a, cons
         if (cols <= 1024) DFDX_SOFTMAX_REG(1, 16);
     }
 #undef DFDX_SOFTMAX_REG
+#undef DFDX_SOFTMAX_ROW16
     if constexpr (FWD) softmax_forward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale);
     else softmax_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh);
     return (int)hipGetLastError();
