@@ -29,6 +29,39 @@ template <> struct Elem<__bf16> {
     }
 };
 
+// Sum / maximum over the 64 lanes of a wave, every lane receiving the result, without the LDS crossbar (`__shfl_xor` is a
+// ds_bpermute per step): four DPP steps inside the 16-lane rows (two quad permutations, the half-row and the row
+// mirror), then the rows pairwise and the wave's halves through v_permlane16_swap / v_permlane32_swap.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x141>(v);  // row_half_mirror
+    return v + dpp_move<0x140>(v);  // row_mirror
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_move<0xB1>(v));
+    v = fmaxf(v, dpp_move<0x4E>(v));
+    v = fmaxf(v, dpp_move<0x141>(v));
+    return fmaxf(v, dpp_move<0x140>(v));
+}
+__device__ __forceinline__ float wave64_sum(float v) {
+    v = row16_sum(v);
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);  // rows (0,0,2,2) and (1,1,3,3)
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);      // (lower, lower) and (upper, upper)
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float wave64_max(float v) {
+    v = row16_max(v);
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 // N consecutive elements as f32; N == Elem<T>::VEC moves 16 bytes at once (p must then be 16-byte aligned).
 template <typename T, int N> __device__ __forceinline__ void load_elems(const T *p, float (&v)[N]) {
     if constexpr (N == Elem<T>::VEC) {

@@ -16,11 +16,7 @@ namespace {
 constexpr int WAVES = 4;      // rows in flight per workgroup (forward)
 constexpr int WAVES_BWD = 8;  // backward: more rows per workgroup, so fewer slices of column sums to combine
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
+__device__ __forceinline__ float wave_sum(float v) { return wave64_sum(v); }
 
 // Lane l owns the N-element groups l, l + 64, ... of the row (CH of them; groups past the row end are skipped).
 template <typename T, int N, int CH>

@@ -14,16 +14,8 @@ namespace {
 
 constexpr int WAVES = 4;  // rows per workgroup
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
-}
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
+__device__ __forceinline__ float wave_max(float v) { return wave64_max(v); }
+__device__ __forceinline__ float wave_sum(float v) { return wave64_sum(v); }
 
 // ---- rows held in registers -----------------------------------------------------------------------------------
 // Lane l owns the N-element groups l, l + 64, ... of the row (CH of them; groups past the row end are skipped).
@@ -119,22 +111,6 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_backward_reg_kernel(const 
 // owns the N-element groups j, j + 16, ...  Its maximum and its sums then need four DPP steps that ride on the max / add
 // itself (two quad permutations, the half-row and the row mirror) instead of six cross-lane moves through the LDS
 // crossbar, and a wave keeps four rows' loads in flight.
-template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
-}
-__device__ __forceinline__ float row16_max(float v) {
-    v = fmaxf(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
-    v = fmaxf(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
-    v = fmaxf(v, dpp_move<0x141>(v));  // row_half_mirror
-    return fmaxf(v, dpp_move<0x140>(v));  // row_mirror
-}
-__device__ __forceinline__ float row16_sum(float v) {
-    v += dpp_move<0xB1>(v);
-    v += dpp_move<0x4E>(v);
-    v += dpp_move<0x141>(v);
-    return v + dpp_move<0x140>(v);
-}
-
 template <typename T, int N, int CH>
 __global__ __launch_bounds__(WAVES * 64) void softmax_forward_row16_kernel(const T *x, T *out, int64_t rows, int cols, float scale) {
     const int lane = threadIdx.x % 64, j = lane % 16, sub = lane / 16;
