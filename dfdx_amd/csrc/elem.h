@@ -29,6 +29,16 @@ template <> struct Elem<__bf16> {
     }
 };
 
+// f64 takes part in the plain (row-walking) kernels only: no 16-byte vector path, f64 arithmetic throughout.
+template <> struct Elem<double> {
+    static constexpr int VEC = 2;
+    static __device__ __forceinline__ double load(const double *p) { return *p; }
+    static __device__ __forceinline__ void store(double *p, double v) { *p = v; }
+};
+// The type a kernel computes in: f32 for the 16- and 32-bit element types, f64 for f64.
+template <typename T> struct Acc { typedef float type; };
+template <> struct Acc<double> { typedef double type; };
+
 // Sum / maximum over the 64 lanes of a wave, every lane receiving the result, without the LDS crossbar (`__shfl_xor` is a
 // ds_bpermute per step): four DPP steps inside the 16-lane rows (two quad permutations, the half-row and the row
 // mirror), then the rows pairwise and the wave's halves through v_permlane16_swap / v_permlane32_swap.

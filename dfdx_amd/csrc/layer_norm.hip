@@ -17,6 +17,11 @@ constexpr int WAVES = 4;      // rows in flight per workgroup (forward)
 constexpr int WAVES_BWD = 8;  // backward: more rows per workgroup, so fewer slices of column sums to combine
 
 __device__ __forceinline__ float wave_sum(float v) { return wave64_sum(v); }
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
 
 // Lane l owns the N-element groups l, l + 64, ... of the row (CH of them; groups past the row end are skipped).
 template <typename T, int N, int CH>
@@ -177,20 +182,21 @@ __global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_kernel(con
 // Long or unaligned rows: the same formulas with the row walked from memory once per pass.
 template <typename T>
 __global__ __launch_bounds__(WAVES * 64) void layer_norm_forward_loop_kernel(const T *x, const T *gamma, const T *beta, T *out,
-                                                                             int64_t rows, int cols, float eps) {
+                                                                             int64_t rows, int cols, typename Acc<T>::type eps) {
+    typedef typename Acc<T>::type A;  // f32, or f64 for f64 rows
     const int lane = threadIdx.x % 64;
-    const float inv_n = 1.0f / (float)cols;
+    const A inv_n = A(1) / (A)cols;
     for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
         const T *src = x + row * cols;
-        float s = 0.0f;
+        A s = A(0);
         for (int c = lane; c < cols; c += 64) s += Elem<T>::load(src + c);
-        const float mean = wave_sum(s) * inv_n;
-        float q = 0.0f;
+        const A mean = wave_sum(s) * inv_n;
+        A q = A(0);
         for (int c = lane; c < cols; c += 64) {
-            const float d = Elem<T>::load(src + c) - mean;
+            const A d = Elem<T>::load(src + c) - mean;
             q += d * d;
         }
-        const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_n + eps);
+        const A rstd = A(1) / sqrt(wave_sum(q) * inv_n + eps);
         T *dst = out + row * cols;
         for (int c = lane; c < cols; c += 64)
             Elem<T>::store(dst + c, (Elem<T>::load(src + c) - mean) * rstd * Elem<T>::load(gamma + c) + Elem<T>::load(beta + c));
@@ -201,35 +207,36 @@ __global__ __launch_bounds__(WAVES * 64) void layer_norm_forward_loop_kernel(con
 // wave w adds its rows into partial[slice * WAVES_BWD + w], so `slices` counts waves here.
 template <typename T>
 __global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_loop_kernel(const T *x, const T *gamma, const T *go, T *gx,
-                                                                              float *partial, int64_t rows, int cols, float eps, bool fresh_x) {
+                                                                              typename Acc<T>::type *partial, int64_t rows, int cols, typename Acc<T>::type eps, bool fresh_x) {
+    typedef typename Acc<T>::type A;
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-    const float inv_n = 1.0f / (float)cols;
-    float *pg = partial + ((int64_t)(blockIdx.x * WAVES_BWD + wave) * 2) * cols, *pb = pg + cols;
-    for (int c = lane; c < cols; c += 64) pg[c] = pb[c] = 0.0f;
+    const A inv_n = A(1) / (A)cols;
+    A *pg = partial + ((int64_t)(blockIdx.x * WAVES_BWD + wave) * 2) * cols, *pb = pg + cols;
+    for (int c = lane; c < cols; c += 64) pg[c] = pb[c] = A(0);
     for (int64_t row = (int64_t)blockIdx.x * WAVES_BWD + wave; row < rows; row += (int64_t)gridDim.x * WAVES_BWD) {
         const T *src = x + row * cols, *gs = go + row * cols;
-        float s = 0.0f;
+        A s = A(0);
         for (int c = lane; c < cols; c += 64) s += Elem<T>::load(src + c);
-        const float mean = wave_sum(s) * inv_n;
-        float q = 0.0f;
+        const A mean = wave_sum(s) * inv_n;
+        A q = A(0);
         for (int c = lane; c < cols; c += 64) {
-            const float d = Elem<T>::load(src + c) - mean;
+            const A d = Elem<T>::load(src + c) - mean;
             q += d * d;
         }
-        const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_n + eps);
-        float s1 = 0.0f, s2 = 0.0f;
+        const A rstd = A(1) / sqrt(wave_sum(q) * inv_n + eps);
+        A s1 = A(0), s2 = 0.0f;
         for (int c = lane; c < cols; c += 64) {
-            const float xh = (Elem<T>::load(src + c) - mean) * rstd, g = Elem<T>::load(gs + c), gh = g * Elem<T>::load(gamma + c);
+            const A xh = (Elem<T>::load(src + c) - mean) * rstd, g = Elem<T>::load(gs + c), gh = g * Elem<T>::load(gamma + c);
             pg[c] += g * xh;  // column c of this wave's partial belongs to this lane alone
             pb[c] += g;
             s1 += gh;
             s2 += gh * xh;
         }
-        const float m1 = wave_sum(s1) * inv_n, m2 = wave_sum(s2) * inv_n;
+        const A m1 = wave_sum(s1) * inv_n, m2 = wave_sum(s2) * inv_n;
         T *dst = gx + row * cols;
         for (int c = lane; c < cols; c += 64) {
-            const float xh = (Elem<T>::load(src + c) - mean) * rstd, gh = Elem<T>::load(gs + c) * Elem<T>::load(gamma + c);
-            Elem<T>::store(dst + c, (fresh_x ? 0.0f : Elem<T>::load(dst + c)) + rstd * (gh - m1 - xh * m2));
+            const A xh = (Elem<T>::load(src + c) - mean) * rstd, gh = Elem<T>::load(gs + c) * Elem<T>::load(gamma + c);
+            Elem<T>::store(dst + c, (fresh_x ? A(0) : Elem<T>::load(dst + c)) + rstd * (gh - m1 - xh * m2));
         }
     }
 }
@@ -239,18 +246,19 @@ __global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_loop_kerne
 // sums in order: the result does not depend on timing.
 constexpr int COMBINE_GROUPS = 16;
 template <typename T>
-__global__ __launch_bounds__(64 * COMBINE_GROUPS) void layer_norm_combine_kernel(const float *partial, int slices, int cols, T *grad_gamma,
+__global__ __launch_bounds__(64 * COMBINE_GROUPS) void layer_norm_combine_kernel(const typename Acc<T>::type *partial, int slices, int cols, T *grad_gamma,
                                                                                  T *grad_beta, bool fresh_gamma, bool fresh_beta) {
-    __shared__ float red[COMBINE_GROUPS][2][64];
+    typedef typename Acc<T>::type A;
+    __shared__ A red[COMBINE_GROUPS][2][64];
     const int lane = threadIdx.x % 64, grp = threadIdx.x / 64;
     const int c = blockIdx.x * 64 + lane;
     const int per = (slices + COMBINE_GROUPS - 1) / COMBINE_GROUPS;
     const int j0 = grp * per, j1 = min(slices, j0 + per);
-    float sg = 0.0f, sb = 0.0f;
+    A sg = A(0), sb = 0.0f;
     if (c < cols) {
         int j = j0;
         for (; j + 4 <= j1; j += 4) {
-            float a[4], b[4];
+            A a[4], b[4];
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 a[u] = partial[((int64_t)(j + u) * 2) * cols + c];
@@ -271,24 +279,25 @@ __global__ __launch_bounds__(64 * COMBINE_GROUPS) void layer_norm_combine_kernel
     red[grp][1][lane] = sb;
     __syncthreads();
     if (grp == 0 && c < cols) {
-        float tg = 0.0f, tb = 0.0f;
+        A tg = A(0), tb = 0.0f;
 #pragma unroll
         for (int g = 0; g < COMBINE_GROUPS; g++) {
             tg += red[g][0][lane];
             tb += red[g][1][lane];
         }
-        Elem<T>::store(grad_gamma + c, (fresh_gamma ? 0.0f : Elem<T>::load(grad_gamma + c)) + tg);
-        Elem<T>::store(grad_beta + c, (fresh_beta ? 0.0f : Elem<T>::load(grad_beta + c)) + tb);
+        Elem<T>::store(grad_gamma + c, (fresh_gamma ? A(0) : Elem<T>::load(grad_gamma + c)) + tg);
+        Elem<T>::store(grad_beta + c, (fresh_beta ? A(0) : Elem<T>::load(grad_beta + c)) + tb);
     }
 }
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 template <typename T>
-int forward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, const void *gamma, const void *beta, float eps,
-              void *out) {
+int forward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, const void *gamma, const void *beta,
+              typename Acc<T>::type eps, void *out) {
     constexpr int V = Elem<T>::VEC;
-    const bool vec = cols % V == 0 && aligned16(x) && aligned16(gamma) && aligned16(beta) && aligned16(out);
+    constexpr bool F64 = sizeof(T) == 8;  // the plain kernel only
+    const bool vec = !F64 && cols % V == 0 && aligned16(x) && aligned16(gamma) && aligned16(beta) && aligned16(out);
     const unsigned grid = (unsigned)std::min<int64_t>((rows + WAVES - 1) / WAVES, (int64_t)ctx->compute_units * 16);
     const dim3 block(WAVES * 64);
     hipStream_t s = ctx->stream;
@@ -298,11 +307,13 @@ int forward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, con
                                                                    (int)cols, eps);                                               \
         return (int)hipGetLastError();                                                                                            \
     } while (0)
-    if (vec) {
-        const int64_t groups = cols / V;
-        if (groups <= 64) DFDX_LN_FWD(1);
-        if (groups <= 128) DFDX_LN_FWD(2);
-        if (groups <= 256) DFDX_LN_FWD(4);
+    if constexpr (!F64) {
+        if (vec) {
+            const int64_t groups = cols / V;
+            if (groups <= 64) DFDX_LN_FWD(1);
+            if (groups <= 128) DFDX_LN_FWD(2);
+            if (groups <= 256) DFDX_LN_FWD(4);
+        }
     }
 #undef DFDX_LN_FWD
     layer_norm_forward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)beta, (T *)out, rows, (int)cols, eps);
@@ -310,10 +321,12 @@ int forward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, con
 }
 
 template <typename T>
-int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, const void *gamma, float eps, const void *go,
-               void *gx, void *ggamma, void *gbeta, const bool fresh[3]) {
+int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, const void *gamma, typename Acc<T>::type eps,
+               const void *go, void *gx, void *ggamma, void *gbeta, const bool fresh[3]) {
+    typedef typename Acc<T>::type A;
     constexpr int V = Elem<T>::VEC;
-    const bool vec = cols % V == 0 && aligned16(x) && aligned16(gamma) && aligned16(go) && aligned16(gx);
+    constexpr bool F64 = sizeof(T) == 8;
+    const bool vec = !F64 && cols % V == 0 && aligned16(x) && aligned16(gamma) && aligned16(go) && aligned16(gx);
     const int64_t groups = cols / V;
     const bool reg = vec && groups <= 256;
     // at least 2 rows per wave so that the column sums amortise; two workgroups (16 waves) per compute unit
@@ -322,15 +335,21 @@ int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, co
     const dim3 block(WAVES_BWD * 64);
     hipStream_t s = ctx->stream;
     CtxLock lock(ctx->mu);  // two launches around the shared workspace
-    if (int rc = ensure_workspace(ctx, (size_t)slices * 2 * cols * sizeof(float))) return rc;
-    float *partial = (float *)ctx->workspace;
+    if (int rc = ensure_workspace(ctx, (size_t)slices * 2 * cols * sizeof(A))) return rc;
+    A *partial = (A *)ctx->workspace;
 #define DFDX_LN_BWD(CH)                                                                                                         \
     layer_norm_backward_kernel<T, V, CH><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, \
                                                                 rows, (int)cols, eps, fresh[0])
-    if (reg && groups <= 64) DFDX_LN_BWD(1);
-    else if (reg && groups <= 128) DFDX_LN_BWD(2);
-    else if (reg) DFDX_LN_BWD(4);
-    else layer_norm_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, rows, (int)cols, eps, fresh[0]);
+    bool launched = false;
+    if constexpr (!F64) {
+        if (reg) {
+            if (groups <= 64) DFDX_LN_BWD(1);
+            else if (groups <= 128) DFDX_LN_BWD(2);
+            else DFDX_LN_BWD(4);
+            launched = true;
+        }
+    }
+    if (!launched) layer_norm_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, rows, (int)cols, eps, fresh[0]);
 #undef DFDX_LN_BWD
     HIP_TRY(hipGetLastError());
     layer_norm_combine_kernel<T><<<(unsigned)((cols + 63) / 64), 64 * COMBINE_GROUPS, 0, s>>>(partial, slices, (int)cols, (T *)ggamma, (T *)gbeta, fresh[1], fresh[2]);
@@ -352,12 +371,13 @@ int dfdx_rocm_layer_norm_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, in
     if (!dims_ok(rows, cols)) return DFDX_ROCM_ERR_INVALID_ARG;
     if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
     if (!x || !gamma || !beta || !out) return DFDX_ROCM_ERR_INVALID_ARG;
-    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    if (dtype < DFDX_ROCM_F32 || dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_UNSUPPORTED;
     if (int e = settle(ctx, x)) return e;
     if (int e = settle(ctx, gamma)) return e;
     if (int e = settle(ctx, beta)) return e;
-    if (int e = settle_output(ctx, out, (size_t)(rows * cols) * (dtype == DFDX_ROCM_F32 ? 4 : 2), false, nullptr)) return e;
+    if (int e = settle_output(ctx, out, (size_t)(rows * cols) * (dtype == DFDX_ROCM_F64 ? 8 : dtype == DFDX_ROCM_F32 ? 4 : 2), false, nullptr)) return e;
     switch (dtype) {
+    case DFDX_ROCM_F64: return forward_t<double>(ctx, rows, cols, x, gamma, beta, epsilon, out);
     case DFDX_ROCM_F32: return forward_t<float>(ctx, rows, cols, x, gamma, beta, (float)epsilon, out);
     case DFDX_ROCM_F16: return forward_t<_Float16>(ctx, rows, cols, x, gamma, beta, (float)epsilon, out);
     case DFDX_ROCM_BF16: return forward_t<__bf16>(ctx, rows, cols, x, gamma, beta, (float)epsilon, out);
@@ -371,8 +391,8 @@ int dfdx_rocm_layer_norm_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, i
     if (!dims_ok(rows, cols)) return DFDX_ROCM_ERR_INVALID_ARG;
     if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
     if (!x || !gamma || !grad_x || !grad_gamma || !grad_beta || !grad_out) return DFDX_ROCM_ERR_INVALID_ARG;
-    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
-    const size_t es = dtype == DFDX_ROCM_F32 ? 4 : 2;
+    if (dtype < DFDX_ROCM_F32 || dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_UNSUPPORTED;
+    const size_t es = dtype == DFDX_ROCM_F64 ? 8 : dtype == DFDX_ROCM_F32 ? 4 : 2;
     bool fresh[3] = {false, false, false};  // gradients whose zero fill is still deferred: stored without being read
     if (int e = settle(ctx, x)) return e;
     if (int e = settle(ctx, gamma)) return e;
@@ -381,6 +401,7 @@ int dfdx_rocm_layer_norm_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, i
     if (int e = settle_output(ctx, grad_gamma, (size_t)cols * es, true, &fresh[1])) return e;
     if (int e = settle_output(ctx, grad_beta, (size_t)cols * es, true, &fresh[2])) return e;
     switch (dtype) {
+    case DFDX_ROCM_F64: return backward_t<double>(ctx, rows, cols, x, gamma, epsilon, grad_out, grad_x, grad_gamma, grad_beta, fresh);
     case DFDX_ROCM_F32: return backward_t<float>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta, fresh);
     case DFDX_ROCM_F16: return backward_t<_Float16>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta, fresh);
     case DFDX_ROCM_BF16: return backward_t<__bf16>(ctx, rows, cols, x, gamma, (float)epsilon, grad_out, grad_x, grad_gamma, grad_beta, fresh);

@@ -33,15 +33,24 @@ template <typename Index> __device__ __forceinline__ int64_t view_offset(const V
 template <typename T, int N, typename Index>
 __global__ __launch_bounds__(256) void reshape_forward_kernel(const T *inp, T *out, ViewDims d, Index groups) {
     for (Index g = (Index)blockIdx.x * 256 + threadIdx.x; g < groups; g += (Index)gridDim.x * 256) {
-        float v[N];
-        load_elems<T, N>(inp + view_offset<Index>(d, g), v);
-        store_elems<T, N>(out + (int64_t)g * N, v);
+        if constexpr (sizeof(T) == 8) {  // f64: one element per thread (N == 1)
+            out[(int64_t)g] = inp[view_offset<Index>(d, g)];
+        } else {
+            float v[N];
+            load_elems<T, N>(inp + view_offset<Index>(d, g), v);
+            store_elems<T, N>(out + (int64_t)g * N, v);
+        }
     }
 }
 
 template <typename T, int N, typename Index>
 __global__ __launch_bounds__(256) void reshape_backward_kernel(T *grad_inp, const T *grad_out, ViewDims d, Index groups, bool fresh) {
     for (Index g = (Index)blockIdx.x * 256 + threadIdx.x; g < groups; g += (Index)gridDim.x * 256) {
+        if constexpr (sizeof(T) == 8) {  // f64: one element per thread (N == 1)
+            T *dst64 = grad_inp + view_offset<Index>(d, g);
+            *dst64 = (fresh ? T(0) : *dst64) + grad_out[(int64_t)g];
+            continue;
+        }
         float v[N], old[N];
         load_elems<T, N>(grad_out + (int64_t)g * N, v);
         T *dst = grad_inp + view_offset<Index>(d, g);
@@ -79,7 +88,7 @@ __global__ __launch_bounds__(256) void reshape_backward_reduce_kernel(T *grad_in
             dst += i * d.keep_dst[a];
             src0 += i * d.keep_src[a];
         }
-        float sum = 0.0f;
+        typename Acc<T>::type sum = 0;
         for (int64_t r = 0; r < folded; r++) {
             int64_t src = src0, t = r;
             for (int a = d.nbro - 1; a >= 0; a--) {
@@ -152,7 +161,7 @@ int launch_t(dfdx_rocm_ctx *ctx, int rank, const int64_t *shape, const int64_t *
     for (int a = 0; a < n; a++) total *= cs[a];
     constexpr int V = Elem<T>::VEC;
     const void *strided = FWD ? src : dst;
-    bool vec = cst[n - 1] == 1 && cs[n - 1] % V == 0 && aligned16(src) && aligned16(dst);
+    bool vec = sizeof(T) != 8 && cst[n - 1] == 1 && cs[n - 1] % V == 0 && aligned16(src) && aligned16(dst);
     for (int a = 0; a + 1 < n && vec; a++) vec = cst[a] % V == 0;
     (void)strided;
     const int g = vec ? V : 1;
@@ -171,9 +180,17 @@ int launch_t(dfdx_rocm_ctx *ctx, int rank, const int64_t *shape, const int64_t *
         if constexpr (FWD) reshape_forward_kernel<T, N, IDX><<<grid, 256, 0, s>>>((const T *)src, (T *)dst, d, (IDX)groups); \
         else reshape_backward_kernel<T, N, IDX><<<grid, 256, 0, s>>>((T *)dst, (const T *)src, d, (IDX)groups, fresh); \
     } while (0)
-    if (vec && small) DFDX_RESHAPE(V, uint32_t);
-    else if (vec) DFDX_RESHAPE(V, uint64_t);
-    else if (small) DFDX_RESHAPE(1, uint32_t);
+    if constexpr (sizeof(T) != 8) {
+        if (vec && small) {
+            DFDX_RESHAPE(V, uint32_t);
+            return (int)hipGetLastError();
+        }
+        if (vec) {
+            DFDX_RESHAPE(V, uint64_t);
+            return (int)hipGetLastError();
+        }
+    }
+    if (small) DFDX_RESHAPE(1, uint32_t);
     else DFDX_RESHAPE(1, uint64_t);
 #undef DFDX_RESHAPE
     return (int)hipGetLastError();
@@ -193,16 +210,17 @@ int dispatch(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, cons
     }
     if (total == 0) return DFDX_ROCM_OK;
     if (!src || !dst) return DFDX_ROCM_ERR_INVALID_ARG;
-    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    if (dtype < DFDX_ROCM_F32 || dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_UNSUPPORTED;
     // Deferred zero fills: the contiguous side covers total elements; the strided side covers its buffer when the view
     // is a permutation of a contiguous layout (a backward through such a view then stores 0 + value).
-    const size_t es = dtype == DFDX_ROCM_F32 ? 4 : 2;
+    const size_t es = dtype == DFDX_ROCM_F64 ? 8 : dtype == DFDX_ROCM_F32 ? 4 : 2;
     bool fresh = false;
     if (int e = settle(ctx, src)) return e;
     if (int e = settle_output(ctx, dst, FWD ? (size_t)total * es : dense_bytes(rank, shape, strides, es), !FWD, broadcast ? nullptr : &fresh))
         return e;
     if (broadcast) {
         switch (dtype) {
+        case DFDX_ROCM_F64: return launch_reduce<double>(ctx, rank, shape, strides, src, dst);
         case DFDX_ROCM_F32: return launch_reduce<float>(ctx, rank, shape, strides, src, dst);
         case DFDX_ROCM_F16: return launch_reduce<_Float16>(ctx, rank, shape, strides, src, dst);
         case DFDX_ROCM_BF16: return launch_reduce<__bf16>(ctx, rank, shape, strides, src, dst);
@@ -210,6 +228,7 @@ int dispatch(dfdx_rocm_ctx *ctx, int dtype, int rank, const int64_t *shape, cons
         }
     }
     switch (dtype) {
+    case DFDX_ROCM_F64: return launch_t<double, FWD>(ctx, rank, shape, strides, src, dst, fresh);
     case DFDX_ROCM_F32: return launch_t<float, FWD>(ctx, rank, shape, strides, src, dst, fresh);
     case DFDX_ROCM_F16: return launch_t<_Float16, FWD>(ctx, rank, shape, strides, src, dst, fresh);
     case DFDX_ROCM_BF16: return launch_t<__bf16, FWD>(ctx, rank, shape, strides, src, dst, fresh);

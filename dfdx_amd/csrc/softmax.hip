@@ -234,6 +234,44 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_backward_loop_kernel(const
     }
 }
 
+// ---- f64: one wave per row, three passes over memory, f64 arithmetic ------------------------------------------
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ double wave_max_f64(double v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v = fmax(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__global__ __launch_bounds__(WAVES * 64) void softmax_forward_f64_kernel(const double *x, double *out, int64_t rows, int cols, double scale) {
+    const int lane = threadIdx.x % 64;
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const double *src = x + row * cols;
+        double m = -DBL_MAX;
+        for (int c = lane; c < cols; c += 64) m = fmax(m, src[c] * scale);
+        m = wave_max_f64(m);
+        double s = 0.0;
+        for (int c = lane; c < cols; c += 64) s += exp(src[c] * scale - m);
+        s = wave_sum_f64(s);
+        double *dst = out + row * cols;
+        for (int c = lane; c < cols; c += 64) dst[c] = exp(src[c] * scale - m) / s;
+    }
+}
+__global__ __launch_bounds__(WAVES * 64) void softmax_backward_f64_kernel(const double *p, const double *go, double *gx, int64_t rows,
+                                                                          int cols, double scale, bool fresh) {
+    const int lane = threadIdx.x % 64;
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const double *ps = p + row * cols, *gs = go + row * cols;
+        double dot = 0.0;
+        for (int c = lane; c < cols; c += 64) dot += ps[c] * gs[c];
+        dot = wave_sum_f64(dot);
+        double *dst = gx + row * cols;
+        for (int c = lane; c < cols; c += 64) dst[c] = (fresh ? 0.0 : dst[c]) + scale * (ps[c] * (gs[c] - dot));
+    }
+}
+
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 template <typename T, bool FWD>
@@ -285,12 +323,18 @@ int dispatch(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const vo
     if (rows < 0 || cols < 0 || cols >= (1ll << 31)) return DFDX_ROCM_ERR_INVALID_ARG;
     if (rows == 0 || cols == 0) return DFDX_ROCM_OK;
     if (!a || !c || (!FWD && !b)) return DFDX_ROCM_ERR_INVALID_ARG;
-    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    if (dtype < DFDX_ROCM_F32 || dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_UNSUPPORTED;
     bool fresh = false;  // a gradient whose zero fill is still deferred: stored without being read
     if (int e = settle(ctx, a)) return e;
     if (int e = settle(ctx, b)) return e;
-    if (int e = settle_output(ctx, c, (size_t)(rows * cols) * (dtype == DFDX_ROCM_F32 ? 4 : 2), !FWD, &fresh)) return e;
+    if (int e = settle_output(ctx, c, (size_t)(rows * cols) * (dtype == DFDX_ROCM_F64 ? 8 : dtype == DFDX_ROCM_F32 ? 4 : 2), !FWD, &fresh)) return e;
     switch (dtype) {
+    case DFDX_ROCM_F64: {
+        const unsigned grid = (unsigned)std::min<int64_t>((rows + WAVES - 1) / WAVES, (int64_t)ctx->compute_units * 16);
+        if constexpr (FWD) softmax_forward_f64_kernel<<<grid, WAVES * 64, 0, ctx->stream>>>((const double *)a, (double *)c, rows, (int)cols, (double)scale);
+        else softmax_backward_f64_kernel<<<grid, WAVES * 64, 0, ctx->stream>>>((const double *)a, (const double *)b, (double *)c, rows, (int)cols, (double)scale, fresh);
+        return (int)hipGetLastError();
+    }
     case DFDX_ROCM_F32: return launch_t<float, FWD>(ctx, rows, cols, a, b, c, scale, fresh);
     case DFDX_ROCM_F16: return launch_t<_Float16, FWD>(ctx, rows, cols, a, b, c, scale, fresh);
     case DFDX_ROCM_BF16: return launch_t<__bf16, FWD>(ctx, rows, cols, a, b, c, scale, fresh);

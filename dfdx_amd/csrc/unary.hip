@@ -95,6 +95,31 @@ __global__ __launch_bounds__(256) void add_backward_kernel(const T *go, T *gl, T
     }
 }
 
+// ---- f64: the reference's fourth element type (its CI runs every test in f64 as well); plain kernels, f64 arithmetic
+enum { F64_SCALE, F64_SCALE_ACC, F64_RELU_FWD, F64_RELU_BWD, F64_ADD_FWD, F64_ADD_BWD };
+template <int OP>
+__global__ __launch_bounds__(256) void unary_f64_kernel(const double *a, const double *b, double *c, double *d, int64_t len, double s,
+                                                        bool fresh_c, bool fresh_d) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < len; i += (int64_t)gridDim.x * 256) {
+        if constexpr (OP == F64_SCALE) c[i] = s * a[i];
+        else if constexpr (OP == F64_SCALE_ACC) c[i] = (fresh_c ? 0.0 : c[i]) + s * a[i];
+        else if constexpr (OP == F64_RELU_FWD) c[i] = fmax(a[i], 0.0);
+        else if constexpr (OP == F64_RELU_BWD) c[i] = (fresh_c ? 0.0 : c[i]) + (a[i] > 0.0 ? b[i] : 0.0);
+        else if constexpr (OP == F64_ADD_FWD) c[i] = a[i] + b[i];
+        else {
+            const double g = a[i];
+            c[i] = (fresh_c ? 0.0 : c[i]) + g;
+            d[i] = (fresh_d ? 0.0 : d[i]) + g;
+        }
+    }
+}
+template <int OP>
+int launch_f64(dfdx_rocm_ctx *ctx, int64_t len, const void *a, const void *b, void *c, void *d, double s, bool fresh_c, bool fresh_d) {
+    const unsigned grid = (unsigned)std::min<int64_t>((len + 255) / 256, (int64_t)ctx->compute_units * 16);
+    unary_f64_kernel<OP><<<grid, 256, 0, ctx->stream>>>((const double *)a, (const double *)b, (double *)c, (double *)d, len, s, fresh_c, fresh_d);
+    return (int)hipGetLastError();
+}
+
 template <typename T> float round_scalar(double s) {
     T tmp;
     float f = (float)s;
@@ -127,11 +152,12 @@ template <bool ACC> int dispatch(dfdx_rocm_ctx *ctx, int dtype, int64_t len, con
     if (len < 0) return DFDX_ROCM_ERR_INVALID_ARG;
     if (len == 0) return DFDX_ROCM_OK;
     if (!x || !out) return DFDX_ROCM_ERR_INVALID_ARG;
-    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    if (dtype < DFDX_ROCM_F32 || dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_UNSUPPORTED;
     bool fresh = false;  // a gradient whose zero fill is still deferred: stored without being read
     if (int e = settle(ctx, x)) return e;
-    if (int e = settle_output(ctx, out, (size_t)len * (dtype == DFDX_ROCM_F32 ? 4 : 2), ACC, &fresh)) return e;
+    if (int e = settle_output(ctx, out, (size_t)len * (dtype == DFDX_ROCM_F64 ? 8 : dtype == DFDX_ROCM_F32 ? 4 : 2), ACC, &fresh)) return e;
     switch (dtype) {
+    case DFDX_ROCM_F64: return launch_f64<ACC ? F64_SCALE_ACC : F64_SCALE>(ctx, len, x, nullptr, out, nullptr, scalar, fresh, false);
     case DFDX_ROCM_F32: return launch_t<float, ACC>(ctx, len, x, scalar, out, fresh);
     case DFDX_ROCM_F16: return launch_t<_Float16, ACC>(ctx, len, x, scalar, out, fresh);
     case DFDX_ROCM_BF16: return launch_t<__bf16, ACC>(ctx, len, x, scalar, out, fresh);
@@ -167,15 +193,18 @@ template <int OP> int dispatch_op(dfdx_rocm_ctx *ctx, int dtype, int64_t len, co
     if (len < 0) return DFDX_ROCM_ERR_INVALID_ARG;
     if (len == 0) return DFDX_ROCM_OK;
     if (!a || !c || (OP != OP_RELU_FWD && OP != OP_ADD_BWD && !b) || (OP == OP_ADD_BWD && !d)) return DFDX_ROCM_ERR_INVALID_ARG;
-    if (dtype != DFDX_ROCM_F32 && dtype != DFDX_ROCM_F16 && dtype != DFDX_ROCM_BF16) return DFDX_ROCM_ERR_UNSUPPORTED;
+    if (dtype < DFDX_ROCM_F32 || dtype > DFDX_ROCM_F64) return DFDX_ROCM_ERR_UNSUPPORTED;
     bool fresh_c = false, fresh_d = false;  // gradients whose zero fill is still deferred: stored without being read
     constexpr bool BWD = OP == OP_RELU_BWD || OP == OP_ADD_BWD;
-    const size_t bytes = (size_t)len * (dtype == DFDX_ROCM_F32 ? 4 : 2);
+    const size_t bytes = (size_t)len * (dtype == DFDX_ROCM_F64 ? 8 : dtype == DFDX_ROCM_F32 ? 4 : 2);
     if (int e = settle(ctx, a)) return e;
     if (int e = settle(ctx, b)) return e;
     if (int e = settle_output(ctx, c, bytes, BWD, &fresh_c)) return e;
     if (int e = settle_output(ctx, d, bytes, BWD, &fresh_d)) return e;
     switch (dtype) {
+    case DFDX_ROCM_F64:
+        return launch_f64<OP == OP_RELU_FWD ? F64_RELU_FWD : OP == OP_RELU_BWD ? F64_RELU_BWD : OP == OP_ADD_FWD ? F64_ADD_FWD : F64_ADD_BWD>(
+            ctx, len, a, b, c, d, 0.0, fresh_c, fresh_d);
     case DFDX_ROCM_F32: return launch_op<float, OP>(ctx, len, a, b, c, d, fresh_c, fresh_d);
     case DFDX_ROCM_F16: return launch_op<_Float16, OP>(ctx, len, a, b, c, d, fresh_c, fresh_d);
     case DFDX_ROCM_BF16: return launch_op<__bf16, OP>(ctx, len, a, b, c, d, fresh_c, fresh_d);

@@ -24,6 +24,9 @@
  *     blocks until it is done.
  *   - f16 and bf16 products accumulate in f32 and round to nearest even once
  *     on store; f32 accumulates in f32; f64 in f64.
+ *   - Every entry point takes all four element types, conv2d excepted (f16,
+ *     bf16, f32): the ops around the products evaluate their formula in f32
+ *     for the 16- and 32-bit types and round once, and in f64 for f64.
  */
 #ifndef DFDX_ROCM_H
 #define DFDX_ROCM_H

@@ -27,8 +27,15 @@ import oracle
 from helpers import row_major_strides
 
 
+def wt(dtype: str):
+    """The numpy type the glue computes in: float32, or float64 for f64 tensors."""
+    return np.float64 if dtype == "f64" else np.float32
+
+
 def rt(x32: np.ndarray, dtype: str) -> np.ndarray:
     """Round float32 values to the storage dtype and back (what storing into a tensor of that dtype does)."""
+    if dtype == "f64":
+        return np.asarray(x32, dtype=np.float64)
     if dtype == "f32":
         return x32.astype(np.float32)
     if dtype == "f16":
@@ -38,11 +45,11 @@ def rt(x32: np.ndarray, dtype: str) -> np.ndarray:
 
 def st(x32: np.ndarray, dtype: str) -> np.ndarray:
     """float32 values -> flat storage array."""
-    return oracle.to_storage(np.ascontiguousarray(x32, dtype=np.float32).reshape(-1), dtype)
+    return oracle.to_storage(np.ascontiguousarray(x32, dtype=wt(dtype)).reshape(-1), dtype)
 
 
 def val(storage: np.ndarray, dtype: str) -> np.ndarray:
-    return oracle.to_f64(storage, dtype).astype(np.float32)
+    return oracle.to_f64(storage, dtype).astype(wt(dtype))
 
 
 class View:
@@ -88,22 +95,22 @@ def linear_fwd(be, dtype, x: View, w: np.ndarray, b: np.ndarray, o: int, i: int)
 def linear_bwd(be, dtype, x: View, gx, w, gw, gb, gy_storage, o: int, i: int):
     be.backward(x, gx, View(w, (i, o), (1, i)), gw, gy_storage)
     g = val(gy_storage, dtype).reshape(-1, o)
-    gb[:] = st(rt(val(gb, dtype) + rt(g.sum(axis=0, dtype=np.float32), dtype), dtype), dtype)
+    gb[:] = st(rt(val(gb, dtype) + rt(g.sum(axis=0, dtype=g.dtype), dtype), dtype), dtype)
 
 
 def softmax_fwd(x, dtype):
     e = np.exp(x - x.max(axis=-1, keepdims=True))
-    return rt(e / e.sum(axis=-1, keepdims=True, dtype=np.float32), dtype)
+    return rt(e / e.sum(axis=-1, keepdims=True, dtype=e.dtype), dtype)
 
 
 def softmax_bwd(p, gp):
-    return p * (gp - (gp * p).sum(axis=-1, keepdims=True, dtype=np.float32))
+    return p * (gp - (gp * p).sum(axis=-1, keepdims=True, dtype=p.dtype))
 
 
 def layernorm_fwd(x, gamma, beta, dtype, eps=1e-5):
-    mean = x.mean(axis=-1, keepdims=True, dtype=np.float32)
-    var = ((x - mean) ** 2).mean(axis=-1, keepdims=True, dtype=np.float32)
-    inv = 1.0 / np.sqrt(var + np.float32(eps))
+    mean = x.mean(axis=-1, keepdims=True, dtype=x.dtype)
+    var = ((x - mean) ** 2).mean(axis=-1, keepdims=True, dtype=x.dtype)
+    inv = 1.0 / np.sqrt(var + x.dtype.type(eps))
     xhat = (x - mean) * inv
     return rt(xhat * gamma + beta, dtype), (xhat, inv)
 
@@ -112,8 +119,9 @@ def layernorm_bwd(gy, gamma, cache):
     xhat, inv = cache
     g = gy * gamma
     n = xhat.shape[-1]
-    gx = inv * (g - g.mean(axis=-1, keepdims=True, dtype=np.float32) - xhat * (g * xhat).mean(axis=-1, keepdims=True, dtype=np.float32))
-    return gx, (gy * xhat).reshape(-1, n).sum(axis=0, dtype=np.float32), gy.reshape(-1, n).sum(axis=0, dtype=np.float32)
+    t = xhat.dtype
+    gx = inv * (g - g.mean(axis=-1, keepdims=True, dtype=t) - xhat * (g * xhat).mean(axis=-1, keepdims=True, dtype=t))
+    return gx, (gy * xhat).reshape(-1, n).sum(axis=0, dtype=t), gy.reshape(-1, n).sum(axis=0, dtype=t)
 
 
 PARAMS = ("wq", "bq", "wk", "bk", "wv", "bv", "wo", "bo", "g1", "be1", "w1", "b1", "w2", "b2", "g2", "be2")
@@ -149,7 +157,7 @@ def encoder_block(be, dtype, p, x32, B, S, d, H, ff, gout):
     kv = View(k, (B, S, H, D)).permute(0, 2, 3, 1)   # (B,H,D,S)
     vv = View(v, (B, S, H, D)).permute(0, 2, 1, 3)
     scores = be.forward(qv, kv)                                           # (B,H,S,S)
-    scaled = rt(val(scores, dtype).reshape(B, H, S, S) * np.float32(1.0 / np.sqrt(D)), dtype)
+    scaled = rt(val(scores, dtype).reshape(B, H, S, S) * wt(dtype)(1.0 / np.sqrt(D)), dtype)
     probs = softmax_fwd(scaled, dtype)
     pst = st(probs, dtype)
     tokens = be.forward(View(pst, (B, H, S, S)), vv)                      # (B,H,S,D) contiguous
@@ -189,7 +197,7 @@ def encoder_block(be, dtype, p, x32, B, S, d, H, ff, gout):
     gp, gv = z(B * H * S * S), z(T * d)
     be.backward(View(pst, (B, H, S, S)), gp, vv, gv, gtokens)
     gscaled = rt(softmax_bwd(probs, val(gp, dtype).reshape(B, H, S, S)), dtype)
-    gscores = st(rt(gscaled * np.float32(1.0 / np.sqrt(D)), dtype), dtype)
+    gscores = st(rt(gscaled * wt(dtype)(1.0 / np.sqrt(D)), dtype), dtype)
     gq, gk = z(T * d), z(T * d)
     be.backward(qv, gq, kv, gk, gscores)
     gx = z(T * d)                                             # x feeds three Linears: three accumulations into one buffer

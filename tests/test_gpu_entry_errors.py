@@ -101,13 +101,15 @@ def test_layer_norm_relu_add_argument_checks():
     assert lib.dfdx_rocm_layer_norm_forward(ctx, 0, I64(-1), I64(4), p, p, p, F64(1e-5), p) == INVALID
     assert lib.dfdx_rocm_layer_norm_forward(ctx, 0, I64(2), I64(1 << 24), p, p, p, F64(1e-5), p) == INVALID
     assert lib.dfdx_rocm_layer_norm_forward(ctx, 0, I64(2), I64(4), p, VP(), p, F64(1e-5), p) == INVALID
-    assert lib.dfdx_rocm_layer_norm_forward(ctx, 3, I64(2), I64(4), p, p, p, F64(1e-5), p) == UNSUPPORTED
+    assert lib.dfdx_rocm_layer_norm_forward(ctx, 3, I64(2), I64(4), p, p, p, F64(1e-5), p) == 0             # f64 is served
+    assert lib.dfdx_rocm_layer_norm_forward(ctx, 9, I64(2), I64(4), p, p, p, F64(1e-5), p) == UNSUPPORTED   # no such element type
     assert lib.dfdx_rocm_layer_norm_forward(ctx, 0, I64(0), I64(4), VP(), VP(), VP(), F64(1e-5), VP()) == 0
     assert lib.dfdx_rocm_layer_norm_backward(ctx, 0, I64(2), I64(4), p, p, F64(1e-5), p, p, VP(), p) == INVALID
     assert lib.dfdx_rocm_layer_norm_backward(ctx, 0, I64(2), I64(0), VP(), VP(), F64(1e-5), VP(), VP(), VP(), VP()) == 0
     assert lib.dfdx_rocm_relu_forward(ctx, 0, I64(-1), p, p) == INVALID
     assert lib.dfdx_rocm_relu_forward(ctx, 0, I64(4), VP(), p) == INVALID
-    assert lib.dfdx_rocm_relu_forward(ctx, 3, I64(4), p, p) == UNSUPPORTED
+    assert lib.dfdx_rocm_relu_forward(ctx, 3, I64(4), p, p) == 0
+    assert lib.dfdx_rocm_relu_forward(ctx, 9, I64(4), p, p) == UNSUPPORTED
     assert lib.dfdx_rocm_relu_backward(ctx, 0, I64(4), p, p, VP()) == INVALID
     assert lib.dfdx_rocm_relu_forward(ctx, 0, I64(0), VP(), VP()) == 0
     assert lib.dfdx_rocm_add_forward(ctx, 0, I64(4), p, VP(), p) == INVALID
