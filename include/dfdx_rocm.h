@@ -313,8 +313,10 @@ int dfdx_rocm_scalar_mul_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, do
  * exp(t - max) / sum exp(t - max)), applied to scale * x so that attention's
  * scalar multiplication can be folded in (scale = 1 for a plain softmax).
  * The reference composes it from max / sub / exp / sum / div kernels, each
- * rounding to the element type; here a row is processed in f32 and rounded
- * once.  out may be x.  Backward of the composition, from the saved output:
+ * rounding to the element type; here a row is processed in f32 (f64 rows in
+ * f64) and rounded once.  `scale` is a float: an f64 caller whose scalar has
+ * no exact float value applies dfdx_rocm_scalar_mul_forward first and passes
+ * 1.  out may be x.  Backward of the composition, from the saved output:
  * grad_x[r][c] += scale * out[r][c] * (grad_out[r][c] - sum_j grad_out[r][j] * out[r][j]). */
 int dfdx_rocm_softmax_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t rows, int64_t cols, const void *x, float scale,
                               void *out);
