@@ -124,7 +124,21 @@ def test_linear_backward_seeded(dtype, rows, i, o):
 # gradient is produced by the same launch (one more MFMA per A fragment in the work items of tile column 0) instead of
 # by the reduction kernels.  Both tile families, split and unsplit contractions, edge tiles in either direction.
 FUSED_SHAPES = [(8192, 1024, 1024), (4096, 1024, 4096), (512, 256, 512), (640, 264, 1000), (128, 64, 8), (2048, 4096, 1024),
-                (64, 1024, 1024)]
+                (64, 1024, 1024), (2048, 128, 256), (4096, 256, 4096), (8192, 1024, 4096)]
+
+
+def test_fused_shapes_reach_every_tile_family_that_sums_rows():
+    """The weight-gradient products of FUSED_SHAPES are planned on all four LDS-DMA tiles that can carry the row sums
+    (the 256 x 64 tile serves outputs of at most 64 columns: too few tile columns to share an A tile)."""
+    dev = device()
+    seen = set()
+    probe = dev.zeros("f16", (16,))
+    for rows, i, o in FUSED_SHAPES:
+        d = dev.gemm_desc("f16", i, rows, o, probe.ptr, (1, i), probe.ptr, (o, 1), probe.ptr, (1, i), accumulate=True)
+        name = dev.gemm_plan(d)[2]
+        if "_dma_" in name and "splitk" in name:
+            seen.add(name.split("_dma_")[1].split("x64_")[0])
+    assert {"256x256", "256x128", "128x128", "128x64"} <= seen, seen
 
 
 # f32: the k-sliced small kernel produces the row sums (config 1's Linear and smaller)
