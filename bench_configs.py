@@ -124,8 +124,8 @@ def main():
                 torch.cuda.synchronize()
             print(json.dumps({"probe": names}))
         return
-    tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
-    esz = {"f16": 2, "bf16": 2, "f32": 4}
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32, "f64": torch.float64}
+    esz = {"f16": 2, "bf16": 2, "f32": 4, "f64": 8}
     only = set(filter(None, args.only.split(",")))
     rows = []
 
@@ -219,17 +219,20 @@ def main():
 
     # ---- config 1: Linear 512 -> 256 on 64 rows, f32 (latency-bound) ------------------------------------------
     if want("c1"):
-        dt, (r, i, o), es = "f32", (64, 512, 256), 4
-        x, w, go = rnd((r, i), dt), rnd((o, i), dt, 0.04), rnd((r, o), dt)
-        y, gx, gw = zeros((r, o), dt), zeros((r, i), dt), zeros((o, i), dt)
-        fl = 2 * r * i * o
-        gemm("c1", "Linear fwd 64x512x256 NT", dev.gemm_desc(dt, r, i, o, P(x), (i, 1), P(w), (1, i), P(y), (o, 1)),
-             fl, es * (r * i + i * o + r * o), 200, bufs=(x, w, y))
-        gemm("c1", "dX 64x256x512 NN acc", dev.gemm_desc(dt, r, o, i, P(go), (o, 1), P(w), (i, 1), P(gx), (i, 1), accumulate=True),
-             fl, es * (r * o + i * o + 2 * r * i), 200, bufs=(go, w, gx))
-        gemm("c1", "dW 512x64x256 TN col-major C acc",
-             dev.gemm_desc(dt, i, r, o, P(x), (1, i), P(go), (o, 1), P(gw), (1, i), accumulate=True),
-             fl, es * (r * o + r * i + 2 * i * o), 200, bufs=(x, go, gw))
+        # the configuration itself is f32; the same three products in the other element types follow it
+        for dt, es in (("f32", 4), ("f16", 2), ("bf16", 2), ("f64", 8)):
+            r, i, o = 64, 512, 256
+            tag = "" if dt == "f32" else f" [{dt}]"
+            x, w, go = rnd((r, i), dt), rnd((o, i), dt, 0.04), rnd((r, o), dt)
+            y, gx, gw = zeros((r, o), dt), zeros((r, i), dt), zeros((o, i), dt)
+            fl = 2 * r * i * o
+            gemm("c1", "Linear fwd 64x512x256 NT" + tag, dev.gemm_desc(dt, r, i, o, P(x), (i, 1), P(w), (1, i), P(y), (o, 1)),
+                 fl, es * (r * i + i * o + r * o), 200, bufs=(x, w, y))
+            gemm("c1", "dX 64x256x512 NN acc" + tag, dev.gemm_desc(dt, r, o, i, P(go), (o, 1), P(w), (i, 1), P(gx), (i, 1), accumulate=True),
+                 fl, es * (r * o + i * o + 2 * r * i), 200, bufs=(go, w, gx))
+            gemm("c1", "dW 512x64x256 TN col-major C acc" + tag,
+                 dev.gemm_desc(dt, i, r, o, P(x), (1, i), P(go), (o, 1), P(gw), (1, i), accumulate=True),
+                 fl, es * (r * o + r * i + 2 * i * o), 200, bufs=(x, go, gw))
 
     # ---- config 3: [32,512,1024] x [1024,1024], f16, broadcast rhs ---------------------------------------------
     if want("c3"):

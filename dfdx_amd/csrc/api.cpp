@@ -287,7 +287,7 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
         return DFDX_ROCM_OK;
     case DFDX_ROCM_KERNEL_MFMA: {
         int v = d->variant;
-        if (is16 && (v == 0 || v >= mfma16_dma_first_variant())) {  // LDS-DMA family: tile and split count together
+        if (is16 && (v == 0 || (v >= mfma16_dma_first_variant() && v != mfma16_small_variant()))) {  // LDS-DMA family: tile and split count together
             int dv = 0, splits = 1;
             mfma16dma_plan_split(p, ctx->compute_units, v ? v - mfma16_dma_first_variant() + 1 : 0, forced_splits, &dv, &splits);
             if (dv) {
@@ -315,11 +315,20 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
         *plan = {DFDX_ROCM_KERNEL_GEMV, 0, 1};
         return DFDX_ROCM_OK;
     }
+    // The small-product kernel where its estimate beats the family's (the f32 family weighs it among its own variants);
+    // not where the caller fixed the order of the contraction.
+    const bool may_small = forced_splits == 0 && (is16 || is64) && small_supported(p);
+    const double t_small = may_small ? small_time(p, ctx->compute_units) : 1e300;
+    const Plan small_plan = {DFDX_ROCM_KERNEL_MFMA, is16 ? mfma16_small_variant() : mfma64_small_variant(), 1};
     if (is16) {
         int dv = 0, splits = 1;
-        mfma16dma_plan_split(p, ctx->compute_units, 0, forced_splits, &dv, &splits);
+        double t_dma = 1e300;
+        mfma16dma_plan_split(p, ctx->compute_units, 0, forced_splits, &dv, &splits, &t_dma);
         if (dv) {
-            *plan = {DFDX_ROCM_KERNEL_MFMA, dv + mfma16_dma_first_variant() - 1, splits};
+            // that family's estimate ranks its own tiles and split counts; on products of a few microseconds it runs
+            // 1 - 2 us above the clock, and 8 us above it for a split plan
+            t_dma -= splits > 1 ? 6.5e-6 : 1.5e-6;
+            *plan = t_small < t_dma ? small_plan : Plan{DFDX_ROCM_KERNEL_MFMA, dv + mfma16_dma_first_variant() - 1, splits};
             return DFDX_ROCM_OK;
         }
     }
@@ -329,6 +338,13 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
         *plan = {DFDX_ROCM_KERNEL_MFMA, v,
                  is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits)
                       : is16 ? mfma16_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
+        if (may_small && t_small < (is16 ? mfma16_staged_time(p, v, plan->splits, ctx->compute_units) : mfma64_time(p, v, ctx->compute_units)))
+            *plan = small_plan;
+        return DFDX_ROCM_OK;
+    }
+    // no tiled kernel takes these strides: the small-product kernel takes any, up to the size where 16 x 16 tiles pay
+    if (may_small && (double)p.m * (double)p.n * (double)p.k <= 134217728.0) {
+        *plan = small_plan;
         return DFDX_ROCM_OK;
     }
     *plan = {DFDX_ROCM_KERNEL_GENERIC, 0, 1};
@@ -409,15 +425,19 @@ int gemm_with_colsum(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, void *
     GemmProblem p;
     if (int e = make_problem(desc, &p, colsum_b)) return e;
     if (p.m == 0) return DFDX_ROCM_OK;
-    if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
-    Plan plan;
+    Plan plan;  // from the product as the caller states it: a pending zero fill of C must not change which kernel runs
     if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
     bool can = p.ksum && plan.kernel == DFDX_ROCM_KERNEL_MFMA;
     if (can && (p.dtype == DT_F16 || p.dtype == DT_BF16))
-        can = plan.variant >= mfma16_dma_first_variant() &&
-              mfma16dma_ksum_supported(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
+        can = plan.variant == mfma16_small_variant()
+                  ? small_ksum_supported(p)
+                  : plan.variant >= mfma16_dma_first_variant() &&
+                        mfma16dma_ksum_supported(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
     else if (can && p.dtype == DT_F32)
         can = plan.splits <= 1 && mfma32_ksum_supported(p, plan.variant);
+    else if (can && p.dtype == DT_F64)
+        can = plan.variant == mfma64_small_variant() && small_ksum_supported(p);
     else
         can = false;
     if (can) {
@@ -680,9 +700,9 @@ int dfdx_rocm_gemm(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc) {
     GemmProblem p;
     if (int e = make_problem(desc, &p)) return e;
     if (p.m == 0) return DFDX_ROCM_OK;
-    if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
-    Plan plan;
+    Plan plan;  // from the product as the caller states it: a pending zero fill of C must not change which kernel runs
     if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
     return run_plan(ctx, p, plan);
 }
 
@@ -691,9 +711,9 @@ int dfdx_rocm_gemm_noalloc(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc) 
     GemmProblem p;
     if (int e = make_problem(desc, &p)) return e;
     if (p.m == 0) return DFDX_ROCM_OK;
-    if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
-    Plan plan;
+    Plan plan;  // from the product as the caller states it: a pending zero fill of C must not change which kernel runs
     if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
     return run_plan(ctx, p, plan, /*static_scratch=*/true);
 }
 
@@ -741,8 +761,8 @@ int dfdx_rocm_gemm_time_rotating(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *
             *avg_ms = 0.0f;
             return DFDX_ROCM_OK;
         }
-        if (int e = settle_operands(ctx, &problems[(size_t)i], /*may_overwrite=*/false)) return e;
         if (int e = make_plan(ctx, &descs[i], problems[(size_t)i], &plans[(size_t)i])) return e;
+        if (int e = settle_operands(ctx, &problems[(size_t)i], /*may_overwrite=*/false)) return e;
     }
     for (int i = 0; i < warmup; i++)
         if (int e = run_plan(ctx, problems[(size_t)(i % count)], plans[(size_t)(i % count)])) return e;

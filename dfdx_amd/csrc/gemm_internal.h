@@ -29,7 +29,8 @@ struct GemmProblem {
     // Optional second result, in the element type: the sums of one operand over the contraction (and over the batches
     // of a reduced product), ksum[i] (+)= sum_k A[i,k] (KSUM_OF_A, length m) or ksum[j] (+)= sum_k B[k,j] (KSUM_OF_B,
     // length n).  `Linear`'s bias gradient is the latter for the weight-gradient product x^T . grad_out.  Only some
-    // kernels produce it (mfma16dma_ksum_supported); the caller clears `ksum` and runs the reduction itself otherwise.
+    // kernels produce it (mfma16dma_ksum_supported, small_ksum_supported); the caller clears `ksum` and runs the reduction
+    // itself otherwise.
     void *ksum = nullptr;
     int ksum_of = KSUM_NONE;
     int ksum_accumulate = 0;
@@ -86,10 +87,12 @@ int mfma16_variant_count();
 const char *mfma16_variant_name(int variant);
 bool mfma16_supported(const GemmProblem &p, int variant);
 int mfma16_pick_variant(const GemmProblem &p, int compute_units);
-int mfma16_dma_first_variant();  // variant ids >= this are the LDS-DMA kernels
+int mfma16_dma_first_variant();  // variant ids >= this are the LDS-DMA kernels ...
+int mfma16_small_variant();      // ... except the last one, the small-product kernel
 // split-k of the register-staged variants (ids below mfma16_dma_first_variant)
 int mfma16_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits);
 size_t mfma16_workspace_bytes(const GemmProblem &p, int variant, int splits);
+double mfma16_staged_time(const GemmProblem &p, int variant, int splits, int compute_units);  // estimated seconds
 hipError_t launch_mfma16(const GemmProblem &p, int variant, hipStream_t stream);
 // The same product with B given as a patch matrix (`p.b` = channel 0 of the first image, b_b1 / b_b2 = image and group
 // strides, b_rs / b_cs unused): register-staged kernels only, tile chosen inside.  Returns hipErrorNotSupported when
@@ -104,9 +107,9 @@ bool mfma16dma_supported(const GemmProblem &p, int variant);
 int mfma16dma_pick_variant(const GemmProblem &p, int compute_units);
 hipError_t launch_mfma16dma(const GemmProblem &p, int variant, hipStream_t stream);
 // Split-k planning for the LDS-DMA kernels: picks tile variant and split count together.  `forced_splits`
-// > 0 overrides the count (clamped to what the k extent allows).  Returns the workspace bytes needed.
+// > 0 overrides the count (clamped to what the k extent allows).  `seconds` (may be null) receives the estimate.
 void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_variant, int forced_splits, int *variant,
-                          int *splits);
+                          int *splits, double *seconds = nullptr);
 size_t mfma16dma_workspace_bytes(const GemmProblem &p, int variant, int splits);
 bool mfma16dma_ksum_supported(const GemmProblem &p, int variant, int splits);  // can this plan also produce p.ksum?
 
@@ -130,7 +133,16 @@ int mfma64_variant_count();
 const char *mfma64_variant_name(int variant);
 bool mfma64_supported(const GemmProblem &p, int variant);
 int mfma64_pick_variant(const GemmProblem &p, int compute_units);
+int mfma64_small_variant();
+double mfma64_time(const GemmProblem &p, int variant, int compute_units);  // estimated seconds of a tiled variant
 hipError_t launch_mfma64(const GemmProblem &p, int variant, hipStream_t stream);
+
+// ---- small products in every element type (gemm_small.hip): 16 x 16 tiles, the contraction cut over the waves ----
+// Any operand strides, one product per launch, row-major C.  Each family lists it as its last variant.
+bool small_supported(const GemmProblem &p);
+bool small_ksum_supported(const GemmProblem &p);  // p.ksum of A as a second result
+double small_time(const GemmProblem &p, int compute_units);  // estimated seconds
+hipError_t launch_small(const GemmProblem &p, hipStream_t stream);
 
 // ---- bandwidth-bound vector products (gemv.hip) ----
 bool gemv_supported(const GemmProblem &p);

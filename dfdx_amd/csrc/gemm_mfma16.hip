@@ -566,14 +566,18 @@ inline bool needs_window(const GemmProblem &p, const OperandLayout &la, const Op
 
 }  // namespace
 
-// Variant ids 1..kNumVariants are the register-staged kernels of this file; higher ids are the LDS-DMA kernels.
-int mfma16_variant_count() { return kNumVariants + mfma16dma_variant_count(); }
+// Variant ids 1..kNumVariants are the register-staged kernels of this file; higher ids are the LDS-DMA kernels; the
+// last id is the small-product kernel (gemm_small.hip).
+int mfma16_small_variant() { return kNumVariants + mfma16dma_variant_count() + 1; }
+int mfma16_variant_count() { return mfma16_small_variant(); }
 const char *mfma16_variant_name(int v) {
+    if (v == mfma16_small_variant()) return "small_16x16_ksliced";
     if (v > kNumVariants) return mfma16dma_variant_name(v - kNumVariants);
     return (v >= 1) ? kVariants[v - 1].name : "?";
 }
 
 bool mfma16_supported(const GemmProblem &p, int variant) {
+    if (variant == mfma16_small_variant()) return (p.dtype == DT_F16 || p.dtype == DT_BF16) && small_supported(p);
     if (variant > kNumVariants) return mfma16dma_supported(p, variant - kNumVariants);
     if (p.dtype != DT_F16 && p.dtype != DT_BF16) return false;
     if (variant < 1) return false;
@@ -655,6 +659,21 @@ int mfma16_plan_splits(const GemmProblem &p, int variant, int compute_units, int
     return (int)s;
 }
 
+// Estimated seconds of a register-staged variant, for the comparison with the small-product kernel: a lone workgroup's
+// k tile takes 1.1 us (load -> LDS -> MFMA chain: 64 x 64 x 64 tiles measure 3.0 / 5.5 / 7.5 us for 1 / 3 / 5 k tiles),
+// a full chip runs at the variant's rate; a split adds its second launch.
+double mfma16_staged_time(const GemmProblem &p, int variant, int splits, int compute_units) {
+    if (variant < 1 || variant > kNumVariants) return 1e300;
+    const Variant &t = kVariants[variant - 1];
+    const int cus = std::max(1, compute_units);
+    const double rate[kNumVariants] = {1.0, 0.8, 0.60, 0.73, 0.54, 0.46};
+    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+    const int64_t total_iters = ((p.k + t.bk - 1) / t.bk) * (p.reduce ? p.nb1 * p.nb2 : 1);
+    const double blocks = (double)((p.m + t.bm - 1) / t.bm) * (double)((p.n + t.bn - 1) / t.bn) * (double)nbatch * splits;
+    const double step = std::max(1.1e-6, 2.0 * t.bm * t.bn * t.bk / (rate[variant - 1] * 821e12 / 256));
+    return 2.5e-6 + std::max(1.0, blocks / cus) * (double)((total_iters + splits - 1) / splits) * step + (splits > 1 ? 4e-6 : 0.0);
+}
+
 static void ws_layout16(const GemmProblem &p, int variant, int64_t *ld, int64_t *split_stride) {
     const Variant &v = kVariants[variant - 1];
     *ld = ((p.n + v.bn - 1) / v.bn) * v.bn;
@@ -669,6 +688,7 @@ size_t mfma16_workspace_bytes(const GemmProblem &p, int variant, int splits) {
 }
 
 hipError_t launch_mfma16(const GemmProblem &g, int variant, hipStream_t stream) {
+    if (variant == mfma16_small_variant()) return mfma16_supported(g, variant) ? launch_small(g, stream) : hipErrorInvalidValue;
     if (variant > kNumVariants) return launch_mfma16dma(g, variant - kNumVariants, stream);
     if (!mfma16_supported(g, variant)) return hipErrorInvalidValue;
     const Variant &v = kVariants[variant - 1];

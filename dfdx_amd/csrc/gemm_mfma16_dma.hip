@@ -1017,7 +1017,7 @@ constexpr double kSplitLaunch = 7e-6, kSplitPerPiece = 0.25e-6;  // 1024^3: 12.4
 }  // namespace
 
 void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_variant, int forced_splits, int *variant,
-                          int *splits) {
+                          int *splits, double *seconds) {
     *variant = 0;
     *splits = 1;
     const int cus = std::max(1, compute_units);
@@ -1067,6 +1067,7 @@ void mfma16dma_plan_split(const GemmProblem &p, int compute_units, int forced_va
             }
         }
     }
+    if (seconds) *seconds = best;
 }
 
 // layout of the split-k workspace: [splits][tiles_m * BM][tiles_n * BN] f32, then -- row sums of A asked for --

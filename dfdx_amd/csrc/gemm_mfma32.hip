@@ -541,114 +541,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma32_dma_kernel(
     store_tiles32<TM, TN>(p, acc, bm0, bn0, wm0, wn0, l32, lh, batch, split);
 }
 
-// ---- small products: one 16 x 16 tile of C per workgroup, the contraction cut over its waves ------------------------
-// A product of a few MFLOP (a Linear layer on 64 rows) is bound by the chain launch -> load -> MFMA -> store, not by any
-// rate: the tiled kernels above walk k in steps behind one another (9.7 us for 64 x 512 x 256 in four k pieces plus the
-// combining launch).  Here every wave of a workgroup takes one slice of k, requests ALL its operand values at once --
-// straight into the registers the MFMA reads, no LDS staging, any strides -- runs its v_mfma_f32_16x16x4 chain on two
-// accumulators, and the slices meet in LDS, added in wave order (the result does not depend on timing).  Lane l supplies
-// A[row l % 16][k] and B[k][col l % 16] for k = 16 s + 4 (l / 16) + c in MFMA c of step s: four consecutive k per lane, one
-// 16-byte load where the operand is stored along k.
-struct SmallParams {
-    const float *a, *b;
-    float *c;
-    const float *bias;
-    int m, n, k, tiles_n;
-    int64_t a_rs, a_cs, b_rs, b_cs, ldc;
-    int accumulate, bias_mode;
-    int a_vec, b_vec;  // the operand is stored along k and every 4-k group of a row is one aligned 16-byte piece
-    int slice;         // k per wave, a multiple of 16
-    // second result (may be null): ksum[i] (+)= sum_k A[i][k], produced by the workgroups of tile column 0 from the A
-    // values they hold anyway (Linear's bias gradient out of the weight-gradient launch)
-    float *ksum;
-    int ksum_accumulate;
-};
-
-template <int WAVES> __global__ __launch_bounds__(WAVES * 64) void gemm_small32_kernel(const SmallParams p) {
-    __shared__ float part[WAVES][256];
-    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-    const int r16 = lane % 16, q = lane / 16;
-    const int tm = blockIdx.x / p.tiles_n, tn = blockIdx.x % p.tiles_n;
-    const int row = tm * 16 + r16, col = tn * 16 + r16;
-    const bool row_ok = row < p.m, col_ok = col < p.n;
-    const float *ap = p.a + (int64_t)(row_ok ? row : 0) * p.a_rs;
-    const float *bp = p.b + (int64_t)(col_ok ? col : 0) * p.b_cs;
-    const int k0 = wave * p.slice, k1 = min(p.k, k0 + p.slice);
-    auto fetch = [&](const float *base, int64_t kstride, bool ok, bool vec, int kk) -> f32x4 {
-        f32x4 v = {0.f, 0.f, 0.f, 0.f};
-        if (!ok || kk >= k1) return v;
-        if (vec && kk + 3 < k1) return *(const f32x4 *)(base + kk);
-#pragma unroll
-        for (int c = 0; c < 4; c++)
-            if (kk + c < k1) v[c] = base[(int64_t)(kk + c) * kstride];
-        return v;
-    };
-    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-    const bool sums = p.ksum && tn == 0;
-    float rsum = 0.0f;  // of A[row r16][this lane's k values]
-    for (int kb = k0; kb < k1; kb += 64) {  // four steps of 16 k per pass: 8 loads in flight per lane
-        f32x4 av[4], bv[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            av[u] = fetch(ap, p.a_cs, row_ok, p.a_vec, kb + 16 * u + 4 * q);
-            bv[u] = fetch(bp, p.b_rs, col_ok, p.b_vec, kb + 16 * u + 4 * q);
-        }
-        if (sums) {
-#pragma unroll
-            for (int u = 0; u < 4; u++) rsum += (av[u][0] + av[u][1]) + (av[u][2] + av[u][3]);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; u++)
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                if (u % 2 == 0) acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u][c], bv[u][c], acc0, 0, 0, 0);
-                else acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u][c], bv[u][c], acc1, 0, 0, 0);
-            }
-    }
-    // lane l, register r: C[tm * 16 + 4 * (l / 16) + r][tn * 16 + l % 16]
-    f32x4 sum = acc0 + acc1;
-    __shared__ float part_rows[WAVES][16];
-    if (sums) {  // uniform over the workgroup
-        rsum += __shfl_xor(rsum, 16, 64);
-        rsum += __shfl_xor(rsum, 32, 64);
-        if (lane < 16) part_rows[wave][lane] = rsum;
-    }
-    if constexpr (WAVES > 1) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) part[wave][r * 64 + lane] = sum[r];
-        __syncthreads();
-        if (wave != 0) return;
-        sum = f32x4{part[0][lane], part[0][64 + lane], part[0][128 + lane], part[0][192 + lane]};
-#pragma unroll
-        for (int w = 1; w < WAVES; w++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) sum[r] += part[w][r * 64 + lane];
-    }
-    if (sums && lane < 16 && row_ok) {  // slices in wave order, then the old value unless the gradient is fresh
-        float v = part_rows[0][lane];
-#pragma unroll
-        for (int w = 1; w < WAVES; w++) v += part_rows[w][lane];
-        p.ksum[row] = (p.ksum_accumulate ? p.ksum[row] : 0.0f) + v;
-    }
-    if (!col_ok) return;
-    const float cb = p.bias_mode == BIAS_PER_COL ? p.bias[col] : 0.0f;
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int orow = tm * 16 + 4 * q + r;
-        if (orow >= p.m) break;
-        float *dst = p.c + (int64_t)orow * p.ldc + col;
-        float v = sum[r] + cb;
-        if (p.bias_mode == BIAS_PER_ROW) v += p.bias[orow];
-        if (p.accumulate) v += *dst;
-        *dst = v;
-    }
-}
-
 struct Variant {
     const char *name;
     int bm, bn, bk, waves_m, waves_n;
     bool dma;    // the LDS-DMA form: aligned operands, K % 32 == 0
-    bool small;  // the 16 x 16 tile with the contraction cut over the waves (any strides, no batch)
+    bool small;  // the 16 x 16 tile with the contraction cut over the waves (gemm_small.hip: any strides, no batch)
 };
 constexpr Variant kVariants[] = {
     {"256x256x32_w2x4", 256, 256, 32, 2, 4, false},
@@ -744,8 +641,7 @@ inline bool needs_window(const GemmProblem &p, const OperandLayout &la, const Op
 
 int mfma32_variant_count() { return kNumVariants; }
 bool mfma32_ksum_supported(const GemmProblem &p, int variant) {
-    return p.ksum && p.ksum_of == KSUM_OF_A && variant >= 1 && variant <= kNumVariants && kVariants[variant - 1].small &&
-           mfma32_supported(p, variant) && ((uintptr_t)p.ksum & 3u) == 0;
+    return variant >= 1 && variant <= kNumVariants && kVariants[variant - 1].small && p.dtype == DT_F32 && small_ksum_supported(p);
 }
 const char *mfma32_variant_name(int v) { return (v >= 1 && v <= kNumVariants) ? kVariants[v - 1].name : "?"; }
 
@@ -756,11 +652,7 @@ bool mfma32_supported(const GemmProblem &p, int variant) {
     if (p.m > (1 << 30) || p.n > (1 << 30) || p.k > (1 << 30)) return false;
     if (p.c_cs != 1 && p.n != 1) return false;
     if (p.n > 1 && p.m > 1 && p.c_rs < p.n) return false;
-    if (kVariants[variant - 1].small) {  // any operand strides; one product per launch; a grid of 16 x 16 tiles
-        if (p.nb1 * p.nb2 != 1) return false;
-        if (((uintptr_t)p.a | (uintptr_t)p.b | (uintptr_t)p.c) & 3u) return false;
-        return ((p.m + 15) / 16) * ((p.n + 15) / 16) < (1ll << 20);
-    }
+    if (kVariants[variant - 1].small) return small_supported(p);
     const OperandLayout la = classify(p.m, p.k, p.a_rs, p.a_cs);
     const OperandLayout lb = classify(p.n, p.k, p.b_cs, p.b_rs);
     if (!la.ok || !lb.ok) return false;
@@ -789,21 +681,9 @@ constexpr int kPerCu32[kNumVariants] = {1, 1, 1, 2, 2, 4, 1, 1};  // workgroups 
 constexpr double kCuFlops32 = 130e12 / 256, kSplitLaunch32 = 2.5e-6, kWorkspaceBw32 = 4.5e12;
 constexpr double kStepLatency32 = 1.0e-6;  // a k step of a lone small workgroup is bound by its load -> LDS -> MFMA chain
 
-// waves per workgroup of the small kernel: slices of at least 32 k
-int small_waves(int64_t k) { return k >= 256 ? 8 : k >= 128 ? 4 : k >= 64 ? 2 : 1; }
-
 double plan_time32(const GemmProblem &p, int v, int64_t s, int compute_units) {
     const Variant &t = kVariants[v - 1];
-    if (t.small) {
-        // one launch; a compute unit holds 2048 / (64 * waves) workgroups at once, each of which spends about a
-        // microsecond on its load round trip and 0.1 us per 16 k of its slice; no operand value is shared between
-        // workgroups, so every tile pulls its 16 rows and 16 columns through the caches again
-        const int waves = small_waves(p.k);
-        const int64_t tiles = ((p.m + 15) / 16) * ((p.n + 15) / 16);
-        const double held = (double)std::max(1, compute_units) * (32 / waves);
-        const double per_wg = 1.0e-6 + 0.1e-6 * (double)((p.k / waves + 15) / 16);
-        return 3.0e-6 + std::max(1.0, (double)tiles / held) * per_wg + (double)tiles * 128.0 * (double)p.k / 10e12;
-    }
+    if (t.small) return small_time(p, compute_units);
     const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
     const int64_t total_iters = ((p.k + t.bk - 1) / t.bk) * (p.reduce ? p.nb1 * p.nb2 : 1);
     const int64_t items = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn) * nbatch * s;
@@ -882,30 +762,6 @@ int mfma32_pick_variant(const GemmProblem &p, int compute_units, int forced_spli
 }
 
 static hipError_t launch_tiles(const Params &p, int variant, bool a_kc, bool b_kc, hipStream_t stream);
-
-static hipError_t launch_small(const GemmProblem &g, hipStream_t stream) {
-    SmallParams p;
-    p.a = (const float *)g.a; p.b = (const float *)g.b; p.c = (float *)g.c; p.bias = (const float *)g.bias;
-    p.m = (int)g.m; p.n = (int)g.n; p.k = (int)g.k;
-    p.tiles_n = (int)((g.n + 15) / 16);
-    p.a_rs = g.a_rs; p.a_cs = g.a_cs; p.b_rs = g.b_rs; p.b_cs = g.b_cs;
-    p.ldc = g.m == 1 ? g.n : g.c_rs;
-    p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
-    p.a_vec = g.a_cs == 1 && (g.m == 1 || g.a_rs % 4 == 0) && aligned16(g.a);
-    p.b_vec = g.b_rs == 1 && (g.n == 1 || g.b_cs % 4 == 0) && aligned16(g.b);
-    p.ksum = (g.ksum && g.ksum_of == KSUM_OF_A) ? (float *)g.ksum : nullptr;
-    p.ksum_accumulate = g.ksum_accumulate;
-    const int waves = small_waves(g.k);
-    p.slice = (int)(((g.k + waves - 1) / waves + 15) / 16 * 16);
-    const dim3 grid((unsigned)(((g.m + 15) / 16) * p.tiles_n));
-    switch (waves) {
-    case 8: gemm_small32_kernel<8><<<grid, 512, 0, stream>>>(p); break;
-    case 4: gemm_small32_kernel<4><<<grid, 256, 0, stream>>>(p); break;
-    case 2: gemm_small32_kernel<2><<<grid, 128, 0, stream>>>(p); break;
-    default: gemm_small32_kernel<1><<<grid, 64, 0, stream>>>(p); break;
-    }
-    return hipGetLastError();
-}
 
 hipError_t launch_mfma32(const GemmProblem &g, int variant, hipStream_t stream) {
     if (!mfma32_supported(g, variant)) return hipErrorInvalidValue;

@@ -13,6 +13,7 @@
 // Lane l of a wave supplies A[row l % 16][k = l / 16] and B[k = l / 16][col l % 16] and receives, in register r of a
 // tile, C[row 4 * r + l / 16][col l % 16].
 #include "gemm_internal.h"
+#include <algorithm>
 
 namespace dfdx_rocm {
 namespace {
@@ -200,12 +201,18 @@ template <int BM, int BN, int WM, int WN> hipError_t launch_layout(const Params 
 
 }  // namespace
 
-int mfma64_variant_count() { return kNumVariants; }
-const char *mfma64_variant_name(int v) { return (v >= 1 && v <= kNumVariants) ? kVariants[v - 1].name : "?"; }
+// The last id is the small-product kernel (gemm_small.hip).
+int mfma64_small_variant() { return kNumVariants + 1; }
+int mfma64_variant_count() { return mfma64_small_variant(); }
+const char *mfma64_variant_name(int v) {
+    if (v == mfma64_small_variant()) return "small_16x16_ksliced";
+    return (v >= 1 && v <= kNumVariants) ? kVariants[v - 1].name : "?";
+}
 
 // Row-major C (unit column stride); the operands may have any non-negative strides (every access is one element; the
 // unit-stride axis only decides which access pattern coalesces).
 bool mfma64_supported(const GemmProblem &p, int variant) {
+    if (variant == mfma64_small_variant()) return p.dtype == DT_F64 && small_supported(p);
     if (p.dtype != DT_F64 || variant < 1 || variant > kNumVariants) return false;
     if (p.m < 1 || p.n < 1 || p.k < 1 || p.m >= (1 << 30) || p.n >= (1 << 30) || p.k >= (1 << 30)) return false;
     if (p.c_cs != 1 && p.n != 1) return false;
@@ -228,8 +235,23 @@ int mfma64_pick_variant(const GemmProblem &p, int compute_units) {
     return big * 2 >= compute_units ? 1 : 2;
 }
 
+// Estimated seconds of a tiled variant, for the comparison with the small-product kernel: a k tile of 16 takes a lone
+// workgroup 1.25 us (64 x 64 tiles measure 9 / 14 / 24 / 44 / 84 us for k = 64 ... 1024), or its flops at the compute
+// unit's share of 50 TFLOP/s once that is more.
+double mfma64_time(const GemmProblem &p, int variant, int compute_units) {
+    if (variant < 1 || variant > kNumVariants) return 1e300;
+    const Variant &t = kVariants[variant - 1];
+    const int cus = std::max(1, compute_units);
+    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+    const double blocks = (double)((p.m + t.bm - 1) / t.bm) * (double)((p.n + t.bn - 1) / t.bn) * (double)nbatch;
+    const double steps = (double)((p.k + 15) / 16) * (double)(p.reduce ? p.nb1 * p.nb2 : 1);
+    const double step = std::max(1.25e-6, 2.0 * t.bm * t.bn * 16 / (50e12 / 256));
+    return 4e-6 + std::max(1.0, blocks / cus) * steps * step;
+}
+
 hipError_t launch_mfma64(const GemmProblem &g, int variant, hipStream_t stream) {
     if (!mfma64_supported(g, variant)) return hipErrorInvalidValue;
+    if (variant == mfma64_small_variant()) return launch_small(g, stream);
     const Variant &v = kVariants[variant - 1];
     Params p;
     p.a = (const double *)g.a; p.b = (const double *)g.b; p.c = (double *)g.c; p.bias = (const double *)g.bias;

@@ -1,0 +1,316 @@
+// Small products in every element type: one 16 x 16 tile of C per workgroup, the contraction cut over its waves.
+//
+// A product of a few MFLOP (a Linear layer on 64 rows, the reference's own test shapes) is bound by the chain
+// launch -> load -> MFMA -> store, not by any rate, and the tiled kernels walk k in steps behind one another (9.7 us for
+// f32 64 x 512 x 256 as four k pieces plus the combining launch).  Here every wave of a workgroup takes one slice of k,
+// requests ALL the operand values of a pass at once -- straight into the registers the MFMA reads, no LDS staging, any
+// strides -- runs its MFMA chain on two accumulators, and the slices meet in LDS, added in wave order (the result does
+// not depend on timing).  Lane l supplies A[row l % 16][k] and B[k][col l % 16] for the four consecutive
+// k = 16 s + 4 (l / 16) + c, c < 4, of step s: one vector load where the operand is stored along k and aligned.  The
+// 16-bit types feed the four values to one v_mfma_f32_16x16x16, f32 and f64 to four v_mfma_*_16x16x4 (whose lane group
+// l / 16 is the k index: any bijection between (lane group, instruction) and k serves, as long as A and B share it).
+//
+// Optional second result: the sums of A's rows over k, from the values the workgroups of tile column 0 hold anyway
+// (Linear's bias gradient out of the weight-gradient launch).
+#include "gemm_internal.h"
+#include <algorithm>
+
+namespace dfdx_rocm {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct SmallParams {
+    const void *a, *b;
+    void *c;
+    const void *bias;
+    int m, n, k, tiles_n;
+    int64_t a_rs, a_cs, b_rs, b_cs, ldc;
+    int accumulate, bias_mode;
+    int a_vec, b_vec;  // the operand is stored along k and every 4-k group of a row is one aligned vector
+    int slice;         // k per wave, a multiple of 16
+    void *ksum;        // may be null: ksum[i] (+)= sum_k A[i][k]
+    int ksum_accumulate;
+};
+
+// Per element type: the accumulator type, four k-values of one row as the MFMA wants them, the MFMA step, and which row
+// of the 16 x 16 tile register r of lane l holds.
+template <typename T> struct Small;
+template <> struct Small<float> {
+    typedef float acc_t;
+    typedef f32x4 acc4;
+    typedef f32x4 pack;
+    static __device__ __forceinline__ pack zero() { return pack{0.f, 0.f, 0.f, 0.f}; }
+    static __device__ __forceinline__ pack vec(const float *p) { return *(const f32x4 *)p; }
+    static __device__ __forceinline__ void set(pack &v, int c, const float *p) { v[c] = *p; }
+    static __device__ __forceinline__ acc4 mma(pack a, pack b, acc4 acc) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[c], b[c], acc, 0, 0, 0);
+        return acc;
+    }
+    static __device__ __forceinline__ float sum4(pack v) { return (v[0] + v[1]) + (v[2] + v[3]); }
+    static __device__ __forceinline__ int out_row(int r, int q) { return 4 * q + r; }
+    static __device__ __forceinline__ float load(const float *p) { return *p; }
+    static __device__ __forceinline__ void store(float *p, float v) { *p = v; }
+};
+template <> struct Small<double> {
+    typedef double acc_t;
+    typedef f64x4 acc4;
+    typedef f64x4 pack;
+    static __device__ __forceinline__ pack zero() { return pack{0.0, 0.0, 0.0, 0.0}; }
+    static __device__ __forceinline__ pack vec(const double *p) {
+        typedef double f64x2 __attribute__((ext_vector_type(2)));
+        const f64x2 lo = *(const f64x2 *)p, hi = *(const f64x2 *)(p + 2);
+        return pack{lo[0], lo[1], hi[0], hi[1]};
+    }
+    static __device__ __forceinline__ void set(pack &v, int c, const double *p) { v[c] = *p; }
+    static __device__ __forceinline__ acc4 mma(pack a, pack b, acc4 acc) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc = __builtin_amdgcn_mfma_f64_16x16x4f64(a[c], b[c], acc, 0, 0, 0);
+        return acc;
+    }
+    static __device__ __forceinline__ double sum4(pack v) { return (v[0] + v[1]) + (v[2] + v[3]); }
+    static __device__ __forceinline__ int out_row(int r, int q) { return 4 * r + q; }  // f64: register r is row 4 r + l / 16
+    static __device__ __forceinline__ double load(const double *p) { return *p; }
+    static __device__ __forceinline__ void store(double *p, double v) { *p = v; }
+};
+template <> struct Small<_Float16> {
+    typedef float acc_t;
+    typedef f32x4 acc4;
+    typedef f16x4 pack;
+    static __device__ __forceinline__ pack zero() { return pack{0, 0, 0, 0}; }
+    static __device__ __forceinline__ pack vec(const _Float16 *p) { return *(const f16x4 *)p; }
+    static __device__ __forceinline__ void set(pack &v, int c, const _Float16 *p) { v[c] = *p; }
+    static __device__ __forceinline__ acc4 mma(pack a, pack b, acc4 acc) { return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, acc, 0, 0, 0); }
+    static __device__ __forceinline__ float sum4(pack v) { return ((float)v[0] + (float)v[1]) + ((float)v[2] + (float)v[3]); }
+    static __device__ __forceinline__ int out_row(int r, int q) { return 4 * q + r; }
+    static __device__ __forceinline__ float load(const _Float16 *p) { return (float)*p; }
+    static __device__ __forceinline__ void store(_Float16 *p, float v) { *p = (_Float16)v; }
+};
+template <> struct Small<__bf16> {
+    typedef float acc_t;
+    typedef f32x4 acc4;
+    typedef i16x4 pack;
+    static __device__ __forceinline__ float widen(short b) { return __uint_as_float((uint32_t)(uint16_t)b << 16); }
+    static __device__ __forceinline__ pack zero() { return pack{0, 0, 0, 0}; }
+    static __device__ __forceinline__ pack vec(const __bf16 *p) { return *(const i16x4 *)p; }
+    static __device__ __forceinline__ void set(pack &v, int c, const __bf16 *p) { v[c] = *(const short *)p; }
+    static __device__ __forceinline__ acc4 mma(pack a, pack b, acc4 acc) { return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, acc, 0, 0, 0); }
+    static __device__ __forceinline__ float sum4(pack v) { return (widen(v[0]) + widen(v[1])) + (widen(v[2]) + widen(v[3])); }
+    static __device__ __forceinline__ int out_row(int r, int q) { return 4 * q + r; }
+    static __device__ __forceinline__ float load(const __bf16 *p) { return widen(*(const short *)p); }
+    static __device__ __forceinline__ void store(__bf16 *p, float v) {  // round to nearest even, quiet NaNs
+        const uint32_t x = __float_as_uint(v);
+        *(uint16_t *)p = ((x & 0x7fffffffu) > 0x7f800000u) ? (uint16_t)((x >> 16) | 0x40u) : (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
+    }
+};
+
+template <typename T, int WAVES> __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(const SmallParams p) {
+    typedef Small<T> S;
+    typedef typename S::acc_t A;
+    typedef typename S::acc4 A4;
+    typedef typename S::pack Pack;
+    __shared__ A part[WAVES][256];
+    __shared__ A part_rows[WAVES][16];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int r16 = lane % 16, q = lane / 16;
+    const int tm = blockIdx.x / p.tiles_n, tn = blockIdx.x % p.tiles_n;
+    const int row = tm * 16 + r16, col = tn * 16 + r16;
+    const bool row_ok = row < p.m, col_ok = col < p.n;
+    const T *ap = (const T *)p.a + (int64_t)(row_ok ? row : 0) * p.a_rs;
+    const T *bp = (const T *)p.b + (int64_t)(col_ok ? col : 0) * p.b_cs;
+    const int k0 = wave * p.slice, k1 = min(p.k, k0 + p.slice);
+    // Four k values of a pass that the slice's end cuts: every lane loads from an address inside the slice and the values
+    // beyond the end (or of a row / column beyond m / n) are replaced by zeros afterwards -- no branch per value, so all
+    // the loads of a pass are in flight together.
+    auto fetch = [&](const T *base, int64_t kstride, bool ok, bool vec, int kk) -> Pack {
+        if (vec && kk + 3 < k1) return ok ? S::vec(base + kk) : S::zero();
+        Pack v = S::zero();
+        const Pack z = S::zero();
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            S::set(v, c, base + (int64_t)max(0, min(kk + c, k1 - 1)) * kstride);
+            if (!ok || kk + c >= k1) v[c] = z[c];
+        }
+        return v;
+    };
+    A4 acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+    const bool sums = p.ksum && tn == 0;
+    A rsum = 0;  // of A[row r16][this lane's k values]
+    // Passes of four steps of 16 k (8 loads per lane each), the loads of the next pass in flight behind the MFMAs of this
+    // one (not f64).
+    Pack av[4], bv[4], an[4], bn[4];
+    // A pass that lies inside the slice is loaded without a test per value: the rows and columns beyond m and n read
+    // row / column 0 (their results are never stored), and the branches on the layout are the same for the whole launch.
+    auto whole = [&](const T *base, int64_t kstride, bool vec, int kk) -> Pack {
+        if (vec) return S::vec(base + kk);
+        Pack v = S::zero();
+#pragma unroll
+        for (int c = 0; c < 4; c++) S::set(v, c, base + (int64_t)(kk + c) * kstride);
+        return v;
+    };
+    auto load_pass = [&](Pack *a, Pack *b, int kb) {
+        if (kb + 64 <= k1) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                a[u] = whole(ap, p.a_cs, p.a_vec, kb + 16 * u + 4 * q);
+                b[u] = whole(bp, p.b_rs, p.b_vec, kb + 16 * u + 4 * q);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                a[u] = fetch(ap, p.a_cs, row_ok, p.a_vec, kb + 16 * u + 4 * q);
+                b[u] = fetch(bp, p.b_rs, col_ok, p.b_vec, kb + 16 * u + 4 * q);
+            }
+        }
+    };
+    auto use_pass = [&](const Pack *a, const Pack *b) {
+        if (sums) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) rsum += S::sum4(a[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (u % 2 == 0) acc0 = S::mma(a[u], b[u], acc0);
+            else acc1 = S::mma(a[u], b[u], acc1);
+        }
+    };
+    if constexpr (sizeof(T) < 8) {
+        load_pass(av, bv, k0);
+        for (int kb = k0; kb < k1; kb += 128) {  // k0, k1 and kb are the same in every lane of a wave
+            if (kb + 64 < k1) load_pass(an, bn, kb + 64);
+            use_pass(av, bv);
+            if (kb + 64 < k1) {
+                if (kb + 128 < k1) load_pass(av, bv, kb + 128);
+                use_pass(an, bn);
+            }
+        }
+    } else {  // f64: two passes of operands would halve the waves a compute unit holds
+        for (int kb = k0; kb < k1; kb += 64) {
+            load_pass(av, bv, kb);
+            use_pass(av, bv);
+        }
+    }
+    A4 sum = acc0 + acc1;
+    if (sums) {  // uniform over the workgroup
+        rsum += __shfl_xor(rsum, 16, 64);
+        rsum += __shfl_xor(rsum, 32, 64);
+        if (lane < 16) part_rows[wave][lane] = rsum;
+    }
+    if constexpr (WAVES > 1) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) part[wave][r * 64 + lane] = sum[r];
+        __syncthreads();
+        if (wave != 0) return;
+        sum = A4{part[0][lane], part[0][64 + lane], part[0][128 + lane], part[0][192 + lane]};
+#pragma unroll
+        for (int w = 1; w < WAVES; w++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) sum[r] += part[w][r * 64 + lane];
+    }
+    if (sums && lane < 16 && row_ok) {  // slices in wave order, then the old value unless the gradient is fresh
+        A v = part_rows[0][lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) v += part_rows[w][lane];
+        T *dst = (T *)p.ksum + row;
+        S::store(dst, (p.ksum_accumulate ? S::load(dst) : A(0)) + v);
+    }
+    if (!col_ok) return;
+    const A cb = p.bias_mode == BIAS_PER_COL ? S::load((const T *)p.bias + col) : A(0);
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int orow = tm * 16 + S::out_row(r, q);
+        if (orow >= p.m) continue;
+        T *dst = (T *)p.c + (int64_t)orow * p.ldc + col;
+        A v = sum[r] + cb;
+        if (p.bias_mode == BIAS_PER_ROW) v += S::load((const T *)p.bias + orow);
+        if (p.accumulate) v += S::load(dst);
+        S::store(dst, v);
+    }
+}
+
+inline size_t elem_size(int dt) { return dt == DT_F64 ? 8 : dt == DT_F32 ? 4 : 2; }
+// waves per workgroup: slices of at least 32 k; sixteen once each of them has two passes to overlap (not f64, whose two
+// passes of operands fill the 128 registers a lane of such a workgroup may have)
+inline int small_waves(int dtype, int64_t k) {
+    return (k >= 2048 && dtype != DT_F64) ? 16 : k >= 256 ? 8 : k >= 128 ? 4 : k >= 64 ? 2 : 1;
+}
+
+template <typename T> hipError_t launch_t(const SmallParams &p, int waves, dim3 grid, hipStream_t stream) {
+    switch (waves) {
+    case 16:
+        if constexpr (sizeof(T) < 8) gemm_small_kernel<T, 16><<<grid, 1024, 0, stream>>>(p);
+        else return hipErrorInvalidValue;
+        break;
+    case 8: gemm_small_kernel<T, 8><<<grid, 512, 0, stream>>>(p); break;
+    case 4: gemm_small_kernel<T, 4><<<grid, 256, 0, stream>>>(p); break;
+    case 2: gemm_small_kernel<T, 2><<<grid, 128, 0, stream>>>(p); break;
+    default: gemm_small_kernel<T, 1><<<grid, 64, 0, stream>>>(p); break;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool small_supported(const GemmProblem &p) {
+    if (p.dtype < DT_F32 || p.dtype > DT_F64) return false;
+    if (p.m < 1 || p.n < 1 || p.k < 1 || p.k >= (1ll << 30)) return false;
+    if (p.c_cs != 1 && p.n != 1) return false;
+    if (p.n > 1 && p.m > 1 && p.c_rs < p.n) return false;
+    if (p.nb1 * p.nb2 != 1) return false;  // one product per launch
+    const uintptr_t mask = elem_size(p.dtype) - 1;
+    if (((uintptr_t)p.a | (uintptr_t)p.b | (uintptr_t)p.c | (uintptr_t)p.bias) & mask) return false;
+    return ((p.m + 15) / 16) * ((p.n + 15) / 16) < (1ll << 20);
+}
+
+bool small_ksum_supported(const GemmProblem &p) {
+    return p.ksum && p.ksum_of == KSUM_OF_A && small_supported(p) && ((uintptr_t)p.ksum & (elem_size(p.dtype) - 1)) == 0;
+}
+
+// Estimated time, fitted to timings on a 256-CU MI355X: the launch; the chain of loads of one workgroup, which grows
+// with the whole contraction however many waves share it (3.4 ns per k, twice that for f64: the 16 rows of a load
+// instruction lie a row stride apart); an operand that is not stored along k costs a 2- or 4-byte load per value; and
+// no operand value is shared between workgroups, so every tile pulls its 16 rows and 16 columns through the caches again
+// (5 - 8 TB/s over the whole chip).
+double small_time(const GemmProblem &p, int compute_units) {
+    const double tiles = (double)((p.m + 15) / 16) * (double)((p.n + 15) / 16);
+    const double es = (double)elem_size(p.dtype);
+    const double chain = std::max(0.5e-6, (double)p.k * (p.dtype == DT_F64 ? 6.8e-9 : 3.4e-9));
+    const double gather = p.dtype == DT_F64 ? 0.0 : (p.dtype == DT_F32 ? 0.4e-6 : 0.9e-6) * ((p.a_cs != 1) + (p.b_rs != 1));
+    const double bandwidth = (p.dtype == DT_F64 ? 8e12 : p.dtype == DT_F32 ? 7.5e12 : 5e12) * std::max(1, compute_units) / 256.0;
+    return 2.1e-6 + chain + gather + tiles * 32.0 * es * (double)p.k / bandwidth;
+}
+
+hipError_t launch_small(const GemmProblem &g, hipStream_t stream) {
+    if (!small_supported(g) || g.splits > 1) return hipErrorInvalidValue;
+    const size_t es = elem_size(g.dtype);
+    const uintptr_t vmask = 4 * es >= 16 ? 15 : 4 * es - 1;  // four elements: 8 bytes (16-bit), 16 bytes (f32; f64 as two halves)
+    SmallParams p;
+    p.a = g.a; p.b = g.b; p.c = g.c; p.bias = g.bias;
+    p.m = (int)g.m; p.n = (int)g.n; p.k = (int)g.k;
+    p.tiles_n = (int)((g.n + 15) / 16);
+    p.a_rs = g.a_rs; p.a_cs = g.a_cs; p.b_rs = g.b_rs; p.b_cs = g.b_cs;
+    p.ldc = g.m == 1 ? g.n : g.c_rs;
+    p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
+    const int64_t vq = (int64_t)((vmask + 1) / es);  // row stride must keep the vectors aligned
+    p.a_vec = g.a_cs == 1 && (g.m == 1 || g.a_rs % vq == 0) && ((uintptr_t)g.a & vmask) == 0;
+    p.b_vec = g.b_rs == 1 && (g.n == 1 || g.b_cs % vq == 0) && ((uintptr_t)g.b & vmask) == 0;
+    p.ksum = (g.ksum && g.ksum_of == KSUM_OF_A) ? g.ksum : nullptr;
+    p.ksum_accumulate = g.ksum_accumulate;
+    const int waves = small_waves(g.dtype, g.k);
+    p.slice = (int)(((g.k + waves - 1) / waves + 15) / 16 * 16);
+    const dim3 grid((unsigned)(((g.m + 15) / 16) * p.tiles_n));
+    switch (g.dtype) {
+    case DT_F32: return launch_t<float>(p, waves, grid, stream);
+    case DT_F16: return launch_t<_Float16>(p, waves, grid, stream);
+    case DT_BF16: return launch_t<__bf16>(p, waves, grid, stream);
+    case DT_F64: return launch_t<double>(p, waves, grid, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace dfdx_rocm

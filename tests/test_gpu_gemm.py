@@ -88,13 +88,16 @@ def test_generic_k_zero_and_empty():
 
 
 def test_doubly_strided_operand_takes_generic_path():
-    """Neither stride is 1 (reachable through user permutes/slices): Cuda panics there (mod.rs:323), Cpu does not.  16-bit
-    products take the generic kernel; a small f32 product takes the k-sliced 16 x 16 kernel, which reads its operands
-    element by element and accepts any strides; a large f32 one the generic kernel again."""
+    """Neither stride is 1 (reachable through user permutes/slices): Cuda panics there (mod.rs:323), Cpu does not.  A small
+    product takes the k-sliced 16 x 16 kernel, which reads such an operand element by element and accepts any strides; a
+    large one the generic kernel."""
     dev = device()
     g = rng(5)
-    for dtype, (m, k, n), family, kernel_name in (("f16", (40, 24, 16), KERNEL_GENERIC, "generic"),
+    for dtype, (m, k, n), family, kernel_name in (("f16", (40, 24, 16), KERNEL_MFMA, "mfma16_small_16x16_ksliced"),
+                                                  ("bf16", (40, 24, 16), KERNEL_MFMA, "mfma16_small_16x16_ksliced"),
                                                   ("f32", (40, 24, 16), KERNEL_MFMA, "mfma32_small_16x16_ksliced"),
+                                                  ("f64", (40, 24, 16), KERNEL_MFMA, "mfma64_small_16x16_ksliced"),
+                                                  ("f16", (600, 520, 440), KERNEL_GENERIC, "generic"),
                                                   ("f32", (600, 520, 440), KERNEL_GENERIC, "generic")):
         a = oracle.to_storage(g.standard_normal(m * (2 * k + 3)), dtype)
         astr = (2 * k + 3, 2)
@@ -167,17 +170,27 @@ def test_mfma_column_major_c(dtype, layout):
     run_case(dtype, 264, 72, 136, layout, True, KERNEL_MFMA, 0, c_colmajor=True, pads=(0, 8, 8))
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16", "f64"])
 @pytest.mark.parametrize("layout", list(LAYOUTS))
-def test_small_f32_kernel_tails_bias_and_wave_counts(layout):
-    """The 16 x 16 kernel that cuts k over the waves of a workgroup: extents that are no multiple of 16 or 4 in any
-    direction, every wave count (k = 20 .. 600: 1, 2, 4, 8 slices), bias per column and (column-major C) per row, beta = 1,
-    padded rows (vector loads off / on).  Config 1's three products take it on their own."""
+def test_small_kernel_tails_bias_and_wave_counts(layout, dtype):
+    """The 16 x 16 kernel that cuts k over the waves of a workgroup, the last variant of every family: extents that are no
+    multiple of 16 or 4 in any direction, every wave count (k = 20 .. 4096: 1, 2, 4, 8, 16 slices, one to four passes each), bias per column and
+    (column-major C) per row, beta = 1, padded rows (vector loads off / on)."""
     dev = device()
-    small = dev.mfma_variant_count("f32")
-    for i, (m, k, n) in enumerate([(64, 512, 256), (19, 20, 35), (33, 70, 17), (50, 131, 49), (16, 600, 16), (1, 77, 5), (130, 258, 3)]):
+    small = dev.mfma_variant_count(dtype)
+    t = dev.zeros(dtype, (16, 16))
+    assert dev.gemm_plan(dev.gemm_desc(dtype, 16, 16, 16, t.ptr, (16, 1), t.ptr, (16, 1), t.ptr, (16, 1), kernel=KERNEL_MFMA,
+                                       variant=small))[2].endswith("small_16x16_ksliced")
+    for i, (m, k, n) in enumerate([(64, 512, 256), (19, 20, 35), (33, 70, 17), (50, 131, 49), (16, 600, 16), (1, 77, 5), (130, 258, 3),
+                                   (20, 2100, 18), (17, 4096, 33)]):
         for pads in ((0, 0, 0), (3, 1, 5), (8, 4, 4)):
-            run_case("f32", m, k, n, layout, bool(i % 2), KERNEL_MFMA, small, bias=(i % 3 == 0), c_colmajor=(i % 3 == 1 and n > 1),
+            run_case(dtype, m, k, n, layout, bool(i % 2), KERNEL_MFMA, small, bias=(i % 3 == 0), c_colmajor=(i % 3 == 1 and n > 1),
                      seed=60 + i, pads=pads)
+
+
+def test_small_f32_products_plan_the_small_kernel():
+    """Config 1's three products take the small kernel on their own; a caller that asks for the plain k order does not."""
+    dev = device()
     x, w, y = dev.tensor(np.zeros(64 * 512, np.float32), "f32"), dev.tensor(np.zeros(256 * 512, np.float32), "f32"), dev.tensor(np.zeros(64 * 256, np.float32), "f32")
     for desc in (dev.gemm_desc("f32", 64, 512, 256, x.ptr, (512, 1), w.ptr, (1, 512), y.ptr, (256, 1)),
                  dev.gemm_desc("f32", 64, 256, 512, y.ptr, (256, 1), w.ptr, (512, 1), x.ptr, (512, 1), accumulate=True),
@@ -230,7 +243,9 @@ def test_auto_dispatch_prefers_mfma_when_aligned():
     d = dev.gemm_desc("f16", 255, 256, 256, a.ptr, (1, 256), a.ptr, (256, 1), a.ptr, (256, 1))
     assert dev.gemm_plan(d)[0] == KERNEL_MFMA     # M-contiguous A with M % 8 != 0: the MFMA kernel's window loads
     d = dev.gemm_desc("f16", 128, 64, 128, a.ptr, (128, 2), a.ptr, (256, 1), a.ptr, (256, 1))
-    assert dev.gemm_plan(d)[0] == KERNEL_GENERIC  # neither stride of A is 1
+    assert dev.gemm_plan(d)[2] == "mfma16_small_16x16_ksliced"  # neither stride of A is 1: no tiled kernel; small enough
+    d = dev.gemm_desc("f16", 1024, 256, 1024, a.ptr, (512, 2), a.ptr, (1024, 1), a.ptr, (1024, 1))
+    assert dev.gemm_plan(d)[0] == KERNEL_GENERIC  # the same at a size where 16 x 16 tiles no longer pay
     d = dev.gemm_desc("f64", 256, 256, 256, a.ptr, (256, 1), a.ptr, (256, 1), a.ptr, (256, 1))
     assert dev.gemm_plan(d)[0] == KERNEL_MFMA and dev.gemm_plan(d)[2].startswith("mfma64")
 

@@ -143,9 +143,11 @@ def test_fused_shapes_reach_every_tile_family_that_sums_rows():
 
 # f32: the k-sliced small kernel produces the row sums (config 1's Linear and smaller)
 FUSED_F32 = [("f32", 64, 512, 256), ("f32", 100, 40, 24), ("f32", 17, 33, 9), ("f32", 300, 16, 130)]
+# the small-product kernel in the other element types (its row sums come from the tile column 0 workgroups)
+FUSED_SMALL = [(d, *shape) for d in ("f16", "bf16", "f64") for shape in ((64, 512, 256), (100, 40, 24), (17, 33, 9), (300, 16, 130))]
 
 
-@pytest.mark.parametrize("dtype,rows,i,o", [(d, *shape) for d in ("f16", "bf16") for shape in FUSED_SHAPES] + FUSED_F32)
+@pytest.mark.parametrize("dtype,rows,i,o", [(d, *shape) for d in ("f16", "bf16") for shape in FUSED_SHAPES] + FUSED_F32 + FUSED_SMALL)
 def test_linear_backward_bias_gradient_from_the_weight_gradient_launch(dtype, rows, i, o):
     """grad_bias: exact on small integers (sums below 2^8 for bf16, 2^11 for f16 are representable), and twice the
     value after a second call (the first call finds the gradient fresh when its zeros are deferred, the second adds)."""
@@ -164,7 +166,7 @@ def test_linear_backward_bias_gradient_from_the_weight_gradient_launch(dtype, ro
         if deferred:   # NaN patterns that are only DECLARED zero: a read of the old contents would show
             import torch
             from dfdx_amd.rocm import View
-            es = 4 if dtype == "f32" else 2
+            es = {"f64": 8, "f32": 4}.get(dtype, 2)
             raw = torch.full((o * es,), 0xFF, dtype=torch.uint8, device="cuda")
             dev.zero_deferred(raw.data_ptr(), o * es)
             gb, base = View(raw, dtype, (o,), (1,)), np.zeros(o)
