@@ -163,8 +163,13 @@ template <typename T, int WAVES> __global__ __launch_bounds__(WAVES * 64) void g
         } else {
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                a[u] = fetch(ap, p.a_cs, row_ok, p.a_vec, kb + 16 * u + 4 * q);
-                b[u] = fetch(bp, p.b_rs, col_ok, p.b_vec, kb + 16 * u + 4 * q);
+                if (kb + 16 * u < k1) {  // the same in every lane: steps past the end are not loaded at all
+                    a[u] = fetch(ap, p.a_cs, row_ok, p.a_vec, kb + 16 * u + 4 * q);
+                    b[u] = fetch(bp, p.b_rs, col_ok, p.b_vec, kb + 16 * u + 4 * q);
+                } else {
+                    a[u] = S::zero();
+                    b[u] = S::zero();
+                }
             }
         }
     };

@@ -201,7 +201,10 @@ int dfdx_rocm_gemm_noalloc(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc);
  * variant and a short name ("mfma16_256x256x64_kc_kc" ...).  No launch. */
 int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int *kernel, int *variant,
                         char *name, size_t name_len);
-/* Number of MFMA tile variants available for `dtype` (variants are 1..count). */
+/* Number of MFMA tile variants available for `dtype` (variants are 1..count).  The last one
+ * in every type is the small-product kernel (16 x 16 tiles of C, the contraction cut over
+ * the waves of a workgroup; any operand strides, unbatched), which the planner picks by itself
+ * for products of a few microseconds. */
 int dfdx_rocm_mfma_variant_count(int dtype);
 
 /* Times `iters` back-to-back launches of `desc` with HIP events recorded on
