@@ -3,9 +3,9 @@
 // A product of a few MFLOP (a Linear layer on 64 rows, the reference's own test shapes) is bound by the chain
 // launch -> load -> MFMA -> store, not by any rate, and the tiled kernels walk k in steps behind one another (9.7 us for
 // f32 64 x 512 x 256 as four k pieces plus the combining launch).  Here every wave of a workgroup takes one slice of k,
-// requests ALL the operand values of a pass at once -- straight into the registers the MFMA reads, no LDS staging, any
-// strides -- runs its MFMA chain on two accumulators, and the slices meet in LDS, added in wave order (the result does
-// not depend on timing).  Lane l supplies A[row l % 16][k] and B[k][col l % 16] for the four consecutive
+// requests ALL the operand values of a pass (64 k) at once -- straight into the registers the MFMA reads, no LDS staging,
+// any strides --, the next pass's behind them where the registers allow, runs its MFMA chain on two accumulators, and the
+// slices meet in LDS, added in wave order (the result does not depend on timing).  Lane l supplies A[row l % 16][k] and B[k][col l % 16] for the four consecutive
 // k = 16 s + 4 (l / 16) + c, c < 4, of step s: one vector load where the operand is stored along k and aligned.  The
 // 16-bit types feed the four values to one v_mfma_f32_16x16x16, f32 and f64 to four v_mfma_*_16x16x4 (whose lane group
 // l / 16 is the k index: any bijection between (lane group, instruction) and k serves, as long as A and B share it).
@@ -22,7 +22,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef double f64x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 struct SmallParams {
     const void *a, *b;
@@ -109,7 +108,9 @@ template <> struct Small<__bf16> {
     }
 };
 
-template <typename T, int WAVES> __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(const SmallParams p) {
+// LONG: slices of more than one pass.  The one-pass form is kept as short as it can be: at 4 - 5 us a launch, the
+// instructions a longer kernel has to fetch and jump over show (0.3 - 0.6 us on a 64-row Linear layer's gradients).
+template <typename T, int WAVES, bool LONG> __global__ __launch_bounds__(WAVES * 64) void gemm_small_kernel(const SmallParams p) {
     typedef Small<T> S;
     typedef typename S::acc_t A;
     typedef typename S::acc4 A4;
@@ -124,26 +125,36 @@ template <typename T, int WAVES> __global__ __launch_bounds__(WAVES * 64) void g
     const T *ap = (const T *)p.a + (int64_t)(row_ok ? row : 0) * p.a_rs;
     const T *bp = (const T *)p.b + (int64_t)(col_ok ? col : 0) * p.b_cs;
     const int k0 = wave * p.slice, k1 = min(p.k, k0 + p.slice);
-    // Four k values of a pass that the slice's end cuts: every lane loads from an address inside the slice and the values
-    // beyond the end (or of a row / column beyond m / n) are replaced by zeros afterwards -- no branch per value, so all
-    // the loads of a pass are in flight together.
+    // Four k values of a pass that the slice's end may cut.  One-pass form in f32 and f64: a branch per value.  Otherwise
+    // every lane loads from an address inside the slice and the values beyond the end (or of a row / column beyond m / n)
+    // are replaced by zeros afterwards, so that all the loads of the pass are in flight together (16-bit values come one
+    // 2-byte load each, which the branches would space out: 0.3 - 0.7 us on the same gradients).
+    constexpr bool BRANCHY = !LONG && sizeof(T) >= 4;
     auto fetch = [&](const T *base, int64_t kstride, bool ok, bool vec, int kk) -> Pack {
-        if (vec && kk + 3 < k1) return ok ? S::vec(base + kk) : S::zero();
         Pack v = S::zero();
-        const Pack z = S::zero();
+        if constexpr (BRANCHY) {  // (this order of the tests and no test per step measured best of the forms tried)
+            if (!ok || kk >= k1) return v;
+            if (vec && kk + 3 < k1) return S::vec(base + kk);
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            S::set(v, c, base + (int64_t)max(0, min(kk + c, k1 - 1)) * kstride);
-            if (!ok || kk + c >= k1) v[c] = z[c];
+            for (int c = 0; c < 4; c++)
+                if (kk + c < k1) S::set(v, c, base + (int64_t)(kk + c) * kstride);
+        } else {
+            if (vec && kk + 3 < k1) return ok ? S::vec(base + kk) : v;
+            const Pack z = S::zero();
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                S::set(v, c, base + (int64_t)max(0, min(kk + c, k1 - 1)) * kstride);
+                if (!ok || kk + c >= k1) v[c] = z[c];
+            }
         }
         return v;
     };
     A4 acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
     const bool sums = p.ksum && tn == 0;
     A rsum = 0;  // of A[row r16][this lane's k values]
-    // Passes of four steps of 16 k (8 loads per lane each), the loads of the next pass in flight behind the MFMAs of this
-    // one (not f64).
-    Pack av[4], bv[4], an[4], bn[4];
+    // Passes of four steps of 16 k (8 loads per lane each); LONG: the loads of the next pass in flight behind the MFMAs
+    // of this one (not f64).
+    Pack av[4], bv[4];
     // A pass that lies inside the slice is loaded without a test per value: the rows and columns beyond m and n read
     // row / column 0 (their results are never stored), and the branches on the layout are the same for the whole launch.
     auto whole = [&](const T *base, int64_t kstride, bool vec, int kk) -> Pack {
@@ -154,7 +165,7 @@ template <typename T, int WAVES> __global__ __launch_bounds__(WAVES * 64) void g
         return v;
     };
     auto load_pass = [&](Pack *a, Pack *b, int kb) {
-        if (kb + 64 <= k1) {
+        if (LONG && kb + 64 <= k1) {
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 a[u] = whole(ap, p.a_cs, p.a_vec, kb + 16 * u + 4 * q);
@@ -163,7 +174,7 @@ template <typename T, int WAVES> __global__ __launch_bounds__(WAVES * 64) void g
         } else {
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                if (kb + 16 * u < k1) {  // the same in every lane: steps past the end are not loaded at all
+                if (BRANCHY || kb + 16 * u < k1) {  // the same in every lane: steps past the end are not loaded at all
                     a[u] = fetch(ap, p.a_cs, row_ok, p.a_vec, kb + 16 * u + 4 * q);
                     b[u] = fetch(bp, p.b_rs, col_ok, p.b_vec, kb + 16 * u + 4 * q);
                 } else {
@@ -184,7 +195,11 @@ template <typename T, int WAVES> __global__ __launch_bounds__(WAVES * 64) void g
             else acc1 = S::mma(a[u], b[u], acc1);
         }
     };
-    if constexpr (sizeof(T) < 8) {
+    if constexpr (!LONG) {
+        load_pass(av, bv, k0);
+        use_pass(av, bv);
+    } else if constexpr (sizeof(T) < 8) {
+        Pack an[4], bn[4];
         load_pass(av, bv, k0);
         for (int kb = k0; kb < k1; kb += 128) {  // k0, k1 and kb are the same in every lane of a wave
             if (kb + 64 < k1) load_pass(an, bn, kb + 64);
@@ -245,18 +260,21 @@ inline int small_waves(int dtype, int64_t k) {
     return (k >= 2048 && dtype != DT_F64) ? 16 : k >= 256 ? 8 : k >= 128 ? 4 : k >= 64 ? 2 : 1;
 }
 
-template <typename T> hipError_t launch_t(const SmallParams &p, int waves, dim3 grid, hipStream_t stream) {
+template <typename T, bool LONG> hipError_t launch_form(const SmallParams &p, int waves, dim3 grid, hipStream_t stream) {
     switch (waves) {
     case 16:
-        if constexpr (sizeof(T) < 8) gemm_small_kernel<T, 16><<<grid, 1024, 0, stream>>>(p);
+        if constexpr (sizeof(T) < 8 && LONG) gemm_small_kernel<T, 16, true><<<grid, 1024, 0, stream>>>(p);
         else return hipErrorInvalidValue;
         break;
-    case 8: gemm_small_kernel<T, 8><<<grid, 512, 0, stream>>>(p); break;
-    case 4: gemm_small_kernel<T, 4><<<grid, 256, 0, stream>>>(p); break;
-    case 2: gemm_small_kernel<T, 2><<<grid, 128, 0, stream>>>(p); break;
-    default: gemm_small_kernel<T, 1><<<grid, 64, 0, stream>>>(p); break;
+    case 8: gemm_small_kernel<T, 8, LONG><<<grid, 512, 0, stream>>>(p); break;
+    case 4: gemm_small_kernel<T, 4, LONG><<<grid, 256, 0, stream>>>(p); break;
+    case 2: gemm_small_kernel<T, 2, LONG><<<grid, 128, 0, stream>>>(p); break;
+    default: gemm_small_kernel<T, 1, LONG><<<grid, 64, 0, stream>>>(p); break;
     }
     return hipGetLastError();
+}
+template <typename T> hipError_t launch_t(const SmallParams &p, int waves, dim3 grid, hipStream_t stream) {
+    return p.slice > 64 ? launch_form<T, true>(p, waves, grid, stream) : launch_form<T, false>(p, waves, grid, stream);
 }
 
 }  // namespace
