@@ -426,6 +426,9 @@ def main():
                 gemm("gemv", f"vec.mat {dt} (1,{n_})x({n_},{n_})", dev.gemm_desc(dt, 1, n_, n_, P(xv), (n_, 1), P(W), (n_, 1), P(yv), (n_, 1)), 2 * n_ * n_, es * n_ * n_, 100, bufs=(W, xv, yv))
                 gemm("gemv", f"vec.mat {dt}, Linear weight view", dev.gemm_desc(dt, 1, n_, n_, P(xv), (n_, 1), P(W), (1, n_), P(yv), (n_, 1)), 2 * n_ * n_, es * n_ * n_, 100, bufs=(W, xv, yv))
                 gemm("gemv", f"mat.vec {dt} ({n_},{n_})x({n_},)", dev.gemm_desc(dt, n_, n_, 1, P(W), (n_, 1), P(xv), (1, 1), P(yv), (1, 1)), 2 * n_ * n_, es * n_ * n_, 100, bufs=(W, xv, yv))
+                # the weight gradient of the same vec.mat: the rank-1 update grad_W += x^T (x) grad_y (k = 1), C read and written
+                gemm("gemv", f"rank-1 update {dt} ({n_},1)x(1,{n_}) acc", dev.gemm_desc(dt, n_, 1, n_, P(xv), (1, 1), P(yv), (n_, 1), P(W), (n_, 1), accumulate=True),
+                     2 * n_ * n_, 2 * es * n_ * n_, 100, bufs=(W, xv, yv))
                 del W
 
     # ---- operands off the 16-byte grid: an LM head with 50257 outputs, a first-layer convolution -------------------

@@ -149,6 +149,10 @@ bool gemv_supported(const GemmProblem &p);
 size_t gemv_workspace_bytes(const GemmProblem &p);  // f32 partial sums of the k slices (0 when not sliced)
 hipError_t launch_gemv(const GemmProblem &p, hipStream_t stream);
 
+// ---- rank-1 updates, k = 1 (rank1.hip): every dtype, any strides of the two vectors, row-major C ----
+bool rank1_supported(const GemmProblem &p);
+hipError_t launch_rank1(const GemmProblem &p, hipStream_t stream);
+
 // XCD-aware remap of a linear workgroup id: consecutive ids are dispatched round-robin
 // over the 8 XCDs, so ids that share an XCD (and its L2) are pid, pid+8, pid+16 ...
 // This returns a work index such that each XCD owns one contiguous range of work.

@@ -353,6 +353,30 @@ def test_gemv(dtype, shape, layout):
     run_case(dtype, m, k, n, layout, True, KERNEL_AUTO, 0, seed=4, bias=(dtype == "f32"))
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16", "f64"])
+def test_rank1_updates(dtype):
+    """k = 1 (vec (x) vec, mod.rs:139-144, and the weight gradient of a vec.mat product): the elementwise kernel that
+    streams C by whole rows; wide and narrow C, extents off the 16-byte grid, padded rows, strided vectors, beta = 0 / 1,
+    bias per column and (column-major C) per row.  A single product, so f32 and f64 results equal the rounded product."""
+    from dfdx_amd.rocm import KERNEL_GEMV
+    dev = device()
+    for i, (m, n) in enumerate([(4096, 1024), (3, 5), (130, 24), (2, 4104), (515, 257), (64, 8), (1000, 3)]):
+        a = dev.zeros(dtype, (max(m, n),))
+        plan = dev.gemm_plan(dev.gemm_desc(dtype, m, 1, n, a.ptr, (1, 1), a.ptr, (n, 1), a.ptr, (n, 1)))
+        assert plan[0] == KERNEL_GEMV and plan[2] == "rank1", plan
+        for layout in ("nn", "tt"):
+            for pads in ((0, 0, 0), (3, 5, 8), (1, 1, 3)):
+                run_case(dtype, m, 1, n, layout, bool(i % 2), KERNEL_AUTO, 0, bias=(i % 3 == 0), c_colmajor=(i % 3 == 1), seed=90 + i, pads=pads)
+                run_case(dtype, m, 1, n, layout, not (i % 2), KERNEL_GEMV, 0, bias=(i % 3 == 1), seed=70 + i, pads=pads)
+    if dtype in ("f32", "f64"):
+        g = rng(8)
+        np_t = np.float32 if dtype == "f32" else np.float64
+        x, y = g.standard_normal(300).astype(np_t), g.standard_normal(200).astype(np_t)
+        dx, dy, dc = dev.tensor(x, dtype), dev.tensor(y, dtype), dev.zeros(dtype, (300, 200))
+        dev.gemm(dev.gemm_desc(dtype, 300, 1, 200, dx.ptr, (1, 1), dy.ptr, (200, 1), dc.ptr, (200, 1)))
+        assert np.array_equal(dev.to_host(dc).reshape(300, 200), np.outer(x, y))
+
+
 # ------------------------------------------------------------------ split-k --
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("layout", ["tn", "nt", "nn"])
