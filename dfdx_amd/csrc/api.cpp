@@ -737,7 +737,7 @@ int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int
             std::snprintf(name, name_len, "%s_%s", p.dtype == DT_F32 ? "mfma32" : "mfma16",
                           p.dtype == DT_F32 ? mfma32_variant_name(plan.variant) : mfma16_variant_name(plan.variant));
         else
-            std::snprintf(name, name_len, "%s", plan.kernel != DFDX_ROCM_KERNEL_GEMV ? "generic" : rank1_supported(p) ? "rank1" : "gemv");
+            std::snprintf(name, name_len, "%s", plan.kernel != DFDX_ROCM_KERNEL_GEMV ? "generic" : rank1_supported(p) ? (p.k == 1 ? "rank1" : "thin_k") : "gemv");
     }
     return DFDX_ROCM_OK;
 }

@@ -308,7 +308,8 @@ def test_unaligned_operands_run_on_the_mfma_kernels(dtype, shape):
         da, db = dev.tensor(a, dtype), dev.tensor(b, dtype)
         dc = dev.zeros(dtype, (m, n + pads[2]))
         desc = dev.gemm_desc(dtype, m, k, n, da.ptr, astr, db.ptr, bstr, dc.ptr, (n + pads[2], 1))
-        assert dev.gemm_plan(desc)[0] == KERNEL_MFMA, (shape, layout, dev.gemm_plan(desc))
+        plan = dev.gemm_plan(desc)   # (a contraction of at most eight may go to the row-streaming kernel instead)
+        assert plan[0] == KERNEL_MFMA or (k <= 8 and plan[2] == "thin_k"), (shape, layout, plan)
         run_case(dtype, m, k, n, layout, bool(i % 2), KERNEL_AUTO, 0, c_colmajor=(i == 3), seed=900 + i, pads=pads)
 
 
@@ -375,6 +376,26 @@ def test_rank1_updates(dtype):
         dx, dy, dc = dev.tensor(x, dtype), dev.tensor(y, dtype), dev.zeros(dtype, (300, 200))
         dev.gemm(dev.gemm_desc(dtype, 300, 1, 200, dx.ptr, (1, 1), dy.ptr, (200, 1), dc.ptr, (200, 1)))
         assert np.array_equal(dev.to_host(dc).reshape(300, 200), np.outer(x, y))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16", "f64"])
+@pytest.mark.parametrize("k", [2, 3, 4, 5, 8])
+def test_thin_contractions(dtype, k):
+    """k = 2 .. 8 (a Linear layer on a handful of input features, the input gradient of a layer with a handful of outputs):
+    the row-streaming kernel with the sum over k ascending; all four operand layouts, tails, padded rows, beta, bias."""
+    from dfdx_amd.rocm import KERNEL_GEMV
+    dev = device()
+    for i, (m, n) in enumerate([(2048, 1024), (3, 5), (130, 24), (515, 257), (1000, 3)]):
+        a = dev.zeros(dtype, (max(m, n) * k,))
+        plan = dev.gemm_plan(dev.gemm_desc(dtype, m, k, n, a.ptr, (k, 1), a.ptr, (n, 1), a.ptr, (n, 1)))
+        if dtype in ("f32", "f64") or k <= 4:   # 16-bit types: up to k = 4 (beyond, the matrix-core kernels are as fast)
+            assert plan[0] == KERNEL_GEMV and plan[2] == "thin_k", plan
+        else:
+            assert plan[2] != "thin_k", plan
+        for layout in LAYOUTS:
+            run_case(dtype, m, k, n, layout, bool(i % 2), KERNEL_AUTO, 0, bias=(i % 3 == 0), c_colmajor=(i % 3 == 1), seed=40 + i, pads=(i % 3, 2 * (i % 2), 3 * (i % 2)))
+    a = dev.zeros(dtype, (4096,))
+    assert dev.gemm_plan(dev.gemm_desc(dtype, 64, 9, 64, a.ptr, (9, 1), a.ptr, (64, 1), a.ptr, (64, 1)))[2] != "thin_k"
 
 
 # ------------------------------------------------------------------ split-k --
