@@ -26,7 +26,7 @@ def main():
     ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "f32-forms", "mfma-power"],
                     help="counter-collection aids for rocprofv3, nothing is timed: traffic = 3 plain 256 MiB device copies (a kernel "
                          "of known size that calibrates FETCH_SIZE / WRITE_SIZE) then 5 launches of the 4096^3 f16 GEMM; rows = the same copies, then 3 launches each of "
-                         "the HBM-bound rows (config 4 scores and dP, softmax forward and backward on them, the 16384^2 f16 vec.mat); f32-forms = 3 "
+                         "the HBM-bound rows (config 4 scores and dP, the 16384^2 f16 vec.mat and the rank-1 update that is its weight gradient, softmax forward and backward on the scores); f32-forms = 3 "
                          "launches each of the register-staged and the LDS-DMA f32 kernel (256x256 tile) on 4096^3 A.B^T and A.B; variants = 3 "
                          "launches of that GEMM with every f16 MFMA tile variant forced in turn; mfma-power = the stand-alone "
                          "MFMA-only program (built by `make -C dfdx_amd/csrc probe`)")
@@ -100,8 +100,9 @@ def main():
             n_ = 16384
             W, xv, yv = torch.randn(n_, n_, device="cuda").half(), torch.randn(n_, device="cuda").half(), torch.zeros(n_, device="cuda").half()
             gv = dev.gemm_desc("f16", 1, n_, n_, P(xv), (n_, 1), P(W), (n_, 1), P(yv), (n_, 1))
+            r1 = dev.gemm_desc("f16", n_, 1, n_, P(xv), (1, 1), P(yv), (n_, 1), P(W), (n_, 1), accumulate=True)  # W += x (x) y: the gradient of gv
             names = []
-            for desc in (scores, dp, gv):
+            for desc in (scores, dp, gv, r1):
                 names.append(dev.gemm_plan(desc)[2])
                 for _ in range(3):
                     dev.gemm(desc)
