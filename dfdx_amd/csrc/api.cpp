@@ -282,7 +282,7 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
         *plan = {DFDX_ROCM_KERNEL_GENERIC, 0, 1};
         return DFDX_ROCM_OK;
     case DFDX_ROCM_KERNEL_GEMV:  // the bandwidth-bound kernels: vector products and rank-1 updates
-        if (!gemv_supported(p) && !rank1_supported(p)) return DFDX_ROCM_ERR_UNSUPPORTED;
+        if (!gemv_supported(p) && !rank1_supported(p) && !gemv_multi_supported(p)) return DFDX_ROCM_ERR_UNSUPPORTED;
         *plan = {DFDX_ROCM_KERNEL_GEMV, 0, 1};
         return DFDX_ROCM_OK;
     case DFDX_ROCM_KERNEL_MFMA: {
@@ -311,7 +311,7 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
     default:
         return DFDX_ROCM_ERR_INVALID_ARG;
     }
-    if (gemv_supported(p) || rank1_supported(p)) {
+    if (gemv_supported(p) || rank1_supported(p) || gemv_multi_supported(p)) {
         *plan = {DFDX_ROCM_KERNEL_GEMV, 0, 1};
         return DFDX_ROCM_OK;
     }
@@ -380,14 +380,18 @@ int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan, b
         p.splits = plan.splits;
     }
     if (plan.kernel == DFDX_ROCM_KERNEL_GEMV) {
-        if (const size_t need = gemv_workspace_bytes(p)) {
+        const bool multi = !rank1_supported(p) && gemv_multi_supported(p);
+        if (const size_t need = multi ? gemv_multi_workspace_bytes(p) : gemv_workspace_bytes(p)) {
             if (int rc = partials_buffer(ctx, need, static_scratch, &p.workspace)) return rc;
         }
     }
     hipError_t e;
     switch (plan.kernel) {
     case DFDX_ROCM_KERNEL_GENERIC: e = launch_generic(p, ctx->stream); break;
-    case DFDX_ROCM_KERNEL_GEMV: e = rank1_supported(p) ? launch_rank1(p, ctx->stream) : launch_gemv(p, ctx->stream); break;
+    case DFDX_ROCM_KERNEL_GEMV:
+        e = rank1_supported(p) ? launch_rank1(p, ctx->stream)
+                               : gemv_multi_supported(p) ? launch_gemv_multi(p, ctx->stream) : launch_gemv(p, ctx->stream);
+        break;
     case DFDX_ROCM_KERNEL_MFMA:
         e = (p.dtype == DT_F32) ? launch_mfma32(p, plan.variant, ctx->stream)
                                 : (p.dtype == DT_F64) ? launch_mfma64(p, plan.variant, ctx->stream) : launch_mfma16(p, plan.variant, ctx->stream);
@@ -737,7 +741,7 @@ int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int
             std::snprintf(name, name_len, "%s_%s", p.dtype == DT_F32 ? "mfma32" : "mfma16",
                           p.dtype == DT_F32 ? mfma32_variant_name(plan.variant) : mfma16_variant_name(plan.variant));
         else
-            std::snprintf(name, name_len, "%s", plan.kernel != DFDX_ROCM_KERNEL_GEMV ? "generic" : rank1_supported(p) ? (p.k == 1 ? "rank1" : "thin_k") : "gemv");
+            std::snprintf(name, name_len, "%s", plan.kernel != DFDX_ROCM_KERNEL_GEMV ? "generic" : rank1_supported(p) ? (p.k == 1 ? "rank1" : "thin_k") : gemv_multi_supported(p) ? "gemv_multi" : "gemv");
     }
     return DFDX_ROCM_OK;
 }

@@ -149,6 +149,11 @@ bool gemv_supported(const GemmProblem &p);
 size_t gemv_workspace_bytes(const GemmProblem &p);  // f32 partial sums of the k slices (0 when not sliced)
 hipError_t launch_gemv(const GemmProblem &p, hipStream_t stream);
 
+// ---- two to eight vectors against one streamed matrix (gemv_multi.hip): M or N of 2 .. 8, the other operand a megabyte at least ----
+bool gemv_multi_supported(const GemmProblem &p);
+size_t gemv_multi_workspace_bytes(const GemmProblem &p);
+hipError_t launch_gemv_multi(const GemmProblem &p, hipStream_t stream);
+
 // ---- rank-1 updates and thin contractions, k = 1 .. 8 (rank1.hip): every dtype, any operand strides, row-major C ----
 bool rank1_supported(const GemmProblem &p);
 hipError_t launch_rank1(const GemmProblem &p, hipStream_t stream);

@@ -354,6 +354,31 @@ def test_gemv(dtype, shape, layout):
     run_case(dtype, m, k, n, layout, True, KERNEL_AUTO, 0, seed=4, bias=(dtype == "f32"))
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", [(2, 1024, 1032), (3, 2056, 520), (4, 4096, 1024), (5, 1032, 2048), (8, 8200, 264), (7, 264, 8200),
+                                   (1032, 1024, 2), (520, 2056, 3), (2048, 1032, 8), (8200, 264, 6)])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn"])
+def test_gemv_multi(dtype, shape, layout):
+    """2 .. 8 vectors against one streamed matrix (a Linear layer on a batch of a few rows; the gradients of a layer with a
+    few outputs): every layout the matrix can be streamed in, either operand as the small one, beta = 0 / 1, bias,
+    column-major C."""
+    from dfdx_amd.rocm import KERNEL_GEMV
+    m, k, n = shape
+    dev = device()
+    a = dev.zeros(dtype, (max(m, n) * k,))
+    at, bt = LAYOUTS[layout]
+    astr = (1, m) if at else (k, 1)
+    bstr = (1, k) if bt else (n, 1)
+    plan = dev.gemm_plan(dev.gemm_desc(dtype, m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1)))
+    # the matrix must be walkable in 16-byte pieces along its outputs ("cols") or along k ("dots": then the vectors must be
+    # contiguous in k as well); of the three layouts only A.B with the few columns in B is neither
+    if not (n <= 8 and layout == "nn"):
+        assert plan[0] == KERNEL_GEMV and plan[2] == "gemv_multi", (shape, layout, plan)
+    run_case(dtype, m, k, n, layout, False, KERNEL_AUTO, 0, seed=5, bias=True)
+    run_case(dtype, m, k, n, layout, True, KERNEL_AUTO, 0, seed=6, c_colmajor=True, bias=(dtype == "f32"))
+    run_case(dtype, m, k, n, layout, True, KERNEL_AUTO, 0, seed=7, pads=(8, 8, 3))
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16", "f64"])
 def test_rank1_updates(dtype):
     """k = 1 (vec (x) vec, mod.rs:139-144, and the weight gradient of a vec.mat product): the elementwise kernel that
