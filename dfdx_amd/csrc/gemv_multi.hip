@@ -1,5 +1,6 @@
 // A few vectors against one large matrix: (2..8, K).(K, N) and (M, K).(K, 2..8) -- a Linear layer on a batch of a
-// handful of rows, the gradients of a layer with a handful of outputs.  Like the vector products of gemv.hip these are
+// handful of rows, the gradients of a layer with a handful of outputs.  (Sixteen vectors were tried and dropped: 128 sums per
+// thread, and only the f32 weight gradient of a 10-output layer gained, 20 against 35 - 41 us.)  Like the vector products of gemv.hip these are
 // bound by streaming the matrix once from HBM; a matrix-core tile would be 7/8 empty and, worse, leave most of the chip
 // without a workgroup unless the contraction is split and combined by a second launch (16 x 4096 x 4096 f16: 15.8 us on
 // the tiled kernels against 6 us for the bytes).  Same two forms as gemv.hip over
@@ -28,7 +29,10 @@ struct MultiParams {
     float *ws;
 };
 
-constexpr int KCHUNK = 1024;  // k values of a slice in the cols form: R x KCHUNK values in LDS
+// k values of a slice in the cols form: R x kchunk_of(R) values in LDS (32 KiB of f32 at most)
+constexpr int kchunk_of(int r) { return r > 8 ? 512 : 1024; }
+// matrix rows a wave of the dots form takes: 4 * R or 2 * R sums per lane
+constexpr int rows_of(int r) { return r > 8 ? 2 : 4; }
 
 template <typename T, int N> __device__ __forceinline__ void unpack16(const T *p, float (&v)[N]) {
     const u32x4 raw = *(const u32x4 *)p;
@@ -77,7 +81,7 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_c
     constexpr int VEC = Elem<T>::VEC;
     constexpr bool PAIRS = sizeof(T) == 2;
     typedef typename std::conditional<PAIRS, T, float>::type S;  // what the vector slices are kept as
-    __shared__ __align__(16) S vsh[R][KCHUNK];
+    __shared__ __align__(16) S vsh[R][kchunk_of(R)];
     __shared__ float red[4][64 * VEC];
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int j0 = (blockIdx.x * 64 + lane) * VEC;
@@ -160,18 +164,19 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_c
     }
 #pragma unroll
     for (int r = 0; r < R; r++) {  // the four waves' sums of one vector at a time through the same buffer
-        if (r >= p.r) break;       // the same in every thread
+        if (r < p.r) {             // the same in every thread
 #pragma unroll
-        for (int e = 0; e < VEC; e++) red[wave][lane * VEC + e] = acc[r][e];
-        __syncthreads();
-        for (int o = tid; o < 64 * VEC; o += 256) {
-            const int j = blockIdx.x * 64 * VEC + o;
-            if (j >= p.j) continue;
-            const float v = ((red[0][o] + red[1][o]) + red[2][o]) + red[3][o];
-            if (p.kslices > 1) p.ws[((int64_t)blockIdx.y * p.r + r) * p.j + j] = v;
-            else finish<T>(p, r, j, v);
+            for (int e = 0; e < VEC; e++) red[wave][lane * VEC + e] = acc[r][e];
+            __syncthreads();
+            for (int o = tid; o < 64 * VEC; o += 256) {
+                const int j = blockIdx.x * 64 * VEC + o;
+                if (j >= p.j) continue;
+                const float v = ((red[0][o] + red[1][o]) + red[2][o]) + red[3][o];
+                if (p.kslices > 1) p.ws[((int64_t)blockIdx.y * p.r + r) * p.j + j] = v;
+                else finish<T>(p, r, j, v);
+            }
+            __syncthreads();
         }
-        __syncthreads();
     }
 }
 
@@ -192,7 +197,7 @@ template <int NV, int N> __device__ __forceinline__ void halve(float (&vals)[NV]
 }
 
 template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_dots_kernel(const MultiParams p) {
-    constexpr int VEC = Elem<T>::VEC, J = 4;
+    constexpr int VEC = Elem<T>::VEC, J = rows_of(R);
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int j0 = (blockIdx.x * 4 + wave) * J;
     if (j0 >= p.j) return;
@@ -317,10 +322,11 @@ Shape classify(const GemmProblem &g) {
 void plan_slices(Shape &s, int dtype) {
     MultiParams &p = s.p;
     const int vec = dtype == DT_F32 ? 4 : 8;
-    const int64_t blocks_j = s.cols ? (p.j + 64 * vec - 1) / (64 * vec) : (p.j + 15) / 16;
+    const int kchunk_max = kchunk_of(p.r), per_wg = 4 * rows_of(p.r);
+    const int64_t blocks_j = s.cols ? (p.j + 64 * vec - 1) / (64 * vec) : (p.j + per_wg - 1) / per_wg;
     int slices = 1;
     if (s.cols) {
-        slices = (p.k + KCHUNK - 1) / KCHUNK;  // the vector slices must fit the LDS buffer
+        slices = (p.k + kchunk_max - 1) / kchunk_max;  // the vector slices must fit the LDS buffer
         while (blocks_j * slices < 1024 && p.k / (slices * 2) >= 64) slices *= 2;
     } else {
         // a wave of this form is heavy (4 + R loads a step): it takes eight of them per SIMD to hide the latency of HBM
@@ -328,7 +334,7 @@ void plan_slices(Shape &s, int dtype) {
     }
     int chunk = (p.k + slices - 1) / slices;
     chunk = (chunk + vec - 1) / vec * vec;
-    if (s.cols && chunk > KCHUNK) chunk = KCHUNK;
+    if (s.cols && chunk > kchunk_max) chunk = kchunk_max;
     p.kchunk = chunk;
     p.kslices = (p.k + chunk - 1) / chunk;
 }
@@ -340,7 +346,8 @@ template <typename T, int R> hipError_t launch_r(const Shape &s, hipStream_t str
         dim3 grid((unsigned)((p.j + 64 * VEC - 1) / (64 * VEC)), (unsigned)p.kslices);
         gemv_multi_cols_kernel<T, R><<<grid, 256, 0, stream>>>(p);
     } else {
-        dim3 grid((unsigned)((p.j + 15) / 16), (unsigned)p.kslices);
+        constexpr int PER_WG = 4 * rows_of(R);
+        dim3 grid((unsigned)((p.j + PER_WG - 1) / PER_WG), (unsigned)p.kslices);
         gemv_multi_dots_kernel<T, R><<<grid, 256, 0, stream>>>(p);
     }
     if (p.kslices > 1) {

@@ -360,8 +360,8 @@ def test_gemv(dtype, shape, layout):
 @pytest.mark.parametrize("layout", ["nn", "nt", "tn"])
 def test_gemv_multi(dtype, shape, layout):
     """2 .. 8 vectors against one streamed matrix (a Linear layer on a batch of a few rows; the gradients of a layer with a
-    few outputs): every layout the matrix can be streamed in, either operand as the small one, beta = 0 / 1, bias,
-    column-major C."""
+    few outputs): every layout the matrix can be streamed in, either operand as the small one,
+    beta = 0 / 1, bias, column-major C."""
     from dfdx_amd.rocm import KERNEL_GEMV
     m, k, n = shape
     dev = device()
