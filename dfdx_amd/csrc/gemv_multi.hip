@@ -277,7 +277,7 @@ inline bool al16(const void *q) { return ((uintptr_t)q & 15u) == 0; }
 Shape classify(const GemmProblem &g) {
     Shape s{};
     if (g.dtype == DT_F64 || g.reduce || g.nb1 * g.nb2 != 1 || g.k < 1 || g.k >= (1ll << 31)) return s;
-    if (g.m >= (1ll << 31) || g.n >= (1ll << 31)) return s;
+    if (g.m >= (1ll << 30) || g.n >= (1ll << 30)) return s;  // 32-bit output indices with room for a block past the end
     if (g.c_rs < 1 || g.c_cs < 1) return s;  // no aliased outputs
     MultiParams &p = s.p;
     const int vec = g.dtype == DT_F32 ? 4 : 8;

@@ -225,7 +225,7 @@ bool rank1_supported(const GemmProblem &g) {
     const int kmost = (g.dtype == DT_F16 || g.dtype == DT_BF16) ? 4 : 8;
     if (g.k < 1 || g.k > kmost || g.m < 2 || g.n < 2 || g.reduce || g.nb1 * g.nb2 != 1) return false;
     if (g.c_cs != 1 || g.c_rs < g.n) return false;
-    if (g.m >= (1ll << 31) || g.n >= (1ll << 31)) return false;
+    if (g.m >= (1ll << 30) || g.n >= (1ll << 30)) return false;  // 32-bit row and column indices with room for a block past the end
     const int vec = (int)(16 / dtype_size(g.dtype));
     if (((g.n + vec - 1) / vec + 255) / 256 > 65535) return false;  // column blocks are grid.y
     const uintptr_t mask = dtype_size(g.dtype) - 1;
