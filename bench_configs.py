@@ -22,7 +22,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
-    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them)")
+    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them, shapes = shape classes outside the configurations: few rows or columns, thin contractions, rank-1 updates, mid-size products)")
     ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "f32-forms", "mfma-power"],
                     help="counter-collection aids for rocprofv3, nothing is timed: traffic = 3 plain 256 MiB device copies (a kernel "
                          "of known size that calibrates FETCH_SIZE / WRITE_SIZE) then 5 launches of the 4096^3 f16 GEMM; rows = the same copies, then 3 launches each of "
@@ -431,6 +431,26 @@ def main():
                 gemm("gemv", f"rank-1 update {dt} ({n_},1)x(1,{n_}) acc", dev.gemm_desc(dt, n_, 1, n_, P(xv), (1, 1), P(yv), (n_, 1), P(W), (n_, 1), accumulate=True),
                      2 * n_ * n_, 2 * es * n_ * n_, 100, bufs=(W, xv, yv))
                 del W
+
+    # ---- shapes outside the five configurations: few rows or columns, thin contractions, rank-1 updates, mid-size --------
+    if "shapes" in only:   # on request: which kernel the planner gives each shape class, and what it costs
+        cases = [  # (m, k, n, layout of A and B: n = stored as indexed, t = stored transposed)
+            (64, 512, 256, "nt"), (256, 256, 256, "nt"), (100, 300, 200, "nn"), (512, 512, 512, "nt"), (1000, 1000, 1000, "nn"), (2048, 2048, 2048, "nt"),
+            (4096, 1, 4096, "nn"), (4095, 1, 4097, "nn"), (8192, 4, 1024, "nt"), (65536, 8, 256, "nt"), (8192, 10, 1024, "nn"), (4096, 16, 4096, "nn"),
+            (4, 4096, 4096, "nt"), (4, 4096, 4096, "nn"), (8, 1024, 50264, "nt"), (16, 4096, 4096, "nt"), (32, 8192, 8192, "nt"),
+            (65536, 512, 2, "nt"), (8192, 1024, 10, "nt"), (10, 8192, 1024, "tn"), (1024, 8192, 10, "tn"),
+        ]
+        for dt in ("f16", "f32", "f64"):
+            es = esz[dt]
+            for m, k, n, lay in cases:
+                if dt == "f64" and m * k * n > 2 ** 31:
+                    continue
+                a = rnd((k, m) if lay[0] == "t" else (m, k), dt)
+                b = rnd((n, k) if lay[1] == "t" else (k, n), dt)
+                c = zeros((m, n), dt)
+                desc = dev.gemm_desc(dt, m, k, n, P(a), (1, m) if lay[0] == "t" else (k, 1), P(b), (1, k) if lay[1] == "t" else (n, 1), P(c), (n, 1))
+                gemm("shape", f"{dt} {m}x{k}x{n} {lay}", desc, 2 * m * k * n, es * (m * k + k * n + m * n), 100)
+                del a, b, c
 
     # ---- operands off the 16-byte grid: an LM head with 50257 outputs, a first-layer convolution -------------------
     if "edge" in only:   # on request: the scalar kernel's rows take milliseconds each

@@ -750,7 +750,7 @@ int mfma32_pick_variant(const GemmProblem &p, int compute_units, int forced_spli
     for (int v = 1; v <= kNumVariants; v++) {
         if (!mfma32_supported(p, v)) continue;
         // the small kernel adds its k slices in an order of its own: not where the caller asked for the plain k order
-        if (kVariants[v - 1].small && (forced_splits == 1 || (double)p.m * (double)p.n * (double)p.k > 134217728.0)) continue;
+        if (kVariants[v - 1].small && (forced_splits == 1 || (double)p.m * (double)p.n * (double)p.k > 536870912.0)) continue;
         double tm;
         plan_pieces32(p, v, compute_units, forced_splits, &tm);
         if (tm < best_time) {

@@ -294,18 +294,21 @@ bool small_ksum_supported(const GemmProblem &p) {
     return p.ksum && p.ksum_of == KSUM_OF_A && small_supported(p) && ((uintptr_t)p.ksum & (elem_size(p.dtype) - 1)) == 0;
 }
 
-// Estimated time, fitted to timings on a 256-CU MI355X: the launch; the chain of loads of one workgroup, which grows
-// with the whole contraction however many waves share it (3.4 ns per k, twice that for f64: the 16 rows of a load
-// instruction lie a row stride apart); an operand that is not stored along k costs a 2- or 4-byte load per value; and
-// no operand value is shared between workgroups, so every tile pulls its 16 rows and 16 columns through the caches again
-// (5 - 8 TB/s over the whole chip).
+// Estimated time, fitted to timings on a 256-CU MI355X: the launch; then the longer of (a) the chain of loads of one
+// workgroup, which grows with the whole contraction however many waves share it (3.4 ns per k, twice that for f64: the
+// 16 rows of a load instruction lie a row stride apart), and (b) the bytes all workgroups pull through the caches -- no
+// operand value is shared between workgroups, so every tile fetches its 16 rows and 16 columns again (5 - 8 TB/s over
+// the whole chip); an operand that is not stored along k costs a 2- or 4-byte load per value on top, and so does C.
 double small_time(const GemmProblem &p, int compute_units) {
     const double tiles = (double)((p.m + 15) / 16) * (double)((p.n + 15) / 16);
     const double es = (double)elem_size(p.dtype);
     const double chain = std::max(0.5e-6, (double)p.k * (p.dtype == DT_F64 ? 6.8e-9 : 3.4e-9));
     const double gather = p.dtype == DT_F64 ? 0.0 : (p.dtype == DT_F32 ? 0.4e-6 : 0.9e-6) * ((p.a_cs != 1) + (p.b_rs != 1));
     const double bandwidth = (p.dtype == DT_F64 ? 8e12 : p.dtype == DT_F32 ? 7.5e12 : 5e12) * std::max(1, compute_units) / 256.0;
-    return 2.1e-6 + chain + gather + tiles * 32.0 * es * (double)p.k / bandwidth;
+    // C leaves in pieces of 16 elements of a row: 1.5 - 2.5 TB/s (a rank-1 update of 4096^2 through this kernel: 22 - 34 us)
+    const double c_bytes = (double)p.m * (double)p.n * es * (p.accumulate ? 2.0 : 1.0);
+    const double c_rate = (p.dtype == DT_F16 || p.dtype == DT_BF16 ? 1.5e12 : 2.2e12) * std::max(1, compute_units) / 256.0;
+    return 2.1e-6 + gather + std::max(chain, tiles * 32.0 * es * (double)p.k / bandwidth) + c_bytes / c_rate;
 }
 
 hipError_t launch_small(const GemmProblem &g, hipStream_t stream) {

@@ -98,7 +98,8 @@ def test_doubly_strided_operand_takes_generic_path():
                                                   ("f32", (40, 24, 16), KERNEL_MFMA, "mfma32_small_16x16_ksliced"),
                                                   ("f64", (40, 24, 16), KERNEL_MFMA, "mfma64_small_16x16_ksliced"),
                                                   ("f16", (600, 520, 440), KERNEL_GENERIC, "generic"),
-                                                  ("f32", (600, 520, 440), KERNEL_GENERIC, "generic")):
+                                                  ("f32", (600, 520, 440), KERNEL_MFMA, "mfma32_small_16x16_ksliced"),
+                                                  ("f32", (1200, 1040, 880), KERNEL_GENERIC, "generic")):
         a = oracle.to_storage(g.standard_normal(m * (2 * k + 3)), dtype)
         astr = (2 * k + 3, 2)
         b, bstr = make_operand(g, k, n, False, dtype)
