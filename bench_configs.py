@@ -71,7 +71,15 @@ def main():
             a, b, c = (torch.randn(n, n, device="cuda", dtype=torch.float32) for _ in range(3))
             names = []
             for bstr in ((1, n), (n, 1)):
-                for v in (1, dev.mfma_variant_count("f32")):   # the register-staged 256x256 tile, the LDS-DMA form of it
+                probe = dev.gemm_desc("f32", n, n, n, a.data_ptr(), (n, 1), b.data_ptr(), bstr, c.data_ptr(), (n, 1), kernel=KERNEL_MFMA)
+                by_name = {}
+                for v in range(1, dev.mfma_variant_count("f32") + 1):
+                    probe.variant = v
+                    try:
+                        by_name[dev.gemm_plan(probe)[2]] = v
+                    except Exception:   # a variant that does not take this product
+                        pass
+                for v in (by_name["mfma32_256x256x32_w2x4"], by_name["mfma32_dma_256x256x32_w2x4"]):   # the register-staged 256x256 tile, the LDS-DMA form of it
                     desc = dev.gemm_desc("f32", n, n, n, a.data_ptr(), (n, 1), b.data_ptr(), bstr, c.data_ptr(), (n, 1),
                                          kernel=KERNEL_MFMA, variant=v, no_split_k=True)
                     names.append(dev.gemm_plan(desc)[2])
