@@ -20,8 +20,9 @@ namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef double f64x4 __attribute__((ext_vector_type(4)));
-typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
 
 struct SmallParams {
     const void *a, *b;
@@ -31,7 +32,7 @@ struct SmallParams {
     int64_t a_rs, a_cs, b_rs, b_cs, ldc;
     int accumulate, bias_mode;
     int a_vec, b_vec;  // the operand is stored along k and every 4-k group of a row is one aligned vector
-    int slice;         // k per wave, a multiple of 16
+    int slice;         // k per wave, a multiple of the step (16 k; 32 for the 16-bit types)
     void *ksum;        // may be null: ksum[i] (+)= sum_k A[i][k]
     int ksum_accumulate;
 };
@@ -43,6 +44,7 @@ template <> struct Small<float> {
     typedef float acc_t;
     typedef f32x4 acc4;
     typedef f32x4 pack;
+    static constexpr int KL = 4;  // k values a lane supplies per step
     static __device__ __forceinline__ pack zero() { return pack{0.f, 0.f, 0.f, 0.f}; }
     static __device__ __forceinline__ pack vec(const float *p) { return *(const f32x4 *)p; }
     static __device__ __forceinline__ void set(pack &v, int c, const float *p) { v[c] = *p; }
@@ -51,7 +53,7 @@ template <> struct Small<float> {
         for (int c = 0; c < 4; c++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[c], b[c], acc, 0, 0, 0);
         return acc;
     }
-    static __device__ __forceinline__ float sum4(pack v) { return (v[0] + v[1]) + (v[2] + v[3]); }
+    static __device__ __forceinline__ float sum_pack(pack v) { return (v[0] + v[1]) + (v[2] + v[3]); }
     static __device__ __forceinline__ int out_row(int r, int q) { return 4 * q + r; }
     static __device__ __forceinline__ float load(const float *p) { return *p; }
     static __device__ __forceinline__ void store(float *p, float v) { *p = v; }
@@ -60,6 +62,7 @@ template <> struct Small<double> {
     typedef double acc_t;
     typedef f64x4 acc4;
     typedef f64x4 pack;
+    static constexpr int KL = 4;
     static __device__ __forceinline__ pack zero() { return pack{0.0, 0.0, 0.0, 0.0}; }
     static __device__ __forceinline__ pack vec(const double *p) {
         typedef double f64x2 __attribute__((ext_vector_type(2)));
@@ -72,20 +75,23 @@ template <> struct Small<double> {
         for (int c = 0; c < 4; c++) acc = __builtin_amdgcn_mfma_f64_16x16x4f64(a[c], b[c], acc, 0, 0, 0);
         return acc;
     }
-    static __device__ __forceinline__ double sum4(pack v) { return (v[0] + v[1]) + (v[2] + v[3]); }
+    static __device__ __forceinline__ double sum_pack(pack v) { return (v[0] + v[1]) + (v[2] + v[3]); }
     static __device__ __forceinline__ int out_row(int r, int q) { return 4 * r + q; }  // f64: register r is row 4 r + l / 16
     static __device__ __forceinline__ double load(const double *p) { return *p; }
     static __device__ __forceinline__ void store(double *p, double v) { *p = v; }
 };
-template <> struct Small<_Float16> {
+template <> struct Small<_Float16> {  // eight k per lane: one 16-byte load, v_mfma_f32_16x16x32_f16
     typedef float acc_t;
     typedef f32x4 acc4;
-    typedef f16x4 pack;
-    static __device__ __forceinline__ pack zero() { return pack{0, 0, 0, 0}; }
-    static __device__ __forceinline__ pack vec(const _Float16 *p) { return *(const f16x4 *)p; }
+    typedef f16x8 pack;
+    static constexpr int KL = 8;
+    static __device__ __forceinline__ pack zero() { return pack{0, 0, 0, 0, 0, 0, 0, 0}; }
+    static __device__ __forceinline__ pack vec(const _Float16 *p) { return *(const f16x8 *)p; }
     static __device__ __forceinline__ void set(pack &v, int c, const _Float16 *p) { v[c] = *p; }
-    static __device__ __forceinline__ acc4 mma(pack a, pack b, acc4 acc) { return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, acc, 0, 0, 0); }
-    static __device__ __forceinline__ float sum4(pack v) { return ((float)v[0] + (float)v[1]) + ((float)v[2] + (float)v[3]); }
+    static __device__ __forceinline__ acc4 mma(pack a, pack b, acc4 acc) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0); }
+    static __device__ __forceinline__ float sum_pack(pack v) {
+        return (((float)v[0] + (float)v[1]) + ((float)v[2] + (float)v[3])) + (((float)v[4] + (float)v[5]) + ((float)v[6] + (float)v[7]));
+    }
     static __device__ __forceinline__ int out_row(int r, int q) { return 4 * q + r; }
     static __device__ __forceinline__ float load(const _Float16 *p) { return (float)*p; }
     static __device__ __forceinline__ void store(_Float16 *p, float v) { *p = (_Float16)v; }
@@ -93,13 +99,18 @@ template <> struct Small<_Float16> {
 template <> struct Small<__bf16> {
     typedef float acc_t;
     typedef f32x4 acc4;
-    typedef i16x4 pack;
+    typedef i16x8 pack;
+    static constexpr int KL = 8;
     static __device__ __forceinline__ float widen(short b) { return __uint_as_float((uint32_t)(uint16_t)b << 16); }
-    static __device__ __forceinline__ pack zero() { return pack{0, 0, 0, 0}; }
-    static __device__ __forceinline__ pack vec(const __bf16 *p) { return *(const i16x4 *)p; }
+    static __device__ __forceinline__ pack zero() { return pack{0, 0, 0, 0, 0, 0, 0, 0}; }
+    static __device__ __forceinline__ pack vec(const __bf16 *p) { return *(const i16x8 *)p; }
     static __device__ __forceinline__ void set(pack &v, int c, const __bf16 *p) { v[c] = *(const short *)p; }
-    static __device__ __forceinline__ acc4 mma(pack a, pack b, acc4 acc) { return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, acc, 0, 0, 0); }
-    static __device__ __forceinline__ float sum4(pack v) { return (widen(v[0]) + widen(v[1])) + (widen(v[2]) + widen(v[3])); }
+    static __device__ __forceinline__ acc4 mma(pack a, pack b, acc4 acc) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float sum_pack(pack v) {
+        return ((widen(v[0]) + widen(v[1])) + (widen(v[2]) + widen(v[3]))) + ((widen(v[4]) + widen(v[5])) + (widen(v[6]) + widen(v[7])));
+    }
     static __device__ __forceinline__ int out_row(int r, int q) { return 4 * q + r; }
     static __device__ __forceinline__ float load(const __bf16 *p) { return widen(*(const short *)p); }
     static __device__ __forceinline__ void store(__bf16 *p, float v) {  // round to nearest even, quiet NaNs
@@ -115,6 +126,7 @@ template <typename T, int WAVES, bool LONG> __global__ __launch_bounds__(WAVES *
     typedef typename S::acc_t A;
     typedef typename S::acc4 A4;
     typedef typename S::pack Pack;
+    constexpr int KL = S::KL, STEP = 4 * KL, PASS = 4 * STEP;  // k per lane and step, per step of a wave, per pass
     __shared__ A part[WAVES][256];
     __shared__ A part_rows[WAVES][16];
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
@@ -134,15 +146,15 @@ template <typename T, int WAVES, bool LONG> __global__ __launch_bounds__(WAVES *
         Pack v = S::zero();
         if constexpr (BRANCHY) {  // (this order of the tests and no test per step measured best of the forms tried)
             if (!ok || kk >= k1) return v;
-            if (vec && kk + 3 < k1) return S::vec(base + kk);
+            if (vec && kk + KL - 1 < k1) return S::vec(base + kk);
 #pragma unroll
-            for (int c = 0; c < 4; c++)
+            for (int c = 0; c < KL; c++)
                 if (kk + c < k1) S::set(v, c, base + (int64_t)(kk + c) * kstride);
         } else {
-            if (vec && kk + 3 < k1) return ok ? S::vec(base + kk) : v;
+            if (vec && kk + KL - 1 < k1) return ok ? S::vec(base + kk) : v;
             const Pack z = S::zero();
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
+            for (int c = 0; c < KL; c++) {
                 S::set(v, c, base + (int64_t)max(0, min(kk + c, k1 - 1)) * kstride);
                 if (!ok || kk + c >= k1) v[c] = z[c];
             }
@@ -161,22 +173,22 @@ template <typename T, int WAVES, bool LONG> __global__ __launch_bounds__(WAVES *
         if (vec) return S::vec(base + kk);
         Pack v = S::zero();
 #pragma unroll
-        for (int c = 0; c < 4; c++) S::set(v, c, base + (int64_t)(kk + c) * kstride);
+        for (int c = 0; c < KL; c++) S::set(v, c, base + (int64_t)(kk + c) * kstride);
         return v;
     };
     auto load_pass = [&](Pack *a, Pack *b, int kb) {
-        if (LONG && kb + 64 <= k1) {
+        if (LONG && kb + PASS <= k1) {
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                a[u] = whole(ap, p.a_cs, p.a_vec, kb + 16 * u + 4 * q);
-                b[u] = whole(bp, p.b_rs, p.b_vec, kb + 16 * u + 4 * q);
+                a[u] = whole(ap, p.a_cs, p.a_vec, kb + STEP * u + KL * q);
+                b[u] = whole(bp, p.b_rs, p.b_vec, kb + STEP * u + KL * q);
             }
         } else {
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                if (BRANCHY || kb + 16 * u < k1) {  // the same in every lane: steps past the end are not loaded at all
-                    a[u] = fetch(ap, p.a_cs, row_ok, p.a_vec, kb + 16 * u + 4 * q);
-                    b[u] = fetch(bp, p.b_rs, col_ok, p.b_vec, kb + 16 * u + 4 * q);
+                if (BRANCHY || kb + STEP * u < k1) {  // the same in every lane: steps past the end are not loaded at all
+                    a[u] = fetch(ap, p.a_cs, row_ok, p.a_vec, kb + STEP * u + KL * q);
+                    b[u] = fetch(bp, p.b_rs, col_ok, p.b_vec, kb + STEP * u + KL * q);
                 } else {
                     a[u] = S::zero();
                     b[u] = S::zero();
@@ -187,7 +199,7 @@ template <typename T, int WAVES, bool LONG> __global__ __launch_bounds__(WAVES *
     auto use_pass = [&](const Pack *a, const Pack *b) {
         if (sums) {
 #pragma unroll
-            for (int u = 0; u < 4; u++) rsum += S::sum4(a[u]);
+            for (int u = 0; u < 4; u++) rsum += S::sum_pack(a[u]);
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
@@ -201,16 +213,16 @@ template <typename T, int WAVES, bool LONG> __global__ __launch_bounds__(WAVES *
     } else if constexpr (sizeof(T) < 8) {
         Pack an[4], bn[4];
         load_pass(av, bv, k0);
-        for (int kb = k0; kb < k1; kb += 128) {  // k0, k1 and kb are the same in every lane of a wave
-            if (kb + 64 < k1) load_pass(an, bn, kb + 64);
+        for (int kb = k0; kb < k1; kb += 2 * PASS) {  // k0, k1 and kb are the same in every lane of a wave
+            if (kb + PASS < k1) load_pass(an, bn, kb + PASS);
             use_pass(av, bv);
-            if (kb + 64 < k1) {
-                if (kb + 128 < k1) load_pass(av, bv, kb + 128);
+            if (kb + PASS < k1) {
+                if (kb + 2 * PASS < k1) load_pass(av, bv, kb + 2 * PASS);
                 use_pass(an, bn);
             }
         }
     } else {  // f64: two passes of operands would halve the waves a compute unit holds
-        for (int kb = k0; kb < k1; kb += 64) {
+        for (int kb = k0; kb < k1; kb += PASS) {
             load_pass(av, bv, kb);
             use_pass(av, bv);
         }
@@ -263,7 +275,7 @@ inline int small_waves(int dtype, int64_t k) {
 template <typename T, bool LONG> hipError_t launch_form(const SmallParams &p, int waves, dim3 grid, hipStream_t stream) {
     switch (waves) {
     case 16:
-        if constexpr (sizeof(T) < 8 && LONG) gemm_small_kernel<T, 16, true><<<grid, 1024, 0, stream>>>(p);
+        if constexpr (sizeof(T) < 8) gemm_small_kernel<T, 16, LONG><<<grid, 1024, 0, stream>>>(p);
         else return hipErrorInvalidValue;
         break;
     case 8: gemm_small_kernel<T, 8, LONG><<<grid, 512, 0, stream>>>(p); break;
@@ -274,7 +286,7 @@ template <typename T, bool LONG> hipError_t launch_form(const SmallParams &p, in
     return hipGetLastError();
 }
 template <typename T> hipError_t launch_t(const SmallParams &p, int waves, dim3 grid, hipStream_t stream) {
-    return p.slice > 64 ? launch_form<T, true>(p, waves, grid, stream) : launch_form<T, false>(p, waves, grid, stream);
+    return p.slice > 16 * Small<T>::KL ? launch_form<T, true>(p, waves, grid, stream) : launch_form<T, false>(p, waves, grid, stream);
 }
 
 }  // namespace
@@ -295,16 +307,23 @@ bool small_ksum_supported(const GemmProblem &p) {
 }
 
 // Estimated time, fitted to timings on a 256-CU MI355X: the launch; then the longer of (a) the chain of loads of one
-// workgroup, which grows with the whole contraction however many waves share it (3.4 ns per k, twice that for f64: the
-// 16 rows of a load instruction lie a row stride apart), and (b) the bytes all workgroups pull through the caches -- no
+// workgroup, which grows with the whole contraction however many waves share it (the 16 rows of a load instruction lie
+// a row stride apart), and (b) the bytes all workgroups pull through the caches -- no
 // operand value is shared between workgroups, so every tile fetches its 16 rows and 16 columns again (5 - 8 TB/s over
 // the whole chip); an operand that is not stored along k costs a 2- or 4-byte load per value on top, and so does C.
 double small_time(const GemmProblem &p, int compute_units) {
     const double tiles = (double)((p.m + 15) / 16) * (double)((p.n + 15) / 16);
     const double es = (double)elem_size(p.dtype);
-    const double chain = std::max(0.5e-6, (double)p.k * (p.dtype == DT_F64 ? 6.8e-9 : 3.4e-9));
-    const double gather = p.dtype == DT_F64 ? 0.0 : (p.dtype == DT_F32 ? 0.4e-6 : 0.9e-6) * ((p.a_cs != 1) + (p.b_rs != 1));
-    const double bandwidth = (p.dtype == DT_F64 ? 8e12 : p.dtype == DT_F32 ? 7.5e12 : 5e12) * std::max(1, compute_units) / 256.0;
+    const bool half = p.dtype == DT_F16 || p.dtype == DT_BF16;
+    const int strided = (p.a_cs != 1) + (p.b_rs != 1);  // operands not stored along k
+    // per k: 16-byte loads of 16 rows (16-bit types: eight k each, 1.7 ns; f32: four k, 3.4 ns; f64: 6.8 ns)
+    const double per_k = p.dtype == DT_F64 ? 6.8e-9 : half ? 1.7e-9 : 3.4e-9;
+    const double chain = std::max(0.5e-6, (double)p.k * per_k);
+    // an operand that is not stored along k comes one 2- or 4-byte load per value: a fixed cost in the chain, and, where
+    // the operand is large, a rate (16 x 4096 x 4096: f16 9.8 us A.B^T against 22.9 us A.B, f32 18.9 against 24.1)
+    const double strided_values = (p.a_cs != 1 ? (double)p.m * (double)p.k : 0.0) + (p.b_rs != 1 ? (double)p.k * (double)p.n : 0.0);
+    const double gather = p.dtype == DT_F64 ? 0.0 : (half ? 0.9e-6 : 0.4e-6) * strided + strided_values / (half ? 1.3e12 : 3.3e12);
+    const double bandwidth = (p.dtype == DT_F64 ? 8e12 : 7.5e12) * std::max(1, compute_units) / 256.0;
     // C leaves in pieces of 16 elements of a row: 1.5 - 2.5 TB/s (a rank-1 update of 4096^2 through this kernel: 22 - 34 us)
     const double c_bytes = (double)p.m * (double)p.n * es * (p.accumulate ? 2.0 : 1.0);
     const double c_rate = (p.dtype == DT_F16 || p.dtype == DT_BF16 ? 1.5e12 : 2.2e12) * std::max(1, compute_units) / 256.0;
@@ -314,7 +333,8 @@ double small_time(const GemmProblem &p, int compute_units) {
 hipError_t launch_small(const GemmProblem &g, hipStream_t stream) {
     if (!small_supported(g) || g.splits > 1) return hipErrorInvalidValue;
     const size_t es = elem_size(g.dtype);
-    const uintptr_t vmask = 4 * es >= 16 ? 15 : 4 * es - 1;  // four elements: 8 bytes (16-bit), 16 bytes (f32; f64 as two halves)
+    const int kl = es == 2 ? 8 : 4;  // k values per lane and step: 16 bytes (f64: 32 bytes as two halves)
+    const uintptr_t vmask = 15;
     SmallParams p;
     p.a = g.a; p.b = g.b; p.c = g.c; p.bias = g.bias;
     p.m = (int)g.m; p.n = (int)g.n; p.k = (int)g.k;
@@ -328,7 +348,8 @@ hipError_t launch_small(const GemmProblem &g, hipStream_t stream) {
     p.ksum = (g.ksum && g.ksum_of == KSUM_OF_A) ? g.ksum : nullptr;
     p.ksum_accumulate = g.ksum_accumulate;
     const int waves = small_waves(g.dtype, g.k);
-    p.slice = (int)(((g.k + waves - 1) / waves + 15) / 16 * 16);
+    const int step = 4 * kl;
+    p.slice = (int)(((g.k + waves - 1) / waves + step - 1) / step * step);
     const dim3 grid((unsigned)(((g.m + 15) / 16) * p.tiles_n));
     switch (g.dtype) {
     case DT_F32: return launch_t<float>(p, waves, grid, stream);

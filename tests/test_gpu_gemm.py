@@ -444,8 +444,8 @@ def test_split_k_register_staged_family(dtype, splits):
     for i, (m, k, n, layout, pads) in enumerate([(264, 1000, 200, "nn", (8, 8, 8)), (130, 2057, 72, "nt", (1, 3, 5)),
                                                  (96, 4104, 256, "tn", (0, 8, 0))]):
         run_case(dtype, m, k, n, layout, bool(i % 2), KERNEL_MFMA, 0, split_k=splits, seed=700 + i, pads=pads)
-    a = dev.zeros(dtype, (256, 4104))
-    d = dev.gemm_desc(dtype, 256, 4104, 256, a.ptr, (4104, 1), a.ptr, (1, 4104), a.ptr, (256, 1))
+    a = dev.zeros(dtype, (512, 4104))   # (at 256 x 4104 x 256 the small-product kernel is the faster plan)
+    d = dev.gemm_desc(dtype, 512, 4104, 512, a.ptr, (4104, 1), a.ptr, (1, 4104), a.ptr, (512, 1))
     assert "splitk" in dev.gemm_plan(d)[2] and "dma" not in dev.gemm_plan(d)[2], dev.gemm_plan(d)
 
 

@@ -124,7 +124,7 @@ def test_linear_backward_seeded(dtype, rows, i, o):
 # gradient is produced by the same launch (one more MFMA per A fragment in the work items of tile column 0) instead of
 # by the reduction kernels.  Both tile families, split and unsplit contractions, edge tiles in either direction.
 FUSED_SHAPES = [(8192, 1024, 1024), (4096, 1024, 4096), (512, 256, 512), (640, 264, 1000), (128, 64, 8), (2048, 4096, 1024),
-                (64, 1024, 1024), (2048, 128, 256), (4096, 256, 4096), (8192, 1024, 4096)]
+                (64, 1024, 1024), (2048, 128, 256), (4096, 128, 256), (4096, 256, 4096), (8192, 1024, 4096)]
 
 
 def test_fused_shapes_reach_every_tile_family_that_sums_rows():
