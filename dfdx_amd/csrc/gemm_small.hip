@@ -3,12 +3,14 @@
 // A product of a few MFLOP (a Linear layer on 64 rows, the reference's own test shapes) is bound by the chain
 // launch -> load -> MFMA -> store, not by any rate, and the tiled kernels walk k in steps behind one another (9.7 us for
 // f32 64 x 512 x 256 as four k pieces plus the combining launch).  Here every wave of a workgroup takes one slice of k,
-// requests ALL the operand values of a pass (64 k) at once -- straight into the registers the MFMA reads, no LDS staging,
-// any strides --, the next pass's behind them where the registers allow, runs its MFMA chain on two accumulators, and the
-// slices meet in LDS, added in wave order (the result does not depend on timing).  Lane l supplies A[row l % 16][k] and B[k][col l % 16] for the four consecutive
-// k = 16 s + 4 (l / 16) + c, c < 4, of step s: one vector load where the operand is stored along k and aligned.  The
-// 16-bit types feed the four values to one v_mfma_f32_16x16x16, f32 and f64 to four v_mfma_*_16x16x4 (whose lane group
-// l / 16 is the k index: any bijection between (lane group, instruction) and k serves, as long as A and B share it).
+// requests ALL the operand values of a pass (four steps) at once -- straight into the registers the MFMA reads, no LDS
+// staging, any strides --, the next pass's behind them where the registers allow, runs its MFMA chain on two
+// accumulators, and the slices meet in LDS, added in wave order (the result does not depend on timing).  Lane l supplies
+// A[row l % 16][k] and B[k][col l % 16] for KL consecutive k per step, k = 4 KL s + KL (l / 16) + c, c < KL: one 16-byte
+// load where the operand is stored along k and aligned.  The 16-bit types take KL = 8 and feed the eight values to one
+// v_mfma_f32_16x16x32 (with four values and the 16x16x16 instruction the same kernel needed twice the loads:
+// 16 x 4096 x 4096 f16 16.7 -> 9.8 us); f32 and f64 take KL = 4 and four v_mfma_*_16x16x4 (whose lane group l / 16 is
+// the k index: any bijection between (lane group, instruction) and k serves, as long as A and B share it).
 //
 // Optional second result: the sums of A's rows over k, from the values the workgroups of tile column 0 hold anyway
 // (Linear's bias gradient out of the weight-gradient launch).
