@@ -327,7 +327,7 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
         if (dv) {
             // that family's estimate ranks its own tiles and split counts; on products of a few microseconds it runs
             // 1 - 2 us above the clock, and 8 us above it for a split plan
-            t_dma -= splits > 1 ? 6.5e-6 : 1.5e-6;
+            t_dma -= splits > 1 ? 6.5e-6 : 1.0e-6;
             *plan = t_small < t_dma ? small_plan : Plan{DFDX_ROCM_KERNEL_MFMA, dv + mfma16_dma_first_variant() - 1, splits};
             return DFDX_ROCM_OK;
         }
