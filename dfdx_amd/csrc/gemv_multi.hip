@@ -82,7 +82,7 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_c
     constexpr bool PAIRS = sizeof(T) == 2;
     typedef typename std::conditional<PAIRS, T, float>::type S;  // what the vector slices are kept as
     __shared__ __align__(16) S vsh[R][kchunk_of(R)];
-    __shared__ float red[4][64 * VEC];
+    __shared__ float red[4][R < 4 ? R : 4][64 * VEC];
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int j0 = (blockIdx.x * 64 + lane) * VEC;
     const int k0 = blockIdx.y * p.kchunk;
@@ -162,16 +162,21 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_c
             }
         }
     }
+    // the four waves' sums meet in LDS, up to four vectors at a time (two barriers per group, not per vector)
+    constexpr int G = R < 4 ? R : 4;
 #pragma unroll
-    for (int r = 0; r < R; r++) {  // the four waves' sums of one vector at a time through the same buffer
-        if (r < p.r) {             // the same in every thread
+    for (int r0 = 0; r0 < R; r0 += G) {
+        if (r0 < p.r) {  // the same in every thread
 #pragma unroll
-            for (int e = 0; e < VEC; e++) red[wave][lane * VEC + e] = acc[r][e];
+            for (int g = 0; g < G; g++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) red[wave][g][lane * VEC + e] = acc[r0 + g][e];
             __syncthreads();
-            for (int o = tid; o < 64 * VEC; o += 256) {
-                const int j = blockIdx.x * 64 * VEC + o;
-                if (j >= p.j) continue;
-                const float v = ((red[0][o] + red[1][o]) + red[2][o]) + red[3][o];
+            for (int o = tid; o < G * 64 * VEC; o += 256) {
+                const int g = o / (64 * VEC), c = o % (64 * VEC);
+                const int j = blockIdx.x * 64 * VEC + c, r = r0 + g;
+                if (j >= p.j || r >= p.r) continue;
+                const float v = ((red[0][g][c] + red[1][g][c]) + red[2][g][c]) + red[3][g][c];
                 if (p.kslices > 1) p.ws[((int64_t)blockIdx.y * p.r + r) * p.j + j] = v;
                 else finish<T>(p, r, j, v);
             }
