@@ -151,21 +151,24 @@ template <typename T> __global__ __launch_bounds__(256) void gemv_dots_kernel(co
     }
 }
 
-template <typename T> __global__ __launch_bounds__(64) void gemv_combine_kernel(const Params p) {
-    const int j = blockIdx.x * 64 + threadIdx.x;
-    if (j >= p.j) return;
-    const float *src = p.ws + j;
+// Eight lanes per output: lane `part` adds the slices part, part + 8, ... (their loads in flight together), then the
+// eight partial sums meet in a fixed tree of three exchanges: one round trip to the workspace for up to 64 slices.
+template <typename T> __global__ __launch_bounds__(256) void gemv_combine_kernel(const Params p) {
+    const int j = blockIdx.x * 32 + threadIdx.x / 8, part = threadIdx.x % 8;
+    const bool in = j < p.j;
+    const float *src = p.ws + (in ? j : 0);
     float v = 0.0f;
-    int s = 0;
-    for (; s + 8 <= p.kslices; s += 8) {  // eight loads in flight, added in slice order
+    for (int s = part; s < p.kslices; s += 64) {
         float t[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++) t[u] = src[(int64_t)(s + u) * p.j];
+        for (int u = 0; u < 8; u++) t[u] = (s + 8 * u < p.kslices) ? src[(int64_t)(s + 8 * u) * p.j] : 0.0f;
 #pragma unroll
         for (int u = 0; u < 8; u++) v += t[u];
     }
-    for (; s < p.kslices; s++) v += src[(int64_t)s * p.j];
-    finish<T>(p, j, v);
+    v += __shfl_xor(v, 1, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 4, 64);
+    if (in && part == 0) finish<T>(p, j, v);
 }
 
 struct Shape {
@@ -240,7 +243,7 @@ template <typename T> hipError_t launch_t(const Shape &s, hipStream_t stream) {
         dim3 grid((unsigned)((p.j + 3) / 4), (unsigned)p.kslices);
         gemv_dots_kernel<T><<<grid, 256, 0, stream>>>(p);
     }
-    if (p.kslices > 1) gemv_combine_kernel<T><<<dim3((unsigned)((p.j + 63) / 64)), 64, 0, stream>>>(p);
+    if (p.kslices > 1) gemv_combine_kernel<T><<<dim3((unsigned)((p.j + 31) / 32)), 256, 0, stream>>>(p);
     return hipGetLastError();
 }
 
