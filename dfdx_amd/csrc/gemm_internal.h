@@ -154,6 +154,10 @@ bool gemv_multi_supported(const GemmProblem &p);
 size_t gemv_multi_workspace_bytes(const GemmProblem &p);
 hipError_t launch_gemv_multi(const GemmProblem &p, hipStream_t stream);
 
+// ---- thin contractions with large outputs on the matrix cores (gemm_small.hip): k <= 32, f32 / f16 / bf16, row-major C ----
+bool thin_mfma_supported(const GemmProblem &p);
+hipError_t launch_thin_mfma(const GemmProblem &p, hipStream_t stream);
+
 // ---- rank-1 updates and thin contractions, k = 1 .. 8 (rank1.hip): every dtype, any operand strides, row-major C ----
 bool rank1_supported(const GemmProblem &p);
 hipError_t launch_rank1(const GemmProblem &p, hipStream_t stream);

@@ -362,4 +362,192 @@ hipError_t launch_small(const GemmProblem &g, hipStream_t stream) {
     }
 }
 
+
+namespace {
+
+// ---- thin contractions (k <= 32) with large outputs: the matrix cores as a row-streaming kernel ----
+//
+// A product such as 4096 x 16 x 4096 writes 2 K bytes of C per byte it reads: what bounds it is how C leaves the chip.
+// The tiled kernels pad k to their step and reach 2 - 3 TB/s on it.  Here a wave keeps the fragments of 64 columns of B
+// in registers (four 16-column tiles, every k of the product) and walks down the rows of A sixteen at a time: one 16-byte
+// load per lane is a whole 16 x k piece of a row-major A, four (f32: sixteen) MFMAs make a 16 x 64 strip of C, and the
+// strip goes through a wave-private LDS tile so that it leaves as whole rows -- eight (f32: sixteen) lanes with 16 bytes
+// each per row, never the 32-byte row pieces of the accumulator layout.  The MFMA's operands are swapped (B's columns as
+// its rows), which leaves four consecutive columns of one row of C in a lane: the LDS tile is written 16 bytes at a time.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+struct ThinParams {
+    const void *a, *b;
+    void *c;
+    const void *bias;
+    int m, n, k;
+    int64_t a_rs, a_cs, b_rs, b_cs, ldc;
+    int accumulate, bias_mode;
+    int a_vec, b_vec;      // stored along k, every k group of a row / column one aligned 16-byte vector
+    int rows_per_block;    // a multiple of 16
+};
+
+template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thin_kernel(const ThinParams p) {
+    typedef Small<T> S;
+    typedef typename S::pack Pack;
+    constexpr int KL = S::KL, STEP = 4 * KL;
+    constexpr int PIECE = 16 / (int)sizeof(T);  // elements of C a lane stores at once
+    constexpr int PPR = 64 / PIECE;             // such pieces per row of the strip
+    constexpr int RPI = 64 / PPR;               // rows of the strip one store instruction covers
+    constexpr int H = 16 / RPI;                 // store instructions per strip
+    constexpr int LDW = 68;                     // floats per row of the LDS tile (64 + 4: the rows start four banks apart)
+    __shared__ float tile[4][16 * LDW];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r16 = lane % 16, q = lane / 16;
+    const int n0 = blockIdx.x * 256 + wave * 64;
+    if (n0 >= p.n) return;  // (no workgroup barrier below: a wave may leave alone)
+    const int m_begin = blockIdx.y * p.rows_per_block, m_end = min(p.m, m_begin + p.rows_per_block);
+    // a group of k values that the end of k cuts: every load from an address inside the operand, zeros put in afterwards
+    auto fetch = [&](const T *base, int64_t kstride, bool ok, bool vec, int kk) -> Pack {
+        Pack v = S::zero();
+        if (!ok || kk >= p.k) return v;  // (k = 16 in a 16-bit type: half the lanes of every load)
+        if (vec && kk + KL <= p.k) return S::vec(base + kk);
+        const Pack z = S::zero();
+#pragma unroll
+        for (int c = 0; c < KL; c++) {
+            S::set(v, c, base + (int64_t)min(kk + c, p.k - 1) * kstride);
+            if (kk + c >= p.k) v[c] = z[c];
+        }
+        return v;
+    };
+    Pack bf[STEPS][4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const int col = n0 + 16 * t + r16;
+        const bool ok = col < p.n;
+        const T *base = (const T *)p.b + (int64_t)(ok ? col : 0) * p.b_cs;
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) bf[s][t] = fetch(base, p.b_rs, ok, p.b_vec, STEP * s + KL * q);
+    }
+    auto rows_of_a = [&](int m0, Pack (&af)[STEPS]) {
+        const T *base = (const T *)p.a + (int64_t)min(m0 + r16, p.m - 1) * p.a_rs;
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) af[s] = fetch(base, p.a_cs, true, p.a_vec, STEP * s + KL * q);
+    };
+    const int pc = lane % PPR, prow = lane / PPR;
+    const int col = n0 + PIECE * pc;
+    const bool piece_ok = col < p.n;  // n is a multiple of the piece
+    float cb[PIECE];
+#pragma unroll
+    for (int i = 0; i < PIECE; i++) cb[i] = (p.bias_mode == BIAS_PER_COL && piece_ok) ? S::load((const T *)p.bias + col + i) : 0.0f;
+    float *mine = tile[wave];
+    Pack next[STEPS];
+    rows_of_a(m_begin, next);
+    for (int m0 = m_begin; m0 < m_end; m0 += 16) {
+        Pack cur[STEPS];
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) cur[s] = next[s];
+        if (m0 + 16 < m_end) rows_of_a(m0 + 16, next);
+        u32x4 old[H];
+#pragma unroll
+        for (int h = 0; h < H; h++) old[h] = u32x4{0u, 0u, 0u, 0u};
+        if (p.accumulate) {
+#pragma unroll
+            for (int h = 0; h < H; h++) {
+                const int row = m0 + prow + RPI * h;
+                if (row < m_end && piece_ok) old[h] = *(const u32x4 *)((const T *)p.c + (int64_t)row * p.ldc + col);
+            }
+        }
+        f32x4 acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) acc[t] = S::mma(bf[s][t], cur[s], acc[t]);
+        }
+        // register r of lane (r16, q), tile t = C[m0 + r16][n0 + 16 t + 4 q + r]
+#pragma unroll
+        for (int t = 0; t < 4; t++) *(f32x4 *)&mine[r16 * LDW + 16 * t + 4 * q] = acc[t];
+        // the lanes of a wave run its LDS instructions in order: no wait, but the compiler must keep the order too
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int h = 0; h < H; h++) {
+            const int row_l = prow + RPI * h, row = m0 + row_l;
+            float v[PIECE];
+#pragma unroll
+            for (int i = 0; i < PIECE; i += 4) {
+                const f32x4 x = *(const f32x4 *)&mine[row_l * LDW + PIECE * pc + i];
+                v[i] = x[0]; v[i + 1] = x[1]; v[i + 2] = x[2]; v[i + 3] = x[3];
+            }
+            if (row < m_end && piece_ok) {
+                const float rb = p.bias_mode == BIAS_PER_ROW ? S::load((const T *)p.bias + row) : 0.0f;
+                T was[PIECE], out[PIECE];
+                __builtin_memcpy(was, &old[h], 16);
+#pragma unroll
+                for (int i = 0; i < PIECE; i++) {
+                    float x = v[i] + cb[i];
+                    if (p.bias_mode == BIAS_PER_ROW) x += rb;
+                    if (p.accumulate) x += S::load(&was[i]);
+                    S::store(&out[i], x);
+                }
+                u32x4 raw;
+                __builtin_memcpy(&raw, out, 16);
+                *(u32x4 *)((T *)p.c + (int64_t)row * p.ldc + col) = raw;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+template <typename T> hipError_t launch_thin_t(const ThinParams &p, dim3 grid, hipStream_t stream) {
+    if (p.k <= 4 * Small<T>::KL) gemm_thin_kernel<T, 1><<<grid, 256, 0, stream>>>(p);
+    else if constexpr (sizeof(T) == 4) gemm_thin_kernel<T, 2><<<grid, 256, 0, stream>>>(p);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+// rows per workgroup: as many as leave a thousand workgroups (the fragments of B are loaded once per workgroup)
+inline int thin_rows_per_block(const GemmProblem &g) {
+    const int64_t blocks_n = (g.n + 255) / 256;
+    int rows = 256;
+    while (rows > 16 && blocks_n * ((g.m + rows - 1) / rows) < 1024) rows /= 2;
+    return rows;
+}
+
+}  // namespace
+
+// k <= 32 and a large output, row-major with 16-byte aligned rows of whole 16-byte pieces.
+bool thin_mfma_supported(const GemmProblem &g) {
+    if (g.dtype != DT_F32 && g.dtype != DT_F16 && g.dtype != DT_BF16) return false;
+    if (g.k < 1 || g.k > 32 || g.m < 64 || g.n < 64 || g.reduce || g.nb1 * g.nb2 != 1) return false;
+    if (g.m >= (1ll << 30) || g.n >= (1ll << 30)) return false;
+    const int64_t es = (int64_t)elem_size(g.dtype), piece = 16 / es;
+    if (g.c_cs != 1 || g.c_rs < g.n || g.c_rs % piece || g.n % piece || ((uintptr_t)g.c & 15)) return false;
+    // below these sizes of C the small-product and the tiled kernels are as fast or faster (f32 past k = 16 takes two
+    // rounds of MFMAs per strip and only pays on outputs that leave the last-level cache)
+    if (g.m * g.n * es < (es == 2 ? (1ll << 20) : g.k <= 16 ? (4ll << 20) : (64ll << 20))) return false;
+    const int rows = thin_rows_per_block(g);
+    if ((g.m + rows - 1) / rows > 65535) return false;  // row blocks are grid.y
+    const uintptr_t mask = (uintptr_t)es - 1;
+    return (((uintptr_t)g.a | (uintptr_t)g.b | (uintptr_t)g.bias) & mask) == 0;
+}
+
+hipError_t launch_thin_mfma(const GemmProblem &g, hipStream_t stream) {
+    if (!thin_mfma_supported(g)) return hipErrorInvalidValue;
+    const int64_t vq = 16 / (int64_t)elem_size(g.dtype);
+    ThinParams p;
+    p.a = g.a; p.b = g.b; p.c = g.c; p.bias = g.bias;
+    p.m = (int)g.m; p.n = (int)g.n; p.k = (int)g.k;
+    p.a_rs = g.a_rs; p.a_cs = g.a_cs; p.b_rs = g.b_rs; p.b_cs = g.b_cs; p.ldc = g.c_rs;
+    p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
+    p.a_vec = g.a_cs == 1 && g.a_rs % vq == 0 && ((uintptr_t)g.a & 15) == 0;
+    p.b_vec = g.b_rs == 1 && g.b_cs % vq == 0 && ((uintptr_t)g.b & 15) == 0;
+    p.rows_per_block = thin_rows_per_block(g);
+    const dim3 grid((unsigned)((g.n + 255) / 256), (unsigned)((g.m + p.rows_per_block - 1) / p.rows_per_block));
+    switch (g.dtype) {
+    case DT_F32: return launch_thin_t<float>(p, grid, stream);
+    case DT_F16: return launch_thin_t<_Float16>(p, grid, stream);
+    case DT_BF16: return launch_thin_t<__bf16>(p, grid, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 }  // namespace dfdx_rocm

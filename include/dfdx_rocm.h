@@ -63,7 +63,7 @@ enum {
     DFDX_ROCM_KERNEL_AUTO = 0,
     DFDX_ROCM_KERNEL_GENERIC = 1, /* any strides, any dtype (scalar loads, LDS tiled)   */
     DFDX_ROCM_KERNEL_MFMA = 2,    /* matrix-core kernels; variant chosen by `variant`   */
-    DFDX_ROCM_KERNEL_GEMV = 3     /* bandwidth-bound: M or N of 1..8, K of 1..8         */
+    DFDX_ROCM_KERNEL_GEMV = 3     /* bandwidth-bound: M or N of 1..8, K of 1..32        */
 };
 
 /* ---- device context -----------------------------------------------------

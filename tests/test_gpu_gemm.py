@@ -414,7 +414,9 @@ def test_thin_contractions(dtype, k):
     for i, (m, n) in enumerate([(2048, 1024), (3, 5), (130, 24), (515, 257), (1000, 3)]):
         a = dev.zeros(dtype, (max(m, n) * k,))
         plan = dev.gemm_plan(dev.gemm_desc(dtype, m, k, n, a.ptr, (k, 1), a.ptr, (n, 1), a.ptr, (n, 1)))
-        if dtype in ("f32", "f64") or k <= 4:   # 16-bit types: up to k = 4 (beyond, the matrix-core kernels are as fast)
+        if i == 0 and dtype != "f64" and k >= 3:   # a large row-major output: the thin contraction on the matrix cores
+            assert plan[0] == KERNEL_GEMV and plan[2] == "thin_k_mfma", plan
+        elif dtype in ("f32", "f64") or k <= 4:   # 16-bit types: up to k = 4 (beyond, the matrix-core kernels are as fast)
             assert plan[0] == KERNEL_GEMV and plan[2] == "thin_k", plan
         else:
             assert plan[2] != "thin_k", plan
@@ -422,6 +424,38 @@ def test_thin_contractions(dtype, k):
             run_case(dtype, m, k, n, layout, bool(i % 2), KERNEL_AUTO, 0, bias=(i % 3 == 0), c_colmajor=(i % 3 == 1), seed=40 + i, pads=(i % 3, 2 * (i % 2), 3 * (i % 2)))
     a = dev.zeros(dtype, (4096,))
     assert dev.gemm_plan(dev.gemm_desc(dtype, 64, 9, 64, a.ptr, (9, 1), a.ptr, (64, 1), a.ptr, (64, 1)))[2] != "thin_k"
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("k", [3, 9, 16, 17, 31, 32])
+def test_thin_contractions_on_matrix_cores(dtype, k):
+    """k <= 32 with an output of megabytes (a low-rank factor applied to a batch of rows, the product that follows a
+    projection to a handful of features): the row-streaming matrix-core kernel -- all four operand layouts, rows and
+    columns that end inside a strip, padded rows, beta, bias along the columns and (column-major C) along the rows."""
+    from dfdx_amd.rocm import KERNEL_GEMV
+    dev = device()
+    big = dtype == "f32" and k > 16   # f32 takes two rounds of MFMAs there and is planned for outputs of 64 MB and more
+    shapes = [(4096, 4096), (4104, 4100)] if big else [(2048, 1024), (1030, 2056), (4100, 520), (520, 8200), (2048, 1028)]
+    for i, (m, n) in enumerate(shapes):
+        a = dev.zeros(dtype, (max(m, n) * k,))
+        c = dev.zeros(dtype, (m * n,))
+        piece = 4 if dtype == "f32" else 8
+        d = dev.gemm_desc(dtype, m, k, n, a.ptr, (k, 1), a.ptr, (n, 1), c.ptr, (n, 1))
+        plan = dev.gemm_plan(d)
+        if n % piece == 0:
+            assert plan[0] == KERNEL_GEMV and plan[2] == "thin_k_mfma", plan
+        else:
+            assert plan[2] != "thin_k_mfma", plan    # rows that are not whole 16-byte pieces go to the other kernels
+        del a, c
+        for j, layout in enumerate(LAYOUTS):
+            if big and j % 2 != i % 2:
+                continue
+            colmajor = (i + j) % 4 == 3 and m % piece == 0
+            run_case(dtype, m, k, n, layout, bool((i + j) % 2), KERNEL_AUTO, 0, bias=(j % 3 != 1), c_colmajor=colmajor,
+                     seed=90 + 4 * i + j, pads=(j % 3, 2 * (i % 2), 8 * (j % 2)))
+    # small outputs stay with the other kernels
+    a = dev.zeros(dtype, (65536,))
+    assert dev.gemm_plan(dev.gemm_desc(dtype, 256, 16, 256, a.ptr, (16, 1), a.ptr, (256, 1), a.ptr, (256, 1)))[2] != "thin_k_mfma"
 
 
 # ------------------------------------------------------------------ split-k --
