@@ -370,7 +370,7 @@ namespace {
 // A product such as 4096 x 16 x 4096 writes 2 K bytes of C per byte it reads: what bounds it is how C leaves the chip.
 // The tiled kernels pad k to their step and reach 2 - 3 TB/s on it.  Here a wave keeps the fragments of 64 columns of B
 // in registers (four 16-column tiles, every k of the product) and walks down the rows of A sixteen at a time: one 16-byte
-// load per lane is a whole 16 x k piece of a row-major A, four (f32: sixteen) MFMAs make a 16 x 64 strip of C, and the
+// load per lane (f32: four 4-byte loads) is a whole 16 x k piece of a row-major A, four (f32: sixteen) MFMAs make a 16 x 64 strip of C, and the
 // strip goes through a wave-private LDS tile so that it leaves as whole rows -- eight (f32: sixteen) lanes with 16 bytes
 // each per row, never the 32-byte row pieces of the accumulator layout.  The MFMA's operands are swapped (B's columns as
 // its rows), which leaves four consecutive columns of one row of C in a lane: the LDS tile is written 16 bytes at a time.
@@ -401,16 +401,44 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
     const int n0 = blockIdx.x * 256 + wave * 64;
     if (n0 >= p.n) return;  // (no workgroup barrier below: a wave may leave alone)
     const int m_begin = blockIdx.y * p.rows_per_block, m_end = min(p.m, m_begin + p.rows_per_block);
-    // a group of k values that the end of k cuts: every load from an address inside the operand, zeros put in afterwards
-    auto fetch = [&](const T *base, int64_t kstride, bool ok, bool vec, int kk) -> Pack {
+    // The k values of step s that lane group q supplies.  16-bit types: the eight consecutive ones 32 s + 8 q + c, one
+    // 16-byte load where the operand is stored along k (a group that the end of k cuts: every load from an address inside
+    // the operand, zeros put in afterwards; a group beyond k: nothing loaded).  f32: the c-th 16x16x4 MFMA of a step takes
+    // k = 8 (c / 2) + 2 (c % 2) + {0, 4, 1, 5}[q] -- the order in which the tiled f32 kernels contract (their 32x32x2
+    // MFMAs take the pairs (0, 4), (1, 5), (2, 6), (3, 7) of every eight k), so that a product gives the same bits
+    // whether it comes here as one tall matrix or goes to them as a batch.
+    auto fetch = [&](const T *base, int64_t kstride, bool ok, bool vec, int s) -> Pack {
         Pack v = S::zero();
-        if (!ok || kk >= p.k) return v;  // (k = 16 in a 16-bit type: half the lanes of every load)
-        if (vec && kk + KL <= p.k) return S::vec(base + kk);
         const Pack z = S::zero();
+        if constexpr (sizeof(T) == 4) {
+            // loaded as k = 16 s + 4 q + j (one vector where the operand is stored along k), then the wave's halves
+            // trade the odd and even values: two v_permlane32_swap put every value where the order above wants it
+            const int kk = STEP * s + 4 * q;
+            Pack x = S::zero();
+            if (ok && kk < p.k) {
+                if (vec && kk + 4 <= p.k) {
+                    x = S::vec(base + kk);
+                } else {
 #pragma unroll
-        for (int c = 0; c < KL; c++) {
-            S::set(v, c, base + (int64_t)min(kk + c, p.k - 1) * kstride);
-            if (kk + c >= p.k) v[c] = z[c];
+                    for (int j = 0; j < 4; j++) {
+                        S::set(x, j, base + (int64_t)min(kk + j, p.k - 1) * kstride);
+                        if (kk + j >= p.k) x[j] = 0.0f;
+                    }
+                }
+            }
+            const auto r01 = __builtin_amdgcn_permlane32_swap(__float_as_uint(x[0]), __float_as_uint(x[1]), false, false);
+            const auto r23 = __builtin_amdgcn_permlane32_swap(__float_as_uint(x[2]), __float_as_uint(x[3]), false, false);
+            v[0] = __uint_as_float(r01[0]); v[1] = __uint_as_float(r23[0]);
+            v[2] = __uint_as_float(r01[1]); v[3] = __uint_as_float(r23[1]);
+        } else {
+            const int kk = STEP * s + KL * q;
+            if (!ok || kk >= p.k) return v;
+            if (vec && kk + KL <= p.k) return S::vec(base + kk);
+#pragma unroll
+            for (int c = 0; c < KL; c++) {
+                S::set(v, c, base + (int64_t)min(kk + c, p.k - 1) * kstride);
+                if (kk + c >= p.k) v[c] = z[c];
+            }
         }
         return v;
     };
@@ -421,12 +449,12 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
         const bool ok = col < p.n;
         const T *base = (const T *)p.b + (int64_t)(ok ? col : 0) * p.b_cs;
 #pragma unroll
-        for (int s = 0; s < STEPS; s++) bf[s][t] = fetch(base, p.b_rs, ok, p.b_vec, STEP * s + KL * q);
+        for (int s = 0; s < STEPS; s++) bf[s][t] = fetch(base, p.b_rs, ok, p.b_vec, s);
     }
     auto rows_of_a = [&](int m0, Pack (&af)[STEPS]) {
         const T *base = (const T *)p.a + (int64_t)min(m0 + r16, p.m - 1) * p.a_rs;
 #pragma unroll
-        for (int s = 0; s < STEPS; s++) af[s] = fetch(base, p.a_cs, true, p.a_vec, STEP * s + KL * q);
+        for (int s = 0; s < STEPS; s++) af[s] = fetch(base, p.a_cs, true, p.a_vec, s);
     };
     const int pc = lane % PPR, prow = lane / PPR;
     const int col = n0 + PIECE * pc;

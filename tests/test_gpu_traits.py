@@ -110,7 +110,7 @@ def test_matmul_transpose(dtype, dims):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
-@pytest.mark.parametrize("dims", [(5, 4, 3, 2), (6, 40, 64, 72), (3, 200, 136, 264)])
+@pytest.mark.parametrize("dims", [(5, 4, 3, 2), (6, 40, 64, 72), (3, 200, 136, 264), (8, 512, 16, 1024), (4, 1024, 24, 1024)])
 def test_matmul_broadcast(dtype, dims):
     """Br == per-slice 2-D products, grad_rhs == sum over slices (mod.rs:429-457); and Br == Batch3 with
     the rhs stacked, EXACTLY, for out and grad_lhs (mod.rs:460-473)."""
