@@ -385,6 +385,8 @@ struct ThinParams {
     int accumulate, bias_mode;
     int a_vec, b_vec;      // stored along k, every k group of a row / column one aligned 16-byte vector
     int rows_per_block;    // a multiple of 16
+    int nb2;               // batches: blockIdx.z = i1 * nb2 + i2
+    int64_t a_b1, a_b2, b_b1, b_b2, c_b1, c_b2;
 };
 
 template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thin_kernel(const ThinParams p) {
@@ -401,6 +403,10 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
     const int n0 = blockIdx.x * 256 + wave * 64;
     if (n0 >= p.n) return;  // (no workgroup barrier below: a wave may leave alone)
     const int m_begin = blockIdx.y * p.rows_per_block, m_end = min(p.m, m_begin + p.rows_per_block);
+    const int i1 = blockIdx.z / p.nb2, i2 = blockIdx.z % p.nb2;
+    const T *a_mat = (const T *)p.a + i1 * p.a_b1 + i2 * p.a_b2;
+    const T *b_mat = (const T *)p.b + i1 * p.b_b1 + i2 * p.b_b2;
+    T *c_mat = (T *)p.c + i1 * p.c_b1 + i2 * p.c_b2;
     // The k values of step s that lane group q supplies.  16-bit types: the eight consecutive ones 32 s + 8 q + c, one
     // 16-byte load where the operand is stored along k (a group that the end of k cuts: every load from an address inside
     // the operand, zeros put in afterwards; a group beyond k: nothing loaded).  f32: the c-th 16x16x4 MFMA of a step takes
@@ -447,12 +453,12 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
     for (int t = 0; t < 4; t++) {
         const int col = n0 + 16 * t + r16;
         const bool ok = col < p.n;
-        const T *base = (const T *)p.b + (int64_t)(ok ? col : 0) * p.b_cs;
+        const T *base = b_mat + (int64_t)(ok ? col : 0) * p.b_cs;
 #pragma unroll
         for (int s = 0; s < STEPS; s++) bf[s][t] = fetch(base, p.b_rs, ok, p.b_vec, s);
     }
     auto rows_of_a = [&](int m0, Pack (&af)[STEPS]) {
-        const T *base = (const T *)p.a + (int64_t)min(m0 + r16, p.m - 1) * p.a_rs;
+        const T *base = a_mat + (int64_t)min(m0 + r16, p.m - 1) * p.a_rs;
 #pragma unroll
         for (int s = 0; s < STEPS; s++) af[s] = fetch(base, p.a_cs, true, p.a_vec, s);
     };
@@ -477,7 +483,7 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
 #pragma unroll
             for (int h = 0; h < H; h++) {
                 const int row = m0 + prow + RPI * h;
-                if (row < m_end && piece_ok) old[h] = *(const u32x4 *)((const T *)p.c + (int64_t)row * p.ldc + col);
+                if (row < m_end && piece_ok) old[h] = *(const u32x4 *)(c_mat + (int64_t)row * p.ldc + col);
             }
         }
         f32x4 acc[4];
@@ -516,7 +522,7 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
                 }
                 u32x4 raw;
                 __builtin_memcpy(&raw, out, 16);
-                *(u32x4 *)((T *)p.c + (int64_t)row * p.ldc + col) = raw;
+                *(u32x4 *)(c_mat + (int64_t)row * p.ldc + col) = raw;
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -527,14 +533,13 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
 
 template <typename T> hipError_t launch_thin_t(const ThinParams &p, dim3 grid, hipStream_t stream) {
     if (p.k <= 4 * Small<T>::KL) gemm_thin_kernel<T, 1><<<grid, 256, 0, stream>>>(p);
-    else if constexpr (sizeof(T) == 4) gemm_thin_kernel<T, 2><<<grid, 256, 0, stream>>>(p);
-    else return hipErrorInvalidValue;
+    else gemm_thin_kernel<T, 2><<<grid, 256, 0, stream>>>(p);
     return hipGetLastError();
 }
 
 // rows per workgroup: as many as leave a thousand workgroups (the fragments of B are loaded once per workgroup)
 inline int thin_rows_per_block(const GemmProblem &g) {
-    const int64_t blocks_n = (g.n + 255) / 256;
+    const int64_t blocks_n = (g.n + 255) / 256 * g.nb1 * g.nb2;
     int rows = 256;
     while (rows > 16 && blocks_n * ((g.m + rows - 1) / rows) < 1024) rows /= 2;
     return rows;
@@ -542,16 +547,23 @@ inline int thin_rows_per_block(const GemmProblem &g) {
 
 }  // namespace
 
-// k <= 32 and a large output, row-major with 16-byte aligned rows of whole 16-byte pieces.
+// k <= 32 and a large output, row-major with 16-byte aligned rows of whole 16-byte pieces; batches as grid.z.  (The
+// 16-bit types at k = 33 .. 64, two MFMA steps, were measured on the attention-score products, 128 x (1024 x 64 x 1024):
+// 89 us against 73 us of the LDS-DMA tiles -- every workgroup fetches its own fragments of B, and at that k the
+// operands are no longer small next to C.)
 bool thin_mfma_supported(const GemmProblem &g) {
     if (g.dtype != DT_F32 && g.dtype != DT_F16 && g.dtype != DT_BF16) return false;
-    if (g.k < 1 || g.k > 32 || g.m < 64 || g.n < 64 || g.reduce || g.nb1 * g.nb2 != 1) return false;
+    const int64_t es = (int64_t)elem_size(g.dtype), piece = 16 / es, nb = g.nb1 * g.nb2;
+    const int64_t step = es == 2 ? 32 : 16;
+    if (g.k < 1 || g.k > (es == 2 ? step : 2 * step) || g.m < 64 || g.n < 64 || g.reduce || nb < 1 || nb > 65535) return false;
     if (g.m >= (1ll << 30) || g.n >= (1ll << 30)) return false;
-    const int64_t es = (int64_t)elem_size(g.dtype), piece = 16 / es;
     if (g.c_cs != 1 || g.c_rs < g.n || g.c_rs % piece || g.n % piece || ((uintptr_t)g.c & 15)) return false;
-    // below these sizes of C the small-product and the tiled kernels are as fast or faster (f32 past k = 16 takes two
-    // rounds of MFMAs per strip and only pays on outputs that leave the last-level cache)
-    if (g.m * g.n * es < (es == 2 ? (1ll << 20) : g.k <= 16 ? (4ll << 20) : (64ll << 20))) return false;
+    if (nb > 1 && (g.c_b1 % piece || g.c_b2 % piece)) return false;
+    // below these sizes of C the small-product and the tiled kernels are as fast or faster (past one MFMA step a strip
+    // takes two rounds of MFMAs and only pays on outputs that leave the last-level cache)
+    const int64_t bytes = nb * g.m * g.n * es;
+    if (g.k > step && g.n < 1024) return false;  // (f32 16 x 16 x (512 x 32 x 512): 107 us against 92 us of the tiles)
+    if (bytes < (g.k > step ? (64ll << 20) : es == 2 ? (1ll << 20) : (4ll << 20))) return false;
     const int rows = thin_rows_per_block(g);
     if ((g.m + rows - 1) / rows > 65535) return false;  // row blocks are grid.y
     const uintptr_t mask = (uintptr_t)es - 1;
@@ -566,10 +578,13 @@ hipError_t launch_thin_mfma(const GemmProblem &g, hipStream_t stream) {
     p.m = (int)g.m; p.n = (int)g.n; p.k = (int)g.k;
     p.a_rs = g.a_rs; p.a_cs = g.a_cs; p.b_rs = g.b_rs; p.b_cs = g.b_cs; p.ldc = g.c_rs;
     p.accumulate = g.accumulate; p.bias_mode = g.bias ? g.bias_mode : BIAS_NONE;
-    p.a_vec = g.a_cs == 1 && g.a_rs % vq == 0 && ((uintptr_t)g.a & 15) == 0;
-    p.b_vec = g.b_rs == 1 && g.b_cs % vq == 0 && ((uintptr_t)g.b & 15) == 0;
+    p.a_vec = g.a_cs == 1 && g.a_rs % vq == 0 && g.a_b1 % vq == 0 && g.a_b2 % vq == 0 && ((uintptr_t)g.a & 15) == 0;
+    p.b_vec = g.b_rs == 1 && g.b_cs % vq == 0 && g.b_b1 % vq == 0 && g.b_b2 % vq == 0 && ((uintptr_t)g.b & 15) == 0;
     p.rows_per_block = thin_rows_per_block(g);
-    const dim3 grid((unsigned)((g.n + 255) / 256), (unsigned)((g.m + p.rows_per_block - 1) / p.rows_per_block));
+    p.nb2 = (int)g.nb2;
+    p.a_b1 = g.a_b1; p.a_b2 = g.a_b2; p.b_b1 = g.b_b1; p.b_b2 = g.b_b2; p.c_b1 = g.c_b1; p.c_b2 = g.c_b2;
+    const dim3 grid((unsigned)((g.n + 255) / 256), (unsigned)((g.m + p.rows_per_block - 1) / p.rows_per_block),
+                    (unsigned)(g.nb1 * g.nb2));
     switch (g.dtype) {
     case DT_F32: return launch_thin_t<float>(p, grid, stream);
     case DT_F16: return launch_thin_t<_Float16>(p, grid, stream);

@@ -590,6 +590,41 @@ def test_auto_dispatch_seeded_shape_sweep(dtype):
 
 
 # ------------------------------------------------------------------ batched --
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("k", [12, 32])
+def test_batched_thin_contractions(dtype, k):
+    """Attention scores with a head dimension of 32 or less: two batch axes, head-interleaved rows of A, B stored along k
+    (the transposed view of the keys), per batch or shared; beta = 1 and a bias; the row-streaming matrix-core kernel."""
+    from dfdx_amd.rocm import KERNEL_GEMV
+    dev = device()
+    g = rng(43 + k)
+    b1, b2, m, n = 2, 4, 520, 1024 if (dtype == "f32" and k > 16) else 512
+    if dtype == "f32" and k > 16:
+        b1 = 16     # planned for outputs of 64 MB and more there
+    a = oracle.to_storage(g.standard_normal(b1 * m * b2 * k), dtype)   # stored (b1, m, b2, k)
+    a_rs, a_cs, a_b1, a_b2 = b2 * k, 1, m * b2 * k, k
+    A = values(a, dtype, (b1, b2, m, k), (a_b1, a_b2, a_rs, a_cs))
+    da = dev.tensor(a, dtype)
+    for shared in (False, True):
+        nbm = 1 if shared else b1 * b2
+        bmat = oracle.to_storage(g.standard_normal(nbm * n * k), dtype)   # stored (batches, n, k)
+        B = oracle.to_f64(bmat, dtype).reshape((n, k) if shared else (b1, b2, n, k)).swapaxes(-1, -2)
+        bias = oracle.to_storage(g.standard_normal(n), dtype)
+        c0 = oracle.to_storage(g.standard_normal(b1 * b2 * m * n), dtype)
+        db, dbias, dc = dev.tensor(bmat, dtype), dev.tensor(bias, dtype), dev.tensor(c0, dtype)
+        desc = dev.gemm_desc(dtype, m, k, n, da.ptr, (a_rs, a_cs), db.ptr, (1, k), dc.ptr, (n, 1), batch=(b1, b2),
+                             a_batch=(a_b1, a_b2), b_batch=(0, 0) if shared else (b2 * n * k, n * k), c_batch=(b2 * m * n, m * n),
+                             accumulate=shared, bias=dbias.ptr)
+        plan = dev.gemm_plan(desc)
+        announce("batched thin", dtype, k, "shared" if shared else "per batch", plan[2])
+        assert plan[0] == KERNEL_GEMV and plan[2] == "thin_k_mfma", plan
+        dev.gemm(desc)
+        want = A @ B + oracle.to_f64(bias, dtype) + (oracle.to_f64(c0, dtype).reshape(b1, b2, m, n) if shared else 0.0)
+        got = oracle.to_f64(dev.to_host(dc), dtype).reshape(b1, b2, m, n)
+        ulp = {"f32": 2.0 ** -24, "f16": 2.0 ** -11, "bf16": 2.0 ** -8}[dtype]
+        assert_within(dtype, k, got, want, A, B, extra=2 * ulp * np.abs(want).max())
+
+
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("kernel", [KERNEL_GENERIC, KERNEL_MFMA])
 def test_batched_and_reduce(dtype, kernel):
