@@ -109,8 +109,16 @@ def main():
             W, xv, yv = torch.randn(n_, n_, device="cuda").half(), torch.randn(n_, device="cuda").half(), torch.zeros(n_, device="cuda").half()
             gv = dev.gemm_desc("f16", 1, n_, n_, P(xv), (n_, 1), P(W), (n_, 1), P(yv), (n_, 1))
             r1 = dev.gemm_desc("f16", n_, 1, n_, P(xv), (1, 1), P(yv), (n_, 1), P(W), (n_, 1), accumulate=True)  # W += x (x) y: the gradient of gv
+            # thin contractions: a rank-16 factor applied to 8192 rows, and attention scores with a head dimension of 32
+            ta, tb = torch.randn(8192, 16, device="cuda").half(), torch.randn(16, 4096, device="cuda").half()
+            tc = torch.zeros(8192, 4096, device="cuda", dtype=torch.float16)
+            thin = dev.gemm_desc("f16", 8192, 16, 4096, P(ta), (16, 1), P(tb), (4096, 1), P(tc), (4096, 1))
+            q32, k32 = ((torch.randn(Bq, H, S, 32, device="cuda")).half() for _ in range(2))
+            s32 = (H * S * 32, S * 32)
+            thin_scores = dev.gemm_desc("f16", S, 32, S, P(q32), (32, 1), P(k32), (1, 32), P(gs), (S, 1), batch=(Bq, H), a_batch=s32,
+                                        b_batch=s32, c_batch=sSS)
             names = []
-            for desc in (scores, dp, gv, r1):
+            for desc in (scores, dp, gv, r1, thin, thin_scores):
                 names.append(dev.gemm_plan(desc)[2])
                 for _ in range(3):
                     dev.gemm(desc)
