@@ -142,9 +142,10 @@ def test_fused_shapes_reach_every_tile_family_that_sums_rows():
 
 
 # f32: the k-sliced small kernel produces the row sums (config 1's Linear and smaller)
-FUSED_F32 = [("f32", 64, 512, 256), ("f32", 100, 40, 24), ("f32", 17, 33, 9), ("f32", 300, 16, 130)]
+FUSED_F32 = [("f32", 64, 512, 256), ("f32", 100, 40, 24), ("f32", 17, 33, 9), ("f32", 300, 16, 130), ("f32", 12, 2048, 1024)]
 # the small-product kernel in the other element types (its row sums come from the tile column 0 workgroups)
-FUSED_SMALL = [(d, *shape) for d in ("f16", "bf16", "f64") for shape in ((64, 512, 256), (100, 40, 24), (17, 33, 9), (300, 16, 130))]
+FUSED_SMALL = [(d, *shape) for d in ("f16", "bf16", "f64") for shape in ((64, 512, 256), (100, 40, 24), (17, 33, 9), (300, 16, 130),
+                                                                             (24, 2048, 1024))]   # (a handful of rows, a large weight: the thin-contraction kernel, row sums apart)
 
 
 @pytest.mark.parametrize("dtype,rows,i,o", [(d, *shape) for d in ("f16", "bf16") for shape in FUSED_SHAPES] + FUSED_F32 + FUSED_SMALL)
