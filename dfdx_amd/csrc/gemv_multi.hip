@@ -19,6 +19,8 @@
 namespace dfdx_rocm {
 namespace {
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 struct MultiParams {
     const void *vec, *mat, *bias;
     void *out;
@@ -81,7 +83,8 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_c
     constexpr int VEC = Elem<T>::VEC;
     constexpr bool PAIRS = sizeof(T) == 2;
     typedef typename std::conditional<PAIRS, T, float>::type S;  // what the vector slices are kept as
-    __shared__ __align__(16) S vsh[R][kchunk_of(R)];
+    constexpr int KCH = kchunk_of(R);
+    __shared__ __align__(16) S vsh[R][KCH];
     __shared__ float red[4][R < 4 ? R : 4][64 * VEC];
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int j0 = (blockIdx.x * 64 + lane) * VEC;
@@ -96,8 +99,8 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_c
         if constexpr (PAIRS) {
             const uint16_t bits = in ? __builtin_bit_cast(uint16_t, v) : (uint16_t)0;
             vsh[r][kk] = __builtin_bit_cast(T, bits);
-        } else {
-            vsh[r][kk] = in ? Elem<T>::load(&v) : 0.0f;
+        } else {  // a wave's k values (every fourth) side by side: four of them are one 16-byte LDS read
+            vsh[r][(kk & 3) * (KCH / 4) + (kk >> 2)] = in ? Elem<T>::load(&v) : 0.0f;
         }
     }
     __syncthreads();
@@ -142,20 +145,19 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_c
 #pragma unroll
                 for (int u = 0; u < 4; u++) raw[u] = *(const u32x4 *)(col + (int64_t)(kk + 4 * u) * p.mat_k_stride);
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
+                for (int r = 0; r < R; r++) {
+                    const f32x4 v = *(const f32x4 *)&vsh[r][wave * (KCH / 4) + (kk >> 2)];  // k = kk, kk + 4, kk + 8, kk + 12
 #pragma unroll
-                    for (int r = 0; r < R; r++) {
-                        const float v = vsh[r][kk + 4 * u];
+                    for (int u = 0; u < 4; u++)
 #pragma unroll
-                        for (int e = 0; e < VEC; e++) acc[r][e] += v * __uint_as_float(raw[u][e]);
-                    }
+                        for (int e = 0; e < VEC; e++) acc[r][e] += v[u] * __uint_as_float(raw[u][e]);
                 }
             }
             for (; kk < kn; kk += 4) {
                 const u32x4 raw = *(const u32x4 *)(col + (int64_t)kk * p.mat_k_stride);
 #pragma unroll
                 for (int r = 0; r < R; r++) {
-                    const float v = vsh[r][kk];
+                    const float v = vsh[r][wave * (KCH / 4) + (kk >> 2)];
 #pragma unroll
                     for (int e = 0; e < VEC; e++) acc[r][e] += v * __uint_as_float(raw[e]);
                 }
@@ -290,13 +292,15 @@ Shape classify(const GemmProblem &g) {
     if (g.c_rs < 1 || g.c_cs < 1) return s;  // no aliased outputs
     MultiParams &p = s.p;
     const int vec = g.dtype == DT_F32 ? 4 : 8;
-    if (g.m >= 2 && g.m <= 8 && g.n > 8) {  // out[r = i, j] = sum_k a[i, k] b[k, j]
+    // f32 in the cols form keeps up to sixteen vectors (64 accumulators a lane; the 16-bit types would need 128)
+    const int rmax = g.dtype == DT_F32 ? 16 : 8;
+    if (g.m >= 2 && g.m <= rmax && g.n > rmax) {  // out[r = i, j] = sum_k a[i, k] b[k, j]
         p.vec = g.a; p.vec_k_stride = g.a_cs; p.vec_r_stride = g.a_rs;
         p.mat = g.b; p.mat_k_stride = g.b_rs; p.mat_j_stride = g.b_cs;
         p.out_j_stride = g.c_cs; p.out_r_stride = g.c_rs;
         p.j = (int)g.n; p.r = (int)g.m;
         p.bias_j_stride = g.bias_mode == BIAS_PER_COL; p.bias_r_stride = g.bias_mode == BIAS_PER_ROW;
-    } else if (g.n >= 2 && g.n <= 8 && g.m > 8) {  // out[r = j, i] = sum_k b[k, j] a[i, k]
+    } else if (g.n >= 2 && g.n <= rmax && g.m > rmax) {  // out[r = j, i] = sum_k b[k, j] a[i, k]
         p.vec = g.b; p.vec_k_stride = g.b_rs; p.vec_r_stride = g.b_cs;
         p.mat = g.a; p.mat_k_stride = g.a_cs; p.mat_j_stride = g.a_rs;
         p.out_j_stride = g.c_rs; p.out_r_stride = g.c_cs;
@@ -324,6 +328,9 @@ Shape classify(const GemmProblem &g) {
                p.vec_k_stride == 1 && (p.vec_r_stride % vec == 0) && al16(p.vec)) {
         s.ok = true; s.cols = false;
     }
+    // nine to sixteen vectors: where the contraction is long (below, the small-product kernel's k slices are ahead:
+    // 16 x 4096 x 4096 24 against 30 us; 10 x 8192 x 1024 with both operands stored k-major 34.5 -> 17 us here)
+    if (p.r > 8 && !(s.cols && g.k >= 8192)) s.ok = false;
     return s;
 }
 
@@ -354,10 +361,12 @@ template <typename T, int R> hipError_t launch_r(const Shape &s, hipStream_t str
     if (s.cols) {
         dim3 grid((unsigned)((p.j + 64 * VEC - 1) / (64 * VEC)), (unsigned)p.kslices);
         gemv_multi_cols_kernel<T, R><<<grid, 256, 0, stream>>>(p);
-    } else {
+    } else if constexpr (R <= 8) {
         constexpr int PER_WG = 4 * rows_of(R);
         dim3 grid((unsigned)((p.j + PER_WG - 1) / PER_WG), (unsigned)p.kslices);
         gemv_multi_dots_kernel<T, R><<<grid, 256, 0, stream>>>(p);
+    } else {
+        return hipErrorInvalidValue;
     }
     if (p.kslices > 1) {
         const int64_t outs = (int64_t)p.r * p.j;
@@ -366,6 +375,8 @@ template <typename T, int R> hipError_t launch_r(const Shape &s, hipStream_t str
     return hipGetLastError();
 }
 template <typename T> hipError_t launch_t(const Shape &s, hipStream_t stream) {
+    if constexpr (sizeof(T) == 4)
+        if (s.p.r > 8) return launch_r<T, 16>(s, stream);
     return s.p.r <= 2 ? launch_r<T, 2>(s, stream) : s.p.r <= 4 ? launch_r<T, 4>(s, stream) : launch_r<T, 8>(s, stream);
 }
 
