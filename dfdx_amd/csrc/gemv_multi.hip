@@ -292,8 +292,8 @@ Shape classify(const GemmProblem &g) {
     if (g.c_rs < 1 || g.c_cs < 1) return s;  // no aliased outputs
     MultiParams &p = s.p;
     const int vec = g.dtype == DT_F32 ? 4 : 8;
-    // f32 in the cols form keeps up to sixteen vectors (64 accumulators a lane; the 16-bit types would need 128)
-    const int rmax = g.dtype == DT_F32 ? 16 : 8;
+    // the cols form keeps up to sixteen vectors where the contraction is long (see below)
+    const int rmax = 16;
     if (g.m >= 2 && g.m <= rmax && g.n > rmax) {  // out[r = i, j] = sum_k a[i, k] b[k, j]
         p.vec = g.a; p.vec_k_stride = g.a_cs; p.vec_r_stride = g.a_rs;
         p.mat = g.b; p.mat_k_stride = g.b_rs; p.mat_j_stride = g.b_cs;
@@ -330,7 +330,9 @@ Shape classify(const GemmProblem &g) {
     }
     // nine to sixteen vectors: where the contraction is long (below, the small-product kernel's k slices are ahead:
     // 16 x 4096 x 4096 24 against 30 us; 10 x 8192 x 1024 with both operands stored k-major 34.5 -> 17 us here)
-    if (p.r > 8 && !(s.cols && g.k >= 8192)) s.ok = false;
+    // (16-bit types: 128 accumulators a lane, ahead of the split tiles from 16384 terms on -- 10 x 65536 x 256 102 -> 36 us,
+    // 9 x 16384 x 2048 55 -> 35 us; at 8192 the tiles lead, 16 x 8192 x 1024 12.4 against 20 us)
+    if (p.r > 8 && !(s.cols && g.k >= (g.dtype == DT_F32 ? 8192 : 16384))) s.ok = false;
     return s;
 }
 
@@ -375,8 +377,7 @@ template <typename T, int R> hipError_t launch_r(const Shape &s, hipStream_t str
     return hipGetLastError();
 }
 template <typename T> hipError_t launch_t(const Shape &s, hipStream_t stream) {
-    if constexpr (sizeof(T) == 4)
-        if (s.p.r > 8) return launch_r<T, 16>(s, stream);
+    if (s.p.r > 8) return launch_r<T, 16>(s, stream);
     return s.p.r <= 2 ? launch_r<T, 2>(s, stream) : s.p.r <= 4 ? launch_r<T, 4>(s, stream) : launch_r<T, 8>(s, stream);
 }
 

@@ -381,11 +381,11 @@ def test_gemv_multi(dtype, shape, layout):
 
 
 @pytest.mark.parametrize("shape,layout", [((10, 8192, 1024), "tn"), ((1024, 8200, 10), "tn"), ((16, 8192, 520), "nn"), ((9, 16384, 264), "tn"),
-                                          ((264, 8192, 13), "tt")])
+                                          ((264, 8192, 13), "tt"), ((12, 16384, 520), "nn")])
 def test_gemv_multi_nine_to_sixteen_vectors_f32(shape, layout):
     """The weight gradient of a layer with ten outputs over a batch of thousands of rows (both operands stored along the
-    batch): f32 keeps up to sixteen vectors against the streamed matrix where the contraction is long; beta, bias,
-    column-major C.  The 16-bit types and shorter contractions keep their matrix-core plans."""
+    batch): up to sixteen vectors against the streamed matrix where the contraction is long (f32 from 8192 terms, the
+    16-bit types from 16384); beta, bias, column-major C.  Shorter contractions keep their matrix-core plans."""
     from dfdx_amd.rocm import KERNEL_GEMV
     m, k, n = shape
     dev = device()
@@ -394,7 +394,12 @@ def test_gemv_multi_nine_to_sixteen_vectors_f32(shape, layout):
     astr, bstr = (1, m) if at else (k, 1), (1, k) if bt else (n, 1)
     plan = dev.gemm_plan(dev.gemm_desc("f32", m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1)))
     assert plan[0] == KERNEL_GEMV and plan[2] == "gemv_multi", (shape, layout, plan)
-    assert dev.gemm_plan(dev.gemm_desc("f16", m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1)))[2] != "gemv_multi"
+    assert dev.gemm_plan(dev.gemm_desc("f16", m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1)))[2] == ("gemv_multi" if k >= 16384 else
+                                                                                                  dev.gemm_plan(dev.gemm_desc("f16", m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1), kernel=KERNEL_MFMA))[2])
+    if k >= 16384:   # the 16-bit types take the form from 16384 terms on
+        for dt in ("f16", "bf16"):
+            run_case(dt, m, k, n, layout, True, KERNEL_AUTO, 0, seed=18, bias=True, pads=(8, 8, 3))
+            run_case(dt, m, k, n, layout, False, KERNEL_AUTO, 0, seed=19, c_colmajor=True)
     assert dev.gemm_plan(dev.gemm_desc("f32", m, 4096, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1)))[2] != "gemv_multi"
     run_case("f32", m, k, n, layout, False, KERNEL_AUTO, 0, seed=15, bias=True)
     run_case("f32", m, k, n, layout, True, KERNEL_AUTO, 0, seed=16, c_colmajor=True, bias=True)
