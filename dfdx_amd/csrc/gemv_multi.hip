@@ -345,7 +345,11 @@ void plan_slices(Shape &s, int dtype) {
     int slices = 1;
     if (s.cols) {
         slices = (p.k + kchunk_max - 1) / kchunk_max;  // the vector slices must fit the LDS buffer
-        while (blocks_j * slices < 1024 && p.k / (slices * 2) >= 64) slices *= 2;
+        // few column blocks (a narrow matrix with a long k): half as many workgroups -- every slice adds R x j partial sums
+        // for the combining launch, and with few outputs that launch walks long chains of them (8 x 16384 x 1024 f32:
+        // 24.0 -> 17.7 us, 8 x 65536 x 256: 28.9 -> 22.1 us; 4096 columns and more are faster with the thousand)
+        const int want = blocks_j <= 4 ? 512 : 1024;
+        while (blocks_j * slices < want && p.k / (slices * 2) >= 64) slices *= 2;
     } else {
         // a wave of this form is heavy (4 + R loads a step): it takes eight of them per SIMD to hide the latency of HBM
         while (blocks_j * slices < 2048 && p.k / (slices * 2) >= 64 * vec) slices *= 2;
