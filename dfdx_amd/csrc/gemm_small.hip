@@ -370,11 +370,12 @@ namespace {
 // A product such as 4096 x 16 x 4096 writes 2 K bytes of C per byte it reads: what bounds it is how C leaves the chip.
 // The tiled kernels pad k to their step and reach 2 - 3 TB/s on it.  Here a wave keeps the fragments of 64 columns of B
 // in registers (four 16-column tiles, every k of the product) and walks down the rows of A sixteen at a time: one 16-byte
-// load per lane (f32: four 4-byte loads) is a whole 16 x k piece of a row-major A, four (f32: sixteen) MFMAs make a 16 x 64 strip of C, and the
+// load per lane is a whole 16 x k piece of a row-major A, four (f32: sixteen) MFMAs make a 16 x 64 strip of C, and the
 // strip goes through a wave-private LDS tile so that it leaves as whole rows -- eight (f32: sixteen) lanes with 16 bytes
 // each per row, never the 32-byte row pieces of the accumulator layout.  The MFMA's operands are swapped (B's columns as
 // its rows), which leaves four consecutive columns of one row of C in a lane: the LDS tile is written 16 bytes at a time.
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));  // element-aligned: global memory takes such 16-byte accesses
 
 struct ThinParams {
     const void *a, *b;
@@ -389,7 +390,7 @@ struct ThinParams {
     int64_t a_b1, a_b2, b_b1, b_b2, c_b1, c_b2;
 };
 
-template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thin_kernel(const ThinParams p) {
+template <typename T, int STEPS, bool ALIGNED> __global__ __launch_bounds__(256) void gemm_thin_kernel(const ThinParams p) {
     typedef Small<T> S;
     typedef typename S::pack Pack;
     constexpr int KL = S::KL, STEP = 4 * KL;
@@ -464,10 +465,12 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
     };
     const int pc = lane % PPR, prow = lane / PPR;
     const int col = n0 + PIECE * pc;
-    const bool piece_ok = col < p.n;  // n is a multiple of the piece
+    // ALIGNED: every row of C starts on a 16-byte boundary.  Otherwise the pieces move as unaligned 16-byte accesses; the
+    // last piece of a row, where n cuts it, element by element.
+    const bool piece_ok = col < p.n, whole = col + PIECE <= p.n;
     float cb[PIECE];
 #pragma unroll
-    for (int i = 0; i < PIECE; i++) cb[i] = (p.bias_mode == BIAS_PER_COL && piece_ok) ? S::load((const T *)p.bias + col + i) : 0.0f;
+    for (int i = 0; i < PIECE; i++) cb[i] = (p.bias_mode == BIAS_PER_COL && col + i < p.n) ? S::load((const T *)p.bias + col + i) : 0.0f;
     float *mine = tile[wave];
     Pack next[STEPS];
     rows_of_a(m_begin, next);
@@ -483,7 +486,18 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
 #pragma unroll
             for (int h = 0; h < H; h++) {
                 const int row = m0 + prow + RPI * h;
-                if (row < m_end && piece_ok) old[h] = *(const u32x4 *)(c_mat + (int64_t)row * p.ldc + col);
+                if (row < m_end && piece_ok) {
+                    const T *src = c_mat + (int64_t)row * p.ldc + col;
+                    if (whole) {
+                        if constexpr (ALIGNED) old[h] = *(const u32x4 *)src;
+                        else old[h] = *(const u32x4_unaligned *)src;
+                    } else {
+                        T was[PIECE];
+#pragma unroll
+                        for (int i = 0; i < PIECE; i++) was[i] = src[col + i < p.n ? i : 0];
+                        __builtin_memcpy(&old[h], was, 16);
+                    }
+                }
             }
         }
         f32x4 acc[4];
@@ -522,7 +536,15 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
                 }
                 u32x4 raw;
                 __builtin_memcpy(&raw, out, 16);
-                *(u32x4 *)(c_mat + (int64_t)row * p.ldc + col) = raw;
+                T *dst = c_mat + (int64_t)row * p.ldc + col;
+                if (whole) {
+                    if constexpr (ALIGNED) *(u32x4 *)dst = raw;
+                    else *(u32x4_unaligned *)dst = raw;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < PIECE; i++)
+                        if (col + i < p.n) dst[i] = out[i];
+                }
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -531,10 +553,13 @@ template <typename T, int STEPS> __global__ __launch_bounds__(256) void gemm_thi
     }
 }
 
-template <typename T> hipError_t launch_thin_t(const ThinParams &p, dim3 grid, hipStream_t stream) {
-    if (p.k <= 4 * Small<T>::KL) gemm_thin_kernel<T, 1><<<grid, 256, 0, stream>>>(p);
-    else gemm_thin_kernel<T, 2><<<grid, 256, 0, stream>>>(p);
+template <typename T, bool ALIGNED> hipError_t launch_thin_a(const ThinParams &p, dim3 grid, hipStream_t stream) {
+    if (p.k <= 4 * Small<T>::KL) gemm_thin_kernel<T, 1, ALIGNED><<<grid, 256, 0, stream>>>(p);
+    else gemm_thin_kernel<T, 2, ALIGNED><<<grid, 256, 0, stream>>>(p);
     return hipGetLastError();
+}
+template <typename T> hipError_t launch_thin_t(const ThinParams &p, bool aligned, dim3 grid, hipStream_t stream) {
+    return aligned ? launch_thin_a<T, true>(p, grid, stream) : launch_thin_a<T, false>(p, grid, stream);
 }
 
 // rows per workgroup: as many as leave a thousand workgroups (the fragments of B are loaded once per workgroup)
@@ -547,18 +572,17 @@ inline int thin_rows_per_block(const GemmProblem &g) {
 
 }  // namespace
 
-// k <= 32 and a large output, row-major with 16-byte aligned rows of whole 16-byte pieces; batches as grid.z.  (The
+// k <= 32 and a large row-major output (rows off the 16-byte grid move as unaligned pieces); batches as grid.z.  (The
 // 16-bit types at k = 33 .. 64, two MFMA steps, were measured on the attention-score products, 128 x (1024 x 64 x 1024):
 // 89 us against 73 us of the LDS-DMA tiles -- every workgroup fetches its own fragments of B, and at that k the
 // operands are no longer small next to C.)
 bool thin_mfma_supported(const GemmProblem &g) {
     if (g.dtype != DT_F32 && g.dtype != DT_F16 && g.dtype != DT_BF16) return false;
-    const int64_t es = (int64_t)elem_size(g.dtype), piece = 16 / es, nb = g.nb1 * g.nb2;
+    const int64_t es = (int64_t)elem_size(g.dtype), nb = g.nb1 * g.nb2;
     const int64_t step = es == 2 ? 32 : 16;
     if (g.k < 1 || g.k > (es == 2 ? step : 2 * step) || g.m < 64 || g.n < 64 || g.reduce || nb < 1 || nb > 65535) return false;
     if (g.m >= (1ll << 30) || g.n >= (1ll << 30)) return false;
-    if (g.c_cs != 1 || g.c_rs < g.n || g.c_rs % piece || g.n % piece || ((uintptr_t)g.c & 15)) return false;
-    if (nb > 1 && (g.c_b1 % piece || g.c_b2 % piece)) return false;
+    if (g.c_cs != 1 || g.c_rs < g.n) return false;
     // below these sizes of C the small-product and the tiled kernels are as fast or faster (past one MFMA step a strip
     // takes two rounds of MFMAs and only pays on outputs that leave the last-level cache)
     const int64_t bytes = nb * g.m * g.n * es;
@@ -567,7 +591,7 @@ bool thin_mfma_supported(const GemmProblem &g) {
     const int rows = thin_rows_per_block(g);
     if ((g.m + rows - 1) / rows > 65535) return false;  // row blocks are grid.y
     const uintptr_t mask = (uintptr_t)es - 1;
-    return (((uintptr_t)g.a | (uintptr_t)g.b | (uintptr_t)g.bias) & mask) == 0;
+    return (((uintptr_t)g.a | (uintptr_t)g.b | (uintptr_t)g.c | (uintptr_t)g.bias) & mask) == 0;
 }
 
 hipError_t launch_thin_mfma(const GemmProblem &g, hipStream_t stream) {
@@ -585,10 +609,11 @@ hipError_t launch_thin_mfma(const GemmProblem &g, hipStream_t stream) {
     p.a_b1 = g.a_b1; p.a_b2 = g.a_b2; p.b_b1 = g.b_b1; p.b_b2 = g.b_b2; p.c_b1 = g.c_b1; p.c_b2 = g.c_b2;
     const dim3 grid((unsigned)((g.n + 255) / 256), (unsigned)((g.m + p.rows_per_block - 1) / p.rows_per_block),
                     (unsigned)(g.nb1 * g.nb2));
+    const bool aligned = ((uintptr_t)g.c & 15) == 0 && g.c_rs % vq == 0 && (g.nb1 * g.nb2 == 1 || (g.c_b1 % vq == 0 && g.c_b2 % vq == 0));
     switch (g.dtype) {
-    case DT_F32: return launch_thin_t<float>(p, grid, stream);
-    case DT_F16: return launch_thin_t<_Float16>(p, grid, stream);
-    case DT_BF16: return launch_thin_t<__bf16>(p, grid, stream);
+    case DT_F32: return launch_thin_t<float>(p, aligned, grid, stream);
+    case DT_F16: return launch_thin_t<_Float16>(p, aligned, grid, stream);
+    case DT_BF16: return launch_thin_t<__bf16>(p, aligned, grid, stream);
     default: return hipErrorInvalidValue;
     }
 }

@@ -457,28 +457,25 @@ def test_thin_contractions(dtype, k):
 def test_thin_contractions_on_matrix_cores(dtype, k):
     """k <= 32 with an output of megabytes (a low-rank factor applied to a batch of rows, the product that follows a
     projection to a handful of features): the row-streaming matrix-core kernel -- all four operand layouts, rows and
-    columns that end inside a strip, padded rows, beta, bias along the columns and (column-major C) along the rows."""
+    columns that end inside a strip, rows of C on and off the 16-byte grid, a last piece that n cuts, beta, bias along the columns and (column-major C) along the rows."""
     from dfdx_amd.rocm import KERNEL_GEMV
     dev = device()
     big = dtype == "f32" and k > 16   # f32 takes two rounds of MFMAs there and is planned for outputs of 64 MB and more
-    shapes = [(4096, 4096), (4104, 4100)] if big else [(2048, 1024), (1030, 2056), (4100, 520), (520, 8200), (2048, 1028)]
+    shapes = [(4096, 4096), (4104, 4099)] if big else [(2048, 1024), (1030, 2056), (4100, 520), (520, 8200), (2048, 1029), (1031, 2050)]
     for i, (m, n) in enumerate(shapes):
         a = dev.zeros(dtype, (max(m, n) * k,))
         c = dev.zeros(dtype, (m * n,))
-        piece = 4 if dtype == "f32" else 8
         d = dev.gemm_desc(dtype, m, k, n, a.ptr, (k, 1), a.ptr, (n, 1), c.ptr, (n, 1))
         plan = dev.gemm_plan(d)
-        if n % piece == 0:
-            assert plan[0] == KERNEL_GEMV and plan[2] == "thin_k_mfma", plan
-        else:
-            assert plan[2] != "thin_k_mfma", plan    # rows that are not whole 16-byte pieces go to the other kernels
+        assert plan[0] == KERNEL_GEMV and plan[2] == "thin_k_mfma", plan
         del a, c
         for j, layout in enumerate(LAYOUTS):
             if big and j % 2 != i % 2:
                 continue
-            colmajor = (i + j) % 4 == 3 and m % piece == 0
+            colmajor = (i + j) % 4 == 3
+            # rows of C on the 16-byte grid (pad 0 or 8) and off it (pad 3: unaligned pieces; n = 1029: a cut last piece)
             run_case(dtype, m, k, n, layout, bool((i + j) % 2), KERNEL_AUTO, 0, bias=(j % 3 != 1), c_colmajor=colmajor,
-                     seed=90 + 4 * i + j, pads=(j % 3, 2 * (i % 2), 8 * (j % 2)))
+                     seed=90 + 4 * i + j, pads=(j % 3, 2 * (i % 2), (0, 8, 3, 5)[(i + j) % 4]))
     # small outputs stay with the other kernels
     a = dev.zeros(dtype, (65536,))
     assert dev.gemm_plan(dev.gemm_desc(dtype, 256, 16, 256, a.ptr, (16, 1), a.ptr, (256, 1), a.ptr, (256, 1)))[2] != "thin_k_mfma"
