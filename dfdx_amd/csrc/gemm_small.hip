@@ -465,9 +465,10 @@ template <typename T, int STEPS, bool ALIGNED> __global__ __launch_bounds__(256)
     };
     const int pc = lane % PPR, prow = lane / PPR;
     const int col = n0 + PIECE * pc;
-    // ALIGNED: every row of C starts on a 16-byte boundary.  Otherwise the pieces move as unaligned 16-byte accesses; the
-    // last piece of a row, where n cuts it, element by element.
-    const bool piece_ok = col < p.n, whole = col + PIECE <= p.n;
+    // ALIGNED: every row of C starts on a 16-byte boundary and n is a whole number of pieces (the form without the tests
+    // below is 0.3 - 0.8 us faster on a 4096 x 16 x 4096 product).  Otherwise the pieces move as unaligned 16-byte
+    // accesses; the last piece of a row, where n cuts it, element by element.
+    const bool piece_ok = col < p.n, whole = ALIGNED || col + PIECE <= p.n;
     float cb[PIECE];
 #pragma unroll
     for (int i = 0; i < PIECE; i++) cb[i] = (p.bias_mode == BIAS_PER_COL && col + i < p.n) ? S::load((const T *)p.bias + col + i) : 0.0f;
@@ -609,7 +610,7 @@ hipError_t launch_thin_mfma(const GemmProblem &g, hipStream_t stream) {
     p.a_b1 = g.a_b1; p.a_b2 = g.a_b2; p.b_b1 = g.b_b1; p.b_b2 = g.b_b2; p.c_b1 = g.c_b1; p.c_b2 = g.c_b2;
     const dim3 grid((unsigned)((g.n + 255) / 256), (unsigned)((g.m + p.rows_per_block - 1) / p.rows_per_block),
                     (unsigned)(g.nb1 * g.nb2));
-    const bool aligned = ((uintptr_t)g.c & 15) == 0 && g.c_rs % vq == 0 && (g.nb1 * g.nb2 == 1 || (g.c_b1 % vq == 0 && g.c_b2 % vq == 0));
+    const bool aligned = ((uintptr_t)g.c & 15) == 0 && g.c_rs % vq == 0 && g.n % vq == 0 && (g.nb1 * g.nb2 == 1 || (g.c_b1 % vq == 0 && g.c_b2 % vq == 0));
     switch (g.dtype) {
     case DT_F32: return launch_thin_t<float>(p, aligned, grid, stream);
     case DT_F16: return launch_thin_t<_Float16>(p, aligned, grid, stream);
