@@ -115,10 +115,7 @@ template <> struct Small<__bf16> {
     }
     static __device__ __forceinline__ int out_row(int r, int q) { return 4 * q + r; }
     static __device__ __forceinline__ float load(const __bf16 *p) { return widen(*(const short *)p); }
-    static __device__ __forceinline__ void store(__bf16 *p, float v) {  // round to nearest even, quiet NaNs
-        const uint32_t x = __float_as_uint(v);
-        *(uint16_t *)p = ((x & 0x7fffffffu) > 0x7f800000u) ? (uint16_t)((x >> 16) | 0x40u) : (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
-    }
+    static __device__ __forceinline__ void store(__bf16 *p, float v) { *p = (__bf16)v; }
 };
 
 // LONG: slices of more than one pass.  The one-pass form is kept as short as it can be: at 4 - 5 us a launch, the
