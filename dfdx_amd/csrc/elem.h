@@ -21,12 +21,8 @@ template <> struct Elem<__bf16> {
     static __device__ __forceinline__ float load(const __bf16 *p) {
         return __uint_as_float((uint32_t)(*(const uint16_t *)p) << 16);
     }
-    static __device__ __forceinline__ void store(__bf16 *p, float v) {  // round to nearest even, quiet NaNs
-        const uint32_t x = __float_as_uint(v);
-        const uint16_t r = ((x & 0x7fffffffu) > 0x7f800000u) ? (uint16_t)((x >> 16) | 0x40u)
-                                                             : (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
-        *(uint16_t *)p = r;
-    }
+    // round to nearest even, quiet NaNs: the hardware conversion (v_cvt_pk_bf16_f32)
+    static __device__ __forceinline__ void store(__bf16 *p, float v) { *p = (__bf16)v; }
 };
 
 // f64 takes part in the plain (row-walking) kernels only: no 16-byte vector path, f64 arithmetic throughout.
