@@ -30,13 +30,7 @@ template <> struct Conv<__bf16> {
     static __device__ __forceinline__ float load(const __bf16 *p) {
         return __uint_as_float((uint32_t)(*(const uint16_t *)p) << 16);
     }
-    static __device__ __forceinline__ void store(__bf16 *p, float v) {
-        uint32_t x = __float_as_uint(v);
-        uint16_t r;
-        if ((x & 0x7fffffffu) > 0x7f800000u) r = (uint16_t)((x >> 16) | 0x40u);
-        else r = (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);  // RNE
-        *(uint16_t *)p = r;
-    }
+    static __device__ __forceinline__ void store(__bf16 *p, float v) { *p = (__bf16)v; }  // RNE, quiet NaNs (v_cvt_pk_bf16_f32)
 };
 
 constexpr int GT = 64;  // tile edge

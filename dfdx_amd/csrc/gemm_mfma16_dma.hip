@@ -81,11 +81,7 @@ template <> struct Mma<__bf16> {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
     static __device__ __forceinline__ float to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
-    static __device__ __forceinline__ uint16_t from_f32(float v) {
-        uint32_t x = __float_as_uint(v);
-        if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
-        return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);  // round to nearest even
-    }
+    static __device__ __forceinline__ uint16_t from_f32(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }  // RNE, quiet NaNs
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // v_cvt_pk_bf16_f32: RNE, quiet NaNs
         typedef __bf16 b2 __attribute__((ext_vector_type(2)));
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, b2));

@@ -40,11 +40,7 @@ template <> struct Elt<_Float16> {
 template <> struct Elt<__bf16> {
     static constexpr int VEC = 8;
     static __device__ __forceinline__ float load(const __bf16 *p) { return __uint_as_float((uint32_t)(*(const uint16_t *)p) << 16); }
-    static __device__ __forceinline__ void store(__bf16 *p, float v) {
-        uint32_t x = __float_as_uint(v);
-        *(uint16_t *)p = ((x & 0x7fffffffu) > 0x7f800000u) ? (uint16_t)((x >> 16) | 0x40u)
-                                                           : (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
-    }
+    static __device__ __forceinline__ void store(__bf16 *p, float v) { *p = (__bf16)v; }  // RNE, quiet NaNs (v_cvt_pk_bf16_f32)
     static __device__ __forceinline__ void unpack(u32x4 r, float (&o)[8]) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {

@@ -18,12 +18,7 @@ template <> struct Cvt<_Float16> {
 };
 template <> struct Cvt<__bf16> {
     static __device__ __forceinline__ float load(const __bf16 *p) { return __uint_as_float((uint32_t)(*(const uint16_t *)p) << 16); }
-    static __device__ __forceinline__ void store(__bf16 *p, float v) {
-        uint32_t x = __float_as_uint(v);
-        uint16_t r = ((x & 0x7fffffffu) > 0x7f800000u) ? (uint16_t)((x >> 16) | 0x40u)
-                                                       : (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
-        *(uint16_t *)p = r;
-    }
+    static __device__ __forceinline__ void store(__bf16 *p, float v) { *p = (__bf16)v; }  // RNE, quiet NaNs (v_cvt_pk_bf16_f32)
 };
 
 // The row sums that ride along with a split product (`ksum`, one value per row of C, `slots` partial sums each, stored
@@ -107,10 +102,7 @@ template <> struct Bits16<_Float16> {
 };
 template <> struct Bits16<__bf16> {
     static __device__ __forceinline__ float widen(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
-    static __device__ __forceinline__ uint16_t narrow(float v) {
-        uint32_t x = __float_as_uint(v);
-        return ((x & 0x7fffffffu) > 0x7f800000u) ? (uint16_t)((x >> 16) | 0x40u) : (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
-    }
+    static __device__ __forceinline__ uint16_t narrow(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }  // RNE, quiet NaNs
 };
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
