@@ -612,6 +612,29 @@ def test_auto_dispatch_seeded_shape_sweep(dtype):
         run_case(dtype, m, k, n, layout, accumulate, KERNEL_AUTO, 0, c_colmajor=ccol, bias=bias, seed=500 + i, pads=pads)
 
 
+def test_thin_contraction_with_more_than_2_31_output_elements():
+    """70000 x 16 x 32768 in f16: 2.29 G elements of C (4.6 GB), so element offsets pass 2^31 (and byte offsets 2^32) --
+    sampled row blocks, the last rows included, against the f64 product."""
+    from dfdx_amd.rocm import KERNEL_GEMV
+    dev, g = device(), rng(97)
+    m, k, n, dtype = 70000, 16, 32768, "f16"
+    a = oracle.to_storage(g.standard_normal(m * k), dtype)
+    b = oracle.to_storage(g.standard_normal(k * n), dtype)
+    da, db, dc = dev.tensor(a, dtype), dev.tensor(b, dtype), dev.zeros(dtype, (m * n,))
+    desc = dev.gemm_desc(dtype, m, k, n, da.ptr, (k, 1), db.ptr, (n, 1), dc.ptr, (n, 1))
+    plan = dev.gemm_plan(desc)
+    announce("gemm beyond 2^31 elements", dtype, (m, k, n), plan[2])
+    assert plan[0] == KERNEL_GEMV and plan[2] == "thin_k_mfma", plan
+    dev.gemm(desc)
+    dev.synchronize()
+    A, B = oracle.to_f64(a, dtype).reshape(m, k), oracle.to_f64(b, dtype).reshape(k, n)
+    for r0 in (0, 1008, 32768, 65520, 65536, m - 16):   # 65536 rows x 32768 columns = 2^31 elements
+        raw = dc.storage[r0 * n * 2:(r0 + 16) * n * 2].cpu().numpy().view(np.float16)
+        got = raw.astype(np.float64).reshape(16, n)
+        want = A[r0:r0 + 16] @ B
+        assert_within(dtype, k, got, want, A[r0:r0 + 16], B, extra=2.0 ** -11 * float(np.abs(want).max()), what=f"rows {r0}..")
+
+
 # ------------------------------------------------------------------ batched --
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("k", [12, 32])
