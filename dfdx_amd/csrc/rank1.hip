@@ -190,10 +190,13 @@ template <typename T> hipError_t launch_t(const Rank1Params &base, const GemmPro
     while (p.tx_log2 < 8 && (1ll << p.tx_log2) < pieces) p.tx_log2++;
     const int ty = 256 >> p.tx_log2;
     const int64_t blocks_y = (pieces + (1ll << p.tx_log2) - 1) >> p.tx_log2;
-    // rows per thread: two (k = 1) or eight at least, sixteen at most, and about 2048 workgroups in between
+    // rows per thread: two (k = 1) or eight at least, sixteen at most, and about 2048 workgroups in between -- 1024 for the
+    // 16-bit types, whose rows are half as many bytes (4096^2: 10.4 -> 9.3 us; not where unaligned rows are read back
+    // as well, 4095 x 4097 with beta = 1: 13.0 against 13.7 us)
     const int64_t passes = (g.m + ty - 1) / ty * blocks_y;
     const int least = g.k > 1 ? 8 : 2;  // the b pieces a thread gathers first want more rows to pay for them
-    const int per_thread = (int)std::min<int64_t>(16, std::max<int64_t>(least, passes / 2048 / 2 * 2));
+    const int64_t groups = (sizeof(T) == 2 && (aligned || !p.accumulate)) ? 1024 : 2048;
+    const int per_thread = (int)std::min<int64_t>(16, std::max<int64_t>(least, passes / groups / 2 * 2));
     p.rows_per_block = ty * per_thread;
     if (g.k > 1) {  // the staged values of a: rows x KMAX within STAGED_A, an even number of rows per thread
         const int kmax = g.k == 2 ? 2 : g.k <= 4 ? 4 : 8;
