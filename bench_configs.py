@@ -22,24 +22,17 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
-    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them, shapes = shape classes outside the configurations: few rows or columns, thin contractions, rank-1 updates, mid-size products)")
-    ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "f32-forms", "mfma-power"],
+    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them, shapes = shape classes outside the configurations: few rows or columns, thin contractions, rank-1 updates, mid-size products, plancheck = the planner's pick against every forced tile variant and split count on a fixed list of shapes; exits 1 with --strict when a pick is more than --plancheck-slack off the best)")
+    ap.add_argument("--strict", action="store_true", help="plancheck: exit status 1 when a pick is flagged")
+    ap.add_argument("--plancheck-slack", type=float, default=0.10, help="plancheck: flag a pick that is this much slower than the best forced candidate")
+    ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "f32-forms"],
                     help="counter-collection aids for rocprofv3, nothing is timed: traffic = 3 plain 256 MiB device copies (a kernel "
                          "of known size that calibrates FETCH_SIZE / WRITE_SIZE) then 5 launches of the 4096^3 f16 GEMM; rows = the same copies, then 3 launches each of "
                          "the HBM-bound rows (config 4 scores and dP, the 16384^2 f16 vec.mat and the rank-1 update that is its weight gradient, softmax forward and backward on the scores); f32-forms = 3 "
                          "launches each of the register-staged and the LDS-DMA f32 kernel (256x256 tile) on 4096^3 A.B^T and A.B; variants = 3 "
-                         "launches of that GEMM with every f16 MFMA tile variant forced in turn; mfma-power = the stand-alone "
-                         "MFMA-only program (built by `make -C dfdx_amd/csrc probe`)")
+                         "launches of that GEMM with every f16 MFMA tile variant forced in turn")
     ap.add_argument("--no-rotate", action="store_true", help="skip the second timing of the HBM-bound cases over rotating buffer sets")
     args = ap.parse_args()
-    if args.probe == "mfma-power":   # a child process, started before this one touches the GPU
-        import os
-        import subprocess
-
-        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "dfdx_amd", "lib", "probe_mfma_power")
-        if not os.path.exists(exe):
-            sys.exit("bench_configs.py: %s is not built (make -C dfdx_amd/csrc probe)" % exe)
-        sys.exit(subprocess.call([exe]))
     import torch
     from dfdx_amd import Rocm
     from dfdx_amd.rocm import GemmDesc, View
@@ -468,6 +461,72 @@ def main():
                 gemm("shape", f"{dt} {m}x{k}x{n} {lay}", desc, 2 * m * k * n, es * (m * k + k * n + m * n), 100)
                 del a, b, c
 
+    # ---- planner regression check: the automatic pick against every forced candidate ---------------------------------
+    flagged = []
+    if "plancheck" in only:
+        from dfdx_amd.rocm import KERNEL_GEMV, KERNEL_MFMA, RocmError
+
+        # (dtype, m, k, n, layout of A and B (n = stored as indexed, t = transposed), accumulate, batch)
+        T = 8192
+        pc_cases = [("f16", 4096, 4096, 4096, "nn", False, 1), ("f16", 4096, 4096, 4096, "tn", False, 1), ("f16", 4096, 4096, 4096, "nt", False, 1),
+                    ("f32", 4096, 4096, 4096, "nn", False, 1), ("f32", 64, 512, 256, "nt", False, 1), ("f32", 64, 256, 512, "nn", True, 1),
+                    ("f32", 512, 64, 256, "tn", True, 1),
+                    ("f16", 16384, 1024, 1024, "nn", False, 1), ("f16", 16384, 1024, 1024, "nt", True, 1), ("f16", 1024, 16384, 1024, "tn", True, 1),
+                    ("f16", 1024, 64, 1024, "nt", False, 128), ("f16", 1024, 1024, 64, "nn", False, 128), ("f16", 1024, 1024, 64, "tn", True, 128),
+                    ("bf16", T, 1024, 1024, "nt", False, 1), ("bf16", T, 1024, 4096, "nt", False, 1), ("bf16", T, 4096, 1024, "nt", False, 1),
+                    ("bf16", T, 1024, 1024, "nn", True, 1), ("bf16", T, 4096, 1024, "nn", True, 1), ("bf16", T, 1024, 4096, "nn", True, 1),
+                    ("bf16", 1024, T, 1024, "tn", True, 1), ("bf16", 4096, T, 1024, "tn", True, 1), ("bf16", 1024, T, 4096, "tn", True, 1),
+                    ("bf16", 512, 64, 512, "nt", False, 256), ("bf16", 512, 512, 64, "nn", False, 256),
+                    ("f16", 2048, 2048, 2048, "nn", False, 1), ("f16", 1024, 1024, 1024, "nn", False, 1), ("f16", 512, 512, 512, "nt", False, 1),
+                    ("f16", 256, 256, 256, "nt", False, 1), ("f16", 512, 4096, 512, "nn", False, 1), ("f16", 8192, 1024, 8192, "nt", False, 1),
+                    ("f16", 16, 4096, 4096, "nt", False, 1), ("f16", 32, 8192, 8192, "nt", False, 1), ("f16", 4, 4096, 4096, "nt", False, 1),
+                    ("f32", 2048, 2048, 2048, "nn", False, 1), ("f32", 1024, 8192, 1024, "tn", True, 1), ("f32", 8192, 1024, 1024, "nt", False, 1),
+                    ("f32", 512, 512, 512, "nn", False, 1), ("f32", 16, 4096, 4096, "nt", False, 1)]
+        for dt, m, k, n, lay, acc, nb in pc_cases:
+            a = rnd((nb, k, m) if lay[0] == "t" else (nb, m, k), dt)
+            b = rnd((nb, n, k) if lay[1] == "t" else (nb, k, n), dt, k ** -0.5)
+            c = zeros((nb, m, n), dt)
+
+            def pc_desc(kernel=0, variant=0, split=0):
+                return dev.gemm_desc(dt, m, k, n, P(a), (1, m) if lay[0] == "t" else (k, 1), P(b), (1, k) if lay[1] == "t" else (n, 1), P(c), (n, 1),
+                                     accumulate=acc, batch=(nb, 1), a_batch=(m * k, 0), b_batch=(k * n, 0), c_batch=(m * n, 0),
+                                     kernel=kernel, variant=variant, split_k=split, no_split_k=(split == 1))
+
+            def pc_time(desc, iters=20):
+                try:
+                    name = dev.gemm_plan(desc)[2]
+                    return min(dev.gemm_time(desc, 3, iters), dev.gemm_time(desc, 1, iters)), name
+                except RocmError:
+                    return None, None
+
+            auto_ms, auto_name = pc_time(pc_desc())
+            cands = {}
+            for v in range(1, dev.mfma_variant_count(dt) + 1):
+                for split in (1, 2, 4, 8, 16):
+                    if split > 1 and (nb > 1 or k < 64 * 4 * split):
+                        continue
+                    ms, name = pc_time(pc_desc(KERNEL_MFMA, v, split), 10)
+                    if ms and (name not in cands or ms < cands[name]):
+                        cands[name] = ms
+            ms, name = pc_time(pc_desc(KERNEL_GEMV), 10)
+            if ms:
+                cands[name] = ms
+            best_name = min(cands, key=cands.get)
+            auto_ms = min(auto_ms, pc_time(pc_desc())[0])   # once more after the sweep: clocks drift over a run
+            # the same plan under both names is the same launch: what separates the two timings is noise
+            slack = 0.0 if best_name == auto_name else auto_ms / cands[best_name] - 1.0
+            flag = slack > args.plancheck_slack
+            tag = f"{dt} {'b' + str(nb) + ' ' if nb > 1 else ''}{m}x{k}x{n} {lay}{' acc' if acc else ''}"
+            rows.append({"group": "plancheck", "case": tag, "kernel": auto_name, "us": round(auto_ms * 1e3, 2), "best": best_name,
+                         "best_us": round(cands[best_name] * 1e3, 2), "candidates": len(cands), "off_best_pct": round(100 * slack, 1), "flagged": flag})
+            print(f"plan  {tag:34s} auto {auto_ms * 1e3:8.1f} us {auto_name:40s} best of {len(cands):3d} {cands[best_name] * 1e3:8.1f} us {best_name:40s} "
+                  f"{100 * slack:+6.1f} %{'  <<<< FLAG' if flag else ''}", flush=True)
+            if flag:
+                flagged.append(tag)
+            del a, b, c
+        print(f"plancheck: {len(pc_cases)} shapes, {len(flagged)} flagged (pick more than {100 * args.plancheck_slack:.0f} % off the best forced candidate)"
+              + (": " + "; ".join(flagged) if flagged else ""), flush=True)
+
     # ---- operands off the 16-byte grid: an LM head with 50257 outputs, a first-layer convolution -------------------
     if "edge" in only:   # on request: the scalar kernel's rows take milliseconds each
         from dfdx_amd.rocm import KERNEL_GENERIC
@@ -553,6 +612,8 @@ def main():
     if args.json:
         with open(args.json, "w") as f:
             json.dump({"device": dev.device_info(), "rows": rows}, f, indent=1)
+    if args.strict and flagged:
+        sys.exit(1)
 
 
 if __name__ == "__main__":

@@ -45,6 +45,7 @@ static int grow(dfdx_rocm_ctx *ctx, void **buf, size_t *have, size_t bytes) {
         e = hipMalloc(buf, bytes);
     }
     if (e != hipSuccess) {
+        (void)hipGetLastError();  // the failed allocation must not surface again in the next launch check
         *buf = nullptr;
         return (int)e;
     }
@@ -257,7 +258,7 @@ int drop_cache(dfdx_rocm_ctx *ctx) {
     CtxLock lock(ctx->mu);
     if (ctx->cache.empty()) return DFDX_ROCM_OK;
     HIP_TRY(hipStreamSynchronize(ctx->stream));
-    hipError_t first = hipSuccess;
+    hipError_t first = free_retired(ctx);
     for (auto &kv : ctx->cache)
         for (void *p : kv.second) {
             const hipError_t e = hipFree(p);
@@ -279,6 +280,36 @@ inline bool use_rank1(const GemmProblem &p) {
     return rank1_supported(p) && !(p.k >= 3 && thin_mfma_supported(p));
 }
 
+// The bandwidth-bound kernels (`Plan::variant` of a DFDX_ROCM_KERNEL_GEMV plan).
+enum { BW_NONE = 0, BW_RANK1 = 1, BW_GEMV_MULTI = 2, BW_GEMV = 3, BW_THIN_MFMA = 4 };
+
+// Which of them takes `p`, if any.  `plain_order`: the caller asked for the contraction order of the tiled kernels
+// (DFDX_ROCM_GEMM_NO_SPLIT_K: the broadcast-rhs forward and grad_lhs, whose results must equal those of the batched
+// product of the same slices bit for bit, matmul/mod.rs:460-473).  The vector-product kernels cut k into grid slices
+// and sum inside a slice in an order of their own, and the vector-ALU form of the thin contraction sums by fused
+// multiply-adds, so none of them qualifies; a rank-1 update has nothing to order, and the matrix-core form of the thin
+// contraction walks k exactly as the tiles do.
+int bandwidth_kernel(const GemmProblem &p, bool plain_order) {
+    if (plain_order) {
+        if (p.k == 1 && rank1_supported(p)) return BW_RANK1;
+        return thin_mfma_supported(p) ? BW_THIN_MFMA : BW_NONE;
+    }
+    if (use_rank1(p)) return BW_RANK1;
+    if (gemv_multi_supported(p)) return BW_GEMV_MULTI;
+    if (gemv_supported(p)) return BW_GEMV;
+    return thin_mfma_supported(p) ? BW_THIN_MFMA : BW_NONE;
+}
+
+const char *bandwidth_kernel_name(const GemmProblem &p, int which) {
+    switch (which) {
+    case BW_RANK1: return p.k == 1 ? "rank1" : "thin_k";
+    case BW_GEMV_MULTI: return "gemv_multi";
+    case BW_GEMV: return "gemv";
+    case BW_THIN_MFMA: return "thin_k_mfma";
+    default: return "none";
+    }
+}
+
 int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProblem &p, Plan *plan) {
     const bool is16 = p.dtype == DT_F16 || p.dtype == DT_BF16;
     const bool is32 = p.dtype == DT_F32, is64 = p.dtype == DT_F64;
@@ -288,10 +319,12 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
     case DFDX_ROCM_KERNEL_GENERIC:
         *plan = {DFDX_ROCM_KERNEL_GENERIC, 0, 1};
         return DFDX_ROCM_OK;
-    case DFDX_ROCM_KERNEL_GEMV:  // the bandwidth-bound kernels: vector products and rank-1 updates
-        if (!gemv_supported(p) && !rank1_supported(p) && !gemv_multi_supported(p) && !thin_mfma_supported(p)) return DFDX_ROCM_ERR_UNSUPPORTED;
-        *plan = {DFDX_ROCM_KERNEL_GEMV, 0, 1};
+    case DFDX_ROCM_KERNEL_GEMV: {  // the bandwidth-bound kernels, forced: the caller's choice outranks the order flag
+        const int bw = bandwidth_kernel(p, false);
+        if (!bw) return DFDX_ROCM_ERR_UNSUPPORTED;
+        *plan = {DFDX_ROCM_KERNEL_GEMV, bw, 1};
         return DFDX_ROCM_OK;
+    }
     case DFDX_ROCM_KERNEL_MFMA: {
         int v = d->variant;
         if (is16 && (v == 0 || (v >= mfma16_dma_first_variant() && v != mfma16_small_variant()))) {  // LDS-DMA family: tile and split count together
@@ -318,8 +351,8 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
     default:
         return DFDX_ROCM_ERR_INVALID_ARG;
     }
-    if (gemv_supported(p) || rank1_supported(p) || gemv_multi_supported(p) || thin_mfma_supported(p)) {
-        *plan = {DFDX_ROCM_KERNEL_GEMV, 0, 1};
+    if (const int bw = bandwidth_kernel(p, (d->flags & DFDX_ROCM_GEMM_NO_SPLIT_K) != 0)) {
+        *plan = {DFDX_ROCM_KERNEL_GEMV, bw, 1};
         return DFDX_ROCM_OK;
     }
     // The small-product kernel where its estimate beats the family's (the f32 family weighs it among its own variants);
@@ -372,33 +405,46 @@ int partials_buffer(dfdx_rocm_ctx *ctx, size_t need, bool static_scratch, float 
     return DFDX_ROCM_OK;
 }
 
+// The f32 partial sums `plan` needs for `p`, in bytes (0: none).
+size_t partials_bytes(const GemmProblem &p, const Plan &plan) {
+    if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1)
+        return p.dtype == DT_F32 ? mfma32_workspace_bytes(p, plan.variant, plan.splits)
+               : plan.variant < mfma16_dma_first_variant()
+                   ? mfma16_workspace_bytes(p, plan.variant, plan.splits)
+                   : mfma16dma_workspace_bytes(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
+    if (plan.kernel == DFDX_ROCM_KERNEL_GEMV && plan.variant == BW_GEMV_MULTI) return gemv_multi_workspace_bytes(p);
+    if (plan.kernel == DFDX_ROCM_KERNEL_GEMV && plan.variant == BW_GEMV) return gemv_workspace_bytes(p);
+    return 0;
+}
+
+// Makes sure the partial sums of `plan` have a place, BEFORE the caller resolves pending zero fills among the operands:
+// a call that is refused here (scratch too small, out of memory) must leave every declaration as it found it.
+int reserve_partials(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan, bool static_scratch) {
+    GemmProblem p = problem;
+    p.compute_units = ctx->compute_units;
+    float *unused = nullptr;
+    const size_t need = partials_bytes(p, plan);
+    return need ? partials_buffer(ctx, need, static_scratch, &unused) : DFDX_ROCM_OK;
+}
+
 int run_plan(dfdx_rocm_ctx *ctx, const GemmProblem &problem, const Plan &plan, bool static_scratch = false) {
     CtxLock lock(ctx->mu);  // a split plan is two launches around the shared workspace
     GemmProblem p = problem;
     p.splits = 1;
     p.workspace = nullptr;
     p.compute_units = ctx->compute_units;
-    if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1) {
-        const size_t need = p.dtype == DT_F32 ? mfma32_workspace_bytes(p, plan.variant, plan.splits)
-                            : plan.variant < mfma16_dma_first_variant()
-                                ? mfma16_workspace_bytes(p, plan.variant, plan.splits)
-                                : mfma16dma_workspace_bytes(p, plan.variant - mfma16_dma_first_variant() + 1, plan.splits);
+    if (const size_t need = partials_bytes(p, plan)) {
         if (int rc = partials_buffer(ctx, need, static_scratch, &p.workspace)) return rc;
-        p.splits = plan.splits;
     }
-    if (plan.kernel == DFDX_ROCM_KERNEL_GEMV) {
-        const bool multi = !use_rank1(p) && gemv_multi_supported(p);
-        if (const size_t need = multi ? gemv_multi_workspace_bytes(p) : gemv_workspace_bytes(p)) {  // (0 for the thin kernels)
-            if (int rc = partials_buffer(ctx, need, static_scratch, &p.workspace)) return rc;
-        }
-    }
+    if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1) p.splits = plan.splits;
     hipError_t e;
     switch (plan.kernel) {
     case DFDX_ROCM_KERNEL_GENERIC: e = launch_generic(p, ctx->stream); break;
     case DFDX_ROCM_KERNEL_GEMV:
-        e = use_rank1(p) ? launch_rank1(p, ctx->stream)
-            : gemv_multi_supported(p) ? launch_gemv_multi(p, ctx->stream)
-            : gemv_supported(p) ? launch_gemv(p, ctx->stream) : launch_thin_mfma(p, ctx->stream);
+        e = plan.variant == BW_RANK1 ? launch_rank1(p, ctx->stream)
+            : plan.variant == BW_GEMV_MULTI ? launch_gemv_multi(p, ctx->stream)
+            : plan.variant == BW_GEMV ? launch_gemv(p, ctx->stream)
+            : plan.variant == BW_THIN_MFMA ? launch_thin_mfma(p, ctx->stream) : hipErrorInvalidValue;
         break;
     case DFDX_ROCM_KERNEL_MFMA:
         e = (p.dtype == DT_F32) ? launch_mfma32(p, plan.variant, ctx->stream)
@@ -439,6 +485,7 @@ int gemm_with_colsum(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, void *
     if (p.m == 0) return DFDX_ROCM_OK;
     Plan plan;  // from the product as the caller states it: a pending zero fill of C must not change which kernel runs
     if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    if (int e = reserve_partials(ctx, p, plan, false)) return e;
     if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
     bool can = p.ksum && plan.kernel == DFDX_ROCM_KERNEL_MFMA;
     if (can && (p.dtype == DT_F16 || p.dtype == DT_BF16))
@@ -552,10 +599,24 @@ int dfdx_rocm_alloc(dfdx_rocm_ctx *ctx, size_t bytes, int zeroed, void **out) {
     }
     if (!recycled) {
         const hipError_t e = hipMalloc(&p, bytes);
-        if (e == hipErrorOutOfMemory && dfdx_rocm_empty_cache(ctx) == DFDX_ROCM_OK) {
+        if (e == hipErrorOutOfMemory) {
+            // once more with everything the context can give back: the cached buffers and the outgrown workspaces
             (void)hipGetLastError();
-            HIP_TRY(hipMalloc(&p, bytes));  // once more with the cached buffers given back
+            (void)dfdx_rocm_empty_cache(ctx);
+            {
+                CtxLock lock(ctx->mu);
+                if (!ctx->retired.empty()) {
+                    HIP_TRY(hipStreamSynchronize(ctx->stream));
+                    (void)free_retired(ctx);
+                }
+            }
+            const hipError_t again = hipMalloc(&p, bytes);
+            if (again != hipSuccess) {
+                (void)hipGetLastError();
+                return (int)again;
+            }
         } else if (e != hipSuccess) {
+            (void)hipGetLastError();
             return (int)e;
         }
         CtxLock lock(ctx->mu);
@@ -600,6 +661,8 @@ int dfdx_rocm_free(dfdx_rocm_ctx *ctx, void *ptr) {
     }
     HIP_TRY(hipStreamSynchronize(ctx->stream));  // pending kernels may still use the buffer
     HIP_TRY(hipFree(ptr));
+    CtxLock lock(ctx->mu);
+    HIP_TRY(free_retired(ctx));  // the stream is drained: nothing uses the outgrown workspaces either
     return DFDX_ROCM_OK;
 }
 
@@ -665,6 +728,12 @@ int dfdx_rocm_settle_zeros(dfdx_rocm_ctx *ctx) {
     return settle_all(ctx);
 }
 
+int dfdx_rocm_forget_zeros(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes) {
+    if (int e = bind(ctx)) return e;
+    if (!ptr && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
+    return bytes ? drop_pending_inside(ctx, ptr, bytes) : DFDX_ROCM_OK;
+}
+
 int dfdx_rocm_copy_h2d(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t bytes) {
     if (int e = bind(ctx)) return e;
     if ((!dst || !src) && bytes) return DFDX_ROCM_ERR_INVALID_ARG;
@@ -672,6 +741,8 @@ int dfdx_rocm_copy_h2d(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t by
         if (int e = drop_pending_inside(ctx, dst, bytes)) return e;
         HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));  // the host buffer may be reused on return
+        CtxLock lock(ctx->mu);
+        HIP_TRY(free_retired(ctx));
     }
     return DFDX_ROCM_OK;
 }
@@ -683,6 +754,8 @@ int dfdx_rocm_copy_d2h(dfdx_rocm_ctx *ctx, void *dst, const void *src, size_t by
         if (int e = settle_range(ctx, src, bytes)) return e;
         HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));
+        CtxLock lock(ctx->mu);
+        HIP_TRY(free_retired(ctx));
     }
     return DFDX_ROCM_OK;
 }
@@ -714,6 +787,7 @@ int dfdx_rocm_gemm(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc) {
     if (p.m == 0) return DFDX_ROCM_OK;
     Plan plan;  // from the product as the caller states it: a pending zero fill of C must not change which kernel runs
     if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    if (int e = reserve_partials(ctx, p, plan, false)) return e;
     if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
     return run_plan(ctx, p, plan);
 }
@@ -725,6 +799,7 @@ int dfdx_rocm_gemm_noalloc(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc) 
     if (p.m == 0) return DFDX_ROCM_OK;
     Plan plan;  // from the product as the caller states it: a pending zero fill of C must not change which kernel runs
     if (int e = make_plan(ctx, desc, p, &plan)) return e;
+    if (int e = reserve_partials(ctx, p, plan, /*static_scratch=*/true)) return e;
     if (int e = settle_operands(ctx, &p, /*may_overwrite=*/true)) return e;
     return run_plan(ctx, p, plan, /*static_scratch=*/true);
 }
@@ -738,7 +813,7 @@ int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int
     if (p.m != 0)
         if (int e = make_plan(ctx, desc, p, &plan)) return e;
     if (kernel) *kernel = plan.kernel;
-    if (variant) *variant = plan.variant;
+    if (variant) *variant = plan.kernel == DFDX_ROCM_KERNEL_GEMV ? 0 : plan.variant;  // (a tile variant; the bandwidth kernels have none)
     if (name && name_len) {
         if (plan.kernel == DFDX_ROCM_KERNEL_MFMA && plan.splits > 1)
             std::snprintf(name, name_len, "%s_%s_splitk%d", p.dtype == DT_F32 ? "mfma32" : "mfma16",
@@ -749,7 +824,7 @@ int dfdx_rocm_gemm_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc, int
             std::snprintf(name, name_len, "%s_%s", p.dtype == DT_F32 ? "mfma32" : "mfma16",
                           p.dtype == DT_F32 ? mfma32_variant_name(plan.variant) : mfma16_variant_name(plan.variant));
         else
-            std::snprintf(name, name_len, "%s", plan.kernel != DFDX_ROCM_KERNEL_GEMV ? "generic" : use_rank1(p) ? (p.k == 1 ? "rank1" : "thin_k") : gemv_multi_supported(p) ? "gemv_multi" : gemv_supported(p) ? "gemv" : "thin_k_mfma");
+            std::snprintf(name, name_len, "%s", plan.kernel != DFDX_ROCM_KERNEL_GEMV ? "generic" : bandwidth_kernel_name(p, plan.variant));
     }
     return DFDX_ROCM_OK;
 }

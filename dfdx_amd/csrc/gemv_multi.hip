@@ -342,6 +342,8 @@ Shape classify(const GemmProblem &g) {
     } else {
         return s;
     }
+    // the combine kernels number the r * j outputs with a 32-bit index, a block of 256 past the end included
+    if ((int64_t)p.r * (int64_t)p.j >= (1ll << 31) - 256) return s;
     // worth a kernel of its own where streaming the matrix is the cost: a megabyte of it at least
     if ((double)p.j * (double)g.k * (double)dtype_size(g.dtype) < 1048576.0) return s;
     // 16-bit types: once 128-column matrix-core tiles give every compute unit a workgroup they stream the matrix as fast

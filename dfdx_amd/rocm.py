@@ -16,6 +16,7 @@ from __future__ import annotations
 
 import ctypes
 import os
+import weakref
 from dataclasses import dataclass
 from typing import Optional, Sequence
 
@@ -73,7 +74,8 @@ _lib = None
 EXPORTS = [
     "dfdx_rocm_create", "dfdx_rocm_destroy", "dfdx_rocm_strerror", "dfdx_rocm_device_info",
     "dfdx_rocm_alloc", "dfdx_rocm_free", "dfdx_rocm_memset_zero", "dfdx_rocm_copy_h2d", "dfdx_rocm_copy_d2h",
-    "dfdx_rocm_copy_d2d", "dfdx_rocm_synchronize", "dfdx_rocm_zero_deferred", "dfdx_rocm_settle_zeros", "dfdx_rocm_enable_cache", "dfdx_rocm_disable_cache",
+    "dfdx_rocm_copy_d2d", "dfdx_rocm_synchronize", "dfdx_rocm_zero_deferred", "dfdx_rocm_settle_zeros", "dfdx_rocm_forget_zeros",
+    "dfdx_rocm_enable_cache", "dfdx_rocm_disable_cache",
     "dfdx_rocm_empty_cache", "dfdx_rocm_cache_stats", "dfdx_rocm_gemm", "dfdx_rocm_gemm_noalloc", "dfdx_rocm_gemm_plan",
     "dfdx_rocm_mfma_variant_count", "dfdx_rocm_gemm_time", "dfdx_rocm_gemm_time_rotating",
     "dfdx_rocm_matmat_forward", "dfdx_rocm_matmat_backward",
@@ -119,6 +121,7 @@ class View:
     shape: tuple
     strides: tuple
     offset: int = 0             # in elements
+    owner: "object" = None      # keeps an arena's declarations alive exactly as long as views of it exist (zeros_many)
 
     @property
     def ptr(self) -> int:
@@ -127,10 +130,32 @@ class View:
     def permute(self, *axes) -> "View":
         """Zero-copy permute (reference: tensor_ops/permute_to.rs:38-52)."""
         return View(self.storage, self.dtype, tuple(self.shape[a] for a in axes),
-                    tuple(self.strides[a] for a in axes), self.offset)
+                    tuple(self.strides[a] for a in axes), self.offset, self.owner)
 
     def numel_storage(self) -> int:
         return self.storage.numel() // ITEMSIZE[self.dtype]
+
+
+class _Arena:
+    """One allocation that several Views are carved from.  When the last View of it goes, whatever zero declarations
+    its pieces still carry are withdrawn (``dfdx_rocm_forget_zeros``) BEFORE torch gets the memory back, so that a later
+    settle cannot write zeros into memory that has a new owner by then."""
+
+    def __init__(self, dev: "Rocm", raw):
+        self.raw = raw
+        self._fin = weakref.finalize(self, _forget_range, weakref.ref(dev), raw, raw.data_ptr(), raw.numel())
+        self._fin.atexit = False   # at interpreter exit the context goes first and takes its declarations with it
+
+    def forget(self):
+        self._fin()
+
+
+def _forget_range(dev_ref, raw, ptr, nbytes):
+    # `raw` is held by this callback's arguments: the memory is still allocated while the declarations are dropped
+    dev = dev_ref()
+    if dev is not None and getattr(dev, "ctx", None):
+        dev.lib.dfdx_rocm_forget_zeros(dev.ctx, ctypes.c_void_p(ptr), ctypes.c_size_t(nbytes))
+    del raw
 
 
 def _row_major(shape):
@@ -218,6 +243,11 @@ class Rocm:
         accumulates into the whole buffer stores 0 + value, any other first use runs the fill."""
         self._check(self.lib.dfdx_rocm_zero_deferred(self.ctx, ctypes.c_void_p(ptr), ctypes.c_size_t(nbytes)))
 
+    def forget_zeros(self, ptr: int, nbytes: int):
+        """Withdraws the zero declarations inside ``[ptr, ptr + nbytes)`` without filling (``dfdx_rocm_forget_zeros``):
+        what the owner of declared storage calls before it releases that storage unsettled."""
+        self._check(self.lib.dfdx_rocm_forget_zeros(self.ctx, ctypes.c_void_p(ptr), ctypes.c_size_t(nbytes)))
+
     def settle_zeros(self):
         """Runs every deferred fill still pending: needed before code outside the library reads such a buffer."""
         self._check(self.lib.dfdx_rocm_settle_zeros(self.ctx))
@@ -251,19 +281,27 @@ class Rocm:
         small fills are launch-bound (3.5 us for 2 MiB), one large fill runs at the HBM write rate.
         ``deferred``: no fill at all; every piece is declared zero (``zero_deferred``) and the first backward op that
         accumulates into the whole of it stores instead -- read the results through this object (``to_host``) or
-        call ``settle_zeros`` first."""
+        call ``settle_zeros`` first.  The declarations are withdrawn when the last of the returned Views (and of the
+        Views derived from them) is dropped, so the arena never goes back to the allocator with a fill still promised."""
         sizes = [max(int(np.prod(v.shape, dtype=np.int64)) * ITEMSIZE[v.dtype], 16) for v in likes]
         offs, total = [], 0
         for n in sizes:
             offs.append(total)
             total += (n + 255) // 256 * 256
+        owner = None
         if deferred:
             arena = self._torch.empty(max(total, 16), dtype=self._torch.uint8, device=self.device)
-            for o, n in zip(offs, sizes):
-                self.zero_deferred(arena.data_ptr() + o, n)
+            owner = _Arena(self, arena)
+            try:
+                for o, n in zip(offs, sizes):
+                    self.zero_deferred(arena.data_ptr() + o, n)
+            except Exception:
+                owner.forget()
+                raise
         else:
             arena = self._zeroed_bytes(max(total, 16))
-        return [View(arena[o:o + n], v.dtype, tuple(v.shape), _row_major(tuple(v.shape))) for v, o, n in zip(likes, offs, sizes)]
+        return [View(arena[o:o + n], v.dtype, tuple(v.shape), _row_major(tuple(v.shape)), 0, owner)
+                for v, o, n in zip(likes, offs, sizes)]
 
     def _zeroed_bytes(self, nbytes: int):
         """Device memory from torch's allocator, cleared by the library's own fill kernel (``dfdx_rocm_memset_zero``)."""
@@ -544,7 +582,7 @@ class Rocm:
         assert int(np.prod(x.shape, dtype=np.int64)) == int(np.prod(new_shape, dtype=np.int64)), \
             f"left: {int(np.prod(x.shape))}\n right: {int(np.prod(new_shape))}"
         if x.strides == _row_major(x.shape):
-            return View(x.storage, x.dtype, new_shape, _row_major(new_shape), x.offset)
+            return View(x.storage, x.dtype, new_shape, _row_major(new_shape), x.offset, x.owner)
         out = self.empty(x.dtype, new_shape)
         vp = ctypes.c_void_p
         self._check(self.lib.dfdx_rocm_reshape_forward(self.ctx, DTYPES[x.dtype], len(x.shape), _i64arr(x.shape),

@@ -110,10 +110,23 @@ int dfdx_rocm_synchronize(dfdx_rocm_ctx *ctx);
  * up by the pointer a call is given: hand views of it to the library by a
  * pointer inside the buffer.  Code outside this library that reads the memory
  * (another stream, a host copy not made by dfdx_rocm_copy_d2h) must call
- * dfdx_rocm_settle_zeros or dfdx_rocm_synchronize first. */
+ * dfdx_rocm_settle_zeros or dfdx_rocm_synchronize first.
+ * A declaration on storage the caller owns (dfdx_rocm_zero_deferred) lives
+ * until a call consumes it; the library cannot see that storage being
+ * released.  Before the caller frees, reuses or hands back such memory it must
+ * either settle it (dfdx_rocm_settle_zeros, dfdx_rocm_synchronize) or
+ * withdraw the declaration with dfdx_rocm_forget_zeros(ptr, bytes): every
+ * declaration that lies wholly inside [ptr, ptr + bytes) is dropped without a
+ * fill, one that reaches beyond either end is filled now (the memory is still
+ * the caller's at that point).  Otherwise a later settle would write zeros
+ * into memory that belongs to somebody else by then (the reference releases
+ * gradient storage in mid-step: `Gradients::drop_non_leafs`,
+ * tensor/gradients.rs:73-78).  Forgetting a range without declarations is not
+ * an error. */
 #define DFDX_ROCM_ZERO_DEFERRED 2
 int dfdx_rocm_zero_deferred(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes);
 int dfdx_rocm_settle_zeros(dfdx_rocm_ctx *ctx);
+int dfdx_rocm_forget_zeros(dfdx_rocm_ctx *ctx, void *ptr, size_t bytes);
 
 /* The allocation cache of the device (`Cache::try_enable_cache`,
  * `try_disable_cache`, `try_empty_cache`: dfdx-core/src/tensor/
@@ -170,9 +183,10 @@ typedef struct dfdx_rocm_gemm_desc {
 
 /* flags.  Long contractions with few output tiles (weight gradients) are split along k over several
  * workgroups whose f32 partial sums are combined in a fixed order (deterministic).  NO_SPLIT_K keeps the
- * plain k-ascending order; the broadcast-rhs forward / grad_lhs use it so that they stay bit-identical to
- * the batched kernels (dfdx tests assert that equality, matmul/mod.rs:467-472).  SPLIT_K(n) forces n
- * splits (testing / tuning). */
+ * contraction order of the tiled kernels: no split, no k-sliced small-product kernel, and none of the vector-product
+ * kernels for few rows or columns (they cut k into slices too).  The broadcast-rhs forward / grad_lhs use it so that
+ * they stay bit-identical to the batched kernels whatever the number of rows (dfdx tests assert that equality,
+ * matmul/mod.rs:460-473).  SPLIT_K(n) forces n splits (testing / tuning). */
 #define DFDX_ROCM_GEMM_NO_SPLIT_K 1
 #define DFDX_ROCM_GEMM_SPLIT_K(n) (((n) & 0xff) << 8)
 
@@ -189,7 +203,9 @@ int dfdx_rocm_gemm(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *desc);
  * (one copy per GPU, held until the process ends) and calls no hipMalloc /
  * hipFree or any other allocating routine.  A plan whose partial sums do not
  * fit is refused with DFDX_ROCM_ERR_SCRATCH_TOO_SMALL before anything is
- * launched (the caller may then lower or forbid the split through `flags`).
+ * launched and before any pending zero declaration of an operand is touched
+ * (the caller may then lower or forbid the split through `flags`, or call
+ * dfdx_rocm_gemm with the same descriptor).
  * Nothing in the array has to start at zero: every partial sum that is read
  * has been written by the same call.  All calls on one GPU share the array,
  * so calls that overlap on one GPU (two contexts, two streams, two threads)

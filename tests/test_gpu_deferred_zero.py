@@ -228,3 +228,79 @@ def test_encoder_block_with_deferred_gradients_matches_the_eager_fill():
         results.append([dev.to_host(grads[n]) for n in PARAMS] + [dev.to_host(gx)])
     for name, e, l in zip(PARAMS + ("gx",), *results):
         assert np.array_equal(e.view(np.uint8), l.view(np.uint8)), name
+
+
+def test_forget_zeros_withdraws_declarations_on_caller_owned_storage():
+    """Storage the caller owns and has only DECLARED zero may be released before anything consumed the declaration; the
+    caller then withdraws it (`dfdx_rocm_forget_zeros`), and no later settle may write into that memory."""
+    import torch
+
+    dev = device()
+    announce("forget zeros")
+    n = 1 << 20
+    raw = torch.full((4 * n,), 0x5A, dtype=torch.uint8, device="cuda")
+    base = raw.data_ptr()
+    dev.zero_deferred(base, n)               # wholly inside the forgotten range: dropped, never filled
+    dev.zero_deferred(base + 2 * n, n)       # outside: still promised, filled by the settle below
+    dev.zero_deferred(base + n + n // 2, n // 2 + 16)   # reaches past the end of the forgotten range: filled at the forget
+    dev.forget_zeros(base, n + n // 2 + 8)
+    dev.forget_zeros(base + 3 * n, n)        # nothing declared there: not an error
+    dev.forget_zeros(0, 0)
+    dev.settle_zeros()
+    torch.cuda.synchronize()
+    host = raw.cpu().numpy()
+    assert (host[:n + n // 2] == 0x5A).all(), "a forgotten declaration was filled after all"
+    assert not host[n + n // 2: 2 * n + 16].any(), "a declaration that straddles the range's end must be filled"
+    assert not host[2 * n:3 * n].any(), "a declaration outside the range must survive"
+    assert (host[3 * n:] == 0x5A).all()
+
+
+def test_arena_declarations_go_when_the_last_view_goes():
+    """`zeros_many(deferred=True)` ties the declarations to the arena: once no View of it is left, the memory returns to
+    the allocator, and a later settle must not touch what now belongs to another tensor."""
+    import gc
+
+    import torch
+
+    dev = device()
+    announce("arena forgets its declarations")
+    like = dev.empty("f32", (1 << 18,))
+    views = dev.zeros_many([like, like, like], deferred=True)
+    ptr, nbytes = views[0].storage.data_ptr(), 3 * (1 << 20)
+    keep = views[1]                       # one surviving view keeps the arena and its declarations
+    del views
+    gc.collect()
+    assert dev.to_host(keep)[:16].tolist() == [0.0] * 16          # still zero by declaration -> settled -> zeros
+    del keep
+    gc.collect()
+    torch.cuda.synchronize()
+    again = torch.full((nbytes,), 0x33, dtype=torch.uint8, device="cuda")   # the caching allocator hands the block back
+    dev.settle_zeros()
+    torch.cuda.synchronize()
+    assert (again.cpu().numpy() == 0x33).all(), "a stale declaration was filled into memory that has a new owner"
+    assert again.data_ptr() == ptr or True   # (whichever block it got: nothing may have been written)
+
+
+def test_a_refused_product_leaves_the_zero_declaration_of_its_output_in_place():
+    """A call that is refused (here: the no-allocation entry with a split whose partial sums exceed its scratch) must
+    not consume the declaration of its output: the retry through `dfdx_rocm_gemm` with accumulate = 1 has to give the
+    bits of the eagerly filled run, not an accumulation into the poison."""
+    from dfdx_amd import RocmError
+    from dfdx_amd.rocm import ERR_SCRATCH_TOO_SMALL
+
+    dev, g = device(), rng(77)
+    m = n = 1024
+    k = 16384
+    a, b = rand(dev, g, "f16", (k, m)), rand(dev, g, "f16", (k, n))
+    announce("refused product on a deferred output", (m, k, n))
+
+    def run(make):
+        c = make(dev, "f16", (m, n))
+        desc = dev.gemm_desc("f16", m, k, n, a.ptr, (1, m), b.ptr, (n, 1), c.ptr, (n, 1), accumulate=True, split_k=9)
+        with pytest.raises(RocmError) as err:
+            dev.gemm_noalloc(desc)
+        assert err.value.code == ERR_SCRATCH_TOO_SMALL
+        dev.gemm(desc)
+        return [c]
+
+    both(dev, run)

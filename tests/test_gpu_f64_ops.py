@@ -118,12 +118,15 @@ def test_reshape_and_bias_f64():
     close(host(dev, gb), gb0 + gy.sum(axis=0), 128)
 
 
-def test_small_encoder_block_entirely_on_the_device_f64():
+@pytest.mark.parametrize("dims", [(2, 32, 64, 4, 128), (2, 24, 96, 4, 160)])
+def test_small_encoder_block_entirely_on_the_device_f64(dims):
+    """Head dimension 16: 1/sqrt(16) is a float, the scale rides in the softmax kernel.  Head dimension 24: it is not,
+    and the block multiplies by the double scalar in an op of its own (multi_head_attention.rs:133-134)."""
     from dfdx_amd.encoder import EncoderBlock
     from encoder_ref import OracleBackend, encoder_block, init_params, val
 
     dev, g = device(), rng(805)
-    B, S, d, H, ff = 2, 32, 64, 4, 128
+    B, S, d, H, ff = dims
     p = init_params(g, d, ff, D, std=0.2)
     for name in ("g1", "g2", "be1", "be2"):
         p[name] = val(p[name], D) + 0.1 * g.standard_normal(d)

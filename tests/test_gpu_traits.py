@@ -84,8 +84,8 @@ def test_linear_literals(case, dtype, fused):
 
 
 # ------------------------------------------------------------------ identities --
-def sample(dev, g, shape, dtype):
-    return upload(dev, g.standard_normal(shape), dtype)
+def sample(dev, g, shape, dtype, scale=1.0):
+    return upload(dev, g.standard_normal(shape) * scale, dtype)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
@@ -135,6 +135,38 @@ def test_matmul_broadcast(dtype, dims):
     assert np.array_equal(dev.to_host(r3), dev.to_host(r)), "Br and Batch3 forward differ bitwise"
     assert np.array_equal(dev.to_host(ga3), dev.to_host(ga)), "Br and Batch3 grad_lhs differ bitwise"
     assert_within(dtype, bsz * m, host(dev, gb3).sum(axis=0), want_gb, A, G, extra=bsz * ulp * np.abs(want_gb).max())
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("dims", [(2, 4, 4096, 4096), (2, 1, 4096, 4096), (16, 1, 16384, 4096), (3, 2, 8192, 1024), (2, 5, 64, 16384)])
+def test_matmul_broadcast_few_rows_exact(dtype, dims):
+    """The reference's exact identity Br == Batch3 with the rhs stacked (mod.rs:460-473) where the broadcast form folds to
+    a FEW rows against a large matrix: a Linear layer on a handful of tokens.  Those shapes would otherwise go to the
+    vector-product kernels, which cut the contraction into grid slices; the broadcast entry points ask for the tiled
+    kernels' contraction order, so forward and grad_lhs must equal the batched product bit for bit whatever the row
+    count.  The stacked rhs is built on the device (up to 4 GiB in f32)."""
+    dev, g = device(), rng(66)
+    bsz, m, k, n = dims
+    announce("broadcast identity, few rows", dtype, dims)
+    from dfdx_amd.rocm import View
+    a, b, go = sample(dev, g, (bsz, m, k), dtype), sample(dev, g, (k, n), dtype, scale=k ** -0.5), sample(dev, g, (bsz, m, n), dtype)
+    r = dev.forward(a, b)
+    ga, gb = dev.zeros_like_storage(a), dev.zeros_like_storage(b)
+    dev.backward(a, ga, b, gb, go)
+    A, B, G = host(dev, a), host(dev, b), host(dev, go)
+    ulp = {"f32": 2.0 ** -24, "f16": 2.0 ** -11, "bf16": 2.0 ** -8}[dtype]
+    assert_within(dtype, k, host(dev, r), A @ B, A, B, extra=ulp * np.abs(A @ B).max(), what="out")
+    assert_within(dtype, n, host(dev, ga), G @ B.T, G, B, extra=ulp * np.abs(G @ B.T).max(), what="grad_lhs")
+    want_gb = np.einsum("bmk,bmn->kn", A, G)
+    assert_within(dtype, bsz * m, host(dev, gb), want_gb, A, G, extra=ulp * np.abs(want_gb).max(), what="grad_rhs")
+    del A, G, want_gb
+
+    b_up = View(b.storage.repeat(bsz), dtype, (bsz, k, n), row_major_strides((bsz, k, n)))
+    r3 = dev.forward(a, b_up)
+    ga3, gb3 = dev.zeros_like_storage(a), dev.zeros_like_storage(b_up)
+    dev.backward(a, ga3, b_up, gb3, go)
+    assert np.array_equal(dev.to_host(r3), dev.to_host(r)), "Br and Batch3 forward differ bitwise"
+    assert np.array_equal(dev.to_host(ga3), dev.to_host(ga)), "Br and Batch3 grad_lhs differ bitwise"
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
