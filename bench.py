@@ -36,6 +36,10 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="wall-clock span of the CPU baseline sample")
     ap.add_argument("--spinup-ms", type=float, default=300.0,
                     help="untimed device spin-up before the first warm-up step (0 disables it)")
+    ap.add_argument("--operands", choices=["uniform", "zeros"], default="uniform",
+                    help="uniform = the benchmark's U(-1,1) entries; zeros = all-zero operands, the same launches without the "
+                         "power that toggling operands draw (a probe of the kernel's cycle count: NOT the headline workload, "
+                         "and the JSON line says so)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -67,6 +71,9 @@ def main():
         gen = torch.Generator(device="cuda").manual_seed(1234)
         a = (torch.rand(N, N, device="cuda", generator=gen) * 2 - 1).to(tdt[dtype])
         b = (torch.rand(N, N, device="cuda", generator=gen) * 2 - 1).to(tdt[dtype])
+        if args.operands == "zeros":
+            a.zero_()
+            b.zero_()
         c = torch.zeros(N, N, device="cuda", dtype=tdt[dtype])
         layouts = {"A.B": ((N, 1), (N, 1)), "At.B": ((1, N), (N, 1)), "A.Bt": ((N, 1), (1, N))}
         if dtype in ("bf16", "f64"):
@@ -135,11 +142,13 @@ def main():
         "value": min(headline["tflops"], headline["kernel_tflops"]), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": headline["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
+        "dtype": "f16", "data": "synthetic" if args.operands == "uniform" else "all-zero operands: a power probe, not the benchmark's workload",
         "config": {"workload": "configs[1]: single square GEMM C=A.B, M=N=K=4096, f16 in / f32 accumulate, row-major A and B ~U(-1,1)",
                    "step": "one GEMM launch (137.44 GFLOP)", "device": info},
         "roofline": {"bound": "mfma", "achieved": headline["kernel_tflops"], "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
                      "frac": round(headline["kernel_tflops"] / PEAK_TFLOPS["f16"], 4), "traffic": traffic,
+                     "traffic_source": ("stored figure: HBM-side bytes per launch of this kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE "
+                                        "runs, profiles/gemm_f16_4096_hbm_traffic.txt -- not measured in this run") if traffic else None,
                      "kernel": headline["kernel"]},
         "cpu_baseline": cpu,
         "cpu_proxy_openblas": proxy,

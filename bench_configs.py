@@ -25,12 +25,13 @@ def main():
     ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them, shapes = shape classes outside the configurations: few rows or columns, thin contractions, rank-1 updates, mid-size products, plancheck = the planner's pick against every forced tile variant and split count on a fixed list of shapes; exits 1 with --strict when a pick is more than --plancheck-slack off the best)")
     ap.add_argument("--strict", action="store_true", help="plancheck: exit status 1 when a pick is flagged")
     ap.add_argument("--plancheck-slack", type=float, default=0.10, help="plancheck: flag a pick that is this much slower than the best forced candidate")
-    ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "f32-forms"],
+    ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "f32-forms", "layouts"],
                     help="counter-collection aids for rocprofv3, nothing is timed: traffic = 3 plain 256 MiB device copies (a kernel "
                          "of known size that calibrates FETCH_SIZE / WRITE_SIZE) then 5 launches of the 4096^3 f16 GEMM; rows = the same copies, then 3 launches each of "
                          "the HBM-bound rows (config 4 scores and dP, the 16384^2 f16 vec.mat and the rank-1 update that is its weight gradient, softmax forward and backward on the scores); f32-forms = 3 "
                          "launches each of the register-staged and the LDS-DMA f32 kernel (256x256 tile) on 4096^3 A.B^T and A.B; variants = 3 "
-                         "launches of that GEMM with every f16 MFMA tile variant forced in turn")
+                         "launches of that GEMM with every f16 MFMA tile variant forced in turn; layouts = 5 launches each of the f16 4096^3 GEMM as "
+                         "A.B^T, A.B and A^T.B, then bf16 A.B (the planner's kernel: one tile, four operand layouts)")
     ap.add_argument("--no-rotate", action="store_true", help="skip the second timing of the HBM-bound cases over rotating buffer sets")
     args = ap.parse_args()
     import torch
@@ -59,6 +60,22 @@ def main():
                 dev.gemm(desc)
             torch.cuda.synchronize()
             print(json.dumps({"probe": "3 x 256 MiB copy, 5 x " + dev.gemm_plan(desc)[2]}))
+        elif args.probe == "layouts":
+            names = []
+            cases = [("f16", (n, 1), (1, n)), ("f16", (n, 1), (n, 1)), ("f16", (1, n), (n, 1))]
+            for dt_, astr, bstr in cases:
+                desc = dev.gemm_desc(dt_, n, n, n, a.data_ptr(), astr, b.data_ptr(), bstr, c.data_ptr(), (n, 1))
+                names.append(dev.gemm_plan(desc)[2] + " A%s B%s" % ("" if astr[1] == 1 else "^T", "" if bstr[1] == 1 else "^T"))
+                for _ in range(5):
+                    dev.gemm(desc)
+                torch.cuda.synchronize()
+            ab, bb, cb = a.bfloat16(), b.bfloat16(), c.bfloat16()
+            desc = dev.gemm_desc("bf16", n, n, n, ab.data_ptr(), (n, 1), bb.data_ptr(), (n, 1), cb.data_ptr(), (n, 1))
+            names.append(dev.gemm_plan(desc)[2] + " bf16 A B")
+            for _ in range(5):
+                dev.gemm(desc)
+            torch.cuda.synchronize()
+            print(json.dumps({"probe": names}))
         elif args.probe == "f32-forms":
             del a, b, c
             a, b, c = (torch.randn(n, n, device="cuda", dtype=torch.float32) for _ in range(3))

@@ -103,7 +103,11 @@ template <int ROWS> __device__ __forceinline__ int mc_swizzle(int k) {
 }
 
 // One operand tile in LDS, filled by LDS-DMA loads (16 B per lane, 1 KB contiguous per wave instruction).
-template <int ROWS, int NWAVES, bool KC> struct DmaTile {
+// PERM (k-contiguous B tiles of wave tiles that are at least 32 columns wide): the fragments of such a tile do not take
+// 16 consecutive rows but the rows 8q + 4 * (fragment parity) + 0..3, q = 0..3, of a 32-row group (see the epilogue: a
+// lane then owns 8 consecutive columns of C without any exchange between lanes).  The swizzle follows the lane that
+// reads the row, (2 * (r / 8 % 4) + r % 4 / 2), so that the banks a fragment read touches are those of the plain order.
+template <int ROWS, int NWAVES, bool KC, bool PERM = false> struct DmaTile {
     static constexpr int BYTES = ROWS * BK * 2;
     static constexpr int INSTRS = BYTES / 1024;
     static constexpr int IPW = INSTRS / NWAVES;
@@ -121,7 +125,7 @@ template <int ROWS, int NWAVES, bool KC> struct DmaTile {
             const int slot = (wave * IPW + i) * 64 + lane;  // 16 B slot index inside the tile
             const int r = slot / CPR, cp = slot % CPR;
             if constexpr (KC) {
-                const int c = cp ^ ((r >> 1) & 7);
+                const int c = PERM ? cp ^ ((((r >> 3) & 3) << 1) | ((r >> 1) & 1)) : cp ^ ((r >> 1) & 7);
                 goff[i] = (uint32_t)(min(r, rows_left - 1) * ld + c * 8) * 2u + (uint32_t)(1024 * (IPW - 1 - i));
             } else {
                 const int c = cp ^ mc_swizzle<ROWS>(r);
@@ -171,8 +175,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
     constexpr int TM = WTM / 16, TN = WTN / 16;
     static_assert(WTM % 64 == 0 && WTN % 16 == 0, "wave tile must be a multiple of 64 x 16");
     constexpr int Q = TM / 4;  // tile rows per quarter of a k step
+    // B stored along k and a wave tile of whole fragment pairs: the rows (n) of B are dealt to the fragments so that the
+    // two accumulators acc[i][2jp], acc[i][2jp + 1] of a lane hold 8 CONSECUTIVE columns of C, n = 32 jp + 8 lq + 0..7
+    // (fragment 2jp + par, MFMA row 4 lq + v  <->  n = 32 jp + 8 lq + 4 par + v), instead of two runs of 4 that the lane
+    // rows would have to trade.  Same products, same k order, same bits; the epilogue loses its cross-lane exchange.
+    constexpr bool PERM = B_KC && TN % 2 == 0;
     using TA = DmaTile<BM, NW, A_KC>;
-    using TB = DmaTile<BN, NW, B_KC>;
+    using TB = DmaTile<BN, NW, B_KC, PERM>;
     constexpr int STAGE_BYTES = TA::BYTES + TB::BYTES;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
@@ -274,7 +283,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
     for (int ks = 0; ks < 2; ks++) {
         const int c = ks * 4 + lq;
         a_off[ks] = (wm0 + l16) * BK * 2 + ((c ^ ((l16 >> 1) & 7)) * 16);
-        b_off[ks] = (wn0 + l16) * BK * 2 + ((c ^ ((l16 >> 1) & 7)) * 16);
+        b_off[ks] = (wn0 + (PERM ? 8 * (l16 / 4) + l16 % 4 : l16)) * BK * 2 + ((c ^ ((l16 >> 1) & 7)) * 16);
     }
     // m/n-contiguous: lane 16*g + L supplies the address of X[k = 8*g + L/4 (+32*ks, +4)][col = w0 + 16*t + 4*(L%4)];
     // the transposing read hands lane L the 4 k-values of column w0 + 16*t + L.  k + 4 and k + 32 leave the
@@ -370,7 +379,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
         [[maybe_unused]] const uint32_t base = lds_addr(sa);
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            if constexpr (B_KC) bf[j] = *(const u32x4 *)(sb + b_off[ks] + j * 16 * BK * 2);
+            if constexpr (B_KC) bf[j] = *(const u32x4 *)(sb + b_off[ks] + (PERM ? (j / 2) * 32 + (j % 2) * 4 : j * 16) * BK * 2);
             else bf[j] = tr_frag(base + b_tr[j], std::integral_constant<int, BN>{}, ks_tag);
         }
     };
@@ -537,9 +546,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
         float *wbase = p.ws + split * p.ws_split_stride;
 #pragma unroll
         for (int i = 0; i < TM; i++) {
-            float *wrow = wbase + (int64_t)(bm0 + wm0 + i * 16 + l16) * p.ws_ld + bn0 + wn0 + lq * 4;
+            float *wrow = wbase + (int64_t)(bm0 + wm0 + i * 16 + l16) * p.ws_ld + bn0 + wn0 + lq * (PERM ? 8 : 4);
 #pragma unroll
-            for (int j = 0; j < TN; j++) *(f32x4 *)(wrow + j * 16) = acc[i][j];
+            for (int j = 0; j < TN; j++) *(f32x4 *)(wrow + (PERM ? (j / 2) * 32 + (j % 2) * 4 : j * 16)) = acc[i][j];
         }
         return ST_SPLIT;
     }
@@ -560,7 +569,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
                 if (p.bias_mode == BIAS_PER_COL) {
 #pragma unroll
                     for (int jp = 0; jp < TN / 2; jp++)
-                        cbias[jp] = *(const u32x4 *)(p.bias + min(bn0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8, p.n - 8));
+                        cbias[jp] = *(const u32x4 *)(p.bias + min(bn0 + wn0 + (PERM ? jp * 32 + lq * 8 : (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8), p.n - 8));
                 }
                 if (p.bias_mode == BIAS_PER_ROW) {
 #pragma unroll
@@ -576,12 +585,17 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
                         float v[8];
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i][2 * jp][e]),
-                                                                            __float_as_uint(acc[i][2 * jp + 1][e]), false, false);
-                            v[e] = __uint_as_float(r[0]);
-                            v[4 + e] = __uint_as_float(r[1]);
+                            if constexpr (PERM) {
+                                v[e] = acc[i][2 * jp][e];
+                                v[4 + e] = acc[i][2 * jp + 1][e];
+                            } else {
+                                const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i][2 * jp][e]),
+                                                                                __float_as_uint(acc[i][2 * jp + 1][e]), false, false);
+                                v[e] = __uint_as_float(r[0]);
+                                v[4 + e] = __uint_as_float(r[1]);
+                            }
                         }
-                        const int gn = bn0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8;
+                        const int gn = bn0 + wn0 + (PERM ? jp * 32 + lq * 8 : (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8);
                         if (!row_ok || gn >= p.n) continue;  // n % 8 == 0 here: all 8 columns are in range
                         if (p.bias_mode == BIAS_PER_ROW) {
 #pragma unroll
@@ -614,7 +628,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
             // + immediate: no address arithmetic in vector registers per access.
             const int wave_u = __builtin_amdgcn_readfirstlane(wave);
             char *const tile_base = (char *)(cbase + (int64_t)(bm0 + (wave_u / WAVES_N) * WTM) * p.ldc + bn0 + (wave_u % WAVES_N) * WTN);
-            const uint32_t lane_off = (uint32_t)(l16 * (int)p.ldc + (lq & 1) * 16 + (lq >> 1) * 8) * 2u;
+            const uint32_t lane_off = (uint32_t)(l16 * (int)p.ldc + (PERM ? lq * 8 : (lq & 1) * 16 + (lq >> 1) * 8)) * 2u;
             const int64_t row_step = p.ldc * 32;  // 16 rows, bytes
             // A wave tile that is 64 columns wide (TN == 4) writes whole 128 B lines: after the 16-lane swaps a lane
             // row holds the left 64 B of matrix row l16 in one register set and the right 64 B in another; lanes
@@ -624,7 +638,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
             // halves from different instructions (and 19 GB/s in 32 B pieces); with half lines the stores of a
             // K = 64 work item take longer to leave the CU than its MFMAs take to compute.
             [[maybe_unused]] const uint32_t line_off =
-                (uint32_t)((l16 & 7) * (int)p.ldc * 2 + (l16 >> 3) * 64 + ((lq & 1) * 2 + (lq >> 1)) * 16);
+                (uint32_t)((l16 & 7) * (int)p.ldc * 2 + (l16 >> 3) * 64 + (PERM ? lq : (lq & 1) * 2 + (lq >> 1)) * 16);
             [[maybe_unused]] const int64_t half_step = p.ldc * 16;  // 8 rows, bytes
             // Pure overwrite of an interior tile, optionally with a per-column bias (every forward product of whole
             // tiles, Linear's fused bias included): no bounds checks, no read of C; the bias values are fetched and
@@ -638,7 +652,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
                 if constexpr (BIAS) {
 #pragma unroll
                     for (int j = 0; j < TN; j++) {
-                        const u32x2 bv = *(const u32x2 *)(p.bias + bn0 + wn0 + j * 16 + lq * 4);
+                        const u32x2 bv = *(const u32x2 *)(p.bias + bn0 + wn0 + (PERM ? (j / 2) * 32 + lq * 8 + (j % 2) * 4 : j * 16 + lq * 4));
                         cb[j][0] = Mma<T>::to_f32((uint16_t)(bv[0] & 0xffffu));
                         cb[j][1] = Mma<T>::to_f32((uint16_t)(bv[0] >> 16));
                         cb[j][2] = Mma<T>::to_f32((uint16_t)(bv[1] & 0xffffu));
@@ -664,9 +678,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
                             }
 #pragma unroll
                         for (int h = 0; h < 2; h++) {
-                            const auto r = __builtin_amdgcn_permlane16_swap(pk[0][h], pk[1][h], false, false);
-                            o[jp][h] = r[0];      // columns 8*(lq/2) + 2h, + 1 of tile 2jp + (lq & 1)
-                            o[jp][2 + h] = r[1];  // columns 8*(lq/2) + 4 + 2h, + 1
+                            if constexpr (PERM) {  // the lane's own 8 consecutive columns, 32 jp + 8 lq + 0..7
+                                o[jp][h] = pk[0][h];
+                                o[jp][2 + h] = pk[1][h];
+                            } else {
+                                const auto r = __builtin_amdgcn_permlane16_swap(pk[0][h], pk[1][h], false, false);
+                                o[jp][h] = r[0];      // columns 8*(lq/2) + 2h, + 1 of tile 2jp + (lq & 1)
+                                o[jp][2 + h] = r[1];  // columns 8*(lq/2) + 4 + 2h, + 1
+                            }
                         }
                     }
                     if constexpr (TN == 4) {
@@ -708,10 +727,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, dma_waves_per_simd(BM, BN, W
                         for (int jp = 0; jp < TN / 2; jp++)
 #pragma unroll
                             for (int e = 0; e < 4; e++) {
-                                const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i0 + i][2 * jp][e]),
-                                                                                __float_as_uint(acc[i0 + i][2 * jp + 1][e]), false, false);
-                                v[jp][e] = __uint_as_float(r[0]);
-                                v[jp][4 + e] = __uint_as_float(r[1]);
+                                if constexpr (PERM) {
+                                    v[jp][e] = acc[i0 + i][2 * jp][e];
+                                    v[jp][4 + e] = acc[i0 + i][2 * jp + 1][e];
+                                } else {
+                                    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i0 + i][2 * jp][e]),
+                                                                                    __float_as_uint(acc[i0 + i][2 * jp + 1][e]), false, false);
+                                    v[jp][e] = __uint_as_float(r[0]);
+                                    v[jp][4 + e] = __uint_as_float(r[1]);
+                                }
                             }
                         if constexpr (TN == 4) {  // whole lines: v[0] becomes rows 0..7, v[1] rows 8..15 (see line_off)
 #pragma unroll
