@@ -22,7 +22,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
-    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them, shapes = shape classes outside the configurations: few rows or columns, thin contractions, rank-1 updates, mid-size products, plancheck = the planner's pick against every forced tile variant and split count on a fixed list of shapes; exits 1 with --strict when a pick is more than --plancheck-slack off the best)")
+    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them, shapes = shape classes outside the configurations: few rows or columns, thin contractions, rank-1 updates, mid-size products, plancheck = the planner's pick against every forced tile variant and split count on a fixed list of shapes; exits 1 with --strict when a pick is more than --plancheck-slack off the best; fewrows = the same check on 128 products of 2 - 16 rows against matrices of 2 - 270 MB)")
     ap.add_argument("--strict", action="store_true", help="plancheck: exit status 1 when a pick is flagged")
     ap.add_argument("--plancheck-slack", type=float, default=0.10, help="plancheck: flag a pick that is this much slower than the best forced candidate")
     ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "f32-forms", "layouts"],
@@ -480,7 +480,7 @@ def main():
 
     # ---- planner regression check: the automatic pick against every forced candidate ---------------------------------
     flagged = []
-    if "plancheck" in only:
+    if "plancheck" in only or "fewrows" in only:
         from dfdx_amd.rocm import KERNEL_GEMV, KERNEL_MFMA, RocmError
 
         # (dtype, m, k, n, layout of A and B (n = stored as indexed, t = transposed), accumulate, batch)
@@ -499,50 +499,63 @@ def main():
                     ("f16", 16, 4096, 4096, "nt", False, 1), ("f16", 32, 8192, 8192, "nt", False, 1), ("f16", 4, 4096, 4096, "nt", False, 1),
                     ("f32", 2048, 2048, 2048, "nn", False, 1), ("f32", 1024, 8192, 1024, "tn", True, 1), ("f32", 8192, 1024, 1024, "nt", False, 1),
                     ("f32", 512, 512, 512, "nn", False, 1), ("f32", 16, 4096, 4096, "nt", False, 1)]
-        for dt, m, k, n, lay, acc, nb in pc_cases:
-            a = rnd((nb, k, m) if lay[0] == "t" else (nb, m, k), dt)
-            b = rnd((nb, n, k) if lay[1] == "t" else (nb, k, n), dt, k ** -0.5)
-            c = zeros((nb, m, n), dt)
+        # a Linear layer on a handful of rows, both weight layouts: where the multi-vector kernel, the k-sliced small kernel and
+        # the split tiles meet
+        few_cases = [(dt, r, k, n, lay, False, 1) for dt in ("f16", "f32") for lay in ("nt", "nn") for r in (2, 4, 8, 16)
+                     for k, n in ((1024, 1024), (2048, 2048), (4096, 4096), (8192, 8192), (4096, 16384), (16384, 4096), (8192, 1024), (1024, 8192))]
 
-            def pc_desc(kernel=0, variant=0, split=0):
-                return dev.gemm_desc(dt, m, k, n, P(a), (1, m) if lay[0] == "t" else (k, 1), P(b), (1, k) if lay[1] == "t" else (n, 1), P(c), (n, 1),
-                                     accumulate=acc, batch=(nb, 1), a_batch=(m * k, 0), b_batch=(k * n, 0), c_batch=(m * n, 0),
-                                     kernel=kernel, variant=variant, split_k=split, no_split_k=(split == 1))
+        def plancheck_run(cases, label):
+            for dt, m, k, n, lay, acc, nb in cases:
+                a = rnd((nb, k, m) if lay[0] == "t" else (nb, m, k), dt)
+                b = rnd((nb, n, k) if lay[1] == "t" else (nb, k, n), dt, k ** -0.5)
+                c = zeros((nb, m, n), dt)
 
-            def pc_time(desc, iters=20):
-                try:
-                    name = dev.gemm_plan(desc)[2]
-                    return min(dev.gemm_time(desc, 3, iters), dev.gemm_time(desc, 1, iters)), name
-                except RocmError:
-                    return None, None
+                def pc_desc(kernel=0, variant=0, split=0):
+                    return dev.gemm_desc(dt, m, k, n, P(a), (1, m) if lay[0] == "t" else (k, 1), P(b), (1, k) if lay[1] == "t" else (n, 1), P(c), (n, 1),
+                                         accumulate=acc, batch=(nb, 1), a_batch=(m * k, 0), b_batch=(k * n, 0), c_batch=(m * n, 0),
+                                         kernel=kernel, variant=variant, split_k=split, no_split_k=(split == 1))
 
-            auto_ms, auto_name = pc_time(pc_desc())
-            cands = {}
-            for v in range(1, dev.mfma_variant_count(dt) + 1):
-                for split in (1, 2, 4, 8, 16):
-                    if split > 1 and (nb > 1 or k < 64 * 4 * split):
-                        continue
-                    ms, name = pc_time(pc_desc(KERNEL_MFMA, v, split), 10)
-                    if ms and (name not in cands or ms < cands[name]):
-                        cands[name] = ms
-            ms, name = pc_time(pc_desc(KERNEL_GEMV), 10)
-            if ms:
-                cands[name] = ms
-            best_name = min(cands, key=cands.get)
-            auto_ms = min(auto_ms, pc_time(pc_desc())[0])   # once more after the sweep: clocks drift over a run
-            # the same plan under both names is the same launch: what separates the two timings is noise
-            slack = 0.0 if best_name == auto_name else auto_ms / cands[best_name] - 1.0
-            flag = slack > args.plancheck_slack
-            tag = f"{dt} {'b' + str(nb) + ' ' if nb > 1 else ''}{m}x{k}x{n} {lay}{' acc' if acc else ''}"
-            rows.append({"group": "plancheck", "case": tag, "kernel": auto_name, "us": round(auto_ms * 1e3, 2), "best": best_name,
-                         "best_us": round(cands[best_name] * 1e3, 2), "candidates": len(cands), "off_best_pct": round(100 * slack, 1), "flagged": flag})
-            print(f"plan  {tag:34s} auto {auto_ms * 1e3:8.1f} us {auto_name:40s} best of {len(cands):3d} {cands[best_name] * 1e3:8.1f} us {best_name:40s} "
-                  f"{100 * slack:+6.1f} %{'  <<<< FLAG' if flag else ''}", flush=True)
-            if flag:
-                flagged.append(tag)
-            del a, b, c
-        print(f"plancheck: {len(pc_cases)} shapes, {len(flagged)} flagged (pick more than {100 * args.plancheck_slack:.0f} % off the best forced candidate)"
-              + (": " + "; ".join(flagged) if flagged else ""), flush=True)
+                def pc_time(desc, iters=20):
+                    try:
+                        name = dev.gemm_plan(desc)[2]
+                        return min(dev.gemm_time(desc, 3, iters), dev.gemm_time(desc, 1, iters)), name
+                    except RocmError:
+                        return None, None
+
+                auto_ms, auto_name = pc_time(pc_desc())
+                cands = {}
+                for v in range(1, dev.mfma_variant_count(dt) + 1):
+                    for split in (1, 2, 4, 8, 16):
+                        if split > 1 and (nb > 1 or k < 64 * 4 * split):
+                            continue
+                        ms, name = pc_time(pc_desc(KERNEL_MFMA, v, split), 10)
+                        if ms and (name not in cands or ms < cands[name]):
+                            cands[name] = ms
+                ms, name = pc_time(pc_desc(KERNEL_GEMV), 10)
+                if ms:
+                    cands[name] = ms
+                best_name = min(cands, key=cands.get)
+                auto_ms = min(auto_ms, pc_time(pc_desc())[0])   # once more after the sweep: clocks drift over a run
+                # the same plan under both names is the same launch: what separates the two timings is noise
+                slack = 0.0 if best_name == auto_name else auto_ms / cands[best_name] - 1.0
+                flag = slack > args.plancheck_slack
+                tag = f"{dt} {'b' + str(nb) + ' ' if nb > 1 else ''}{m}x{k}x{n} {lay}{' acc' if acc else ''}"
+                rows.append({"group": label, "case": tag, "kernel": auto_name, "us": round(auto_ms * 1e3, 2), "best": best_name,
+                             "best_us": round(cands[best_name] * 1e3, 2), "candidates": len(cands), "off_best_pct": round(100 * slack, 1), "flagged": flag})
+                print(f"{label[:5]:5s} {tag:34s} auto {auto_ms * 1e3:8.1f} us {auto_name:40s} best of {len(cands):3d} {cands[best_name] * 1e3:8.1f} us {best_name:40s} "
+                      f"{100 * slack:+6.1f} %{'  <<<< FLAG' if flag else ''}", flush=True)
+                if flag:
+                    flagged.append(tag)
+                del a, b, c
+            mine = [r for r in rows if r["group"] == label]
+            bad = [r["case"] for r in mine if r["flagged"]]
+            print(f"{label}: {len(cases)} shapes, {len(bad)} flagged (pick more than {100 * args.plancheck_slack:.0f} % off the best forced candidate)"
+                  + (": " + "; ".join(bad) if bad else ""), flush=True)
+
+        if "plancheck" in only:
+            plancheck_run(pc_cases, "plancheck")
+        if "fewrows" in only:
+            plancheck_run(few_cases, "fewrows")
 
     # ---- operands off the 16-byte grid: an LM head with 50257 outputs, a first-layer convolution -------------------
     if "edge" in only:   # on request: the scalar kernel's rows take milliseconds each

@@ -2,6 +2,7 @@
 #include "ctx_internal.h"
 #include "gemm_internal.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 
@@ -351,10 +352,18 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
     default:
         return DFDX_ROCM_ERR_INVALID_ARG;
     }
-    if (const int bw = bandwidth_kernel(p, (d->flags & DFDX_ROCM_GEMM_NO_SPLIT_K) != 0)) {
+    // The bandwidth-bound kernels first.  The multi-vector form is weighed against the matrix-core plans by estimated
+    // time (the k-sliced small kernel streams a [n][k] matrix faster for most sizes, the tiles a large [k][n] one); the
+    // others have no rival.
+    const int bw = bandwidth_kernel(p, (d->flags & DFDX_ROCM_GEMM_NO_SPLIT_K) != 0);
+    double t_bw = 1e300;
+    if (bw == BW_GEMV_MULTI) {
+        t_bw = gemv_multi_time(p);
+    } else if (bw) {
         *plan = {DFDX_ROCM_KERNEL_GEMV, bw, 1};
         return DFDX_ROCM_OK;
     }
+    const Plan bw_plan = {DFDX_ROCM_KERNEL_GEMV, BW_GEMV_MULTI, 1};
     // The small-product kernel where its estimate beats the family's (the f32 family weighs it among its own variants);
     // not where the caller fixed the order of the contraction.
     const bool may_small = forced_splits == 0 && (is16 || is64) && small_supported(p);
@@ -369,17 +378,33 @@ int make_plan(dfdx_rocm_ctx *ctx, const dfdx_rocm_gemm_desc *d, const GemmProble
             // 1 - 2 us above the clock, and 8 us above it for a split plan
             t_dma -= splits > 1 ? 6.5e-6 : 1.0e-6;
             *plan = t_small < t_dma ? small_plan : Plan{DFDX_ROCM_KERNEL_MFMA, dv + mfma16_dma_first_variant() - 1, splits};
+            double t_best = std::min(t_small, t_dma);
+            int skinny_splits = 1;
+            double t_skinny = 1e300;
+            if (const int sv = mfma16_skinny_plan(p, ctx->compute_units, forced_splits, &skinny_splits, &t_skinny)) {
+                if (t_skinny < t_best) {
+                    *plan = {DFDX_ROCM_KERNEL_MFMA, sv, skinny_splits};
+                    t_best = t_skinny;
+                }
+            }
+            if (t_bw < t_best) *plan = bw_plan;
             return DFDX_ROCM_OK;
         }
     }
+    double t_family = 1e300;
     int v = is16 ? mfma16_pick_variant(p, ctx->compute_units)
-                 : is32 ? mfma32_pick_variant(p, ctx->compute_units, forced_splits) : is64 ? mfma64_pick_variant(p, ctx->compute_units) : 0;
+                 : is32 ? mfma32_pick_variant(p, ctx->compute_units, forced_splits, &t_family) : is64 ? mfma64_pick_variant(p, ctx->compute_units) : 0;
     if (v > 0) {
         *plan = {DFDX_ROCM_KERNEL_MFMA, v,
                  is32 ? mfma32_plan_splits(p, v, ctx->compute_units, forced_splits)
                       : is16 ? mfma16_plan_splits(p, v, ctx->compute_units, forced_splits) : 1};
-        if (may_small && t_small < (is16 ? mfma16_staged_time(p, v, plan->splits, ctx->compute_units) : mfma64_time(p, v, ctx->compute_units)))
-            *plan = small_plan;
+        if (!is32) t_family = is16 ? mfma16_staged_time(p, v, plan->splits, ctx->compute_units) : mfma64_time(p, v, ctx->compute_units);
+        if (may_small && t_small < t_family) *plan = small_plan;
+        if (t_bw < std::min(t_small, t_family)) *plan = bw_plan;
+        return DFDX_ROCM_OK;
+    }
+    if (bw) {  // no tiled kernel takes these strides, the multi-vector kernel does
+        *plan = t_small < t_bw ? small_plan : bw_plan;
         return DFDX_ROCM_OK;
     }
     // no tiled kernel takes these strides: the small-product kernel takes any, up to the size where 16 x 16 tiles pay

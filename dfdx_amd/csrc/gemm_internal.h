@@ -93,6 +93,8 @@ int mfma16_small_variant();      // ... except the last one, the small-product k
 int mfma16_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits);
 size_t mfma16_workspace_bytes(const GemmProblem &p, int variant, int splits);
 double mfma16_staged_time(const GemmProblem &p, int variant, int splits, int compute_units);  // estimated seconds
+// a few rows or columns against a large matrix: the 64 x 64 register-staged tile with split-k (0 = does not apply)
+int mfma16_skinny_plan(const GemmProblem &p, int compute_units, int forced_splits, int *splits, double *seconds);
 hipError_t launch_mfma16(const GemmProblem &p, int variant, hipStream_t stream);
 // The same product with B given as a patch matrix (`p.b` = channel 0 of the first image, b_b1 / b_b2 = image and group
 // strides, b_rs / b_cs unused): register-staged kernels only, tile chosen inside.  Returns hipErrorNotSupported when
@@ -122,7 +124,7 @@ hipError_t launch_splitk_reduce(const GemmProblem &p, int64_t ws_ld, int64_t ws_
 int mfma32_variant_count();
 const char *mfma32_variant_name(int variant);
 bool mfma32_supported(const GemmProblem &p, int variant);
-int mfma32_pick_variant(const GemmProblem &p, int compute_units, int forced_splits);
+int mfma32_pick_variant(const GemmProblem &p, int compute_units, int forced_splits, double *seconds = nullptr);  // + its estimate
 int mfma32_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits);
 size_t mfma32_workspace_bytes(const GemmProblem &p, int variant, int splits);
 hipError_t launch_mfma32(const GemmProblem &p, int variant, hipStream_t stream);
@@ -152,6 +154,7 @@ hipError_t launch_gemv(const GemmProblem &p, hipStream_t stream);
 // ---- two to eight vectors against one streamed matrix (gemv_multi.hip): M or N of 2 .. 8, the other operand a megabyte at least ----
 bool gemv_multi_supported(const GemmProblem &p);
 size_t gemv_multi_workspace_bytes(const GemmProblem &p);
+double gemv_multi_time(const GemmProblem &p);  // estimated seconds
 hipError_t launch_gemv_multi(const GemmProblem &p, hipStream_t stream);
 
 // ---- thin contractions with large outputs on the matrix cores (gemm_small.hip): k <= 32, f32 / f16 / bf16, row-major C ----

@@ -670,6 +670,37 @@ double mfma16_staged_time(const GemmProblem &p, int variant, int splits, int com
     return 2.5e-6 + std::max(1.0, blocks / cus) * (double)((total_iters + splits - 1) / splits) * step + (splits > 1 ? 4e-6 : 0.0);
 }
 
+// A few rows (or columns) against a large matrix, streamed by the 64 x 64 tile with the contraction split: the tile wastes
+// the least of its rows on such a product and its small LDS footprint puts several workgroups on a compute unit, which
+// is what streaming at the rate of HBM takes (16 x 8192 x 8192 A.B^T: 26.7 us where the 128-row LDS-DMA tiles take 30.6
+// and the k-sliced small kernel 33.5; 8 x 4096 x 4096 A.B: 13.7 us against 15.8).  Returns the variant and its split
+// count with an estimate in seconds, or 0 where the candidate does not apply.
+int mfma16_skinny_plan(const GemmProblem &p, int compute_units, int forced_splits, int *splits, double *seconds) {
+    constexpr int V = 6;  // 64x64x64_w2x2
+    static_assert(kNumVariants >= V, "variant table");
+    *splits = 1;
+    *seconds = 1e300;
+    if (std::min(p.m, p.n) > 64 || forced_splits == 1 || !mfma16_supported(p, V)) return 0;
+    const Variant &t = kVariants[V - 1];
+    const int64_t nbatch = p.reduce ? 1 : p.nb1 * p.nb2;
+    const int64_t total_iters = ((p.k + t.bk - 1) / t.bk) * (p.reduce ? p.nb1 * p.nb2 : 1);
+    if (nbatch != 1 || p.c_cs != 1 || total_iters < 8) return 0;
+    const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn);
+    int64_t s = forced_splits > 0 ? forced_splits : std::min<int64_t>({16, std::max<int64_t>(1, 2 * (int64_t)compute_units / blocks), total_iters / 4});
+    s = std::min<int64_t>(s, total_iters);
+    while (s > 1 && (s - 1) * ((total_iters + s - 1) / s) >= total_iters) s--;  // no empty piece
+    if (s < 2) return 0;
+    const double bytes = ((double)p.m * (double)p.k + (double)p.k * (double)p.n) * 2.0;
+    if (bytes < 8e6) return 0;  // below that the k-sliced small kernel or an unsplit tile is the plan
+    *splits = (int)s;
+    // two launches, then the operands and the f32 partial tiles (written and read back) at the rate of HBM; an operand that
+    // is not stored along k passes through the register transposes of this family
+    const bool along_k = p.a_cs == 1 && p.b_rs == 1;
+    const double partials = (double)s * (double)blocks * t.bm * t.bn * 4.0 * 2.0;
+    *seconds = 6.0e-6 + (bytes * (along_k ? 1.0 : 1.08) + partials) / 6.3e12;
+    return V;
+}
+
 static void ws_layout16(const GemmProblem &p, int variant, int64_t *ld, int64_t *split_stride) {
     const Variant &v = kVariants[variant - 1];
     *ld = ((p.n + v.bn - 1) / v.bn) * v.bn;

@@ -745,13 +745,15 @@ size_t mfma32_workspace_bytes(const GemmProblem &p, int variant, int splits) {
     return (size_t)stride * splits * sizeof(float);
 }
 
-int mfma32_pick_variant(const GemmProblem &p, int compute_units, int forced_splits) {
+int mfma32_pick_variant(const GemmProblem &p, int compute_units, int forced_splits, double *seconds) {
     int best = 0;
     double best_time = 1e300;
     for (int v = 1; v <= kNumVariants; v++) {
         if (!mfma32_supported(p, v)) continue;
         // the small kernel adds its k slices in an order of its own: not where the caller asked for the plain k order
-        if (kVariants[v - 1].small && (forced_splits == 1 || (double)p.m * (double)p.n * (double)p.k > 536870912.0)) continue;
+        // (nor for large products, except those of a few rows or columns: one row of 16 x 16 tiles streams the large
+        // operand once, 16 x 8192 x 8192: 67 us against 103 us on the split 64 x 64 tiles)
+        if (kVariants[v - 1].small && (forced_splits == 1 || ((double)p.m * (double)p.n * (double)p.k > 536870912.0 && std::min(p.m, p.n) > 16))) continue;
         double tm;
         plan_pieces32(p, v, compute_units, forced_splits, &tm);
         if (tm < best_time) {
@@ -759,6 +761,7 @@ int mfma32_pick_variant(const GemmProblem &p, int compute_units, int forced_spli
             best = v;
         }
     }
+    if (seconds) *seconds = best_time;
     return best;
 }
 

@@ -319,14 +319,24 @@ double small_time(const GemmProblem &p, int compute_units) {
     const double per_k = p.dtype == DT_F64 ? 6.8e-9 : half ? 1.7e-9 : 3.4e-9;
     const double chain = std::max(0.5e-6, (double)p.k * per_k);
     // an operand that is not stored along k comes one 2- or 4-byte load per value: a fixed cost in the chain, and, where
-    // the operand is large, a rate (16 x 4096 x 4096: f16 9.8 us A.B^T against 22.9 us A.B, f32 18.9 against 24.1)
+    // the operand is large, a rate (16 x 4096 x 4096: f16 9.8 us A.B^T against 22.9 us A.B, f32 18.9 against 24.1).  With
+    // one row of tiles and only the large operand strided, the gathers of all tiles run beside the chain instead of in
+    // it (4 x 2048 x 2048 f16 A.B 6.6 us, 4 x 1024 x 8192 f32 A.B 13.9 us): the longer of the two counts.
     const double strided_values = (p.a_cs != 1 ? (double)p.m * (double)p.k : 0.0) + (p.b_rs != 1 ? (double)p.k * (double)p.n : 0.0);
-    const double gather = p.dtype == DT_F64 ? 0.0 : (half ? 0.9e-6 : 0.4e-6) * strided + strided_values / (half ? 1.3e12 : 3.3e12);
-    const double bandwidth = (p.dtype == DT_F64 ? 8e12 : 7.5e12) * std::max(1, compute_units) / 256.0;
+    const bool one_row = std::min(p.m, p.n) <= 16 && strided == 1;
+    const double gather = p.dtype == DT_F64 ? 0.0
+                          : (half ? 0.9e-6 : 0.4e-6) * strided + (one_row ? 0.0 : strided_values / (half ? 1.3e12 : 3.3e12));
+    const double gather_stream = p.dtype == DT_F64 || !one_row ? 0.0 : strided_values / (half ? 0.87e12 : 0.8e12);
+    // one row (or column) of tiles: the 16 rows of the small operand are the same for every tile and stay in the caches,
+    // what streams is the large operand, once -- at the rate of HBM when it is larger than the caches hold
+    const double rows_per_tile = std::min(p.m, p.n) <= 16 ? 16.0 : 32.0;
+    const double streamed = tiles * rows_per_tile * es * (double)p.k;
+    const double unique = ((double)p.m + (double)p.n) * (double)p.k * es;
+    const double bandwidth = (unique > 64e6 ? 4.5e12 : p.dtype == DT_F64 ? 8e12 : 7.5e12) * std::max(1, compute_units) / 256.0;
     // C leaves in pieces of 16 elements of a row: 1.5 - 2.5 TB/s (a rank-1 update of 4096^2 through this kernel: 22 - 34 us)
     const double c_bytes = (double)p.m * (double)p.n * es * (p.accumulate ? 2.0 : 1.0);
     const double c_rate = (p.dtype == DT_F16 || p.dtype == DT_BF16 ? 1.5e12 : 2.2e12) * std::max(1, compute_units) / 256.0;
-    return 2.1e-6 + gather + std::max(chain, tiles * 32.0 * es * (double)p.k / bandwidth) + c_bytes / c_rate;
+    return 2.1e-6 + gather + std::max(std::max(chain, streamed / bandwidth), gather_stream) + c_bytes / c_rate;
 }
 
 hipError_t launch_small(const GemmProblem &g, hipStream_t stream) {

@@ -430,6 +430,26 @@ bool gemv_multi_supported(const GemmProblem &g) {
     return s.p.kslices <= 65535;  // the k slices are grid.y
 }
 
+// Estimated seconds, for the planner's comparison with the matrix-core kernels (forced sweeps over 2 - 16 vectors against
+// matrices of 2 MB - 270 MB, both layouts, f16 and f32): the launch (two with the combining pass) plus the matrix at the
+// rate the form streams it.  The 16-bit forms are bound by their multiply-adds, not by memory, once there are more than a
+// few vectors (the rate falls with every vector: 4 x 4096 x 4096 f16 A.B 12.9 us, 8 vectors 17.6 us), f32 hardly.
+double gemv_multi_time(const GemmProblem &g) {
+    Shape s = classify(g);
+    if (!s.ok) return 1e300;
+    plan_slices(s, g.dtype);
+    const bool half = g.dtype != DT_F32;
+    const double bytes = (double)s.p.j * (double)g.k * (double)dtype_size(g.dtype);
+    const double more = (double)s.p.r - 2.0;
+    double rate = s.cols ? (half ? 8.0e12 / (1.0 + 0.19 * more) : 6.3e12 / (1.0 + 0.045 * more))
+                         : (half ? 7.5e12 / (1.0 + 0.13 * more) : 6.0e12 / (1.0 + 0.05 * more));
+    if (half && bytes > 48e6) rate = std::min(rate, s.cols ? 4.8e12 : 5.4e12);  // beyond what the caches hold between launches
+    // two launches (slices + combine) and, in the "cols" form, the vector slices staged through LDS: a matrix of 2 MB takes
+    // 5.7 - 6.5 us as dots and 7.4 - 10.7 us as columns (f16, 2 - 8 vectors), f32 5.6 - 8.1 us
+    const double fixed = !s.cols ? 5.2e-6 + 0.12e-6 * more : half ? 6.5e-6 + 0.45e-6 * more : 5.0e-6 + 0.3e-6 * more;
+    return (s.p.kslices > 1 ? fixed : fixed - 2.0e-6) + bytes / rate;
+}
+
 size_t gemv_multi_workspace_bytes(const GemmProblem &g) {
     Shape s = classify(g);
     if (!s.ok) return 0;

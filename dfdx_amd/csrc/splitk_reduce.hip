@@ -69,8 +69,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, int
     const int row = ((int)blockIdx.x - (ks.ws ? ks.blocks : 0)) * 4 + threadIdx.x / 64;
     if (row >= m || col >= n) return;
     const float *src = ws + (int64_t)row * ws_ld + col;
-    f32x4 v = *(const f32x4 *)src;
-    for (int s = 1; s < splits; s++) v += *(const f32x4 *)(src + s * ws_split_stride);
+    // eight partial sums requested at a time (a tail repeats the last one, unused), added in ascending order: one round
+    // trip to memory per eight splits instead of one per split
+    f32x4 v;
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+        f32x4 part[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) part[u] = *(const f32x4 *)(src + (int64_t)min(s0 + u, splits - 1) * ws_split_stride);
+        if (s0 == 0) v = part[0];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (s0 + u < splits && s0 + u > 0) v += part[u];
+    }
     T *dst = c + (int64_t)row * c_rs + col;
     const float rb = (bias_mode == BIAS_PER_ROW) ? Cvt<T>::load(bias + row) : 0.0f;
     if constexpr (sizeof(T) == 4) {
@@ -122,24 +132,28 @@ __global__ __launch_bounds__(256) void splitk_reduce16_kernel(const float *ws, i
     u32x4 old = {0u, 0u, 0u, 0u}, cb = {0u, 0u, 0u, 0u};
     if (accumulate) old = *(const u32x4 *)dst;
     if (bias_mode == BIAS_PER_COL) cb = *(const u32x4 *)(bias + col);
-    f32x4 lo = *(const f32x4 *)src, hi = *(const f32x4 *)(src + 4);
-    int s = 1;
-    for (; s + 3 < splits; s += 4) {
-        f32x4 a[4], b[4];
+    // eight splits requested at a time (a tail repeats the last one, unused) and added in ascending order: with the old
+    // C values and the bias that is ONE round trip to memory for up to eight splits (a loop that waited for split after
+    // split paid five for eight splits: 9.2 us for the 1024 x 1024 weight gradients)
+    f32x4 lo, hi;
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+        f32x4 a[8], b[8];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            a[u] = *(const f32x4 *)(src + (s + u) * ws_split_stride);
-            b[u] = *(const f32x4 *)(src + (s + u) * ws_split_stride + 4);
+        for (int u = 0; u < 8; u++) {
+            const float *q = src + (int64_t)min(s0 + u, splits - 1) * ws_split_stride;
+            a[u] = *(const f32x4 *)q;
+            b[u] = *(const f32x4 *)(q + 4);
+        }
+        if (s0 == 0) {
+            lo = a[0];
+            hi = b[0];
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            lo += a[u];
-            hi += b[u];
-        }
-    }
-    for (; s < splits; s++) {
-        lo += *(const f32x4 *)(src + s * ws_split_stride);
-        hi += *(const f32x4 *)(src + s * ws_split_stride + 4);
+        for (int u = 0; u < 8; u++)
+            if (s0 + u < splits && s0 + u > 0) {
+                lo += a[u];
+                hi += b[u];
+            }
     }
     const float rb = (bias_mode == BIAS_PER_ROW) ? Bits16<T>::widen(bias[row]) : 0.0f;
     u32x4 out;

@@ -370,14 +370,21 @@ def test_gemv_multi(dtype, shape, layout):
     at, bt = LAYOUTS[layout]
     astr = (1, m) if at else (k, 1)
     bstr = (1, k) if bt else (n, 1)
-    plan = dev.gemm_plan(dev.gemm_desc(dtype, m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1)))
     # the matrix must be walkable in 16-byte pieces along its outputs ("cols") or along k ("dots": then the vectors must be
-    # contiguous in k as well); of the three layouts only A.B with the few columns in B is neither
-    if not (n <= 8 and layout == "nn"):
+    # contiguous in k as well); of the three layouts only A.B with the few columns in B is neither.  The planner weighs
+    # this kernel against the matrix-core plans by estimated time, so the kernel is FORCED here (its family on request
+    # takes the product whenever the kernel supports it) and the automatic plan, whichever it is, runs beside it.
+    if n <= 8 and layout == "nn":
+        forced = KERNEL_AUTO
+    else:
+        forced = KERNEL_GEMV
+        plan = dev.gemm_plan(dev.gemm_desc(dtype, m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1), kernel=KERNEL_GEMV))
         assert plan[0] == KERNEL_GEMV and plan[2] == "gemv_multi", (shape, layout, plan)
-    run_case(dtype, m, k, n, layout, False, KERNEL_AUTO, 0, seed=5, bias=True)
-    run_case(dtype, m, k, n, layout, True, KERNEL_AUTO, 0, seed=6, c_colmajor=True, bias=(dtype == "f32"))
-    run_case(dtype, m, k, n, layout, True, KERNEL_AUTO, 0, seed=7, pads=(8, 8, 3))
+    run_case(dtype, m, k, n, layout, False, forced, 0, seed=5, bias=True)
+    run_case(dtype, m, k, n, layout, True, forced, 0, seed=6, c_colmajor=True, bias=(dtype == "f32"))
+    run_case(dtype, m, k, n, layout, True, forced, 0, seed=7, pads=(8, 8, 3))
+    if forced != KERNEL_AUTO:
+        run_case(dtype, m, k, n, layout, True, KERNEL_AUTO, 0, seed=8, bias=True)
 
 
 @pytest.mark.parametrize("shape,layout", [((10, 8192, 1024), "tn"), ((1024, 8200, 10), "tn"), ((16, 8192, 520), "nn"), ((9, 16384, 264), "tn"),
@@ -392,18 +399,24 @@ def test_gemv_multi_nine_to_sixteen_vectors_f32(shape, layout):
     a = dev.zeros("f32", (max(m, n) * k,))
     at, bt = LAYOUTS[layout]
     astr, bstr = (1, m) if at else (k, 1), (1, k) if bt else (n, 1)
-    plan = dev.gemm_plan(dev.gemm_desc("f32", m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1)))
+    forced = lambda dt, kk: dev.gemm_plan(dev.gemm_desc(dt, m, kk, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1), kernel=KERNEL_GEMV))
+    plan = forced("f32", k)
     assert plan[0] == KERNEL_GEMV and plan[2] == "gemv_multi", (shape, layout, plan)
-    assert dev.gemm_plan(dev.gemm_desc("f16", m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1)))[2] == ("gemv_multi" if k >= 16384 else
-                                                                                                  dev.gemm_plan(dev.gemm_desc("f16", m, k, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1), kernel=KERNEL_MFMA))[2])
     if k >= 16384:   # the 16-bit types take the form from 16384 terms on
+        assert forced("f16", k)[2] == "gemv_multi"
         for dt in ("f16", "bf16"):
-            run_case(dt, m, k, n, layout, True, KERNEL_AUTO, 0, seed=18, bias=True, pads=(8, 8, 3))
-            run_case(dt, m, k, n, layout, False, KERNEL_AUTO, 0, seed=19, c_colmajor=True)
-    assert dev.gemm_plan(dev.gemm_desc("f32", m, 4096, n, a.ptr, astr, a.ptr, bstr, a.ptr, (n, 1)))[2] != "gemv_multi"
-    run_case("f32", m, k, n, layout, False, KERNEL_AUTO, 0, seed=15, bias=True)
-    run_case("f32", m, k, n, layout, True, KERNEL_AUTO, 0, seed=16, c_colmajor=True, bias=True)
-    run_case("f32", m, k, n, layout, True, KERNEL_AUTO, 0, seed=17, pads=(8, 8, 3))
+            run_case(dt, m, k, n, layout, True, KERNEL_GEMV, 0, seed=18, bias=True, pads=(8, 8, 3))
+            run_case(dt, m, k, n, layout, False, KERNEL_GEMV, 0, seed=19, c_colmajor=True)
+            run_case(dt, m, k, n, layout, False, KERNEL_AUTO, 0, seed=20)
+    else:
+        with pytest.raises(RocmError):   # shorter contractions with more than eight vectors: not this kernel's
+            forced("f16", k)
+    with pytest.raises(RocmError):
+        forced("f32", 4096)
+    run_case("f32", m, k, n, layout, False, KERNEL_GEMV, 0, seed=15, bias=True)
+    run_case("f32", m, k, n, layout, True, KERNEL_GEMV, 0, seed=16, c_colmajor=True, bias=True)
+    run_case("f32", m, k, n, layout, True, KERNEL_GEMV, 0, seed=17, pads=(8, 8, 3))
+    run_case("f32", m, k, n, layout, True, KERNEL_AUTO, 0, seed=21, bias=True)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16", "f64"])
