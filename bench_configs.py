@@ -191,8 +191,10 @@ def main():
 
     def gemm(group, name, desc, flop, nbytes, iters=None, bufs=None):
         """`bufs`: the tensors the descriptor points into; given, the case is also timed over rotating copies of them."""
-        iters = iters or args.iters
-        ms = dev.gemm_time(desc, 5, iters)
+        iters = iters or max(args.iters, 100)
+        # 20 warm-up launches: a case of a few launches inherits the clock the case before it left behind (the same 60 us
+        # product measured 60 or 68 us depending on what ran before it with 5 + 30 launches)
+        ms = dev.gemm_time(desc, 20, iters)
         rot_ms, n = None, 0
         if bufs and not args.no_rotate:
             n = nsets(bufs)
