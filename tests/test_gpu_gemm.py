@@ -37,8 +37,9 @@ def run_case(dtype, m, k, n, layout, accumulate, kernel, variant, c_colmajor=Fal
     dbias = dev.tensor(bias_st, dtype) if bias else None
     desc = dev.gemm_desc(dtype, m, k, n, da.ptr, astr, db.ptr, bstr, dc.ptr, cstr, accumulate=accumulate,
                          bias=dbias.ptr if bias else None, kernel=kernel, variant=variant, split_k=split_k)
+    plan_name = dev.gemm_plan(desc)[2]
     announce("gemm", dtype, (m, k, n), layout, "acc" if accumulate else "ovw", "kernel", kernel, "variant", variant,
-             "ccol" if c_colmajor else "crow", "bias" if bias else "", dev.gemm_plan(desc)[2])
+             "ccol" if c_colmajor else "crow", "bias" if bias else "", plan_name)
     dev.gemm(desc)
     dev.synchronize()
     got_st = dev.to_host(dc)
@@ -57,6 +58,7 @@ def run_case(dtype, m, k, n, layout, accumulate, kernel, variant, c_colmajor=Fal
     idx = values(np.arange(c.size, dtype=np.float64), "f64", (m, n), cstr).astype(np.int64)
     mask[idx.reshape(-1)] = False
     assert np.array_equal(oracle.to_f64(got_st, dtype)[mask], oracle.to_f64(c, dtype)[mask])
+    return plan_name
 
 
 # ------------------------------------------------------------------ generic --
@@ -623,6 +625,35 @@ def test_auto_dispatch_seeded_shape_sweep(dtype):
         pads = tuple(int(g.integers(0, 3)) * 8 for _ in range(3)) if kind != 3 else tuple(int(g.integers(0, 5)) for _ in range(3))
         accumulate, ccol, bias = bool(g.integers(0, 2)), bool(g.integers(0, 4) == 0), bool(g.integers(0, 3) == 0)
         run_case(dtype, m, k, n, layout, accumulate, KERNEL_AUTO, 0, c_colmajor=ccol, bias=bias, seed=500 + i, pads=pads)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+def test_auto_dispatch_few_rows_or_columns_sweep(dtype):
+    """The corner of the planner where five kernel families compete: products of 1 ... 64 rows (or columns) against a
+    matrix of 0.5 ... 32 MB -- a Linear layer on a handful of tokens and its gradients.  24 seeded shapes per dtype
+    through KERNEL_AUTO (vector-product kernels, the k-sliced small kernel, LDS-DMA tiles with and without split-k, the
+    split 64 x 64 tile), every operand layout, aligned and unaligned extents, with and without accumulation and bias;
+    the kernels taken are counted so that a sweep that only ever reached one family fails."""
+    g = rng(31000 + ["f16", "bf16", "f32"].index(dtype))
+    few_choices = [1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 24, 32, 48, 64]
+    taken = {}
+    for i in range(24):
+        few = few_choices[int(g.integers(0, len(few_choices)))]
+        aligned = i % 3 != 2
+        gran = 8 if aligned else 1
+        wide = int(g.integers(64, 1025)) * gran if aligned else int(g.integers(500, 4100))
+        k = int(g.integers(4, 257)) * 64 if aligned else int(g.integers(300, 9000))
+        while wide * k > (1 << 24):
+            k //= 2
+        m, n = (few, wide) if g.integers(0, 2) else (wide, few)
+        layout = list(LAYOUTS)[int(g.integers(0, 4))]
+        pads = tuple(int(g.integers(0, 2)) * 8 for _ in range(3)) if aligned else tuple(int(g.integers(0, 3)) for _ in range(3))
+        accumulate, bias = bool(g.integers(0, 2)), bool(g.integers(0, 4) == 0)
+        name = run_case(dtype, m, k, n, layout, accumulate, KERNEL_AUTO, 0, bias=bias, seed=900 + i, pads=pads)
+        family = name.split("_")[0] + ("_small" if "small" in name else "_dma" if "dma" in name else "")
+        taken[family] = taken.get(family, 0) + 1
+    announce("few rows / columns sweep", dtype, taken)
+    assert len(taken) >= 3, f"the sweep reached only {taken}"
 
 
 def test_thin_contraction_with_more_than_2_31_output_elements():
