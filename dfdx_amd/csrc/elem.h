@@ -82,6 +82,25 @@ template <typename T, int N> __device__ __forceinline__ void load_elems(const T 
         for (int i = 0; i < N; i++) v[i] = Elem<T>::load(p + i);
     }
 }
+// The same with the non-temporal form of the 16-byte load (STREAM): for an input that one launch reads once and that is
+// large enough (the callers' rule: 128 MiB or more of read-only input) to push what later ops want out of the caches if it
+// were kept there.  Measured on MI355X in an encoder block (softmax and ReLU gradients of 134 MB tensors): the step as a
+// whole gains 1.2 %, mostly in the GEMMs that run next; small inputs that the previous op has just written lose with it
+// (LayerNorm forward on 16 MB 8.0 -> 10.4 us), hence the size rule.  A compile-time choice: written as a run-time select
+// of the two loads, the compiler merges them into one plain load.
+template <typename T, int N, bool STREAM> __device__ __forceinline__ void load_elems_as(const T *p, float (&v)[N]) {
+    if constexpr (STREAM && N == Elem<T>::VEC) {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 raw = __builtin_nontemporal_load((const u32x4 *)p);
+        T tmp[N];
+        __builtin_memcpy(tmp, &raw, 16);
+#pragma unroll
+        for (int i = 0; i < N; i++) v[i] = Elem<T>::load(&tmp[i]);
+    } else {
+        load_elems<T, N>(p, v);
+    }
+}
+constexpr size_t kStreamInputBytes = (size_t)128 << 20;  // read-only input of one launch from which its loads are non-temporal
 // The same from an address that is only element-aligned (one unaligned 16-byte load; global memory allows it).
 template <typename T, int N> __device__ __forceinline__ void load_elems_unaligned(const T *p, float (&v)[N]) {
     if constexpr (N == Elem<T>::VEC) {

@@ -28,8 +28,13 @@ struct MultiParams {
     int k, j, r;
     int kslices, kchunk;
     int accumulate, has_bias;
+    int stream;  // the matrix is read with non-temporal loads: 256 MiB or more, as in the single-vector kernel (gemv.hip)
     float *ws;
 };
+template <bool STREAM> __device__ __forceinline__ u32x4 ldm(const void *p) {
+    if constexpr (STREAM) return __builtin_nontemporal_load((const u32x4 *)p);
+    else return *(const u32x4 *)p;
+}
 
 // k values of a slice in the cols form: R x kchunk_of(R) values in LDS (32 KiB of f32 at most)
 constexpr int kchunk_of(int r) { return r > 8 ? 512 : 1024; }
@@ -79,7 +84,7 @@ template <typename T> __device__ __forceinline__ void finish(const MultiParams &
 // The cols form.  f32: a wave takes every fourth k and multiplies value by value.  16-bit types: a wave takes every fourth
 // PAIR of k (2 q, 2 q + 1), the vector slices sit in LDS in their own type so that one dword holds a vector's pair, and the
 // two matrix rows of a pair are interleaved column by column into dwords for dot_pair.
-template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_cols_kernel(const MultiParams p) {
+template <typename T, int R, bool STREAM> __global__ __launch_bounds__(256) void gemv_multi_cols_kernel(const MultiParams p) {
     constexpr int VEC = Elem<T>::VEC;
     constexpr bool PAIRS = sizeof(T) == 2;
     typedef typename std::conditional<PAIRS, T, float>::type S;  // what the vector slices are kept as
@@ -117,7 +122,7 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_c
 #pragma unroll
                 for (int u = 0; u < 4; u++) {
                     const int row = kk + 8 * (u / 2) + (u & 1);
-                    raw[u] = *(const u32x4 *)(col + (int64_t)min(row, kn - 1) * p.mat_k_stride);  // (a row past the end meets a zero)
+                    raw[u] = ldm<STREAM>(col + (int64_t)min(row, kn - 1) * p.mat_k_stride);  // (a row past the end meets a zero)
                 }
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
@@ -143,7 +148,7 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_c
             for (; kk + 12 < kn; kk += 16) {  // 4 loads in flight
                 u32x4 raw[4];
 #pragma unroll
-                for (int u = 0; u < 4; u++) raw[u] = *(const u32x4 *)(col + (int64_t)(kk + 4 * u) * p.mat_k_stride);
+                for (int u = 0; u < 4; u++) raw[u] = ldm<STREAM>(col + (int64_t)(kk + 4 * u) * p.mat_k_stride);
 #pragma unroll
                 for (int r = 0; r < R; r++) {
                     const f32x4 v = *(const f32x4 *)&vsh[r][wave * (KCH / 4) + (kk >> 2)];  // k = kk, kk + 4, kk + 8, kk + 12
@@ -154,7 +159,7 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_c
                 }
             }
             for (; kk < kn; kk += 4) {
-                const u32x4 raw = *(const u32x4 *)(col + (int64_t)kk * p.mat_k_stride);
+                const u32x4 raw = ldm<STREAM>(col + (int64_t)kk * p.mat_k_stride);
 #pragma unroll
                 for (int r = 0; r < R; r++) {
                     const float v = vsh[r][wave * (KCH / 4) + (kk >> 2)];
@@ -203,7 +208,7 @@ template <int NV, int N> __device__ __forceinline__ void halve(float (&vals)[NV]
     }
 }
 
-template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_dots_kernel(const MultiParams p) {
+template <typename T, int R, bool STREAM> __global__ __launch_bounds__(256) void gemv_multi_dots_kernel(const MultiParams p) {
     constexpr int VEC = Elem<T>::VEC, J = rows_of(R);
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int j0 = (blockIdx.x * 4 + wave) * J;
@@ -224,7 +229,7 @@ template <typename T, int R> __global__ __launch_bounds__(256) void gemv_multi_d
     for (int kk = lane * VEC; kk < kn; kk += 64 * VEC) {
         u32x4 x[J];
 #pragma unroll
-        for (int jj = 0; jj < J; jj++) x[jj] = *(const u32x4 *)(rows[jj] + kk);
+        for (int jj = 0; jj < J; jj++) x[jj] = ldm<STREAM>(rows[jj] + kk);
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const u32x4 v = *(const u32x4 *)(vecs[r] + kk);
@@ -354,6 +359,7 @@ Shape classify(const GemmProblem &g) {
     p.bias = g.bias;
     p.has_bias = g.bias && g.bias_mode != BIAS_NONE;
     p.accumulate = g.accumulate;
+    p.stream = (double)p.j * (double)g.k * (double)dtype_size(g.dtype) >= 268435456.0;
     const uintptr_t mask = dtype_size(g.dtype) - 1;
     if (((uintptr_t)g.a | (uintptr_t)g.b | (uintptr_t)g.c | (uintptr_t)g.bias) & mask) return s;
     if (!al16(p.mat)) return s;
@@ -401,11 +407,13 @@ template <typename T, int R> hipError_t launch_r(const Shape &s, hipStream_t str
     constexpr int VEC = Elem<T>::VEC;
     if (s.cols) {
         dim3 grid((unsigned)((p.j + 64 * VEC - 1) / (64 * VEC)), (unsigned)p.kslices);
-        gemv_multi_cols_kernel<T, R><<<grid, 256, 0, stream>>>(p);
+        if (p.stream) gemv_multi_cols_kernel<T, R, true><<<grid, 256, 0, stream>>>(p);
+        else gemv_multi_cols_kernel<T, R, false><<<grid, 256, 0, stream>>>(p);
     } else if constexpr (R <= 8) {
         constexpr int PER_WG = 4 * rows_of(R);
         dim3 grid((unsigned)((p.j + PER_WG - 1) / PER_WG), (unsigned)p.kslices);
-        gemv_multi_dots_kernel<T, R><<<grid, 256, 0, stream>>>(p);
+        if (p.stream) gemv_multi_dots_kernel<T, R, true><<<grid, 256, 0, stream>>>(p);
+        else gemv_multi_dots_kernel<T, R, false><<<grid, 256, 0, stream>>>(p);
     } else {
         return hipErrorInvalidValue;
     }

@@ -19,7 +19,7 @@ __device__ __forceinline__ float wave_sum(float v) { return wave64_sum(v); }
 
 // ---- rows held in registers -----------------------------------------------------------------------------------
 // Lane l owns the N-element groups l, l + 64, ... of the row (CH of them; groups past the row end are skipped).
-template <typename T, int N, int CH>
+template <typename T, int N, int CH, bool STREAM>
 __global__ __launch_bounds__(WAVES * 64) void softmax_forward_reg_kernel(const T *x, T *out, int64_t rows, int cols, float scale) {
     const int lane = threadIdx.x % 64;
     for (int64_t row = (int64_t)blockIdx.x * WAVES + threadIdx.x / 64; row < rows; row += (int64_t)gridDim.x * WAVES) {
@@ -30,7 +30,7 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_forward_reg_kernel(const T
         for (int c = 0; c < CH; c++) {
             const int col = (c * 64 + lane) * N;
             if (col < cols) {
-                load_elems<T, N>(src + col, v[c]);
+                load_elems_as<T, N, STREAM>(src + col, v[c]);
 #pragma unroll
                 for (int i = 0; i < N; i++) {
                     v[c][i] *= scale;
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_forward_reg_kernel(const T
 }
 
 // grad_x += scale * p * (g - sum_j g_j p_j); `fresh`: grad_x counts as zero and is not read
-template <typename T, int N, int CH>
+template <typename T, int N, int CH, bool STREAM>
 __global__ __launch_bounds__(WAVES * 64) void softmax_backward_reg_kernel(const T *p, const T *go, T *gx, int64_t rows, int cols,
                                                                           float scale, bool fresh) {
     const int lane = threadIdx.x % 64;
@@ -79,8 +79,8 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_backward_reg_kernel(const 
         for (int c = 0; c < CH; c++) {
             const int col = (c * 64 + lane) * N;
             if (col < cols) {
-                load_elems<T, N>(ps + col, pv[c]);
-                load_elems<T, N>(gs + col, gv[c]);
+                load_elems_as<T, N, STREAM>(ps + col, pv[c]);
+                load_elems_as<T, N, STREAM>(gs + col, gv[c]);
 #pragma unroll
                 for (int i = 0; i < N; i++) dot += pv[c][i] * gv[c][i];
             }
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_backward_reg_kernel(const 
 // owns the N-element groups j, j + 16, ...  Its maximum and its sums then need four DPP steps that ride on the max / add
 // itself (two quad permutations, the half-row and the row mirror) instead of six cross-lane moves through the LDS
 // crossbar, and a wave keeps four rows' loads in flight.
-template <typename T, int N, int CH>
+template <typename T, int N, int CH, bool STREAM>
 __global__ __launch_bounds__(WAVES * 64) void softmax_forward_row16_kernel(const T *x, T *out, int64_t rows, int cols, float scale) {
     const int lane = threadIdx.x % 64, j = lane % 16, sub = lane / 16;
     for (int64_t row0 = ((int64_t)blockIdx.x * WAVES + threadIdx.x / 64) * 4; row0 < rows; row0 += (int64_t)gridDim.x * WAVES * 4) {
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_forward_row16_kernel(const
         for (int c = 0; c < CH; c++) {
             const int col = (c * 16 + j) * N;
             if (col < cols) {
-                load_elems<T, N>(src + col, v[c]);
+                load_elems_as<T, N, STREAM>(src + col, v[c]);
 #pragma unroll
                 for (int i = 0; i < N; i++) {
                     v[c][i] *= scale;
@@ -160,7 +160,7 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_forward_row16_kernel(const
     }
 }
 
-template <typename T, int N, int CH>
+template <typename T, int N, int CH, bool STREAM>
 __global__ __launch_bounds__(WAVES * 64) void softmax_backward_row16_kernel(const T *p, const T *go, T *gx, int64_t rows, int cols,
                                                                             float scale, bool fresh) {
     const int lane = threadIdx.x % 64, j = lane % 16, sub = lane / 16;
@@ -174,8 +174,8 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_backward_row16_kernel(cons
         for (int c = 0; c < CH; c++) {
             const int col = (c * 16 + j) * N;
             if (col < cols) {
-                load_elems<T, N>(ps + col, pv[c]);
-                load_elems<T, N>(gs + col, gv[c]);
+                load_elems_as<T, N, STREAM>(ps + col, pv[c]);
+                load_elems_as<T, N, STREAM>(gs + col, gv[c]);
 #pragma unroll
                 for (int i = 0; i < N; i++) dot += pv[c][i] * gv[c][i];
             }
@@ -283,18 +283,30 @@ int launch_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *a, cons
     const dim3 block(WAVES * 64);
     hipStream_t s = ctx->stream;
     const int n = (int)cols;
+    // read-only input of the launch: x (forward), the probabilities and grad_out (backward)
+    const bool stream = vec && (size_t)rows * (size_t)cols * sizeof(T) * (FWD ? 1 : 2) >= kStreamInputBytes;
+#define DFDX_SOFTMAX_REG_AS(N, CH, STREAM)                                                                             \
+    do {                                                                                                               \
+        if constexpr (FWD) softmax_forward_reg_kernel<T, N, CH, STREAM><<<grid, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale); \
+        else softmax_backward_reg_kernel<T, N, CH, STREAM><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh); \
+        return (int)hipGetLastError();                                                                                 \
+    } while (0)
 #define DFDX_SOFTMAX_REG(N, CH)                                                                                        \
     do {                                                                                                               \
-        if constexpr (FWD) softmax_forward_reg_kernel<T, N, CH><<<grid, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale); \
-        else softmax_backward_reg_kernel<T, N, CH><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh); \
+        if (stream) DFDX_SOFTMAX_REG_AS(N, CH, true);                                                                  \
+        else DFDX_SOFTMAX_REG_AS(N, CH, false);                                                                        \
+    } while (0)
+#define DFDX_SOFTMAX_ROW16_AS(N, CH, STREAM)                                                                           \
+    do {                                                                                                               \
+        const unsigned g16 = (unsigned)std::min<int64_t>((rows + WAVES * 4 - 1) / (WAVES * 4), (int64_t)ctx->compute_units * 16); \
+        if constexpr (FWD) softmax_forward_row16_kernel<T, N, CH, STREAM><<<g16, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale); \
+        else softmax_backward_row16_kernel<T, N, CH, STREAM><<<g16, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh); \
         return (int)hipGetLastError();                                                                                 \
     } while (0)
 #define DFDX_SOFTMAX_ROW16(N, CH)                                                                                      \
     do {                                                                                                               \
-        const unsigned g16 = (unsigned)std::min<int64_t>((rows + WAVES * 4 - 1) / (WAVES * 4), (int64_t)ctx->compute_units * 16); \
-        if constexpr (FWD) softmax_forward_row16_kernel<T, N, CH><<<g16, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale); \
-        else softmax_backward_row16_kernel<T, N, CH><<<g16, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh); \
-        return (int)hipGetLastError();                                                                                 \
+        if (stream) DFDX_SOFTMAX_ROW16_AS(N, CH, true);                                                                \
+        else DFDX_SOFTMAX_ROW16_AS(N, CH, false);                                                                      \
     } while (0)
     if (vec) {
         const int64_t groups = cols / V;
@@ -312,6 +324,8 @@ int launch_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *a, cons
     }
 #undef DFDX_SOFTMAX_REG
 #undef DFDX_SOFTMAX_ROW16
+#undef DFDX_SOFTMAX_REG_AS
+#undef DFDX_SOFTMAX_ROW16_AS
     if constexpr (FWD) softmax_forward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale);
     else softmax_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh);
     return (int)hipGetLastError();

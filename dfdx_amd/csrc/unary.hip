@@ -10,11 +10,11 @@ namespace dfdx_rocm {
 namespace {
 
 // ACC: out[i] += s * x[i] (backward; `fresh`: out counts as zero and is not read), else out[i] = s * x[i]
-template <typename T, int N, bool ACC>
+template <typename T, int N, bool ACC, bool STREAM>
 __global__ __launch_bounds__(256) void scalar_mul_kernel(const T *x, T *out, int64_t groups, float s, bool fresh) {
     for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
         float v[N];
-        load_elems<T, N>(x + g * N, v);
+        load_elems_as<T, N, STREAM>(x + g * N, v);
         if constexpr (ACC) {
             float o[N];
             if (fresh) {
@@ -34,10 +34,10 @@ __global__ __launch_bounds__(256) void scalar_mul_kernel(const T *x, T *out, int
 }
 
 // out = max(x, 0)
-template <typename T, int N> __global__ __launch_bounds__(256) void relu_forward_kernel(const T *x, T *out, int64_t groups) {
+template <typename T, int N, bool STREAM> __global__ __launch_bounds__(256) void relu_forward_kernel(const T *x, T *out, int64_t groups) {
     for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
         float v[N];
-        load_elems<T, N>(x + g * N, v);
+        load_elems_as<T, N, STREAM>(x + g * N, v);
 #pragma unroll
         for (int i = 0; i < N; i++) v[i] = fmaxf(v[i], 0.0f);
         store_elems<T, N>(out + g * N, v);
@@ -45,12 +45,12 @@ template <typename T, int N> __global__ __launch_bounds__(256) void relu_forward
 }
 
 // grad_x += (x > 0 ? 1 : 0) * grad_out; `fresh`: grad_x counts as zero and is not read
-template <typename T, int N>
+template <typename T, int N, bool STREAM>
 __global__ __launch_bounds__(256) void relu_backward_kernel(const T *x, const T *go, T *gx, int64_t groups, bool fresh) {
     for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
         float v[N], d[N], o[N];
-        load_elems<T, N>(x + g * N, v);
-        load_elems<T, N>(go + g * N, d);
+        load_elems_as<T, N, STREAM>(x + g * N, v);
+        load_elems_as<T, N, STREAM>(go + g * N, d);
         if (fresh) {
 #pragma unroll
             for (int i = 0; i < N; i++) o[i] = 0.0f;
@@ -64,11 +64,11 @@ __global__ __launch_bounds__(256) void relu_backward_kernel(const T *x, const T 
 }
 
 // out = a + b
-template <typename T, int N> __global__ __launch_bounds__(256) void add_forward_kernel(const T *a, const T *b, T *out, int64_t groups) {
+template <typename T, int N, bool STREAM> __global__ __launch_bounds__(256) void add_forward_kernel(const T *a, const T *b, T *out, int64_t groups) {
     for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
         float v[N], w[N];
-        load_elems<T, N>(a + g * N, v);
-        load_elems<T, N>(b + g * N, w);
+        load_elems_as<T, N, STREAM>(a + g * N, v);
+        load_elems_as<T, N, STREAM>(b + g * N, w);
 #pragma unroll
         for (int i = 0; i < N; i++) v[i] += w[i];
         store_elems<T, N>(out + g * N, v);
@@ -76,11 +76,11 @@ template <typename T, int N> __global__ __launch_bounds__(256) void add_forward_
 }
 
 // grad_lhs += grad_out, grad_rhs += grad_out (two distinct buffers); fresh_l / fresh_r: that one counts as zero, not read
-template <typename T, int N>
+template <typename T, int N, bool STREAM>
 __global__ __launch_bounds__(256) void add_backward_kernel(const T *go, T *gl, T *gr, int64_t groups, bool fresh_l, bool fresh_r) {
     for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
         float d[N], l[N], r[N];
-        load_elems<T, N>(go + g * N, d);
+        load_elems_as<T, N, STREAM>(go + g * N, d);
 #pragma unroll
         for (int i = 0; i < N; i++) l[i] = r[i] = 0.0f;
         if (!fresh_l) load_elems<T, N>(gl + g * N, l);
@@ -142,8 +142,10 @@ template <typename T, bool ACC> int launch_t(dfdx_rocm_ctx *ctx, int64_t len, co
     const int64_t groups = vec ? len / V : len;
     const unsigned grid = (unsigned)std::min<int64_t>((groups + 255) / 256, (int64_t)ctx->compute_units * 16);
     const float s = round_scalar<T>(scalar);
-    if (vec) scalar_mul_kernel<T, V, ACC><<<grid, 256, 0, ctx->stream>>>((const T *)x, (T *)out, groups, s, fresh);
-    else scalar_mul_kernel<T, 1, ACC><<<grid, 256, 0, ctx->stream>>>((const T *)x, (T *)out, groups, s, fresh);
+    const bool stream = (size_t)len * sizeof(T) >= kStreamInputBytes;
+    if (vec && stream) scalar_mul_kernel<T, V, ACC, true><<<grid, 256, 0, ctx->stream>>>((const T *)x, (T *)out, groups, s, fresh);
+    else if (vec) scalar_mul_kernel<T, V, ACC, false><<<grid, 256, 0, ctx->stream>>>((const T *)x, (T *)out, groups, s, fresh);
+    else scalar_mul_kernel<T, 1, ACC, false><<<grid, 256, 0, ctx->stream>>>((const T *)x, (T *)out, groups, s, fresh);
     return (int)hipGetLastError();
 }
 
@@ -175,15 +177,18 @@ int launch_op(dfdx_rocm_ctx *ctx, int64_t len, const void *a, const void *b, voi
     const int64_t groups = vec ? len / V : len;
     const unsigned grid = (unsigned)std::min<int64_t>((groups + 255) / 256, (int64_t)ctx->compute_units * 16);
     hipStream_t s = ctx->stream;
-#define DFDX_OP(N)                                                                                                       \
+    constexpr int INPUTS = (OP == OP_RELU_BWD || OP == OP_ADD_FWD) ? 2 : 1;  // read-only operands of the op
+    const bool stream = vec && (size_t)len * sizeof(T) * INPUTS >= kStreamInputBytes;
+#define DFDX_OP(N, STREAM)                                                                                                       \
     do {                                                                                                                 \
-        if constexpr (OP == OP_RELU_FWD) relu_forward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (T *)c, groups);    \
-        else if constexpr (OP == OP_RELU_BWD) relu_backward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (const T *)b, (T *)c, groups, fresh_c); \
-        else if constexpr (OP == OP_ADD_FWD) add_forward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (const T *)b, (T *)c, groups);    \
-        else add_backward_kernel<T, N><<<grid, 256, 0, s>>>((const T *)a, (T *)c, (T *)d, groups, fresh_c, fresh_d);      \
+        if constexpr (OP == OP_RELU_FWD) relu_forward_kernel<T, N, STREAM><<<grid, 256, 0, s>>>((const T *)a, (T *)c, groups);    \
+        else if constexpr (OP == OP_RELU_BWD) relu_backward_kernel<T, N, STREAM><<<grid, 256, 0, s>>>((const T *)a, (const T *)b, (T *)c, groups, fresh_c); \
+        else if constexpr (OP == OP_ADD_FWD) add_forward_kernel<T, N, STREAM><<<grid, 256, 0, s>>>((const T *)a, (const T *)b, (T *)c, groups);    \
+        else add_backward_kernel<T, N, STREAM><<<grid, 256, 0, s>>>((const T *)a, (T *)c, (T *)d, groups, fresh_c, fresh_d);      \
     } while (0)
-    if (vec) DFDX_OP(V);
-    else DFDX_OP(1);
+    if (stream) DFDX_OP(V, true);
+    else if (vec) DFDX_OP(V, false);
+    else DFDX_OP(1, false);
 #undef DFDX_OP
     return (int)hipGetLastError();
 }

@@ -152,6 +152,35 @@ def test_relu_and_add_seeded(n, dtype):
     np.testing.assert_array_equal(host(dev, gt), twice)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_relu_add_and_scalar_mul_on_streamed_inputs(dtype):
+    """From 128 MiB of read-only input per launch on, the element-wise kernels load it non-temporally: same bits.
+    2^25 elements: every op in f32 (128 MiB per tensor), the two-input ops (ReLU backward, add forward) in bf16."""
+    dev, g = device(), rng(504)
+    n = 1 << 25
+    announce("relu / add / scalar mul, streamed inputs", n, dtype)
+    small = g.standard_normal(1 << 16)
+    x, y, go = (upload(dev, np.tile(np.roll(small, 17 * i), n >> 16), dtype) for i in range(3))
+    x64, y64, go64 = host(dev, x), host(dev, y), host(dev, go)
+    np.testing.assert_array_equal(host(dev, dev.relu_forward(x)), nn_ops.relu_forward(x64, dtype))
+    gx = dev.tensor(dev.to_host(y), dtype)
+    dev.relu_backward(x, gx, go)
+    np.testing.assert_array_equal(host(dev, gx), nn_ops.relu_backward(x64, y64, go64, dtype))
+    del gx
+    np.testing.assert_array_equal(host(dev, dev.add_forward(x, y)), nn_ops.add_forward(x64, y64, dtype))
+    gl, gr = dev.tensor(dev.to_host(x), dtype), dev.tensor(dev.to_host(y), dtype)
+    dev.add_backward(gl, gr, go)
+    wl, wr = nn_ops.add_backward(x64, y64, go64, dtype)
+    np.testing.assert_array_equal(host(dev, gl), wl)
+    np.testing.assert_array_equal(host(dev, gr), wr)
+    del gl, gr, wl, wr
+    s = 0.25   # a power of two: the product is exact, so a fused and an unfused multiply-add round alike
+    np.testing.assert_array_equal(host(dev, dev.scalar_mul_forward(x, s)), nn_ops.scalar_mul_forward(x64, s, dtype))
+    gi = dev.tensor(dev.to_host(y), dtype)
+    dev.scalar_mul_backward(s, gi, go)
+    np.testing.assert_array_equal(host(dev, gi), nn_ops.scalar_mul_backward(s, y64, go64, dtype))
+
+
 def test_relu_signed_zero_and_nan():
     dev = device()
     announce("relu special values")

@@ -357,6 +357,19 @@ def test_gemv(dtype, shape, layout):
     run_case(dtype, m, k, n, layout, True, KERNEL_AUTO, 0, seed=4, bias=(dtype == "f32"))
 
 
+@pytest.mark.parametrize("case", [("f32", 1, 8192, 8192, "nn"), ("f32", 8192, 8192, 1, "nn"), ("f32", 1, 8192, 8192, "nt"),
+                                  ("f16", 1, 16384, 8192, "nn"), ("f32", 4, 8192, 8192, "nn"), ("f32", 8192, 8192, 3, "tn"),
+                                  ("bf16", 2, 8192, 16384, "nt")],
+                         ids=lambda c: "-".join(map(str, c)))
+def test_vector_products_with_a_streamed_matrix(case):
+    """From 256 MiB of matrix on, the vector-product kernels read it with non-temporal loads (it cannot stay cached
+    between two products): the same sums, one and several vectors, both layouts, beta = 0 and 1."""
+    from dfdx_amd.rocm import KERNEL_GEMV
+    dtype, m, k, n, layout = case
+    run_case(dtype, m, k, n, layout, False, KERNEL_GEMV, 0, seed=21)
+    run_case(dtype, m, k, n, layout, True, KERNEL_GEMV, 0, seed=22)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("shape", [(2, 1024, 1032), (3, 2056, 520), (4, 4096, 1024), (5, 1032, 2048), (8, 8200, 264), (7, 264, 8200),
                                    (1032, 1024, 2), (520, 2056, 3), (2048, 1032, 8), (8200, 264, 6)])
