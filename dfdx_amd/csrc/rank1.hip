@@ -36,24 +36,31 @@ struct Rank1Params {
 // 16 bytes of a row of C as the computing type and back.  ALIGNED: the address is a multiple of 16; otherwise it is only
 // element-aligned (an odd leading dimension or extent) and the access is one unaligned 16-byte load or store, which
 // global memory allows.
-template <typename T, bool ALIGNED> __device__ __forceinline__ void load_row_piece(const T *p, typename Acc<T>::type (&v)[Elem<T>::VEC]) {
+// STREAM (aligned rows only): the non-temporal forms, for an accumulation into 256 MiB of C or more -- read once, written
+// once, too large to be found in the last-level cache by anybody (a weight gradient W += x (x) y on 16384^2: f32 414 ->
+// 372 us, f16 197 -> 188 us; on a 4096^2 that is updated launch after launch the cached forms are faster, 10.1 against 11.5 us).
+template <typename T, bool ALIGNED, bool STREAM = false>
+__device__ __forceinline__ void load_row_piece(const T *p, typename Acc<T>::type (&v)[Elem<T>::VEC]) {
     constexpr int N = Elem<T>::VEC;
     u32x4 raw;
-    if constexpr (ALIGNED) raw = *(const u32x4 *)p;
+    if constexpr (ALIGNED && STREAM) raw = __builtin_nontemporal_load((const u32x4 *)p);
+    else if constexpr (ALIGNED) raw = *(const u32x4 *)p;
     else raw = *(const u32x4_unaligned *)p;
     T tmp[N];
     __builtin_memcpy(tmp, &raw, 16);
 #pragma unroll
     for (int i = 0; i < N; i++) v[i] = Elem<T>::load(&tmp[i]);
 }
-template <typename T, bool ALIGNED> __device__ __forceinline__ void store_row_piece(T *p, const typename Acc<T>::type (&v)[Elem<T>::VEC]) {
+template <typename T, bool ALIGNED, bool STREAM = false>
+__device__ __forceinline__ void store_row_piece(T *p, const typename Acc<T>::type (&v)[Elem<T>::VEC]) {
     constexpr int N = Elem<T>::VEC;
     T tmp[N];
 #pragma unroll
     for (int i = 0; i < N; i++) Elem<T>::store(&tmp[i], v[i]);
     u32x4 raw;
     __builtin_memcpy(&raw, tmp, 16);
-    if constexpr (ALIGNED) *(u32x4 *)p = raw;
+    if constexpr (ALIGNED && STREAM) __builtin_nontemporal_store(raw, (u32x4 *)p);
+    else if constexpr (ALIGNED) *(u32x4 *)p = raw;
     else *(u32x4_unaligned *)p = raw;
 }
 
@@ -63,7 +70,7 @@ __device__ __forceinline__ double fused(double a, double b, double c) { return _
 constexpr int STAGED_A = 4096;  // values of a one workgroup keeps in LDS (k > 1): rows per workgroup x KMAX stays below
 
 // KMAX: 1, or the power of two that holds k.
-template <typename T, bool ALIGNED, int KMAX> __global__ __launch_bounds__(256) void rank1_kernel(const Rank1Params p) {
+template <typename T, bool ALIGNED, int KMAX, bool STREAM = false> __global__ __launch_bounds__(256) void rank1_kernel(const Rank1Params p) {
     typedef typename Acc<T>::type A;
     constexpr int N = Elem<T>::VEC;
     const int tx = 1 << p.tx_log2, ty = 256 >> p.tx_log2;
@@ -144,8 +151,8 @@ template <typename T, bool ALIGNED, int KMAX> __global__ __launch_bounds__(256) 
         for (int e = 0; e < N; e++) o0[e] = o1[e] = 0;
         if (p.accumulate) {
             if (have == N) {
-                load_row_piece<T, ALIGNED>(d0, o0);
-                if (two) load_row_piece<T, ALIGNED>(d1, o1);
+                load_row_piece<T, ALIGNED, STREAM>(d0, o0);
+                if (two) load_row_piece<T, ALIGNED, STREAM>(d1, o1);
             } else {
 #pragma unroll
                 for (int e = 0; e < N; e++)
@@ -168,8 +175,8 @@ template <typename T, bool ALIGNED, int KMAX> __global__ __launch_bounds__(256) 
             o0[e] = v0 + o0[e]; o1[e] = v1 + o1[e];
         }
         if (have == N) {
-            store_row_piece<T, ALIGNED>(d0, o0);
-            if (two) store_row_piece<T, ALIGNED>(d1, o1);
+            store_row_piece<T, ALIGNED, STREAM>(d0, o0);
+            if (two) store_row_piece<T, ALIGNED, STREAM>(d1, o1);
         } else {
 #pragma unroll
             for (int e = 0; e < N; e++)
@@ -205,9 +212,11 @@ template <typename T> hipError_t launch_t(const Rank1Params &base, const GemmPro
     const int64_t blocks_x = (g.m + p.rows_per_block - 1) / p.rows_per_block;
     if (blocks_y > 65535 || blocks_x >= (1ll << 31)) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks_x, (unsigned)blocks_y);
+    const bool streamed = p.accumulate && (double)g.m * (double)g.n * (double)sizeof(T) >= 268435456.0;
 #define DFDX_RANK(KMAX)                                                          \
     do {                                                                         \
-        if (aligned) rank1_kernel<T, true, KMAX><<<grid, 256, 0, stream>>>(p);   \
+        if (aligned && streamed) rank1_kernel<T, true, KMAX, true><<<grid, 256, 0, stream>>>(p); \
+        else if (aligned) rank1_kernel<T, true, KMAX><<<grid, 256, 0, stream>>>(p); \
         else rank1_kernel<T, false, KMAX><<<grid, 256, 0, stream>>>(p);          \
     } while (0)
     if (g.k == 1) DFDX_RANK(1);

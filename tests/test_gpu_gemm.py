@@ -458,6 +458,21 @@ def test_rank1_updates(dtype):
         assert np.array_equal(dev.to_host(dc).reshape(300, 200), np.outer(x, y))
 
 
+@pytest.mark.parametrize("case", [("f32", 8192, 1, 8192), ("f32", 8192, 4, 8192), ("f16", 16384, 1, 8192), ("f64", 4096, 2, 8192)],
+                         ids=lambda c: "-".join(map(str, c)))
+def test_rank1_update_into_a_streamed_output(case):
+    """Accumulating into 256 MiB of C or more, the row-streaming kernel reads and writes C with non-temporal accesses:
+    the same sums as the cached form (and, for comparison, the overwriting product of the same shape, which stays cached)."""
+    dtype, m, k, n = case
+    dev = device()
+    a = dev.zeros(dtype, (8,))
+    plan = dev.gemm_plan(dev.gemm_desc(dtype, m, k, n, a.ptr, (k, 1), a.ptr, (n, 1), a.ptr, (n, 1), accumulate=True))
+    if k == 1 or dtype == "f64":   # (f32 with k = 4 goes to the matrix-core form of the thin kernel: checked all the same)
+        assert plan[2] in ("rank1", "thin_k"), plan
+    run_case(dtype, m, k, n, "nn", True, KERNEL_AUTO, 0, seed=31)
+    run_case(dtype, m, k, n, "nn", False, KERNEL_AUTO, 0, seed=32)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16", "f64"])
 @pytest.mark.parametrize("k", [2, 3, 4, 5, 8])
 def test_thin_contractions(dtype, k):
