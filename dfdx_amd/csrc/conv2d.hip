@@ -7,6 +7,7 @@
 #include <initializer_list>
 #include "elem.h"
 #include "gemm_internal.h"
+#include "conv3x3.h"
 
 #include <cstring>
 
@@ -260,6 +261,28 @@ bool implicit_forward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *f
     return true;
 }
 
+// 3 x 3 filters at unit stride with padding 1, 16-bit types, channel counts in whole chunks: the kernel that keeps a band
+// of the image in LDS and reads every tap's operand from it (conv3x3.hip).  The filters go through the patch buffer in
+// the order that kernel wants.
+template <typename T>
+bool tiled3x3_forward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *filters, const void *img, void *out, int *rc) {
+    if (sizeof(T) != 2 || op.kernel != 3 || op.stride != 1 || op.padding != 1 || op.dilation != 1 || op.groups != 1) return false;
+    if (op.h_out != op.h_in || op.w_out != op.w_in) return false;
+    Conv3x3Problem c{};
+    c.dtype = dtype == DFDX_ROCM_F16 ? DT_F16 : DT_BF16;
+    c.batch = op.batch; c.chan_in = op.chan_in; c.chan_out = op.chan_out; c.h = op.h_in; c.w = op.w_in;
+    c.img = img; c.filters = filters; c.out = out;
+    c.wt = (void *)16;  // any aligned address: the real one needs the lock below
+    if (!conv3x3_supported(c)) return false;
+    CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
+    if ((*rc = ensure_patches(ctx, round256(conv3x3_filter_bytes(c))))) return true;
+    c.wt = ctx->patches;
+    const hipError_t e = launch_conv3x3(c, ctx->stream);
+    if (e == hipErrorNotSupported) return false;
+    *rc = (int)e;
+    return true;
+}
+
 template <typename T>
 int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void *filters, void *out) {
     constexpr int V = Elem<T>::VEC;
@@ -271,6 +294,7 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
     if (per_image >= (1ll << 31) || (int64_t)op.chan_out * np >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
     if (op.kernel > 1) {  // (1x1 filters have no patch matrix to avoid: see `pointwise` below)
         int rc = 0;
+        if (tiled3x3_forward<T>(ctx, dtype, op, filters, img, out, &rc)) return rc;
         if (implicit_forward<T>(ctx, dtype, op, filters, img, out, &rc)) return rc;
     }
     CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context

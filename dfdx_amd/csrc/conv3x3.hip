@@ -1,0 +1,298 @@
+// 3 x 3 convolution at unit stride with padding 1 (f16 / bf16, f32 accumulate, gfx950) without a patch matrix, in
+// global memory or in any other form: the product of `Conv2DKernel::forward` (dfdx-core/src/tensor_ops/conv2d/
+// cpu_kernel.rs:52-98: unfold, then filters . patches per image and group) for the shapes of a residual network's 3 x 3
+// layers.
+//
+//   out[b][o][y][x] = sum over (ky, kx, c) of  filters[o][c][ky][kx] * img[b][c][y + ky - 1][x + kx - 1]
+//
+// as a GEMM per image with M = output channels, N = pixels, K ordered (tap, channel) -- channel fastest.  With that
+// order the 8 consecutive k a lane feeds to one v_mfma_f32_16x16x32 are 8 CHANNELS of ONE pixel at ONE tap, so the B
+// operand of every tap is read from one copy of the image in LDS, stored pixel-major with the channels of a pixel next
+// to each other; the tap only shifts the pixel a lane reads.  The K*K-fold patch matrix never exists.
+//
+// A workgroup (8 waves as 2 x 4, wave tile 32 channels x 64 pixels) owns 64 output channels x 256 consecutive pixels of
+// one image.  Per chunk of 32 input channels it fills
+//   * A: filters[64][9 taps][32 ch] from the re-laid copy wt[o][tap][c] (conv3x3_filters_kernel), rows padded to 37
+//     16-byte pieces so that the 16 rows of a fragment read fall on distinct banks;
+//   * the band of the image its pixels and their neighbours lie in: rows (first row - 1 .. last row + 1) x columns
+//     (-1 .. W) x 32 channels, 80 bytes per pixel (64 + 16 of padding: consecutive pixels on distinct banks), zeros
+//     outside the image.  The image is stored channel-major in memory, so a thread takes two neighbouring pixels of 8
+//     channels (eight 4-byte loads: any even width is aligned), interleaves them with byte permutes and writes two
+//     16-byte pixel records;
+// then runs 9 taps x 8 MFMAs per wave.  One LDS stage (about 75 KB): two workgroups share a compute unit and one fills
+// while the other multiplies.
+#include "gemm_internal.h"
+#include "conv3x3.h"
+#include <algorithm>
+
+namespace dfdx_rocm {
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int NT = 256;        // pixels per workgroup
+constexpr int MT = 64;         // output channels per workgroup
+constexpr int CK = 32;         // input channels per chunk
+constexpr int PIX = 80;        // bytes of a pixel record in LDS (32 channels + padding)
+constexpr int AROW = 37 * 16;  // bytes of a filter row in LDS (9 taps x 32 channels + padding)
+constexpr int A_BYTES = MT * AROW;
+
+template <typename T> struct Mma16;
+template <> struct Mma16<_Float16> {
+    static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, h2));
+    }
+};
+template <> struct Mma16<__bf16> {
+    static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, b2));
+    }
+};
+
+struct Params {
+    const uint16_t *img;  // [B][C][H][W]
+    const uint16_t *wt;   // [O][9][C]
+    uint16_t *out;        // [B][O][H][W]
+    int C, O, H, W, HW;
+    int nblocks, mblocks;  // pixel blocks per image, blocks of 64 output channels
+    int band_rows;         // image rows (with the two halo rows) the LDS band holds
+    uint32_t magic_w, magic_pairs;  // ceil(2^32 / W), ceil(2^32 / (W / 2)): n / W = umulhi(n, magic_w) for n < 2^24
+};
+
+// wt[o][tap][c] = filters[o][c][tap]
+__global__ __launch_bounds__(256) void conv3x3_filters_kernel(const uint16_t *__restrict__ f, uint16_t *__restrict__ wt, int C, int total) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int c = i % C, tap = (i / C) % 9, o = i / (9 * C);
+    wt[i] = f[((int64_t)o * C + c) * 9 + tap];
+}
+
+// UMAX: pixel-pair units of the band a thread may own per chunk (2: four waves per SIMD, 128 registers; 4: two)
+template <typename T, int UMAX>
+__global__ __launch_bounds__(512, UMAX <= 2 ? 4 : 2) void conv3x3_kernel(const Params p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t *const sin = smem + A_BYTES;
+    const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int l16 = lane % 16, lq = lane / 16;
+    const int wm0 = (wave / 4) * 32, wn0 = (wave % 4) * 64;
+    const int W = p.W, WP = W + 2, H = p.H;
+
+    const int mb = blockIdx.x, nb = blockIdx.y, b = blockIdx.z;
+    const int n0 = nb * NT;
+    // (divisions by W and W / 2 as multiplications: the quotients are exact for every n < 2^24 >= H * W)
+    auto div_w = [&](int n) { return (int)__umulhi((uint32_t)n, p.magic_w); };
+    const int ytop = div_w(n0);                           // first image row with a pixel of this block
+    const int ylast = div_w(min(n0 + NT - 1, p.HW - 1));  // last one
+    const int rows = ylast - ytop + 3;                    // band rows: ytop - 1 .. ylast + 1
+
+    // halo columns (x = -1 and x = W) of every band row: zero for the whole launch
+    for (int u = tid; u < rows * 2 * 5; u += 512) {
+        const int r = u / 10, side = (u / 5) % 2, q = u % 5;
+        *(u32x4 *)(sin + (r * WP + side * (W + 1)) * PIX + q * 16) = u32x4{0, 0, 0, 0};
+    }
+
+    // fragment addresses
+    uint32_t a_addr[2], b_addr[4];
+#pragma unroll
+    for (int i = 0; i < 2; i++) a_addr[i] = (uint32_t)((wm0 + 16 * i + l16) * AROW + lq * 16);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int n = min(n0 + wn0 + 16 * j + l16, p.HW - 1);
+        const int y = div_w(n), x = n - y * W;
+        b_addr[j] = (uint32_t)(A_BYTES + ((y - ytop) * WP + x) * PIX + lq * 16);  // tap (0, 0): band row y - ytop, column x
+    }
+
+    f32x4 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const uint16_t *const image = p.img + (int64_t)b * p.C * p.HW;
+    const __amdgpu_buffer_rsrc_t planes = __builtin_amdgcn_make_buffer_rsrc((void *)image, 0, p.C * p.HW * 2, 0x00020000);
+    const uint16_t *const wrows = p.wt + (int64_t)mb * MT * 9 * p.C;
+    const int pairs = W / 2, units = 4 * rows * pairs;
+
+    // What a thread moves per chunk, worked out once: UMAX pixel-pair units of the band (element offset of channel 0 of
+    // the unit's 8 in chunk 0, -1 = the row lies outside the image and is written as zeros; LDS byte offset, -1 = no
+    // such unit) (its five of the 64 x 36 filter pieces are worked out where they are used).
+    int u_src[UMAX], u_dst[UMAX];
+#pragma unroll
+    for (int s = 0; s < UMAX; s++) {
+        const int u = tid + s * 512;
+        const int t = (int)__umulhi((uint32_t)u, p.magic_pairs), xp = u - t * pairs;  // t = cg * rows + r
+        const int cg = (t >= rows) + (t >= 2 * rows) + (t >= 3 * rows), r = t - cg * rows;
+        const int y = ytop - 1 + r;
+        u_src[s] = (u < units && y >= 0 && y < H) ? (8 * cg * H + y) * W + 2 * xp : -1;
+        u_dst[s] = u < units ? A_BYTES + (r * WP + 1 + 2 * xp) * PIX + cg * 16 : -1;
+    }
+    uint32_t d[UMAX][8];
+    u32x4 piece[5];
+    auto request = [&](int c0) {  // the global loads of one chunk: the band first, then the filter pieces
+        // buffer loads: the image of this batch entry as the resource, one 32-bit byte offset per lane shared by the eight
+        // loads of a unit, the channel plane in the scalar offset; a lane with nothing to load points past the end of the
+        // resource and receives zeros
+#pragma unroll
+        for (int s = 0; s < UMAX; s++) {
+            const uint32_t off = u_src[s] >= 0 ? (uint32_t)u_src[s] * 2u : 0xFFFFFFF0u;
+#pragma unroll
+            for (int e = 0; e < 8; e++) d[s][e] = __builtin_amdgcn_raw_buffer_load_b32(planes, (int)off, (c0 + e) * p.HW * 2, 0);
+        }
+        const char *rowbase = (const char *)(wrows + c0);
+#pragma unroll
+        for (int s = 0; s < 5; s++) {
+            const int q = tid + s * 512;  // 64 rows x 36 pieces, not kept in registers across the chunk
+            const int o = min(q / 36, MT - 1), part = q % 36;
+            piece[s] = *(const u32x4 *)(rowbase + (uint32_t)(((o * 9 + part / 4) * p.C + (part % 4) * 8) * 2));
+        }
+    };
+    auto deposit = [&]() {  // ... into LDS: pixel records of two neighbouring pixels x 8 channels, filter pieces as they are
+#pragma unroll
+        for (int s = 0; s < 5; s++) {
+            const int q = tid + s * 512;
+            if (q < MT * 36) *(u32x4 *)(smem + (q / 36) * AROW + (q % 36) * 16) = piece[s];
+        }
+#pragma unroll
+        for (int s = 0; s < UMAX; s++) {
+            if (u_dst[s] >= 0) {
+                u32x4 px0, px1;
+#pragma unroll
+                for (int h = 0; h < 4; h++) {
+                    px0[h] = __builtin_amdgcn_perm(d[s][2 * h + 1], d[s][2 * h], 0x05040100u);  // low halves: pixel 2 xp
+                    px1[h] = __builtin_amdgcn_perm(d[s][2 * h + 1], d[s][2 * h], 0x07060302u);  // high halves: pixel 2 xp + 1
+                }
+                *(u32x4 *)(smem + u_dst[s]) = px0;
+                *(u32x4 *)(smem + u_dst[s] + PIX) = px1;
+            }
+        }
+    };
+
+    request(0);
+    for (int c0 = 0; c0 < p.C; c0 += CK) {
+        __syncthreads();  // the previous chunk's fragments have been read
+        deposit();
+        __syncthreads();
+        if (c0 + CK < p.C) request(c0 + CK);  // the next chunk travels while this one is multiplied
+        // ---- 9 taps x (2 x 4) MFMAs; operands swapped so that a lane ends up with 4 consecutive pixels of one channel
+#pragma unroll
+        for (int ky = 0; ky < 3; ky++)
+#pragma unroll
+            for (int kx = 0; kx < 3; kx++) {
+                const uint32_t shift = (uint32_t)((ky * WP + kx) * PIX);
+                u32x4 fa[2], fb[4];
+#pragma unroll
+                for (int i = 0; i < 2; i++) fa[i] = *(const u32x4 *)(smem + a_addr[i] + (ky * 3 + kx) * 64);
+#pragma unroll
+                for (int j = 0; j < 4; j++) fb[j] = *(const u32x4 *)(smem + b_addr[j] + shift);
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int i = 0; i < 2; i++) acc[i][j] = Mma16<T>::mfma(fb[j], fa[i], acc[i][j]);
+            }
+    }
+
+    // ---- epilogue: lane holds channel o = l16 (per tile) and pixels 4 lq + 0..3 of each 16-pixel tile
+    uint16_t *const obase = p.out + ((int64_t)b * p.O + (int64_t)mb * MT) * p.HW;
+    if (p.HW % 8 == 0) {
+        // 16 bytes per lane: two neighbouring pixel tiles trade halves between the lane rows (v_permlane16_swap on the
+        // packed pairs), after which lane row lq holds pixels 8 (lq / 2) + 0..7 of tile 2 jp + (lq & 1); a store
+        // instruction then writes 64 contiguous bytes of each of 16 channel rows instead of 32
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            uint16_t *orow = obase + (int64_t)(wm0 + 16 * i + l16) * p.HW;
+#pragma unroll
+            for (int jp = 0; jp < 2; jp++) {
+                u32x4 o;
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const uint32_t lo = Mma16<T>::pack2(acc[i][2 * jp][2 * h], acc[i][2 * jp][2 * h + 1]);
+                    const uint32_t hi = Mma16<T>::pack2(acc[i][2 * jp + 1][2 * h], acc[i][2 * jp + 1][2 * h + 1]);
+                    const auto r = __builtin_amdgcn_permlane16_swap(lo, hi, false, false);
+                    o[h] = r[0];
+                    o[2 + h] = r[1];
+                }
+                const int n = n0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8;
+                if (n < p.HW) *(u32x4 *)(orow + n) = o;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            uint16_t *orow = obase + (int64_t)(wm0 + 16 * i + l16) * p.HW;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int n = n0 + wn0 + 16 * j + 4 * lq;
+                if (n < p.HW)  // HW % 4 == 0: all four pixels are in range
+                    *(u32x2 *)(orow + n) = u32x2{Mma16<T>::pack2(acc[i][j][0], acc[i][j][1]), Mma16<T>::pack2(acc[i][j][2], acc[i][j][3])};
+            }
+        }
+    }
+}
+
+}  // namespace
+
+bool conv3x3_supported(const Conv3x3Problem &c) {
+    if (c.dtype != DT_F16 && c.dtype != DT_BF16) return false;
+    if (c.batch < 1 || c.chan_in < CK || c.chan_in % CK || c.chan_out < MT || c.chan_out % MT) return false;
+    if (c.w < 4 || c.w > 254 || c.w % 2 || c.h < 1 || ((int64_t)c.h * c.w) % 4) return false;
+    const int64_t hw = (int64_t)c.h * c.w;
+    if (hw < 128 || hw >= (1 << 24) || (int64_t)c.chan_in * hw >= (1ll << 30)) return false;  // byte offsets of an image fit 31 bits
+    if (((uintptr_t)c.img & 3u) || ((uintptr_t)c.out & 7u) || ((uintptr_t)c.filters & 1u) || ((uintptr_t)c.wt & 15u)) return false;
+    const int band_rows = (int)std::min<int64_t>(c.h, (NT - 1) / c.w + 2) + 2;
+    if ((size_t)A_BYTES + (size_t)band_rows * (c.w + 2) * PIX > 160 * 1024) return false;
+    if (4 * band_rows * (c.w / 2) > 4 * 512) return false;  // units per chunk: at most four per thread
+    return c.batch < 65536 && (hw + NT - 1) / NT < 65536;  // grid.z, grid.y
+}
+
+size_t conv3x3_filter_bytes(const Conv3x3Problem &c) { return (size_t)c.chan_out * 9 * c.chan_in * 2; }
+
+hipError_t launch_conv3x3(const Conv3x3Problem &c, hipStream_t stream) {
+    if (!conv3x3_supported(c)) return hipErrorNotSupported;
+    const int total = c.chan_out * 9 * c.chan_in;
+    conv3x3_filters_kernel<<<(total + 255) / 256, 256, 0, stream>>>((const uint16_t *)c.filters, (uint16_t *)c.wt, c.chan_in, total);
+    Params p;
+    p.img = (const uint16_t *)c.img; p.wt = (const uint16_t *)c.wt; p.out = (uint16_t *)c.out;
+    p.C = c.chan_in; p.O = c.chan_out; p.H = c.h; p.W = c.w; p.HW = c.h * c.w;
+    p.nblocks = (p.HW + NT - 1) / NT; p.mblocks = c.chan_out / MT;
+    p.band_rows = (int)std::min<int64_t>(c.h, (NT - 1) / c.w + 2) + 2;
+    const size_t lds = (size_t)A_BYTES + (size_t)p.band_rows * (c.w + 2) * PIX;
+    p.magic_w = (uint32_t)(((1ull << 32) + c.w - 1) / c.w);
+    p.magic_pairs = (uint32_t)(((1ull << 32) + c.w / 2 - 1) / (c.w / 2));
+    const dim3 grid((unsigned)p.mblocks, (unsigned)p.nblocks, (unsigned)c.batch);
+    const bool few = 4 * p.band_rows * (c.w / 2) <= 2 * 512;
+#define DFDX_CONV3(T, U)                                                                                               \
+    do {                                                                                                               \
+        static PerDevice attr_on;                                                                                      \
+        std::atomic<int> &known = attr_on.here();                                                                      \
+        if (known.load(std::memory_order_acquire) == 0) {                                                              \
+            hipError_t e = hipFuncSetAttribute((const void *)conv3x3_kernel<T, U>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            if (e != hipSuccess) return e;                                                                             \
+            known.store(1, std::memory_order_release);                                                                 \
+        }                                                                                                              \
+        conv3x3_kernel<T, U><<<grid, 512, lds, stream>>>(p);                                                           \
+    } while (0)
+    if (c.dtype == DT_F16) {
+        if (few) DFDX_CONV3(_Float16, 2);
+        else DFDX_CONV3(_Float16, 4);
+    } else {
+        if (few) DFDX_CONV3(__bf16, 2);
+        else DFDX_CONV3(__bf16, 4);
+    }
+#undef DFDX_CONV3
+    return hipGetLastError();
+}
+
+}  // namespace dfdx_rocm

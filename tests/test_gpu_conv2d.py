@@ -104,6 +104,51 @@ def test_conv2d_seeded(cfg, dtype):
                   extra=(batch + 2) * ULP[dtype] * float(np.abs(wgw).max()), what="grad_filters")
 
 
+# 3 x 3 filters at unit stride with padding 1, input channels in chunks of 32, output channels in blocks of 64, an even
+# width and at least 128 pixels: the forward product runs on the kernel that keeps a band of the image in LDS and has no
+# patch matrix in any form (conv3x3.hip).  Shapes: one and several channel chunks / output blocks, pixel blocks that end
+# in the middle of a row or of the image (one partial block; 196, 200 and 280 pixels), H * W off the 8-pixel grid (the
+# 8-byte store form), bands of 3 to 24 rows, an odd height, a width of 112 (four units of the band per thread).
+BAND_CONFIGS = [(2, 32, 64, 16, 16), (1, 64, 64, 14, 14), (3, 96, 128, 20, 14), (2, 64, 64, 56, 56), (2, 128, 192, 28, 28),
+                (1, 32, 64, 9, 112), (2, 64, 64, 31, 12), (1, 64, 64, 112, 112), (5, 32, 64, 8, 16), (2, 32, 64, 50, 4)]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("cfg", BAND_CONFIGS, ids=lambda c: "x".join(map(str, c)))
+def test_conv2d_3x3_forward_from_a_band_in_lds(cfg, dtype):
+    dev, g = device(), rng(504)
+    batch, cin, cout, h, w_ = cfg
+    announce("conv2d 3x3 band kernel", cfg, dtype)
+    op = Conv2DOp.make(batch, cin, cout, h, w_, 3, 1, 1, 1, 1)
+    x = upload(dev, g.standard_normal((batch, cin, h, w_)), dtype)
+    w = upload(dev, g.standard_normal((cout, cin, 3, 3)) / np.sqrt(cin * 9), dtype)
+    y = dev.conv2d_forward(x, w, stride=1, padding=1)
+    assert y.shape == (batch, cout, h, w_)
+    x_h, w_h = dev.to_host(x).reshape(-1), dev.to_host(w).reshape(-1)
+    want = oracle.to_f64(conv2d_forward(dtype, op, x_h, w_h), dtype)
+    assert_within(dtype, cin * 9, host(dev, y).reshape(-1), want, oracle.to_f64(x_h, dtype), oracle.to_f64(w_h, dtype),
+                  extra=ULP[dtype] * float(np.abs(want).max()), what="out")
+    # the same call again gives the same bits (nothing in the kernel depends on timing)
+    y2 = dev.conv2d_forward(x, w, stride=1, padding=1)
+    np.testing.assert_array_equal(dev.to_host(y), dev.to_host(y2))
+
+
+def test_conv2d_3x3_band_kernel_zero_padding_is_exact():
+    """An image of ones against filters of ones: every output is the number of taps inside the image times the channel
+    count -- 4 C in the corners, 6 C on the edges, 9 C inside -- exactly (small integers), whichever rows and columns a
+    pixel block starts and ends on."""
+    dev = device()
+    batch, cin, cout, h, w_ = 2, 64, 64, 23, 18
+    announce("conv2d 3x3 band kernel, ones", batch, cin, cout, h, w_)
+    x = upload(dev, np.ones((batch, cin, h, w_)), "f16")
+    w = upload(dev, np.ones((cout, cin, 3, 3)), "f16")
+    got = host(dev, dev.conv2d_forward(x, w, stride=1, padding=1))
+    ny = 3 - (np.arange(h) == 0) - (np.arange(h) == h - 1)
+    nx = 3 - (np.arange(w_) == 0) - (np.arange(w_) == w_ - 1)
+    want = (ny[:, None] * nx[None, :] * cin).astype(np.float64)
+    np.testing.assert_array_equal(got, np.broadcast_to(want, got.shape))
+
+
 def test_conv2d_unbatched_equals_batch_of_one():
     dev, g = device(), rng(502)
     announce("conv2d unbatched")
