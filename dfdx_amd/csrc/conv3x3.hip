@@ -12,15 +12,15 @@
 //
 // A workgroup (8 waves as 2 x 4, wave tile 32 channels x 64 pixels) owns 64 output channels x 256 consecutive pixels of
 // one image.  Per chunk of 32 input channels it fills
-//   * A: filters[64][9 taps][32 ch] from the re-laid copy wt[o][tap][c] (conv3x3_filters_kernel), rows padded to 37
-//     16-byte pieces so that the 16 rows of a fragment read fall on distinct banks;
+//   * A: filters[64][9 taps][32 ch] from the re-laid copy wt[o][tap][c] (conv3x3_filters_kernel), the four 16-byte
+//     pieces of a tap XOR-swizzled by the row so that the 16 rows of a fragment read fall on distinct banks;
 //   * the band of the image its pixels and their neighbours lie in: rows (first row - 1 .. last row + 1) x columns
-//     (-1 .. W) x 32 channels, 80 bytes per pixel (64 + 16 of padding: consecutive pixels on distinct banks), zeros
-//     outside the image.  The image is stored channel-major in memory, so a thread takes two neighbouring pixels of 8
-//     channels (eight 4-byte loads: any even width is aligned), interleaves them with byte permutes and writes two
-//     16-byte pixel records;
-// then runs 9 taps x 8 MFMAs per wave.  One LDS stage (about 75 KB): two workgroups share a compute unit and one fills
-// while the other multiplies.
+//     (-1 .. W) x 32 channels, 96 bytes per pixel (64 + 32 of padding: 16 consecutive pixels x 4 pieces read without a
+//     bank conflict), zeros outside the image.  The image is stored channel-major in memory, so a thread takes two
+//     neighbouring pixels of 8 channels (eight 4-byte loads: any even width is aligned), interleaves them with byte
+//     permutes and writes two 16-byte pieces of pixel records;
+// then runs 9 taps x 8 MFMAs per wave, the loads of the next chunk in flight meanwhile.  One LDS stage (80 KB at a width
+// of 56): two workgroups share a compute unit.
 #include "gemm_internal.h"
 #include "conv3x3.h"
 #include <algorithm>
@@ -38,8 +38,10 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int NT = 256;        // pixels per workgroup
 constexpr int MT = 64;         // output channels per workgroup
 constexpr int CK = 32;         // input channels per chunk
-constexpr int PIX = 80;        // bytes of a pixel record in LDS (32 channels + padding)
-constexpr int AROW = 37 * 16;  // bytes of a filter row in LDS (9 taps x 32 channels + padding)
+// LDS layouts, both measured free of bank conflicts for the fragment reads (16 rows or pixels x four 16-byte pieces per
+// wave instruction; records of 64 or 80 bytes, or unswizzled 576-byte rows, read at half the rate):
+constexpr int PIX = 96;        // bytes of a pixel record: 32 channels + 32 of padding (an odd multiple of 32 bytes)
+constexpr int AROW = 36 * 16;  // bytes of a filter row: 9 taps x four pieces, piece g of a tap in slot g ^ (row / 2 % 4)
 constexpr int A_BYTES = MT * AROW;
 
 template <typename T> struct Mma16;
@@ -99,15 +101,15 @@ __global__ __launch_bounds__(512, UMAX <= 2 ? 4 : 2) void conv3x3_kernel(const P
     const int rows = ylast - ytop + 3;                    // band rows: ytop - 1 .. ylast + 1
 
     // halo columns (x = -1 and x = W) of every band row: zero for the whole launch
-    for (int u = tid; u < rows * 2 * 5; u += 512) {
-        const int r = u / 10, side = (u / 5) % 2, q = u % 5;
+    for (int u = tid; u < rows * 2 * 4; u += 512) {
+        const int r = u / 8, side = (u / 4) % 2, q = u % 4;
         *(u32x4 *)(sin + (r * WP + side * (W + 1)) * PIX + q * 16) = u32x4{0, 0, 0, 0};
     }
 
     // fragment addresses
     uint32_t a_addr[2], b_addr[4];
 #pragma unroll
-    for (int i = 0; i < 2; i++) a_addr[i] = (uint32_t)((wm0 + 16 * i + l16) * AROW + lq * 16);
+    for (int i = 0; i < 2; i++) a_addr[i] = (uint32_t)((wm0 + 16 * i + l16) * AROW + ((lq ^ ((l16 >> 1) & 3)) * 16));
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int n = min(n0 + wn0 + 16 * j + l16, p.HW - 1);
@@ -163,7 +165,8 @@ __global__ __launch_bounds__(512, UMAX <= 2 ? 4 : 2) void conv3x3_kernel(const P
 #pragma unroll
         for (int s = 0; s < 5; s++) {
             const int q = tid + s * 512;
-            if (q < MT * 36) *(u32x4 *)(smem + (q / 36) * AROW + (q % 36) * 16) = piece[s];
+            const int o = q / 36, part = q % 36;
+            if (q < MT * 36) *(u32x4 *)(smem + o * AROW + ((part & ~3) | ((part & 3) ^ ((o >> 1) & 3))) * 16) = piece[s];
         }
 #pragma unroll
         for (int s = 0; s < UMAX; s++) {
