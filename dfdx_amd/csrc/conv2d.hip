@@ -370,7 +370,23 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     const size_t patch_bytes = pointwise ? 0 : round256((size_t)(chunk * per_image) * sizeof(T));
     const size_t f_bytes = round256((size_t)f_elems * sizeof(T));
     const size_t img_bytes = padded ? round256((size_t)(chunk * op.chan_in * hp) * sizeof(T)) : 0;
-    if (int rc = ensure_patches(ctx, patch_bytes + 2 * f_bytes + 2 * img_bytes)) return rc;
+    // The image gradient of a 3 x 3, unit-stride, padding-1 convolution is such a convolution of grad_out (filters turned
+    // by 180 degrees, channels trading places): the 16-bit types run it on the kernel that reads its taps from a band of
+    // grad_out in LDS (conv3x3.hip) instead of the product with the patch matrix, which only the filter gradient needs then.
+    Conv3x3Problem band{};
+    bool use_band = false;
+    if (sizeof(T) == 2 && op.kernel == 3 && op.stride == 1 && op.padding == 1 && op.dilation == 1 && op.groups == 1 &&
+        op.h_out == op.h_in && op.w_out == op.w_in) {
+        band.dtype = dtype == DFDX_ROCM_F16 ? DT_F16 : DT_BF16;
+        band.chan_in = op.chan_out; band.chan_out = op.chan_in; band.h = op.h_in; band.w = op.w_in;
+        band.batch = (int)chunk;
+        band.img = grad_out; band.filters = filters; band.out = grad_img;
+        band.accumulate = 1; band.transposed_filters = 1;
+        band.wt = (void *)16;  // (placed below)
+        use_band = conv3x3_supported(band);
+    }
+    const size_t wt_bytes = use_band ? round256(conv3x3_filter_bytes(band)) : 0;
+    if (int rc = ensure_patches(ctx, patch_bytes + 2 * f_bytes + 2 * img_bytes + wt_bytes)) return rc;
     T *patches = (T *)ctx->patches;
     T *f_tr = (T *)((char *)ctx->patches + patch_bytes);
     T *grad_f_tr = (T *)((char *)ctx->patches + patch_bytes + f_bytes);
@@ -404,10 +420,17 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
             const unsigned g = (unsigned)((rows_p + 255) / 256);
             pad_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(img_b, img_p, (int)hw, (int)hp, rows_p);
             HIP_TRY(hipGetLastError());
-            pad_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(grad_img_b, grad_img_p, (int)hw, (int)hp, rows_p);
-            HIP_TRY(hipGetLastError());
+            if (!use_band) {
+                pad_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(grad_img_b, grad_img_p, (int)hw, (int)hp, rows_p);
+                HIP_TRY(hipGetLastError());
+            }
         }
-        {   // grad_img (B, G, C/G, H*W) += filters^T (G, C/G, O/G*K*K) . patches (B, G, O/G*K*K, H*W)
+        if (use_band) {
+            band.batch = (int)nb;
+            band.img = go; band.out = grad_img_b;
+            band.wt = (char *)ctx->patches + patch_bytes + 2 * f_bytes + 2 * img_bytes;
+            HIP_TRY(launch_conv3x3(band, ctx->stream));
+        } else {   // grad_img (B, G, C/G, H*W) += filters^T (G, C/G, O/G*K*K) . patches (B, G, O/G*K*K, H*W)
             const int64_t m = cg, k = og * kk, n = hp;
             dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
             d.accumulate = 1;
@@ -417,7 +440,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
             d.c = padded ? grad_img_p : grad_img_b; d.c_rs = n; d.c_cs = 1; d.c_b1 = op.chan_in * n; d.c_b2 = m * n;
             if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
         }
-        if (padded) {
+        if (padded && !use_band) {
             const int64_t total = nb * op.chan_in * hw;
             unpad_rows_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(grad_img_p, grad_img_b, (int)hw, (int)hp, total);
             HIP_TRY(hipGetLastError());

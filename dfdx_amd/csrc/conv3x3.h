@@ -9,8 +9,11 @@ struct Conv3x3Problem {
     int dtype;                 // DT_F16 / DT_BF16
     int batch, chan_in, chan_out, h, w;
     const void *img;           // [batch][chan_in][h][w]
-    const void *filters;       // [chan_out][chan_in][3][3]
+    const void *filters;       // [chan_out][chan_in][3][3]; `transposed_filters`: [chan_in][chan_out][3][3], applied turned
+                               // by 180 degrees (the image gradient of a convolution with these filters: img = its grad_out)
     void *out;                 // [batch][chan_out][h][w]
+    int accumulate = 0;        // out += ... instead of out = ...
+    int transposed_filters = 0;
     void *wt;                  // scratch for the filters as [chan_out][9][chan_in]: conv3x3_filter_bytes(), 16-byte aligned
 };
 

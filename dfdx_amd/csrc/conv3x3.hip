@@ -53,6 +53,7 @@ template <> struct Mma16<_Float16> {
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, h2));
     }
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
 };
 template <> struct Mma16<__bf16> {
     static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
@@ -62,6 +63,7 @@ template <> struct Mma16<__bf16> {
         typedef __bf16 b2 __attribute__((ext_vector_type(2)));
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, b2));
     }
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
 };
 
 struct Params {
@@ -74,16 +76,20 @@ struct Params {
     uint32_t magic_w, magic_pairs;  // ceil(2^32 / W), ceil(2^32 / (W / 2)): n / W = umulhi(n, magic_w) for n < 2^24
 };
 
-// wt[o][tap][c] = filters[o][c][tap]
-__global__ __launch_bounds__(256) void conv3x3_filters_kernel(const uint16_t *__restrict__ f, uint16_t *__restrict__ wt, int C, int total) {
+// wt[o][tap][c] = filters[o][c][tap] -- or, `transposed` (the image gradient: a convolution of grad_out with the filters
+// turned by 180 degrees, input and output channels trading places), wt[c][tap][o] = filters[o][c][8 - tap].
+// `inner` = the extent of wt's last axis, `outer` = that of its first.
+__global__ __launch_bounds__(256) void conv3x3_filters_kernel(const uint16_t *__restrict__ f, uint16_t *__restrict__ wt, int inner, int outer,
+                                                              int transposed, int total) {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
-    const int c = i % C, tap = (i / C) % 9, o = i / (9 * C);
-    wt[i] = f[((int64_t)o * C + c) * 9 + tap];
+    const int c = i % inner, tap = (i / inner) % 9, o = i / (9 * inner);
+    wt[i] = transposed ? f[((int64_t)c * outer + o) * 9 + (8 - tap)] : f[((int64_t)o * inner + c) * 9 + tap];
 }
 
 // UMAX: pixel-pair units of the band a thread may own per chunk (2: four waves per SIMD, 128 registers; 4: two)
-template <typename T, int UMAX>
+// ACC: the result is added to `out` (one rounding: old value and sum meet in f32).
+template <typename T, int UMAX, bool ACC>
 __global__ __launch_bounds__(512, UMAX <= 2 ? 4 : 2) void conv3x3_kernel(const Params p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t *const sin = smem + A_BYTES;
@@ -210,24 +216,42 @@ __global__ __launch_bounds__(512, UMAX <= 2 ? 4 : 2) void conv3x3_kernel(const P
     // ---- epilogue: lane holds channel o = l16 (per tile) and pixels 4 lq + 0..3 of each 16-pixel tile
     uint16_t *const obase = p.out + ((int64_t)b * p.O + (int64_t)mb * MT) * p.HW;
     if (p.HW % 8 == 0) {
-        // 16 bytes per lane: two neighbouring pixel tiles trade halves between the lane rows (v_permlane16_swap on the
-        // packed pairs), after which lane row lq holds pixels 8 (lq / 2) + 0..7 of tile 2 jp + (lq & 1); a store
-        // instruction then writes 64 contiguous bytes of each of 16 channel rows instead of 32
+        // 16 bytes per lane: two neighbouring pixel tiles trade halves between the lane rows (v_permlane16_swap), after
+        // which lane row lq holds pixels 8 (lq / 2) + 0..7 of tile 2 jp + (lq & 1); a store instruction then writes 64
+        // contiguous bytes of each of 16 channel rows instead of 32.  Overwriting, the packed pairs are traded (half as
+        // many instructions); accumulating, the f32 values, which then meet the old ones before the one rounding.
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             uint16_t *orow = obase + (int64_t)(wm0 + 16 * i + l16) * p.HW;
 #pragma unroll
             for (int jp = 0; jp < 2; jp++) {
-                u32x4 o;
-#pragma unroll
-                for (int h = 0; h < 2; h++) {
-                    const uint32_t lo = Mma16<T>::pack2(acc[i][2 * jp][2 * h], acc[i][2 * jp][2 * h + 1]);
-                    const uint32_t hi = Mma16<T>::pack2(acc[i][2 * jp + 1][2 * h], acc[i][2 * jp + 1][2 * h + 1]);
-                    const auto r = __builtin_amdgcn_permlane16_swap(lo, hi, false, false);
-                    o[h] = r[0];
-                    o[2 + h] = r[1];
-                }
                 const int n = n0 + wn0 + (2 * jp + (lq & 1)) * 16 + (lq >> 1) * 8;
+                u32x4 o;
+                if constexpr (ACC) {
+                    float v[8];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc[i][2 * jp][e]), __float_as_uint(acc[i][2 * jp + 1][e]), false, false);
+                        v[e] = __uint_as_float(r[0]);
+                        v[4 + e] = __uint_as_float(r[1]);
+                    }
+                    if (n < p.HW) {
+                        const u32x4 old = *(const u32x4 *)(orow + n);
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            o[e] = Mma16<T>::pack2(v[2 * e] + Mma16<T>::to_f32((uint16_t)(old[e] & 0xffffu)),
+                                                   v[2 * e + 1] + Mma16<T>::to_f32((uint16_t)(old[e] >> 16)));
+                    }
+                } else {
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const uint32_t lo = Mma16<T>::pack2(acc[i][2 * jp][2 * h], acc[i][2 * jp][2 * h + 1]);
+                        const uint32_t hi = Mma16<T>::pack2(acc[i][2 * jp + 1][2 * h], acc[i][2 * jp + 1][2 * h + 1]);
+                        const auto r = __builtin_amdgcn_permlane16_swap(lo, hi, false, false);
+                        o[h] = r[0];
+                        o[2 + h] = r[1];
+                    }
+                }
                 if (n < p.HW) *(u32x4 *)(orow + n) = o;
             }
         }
@@ -238,8 +262,17 @@ __global__ __launch_bounds__(512, UMAX <= 2 ? 4 : 2) void conv3x3_kernel(const P
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int n = n0 + wn0 + 16 * j + 4 * lq;
-                if (n < p.HW)  // HW % 4 == 0: all four pixels are in range
-                    *(u32x2 *)(orow + n) = u32x2{Mma16<T>::pack2(acc[i][j][0], acc[i][j][1]), Mma16<T>::pack2(acc[i][j][2], acc[i][j][3])};
+                if (n < p.HW) {  // HW % 4 == 0: all four pixels are in range
+                    float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+                    if constexpr (ACC) {
+                        const u32x2 old = *(const u32x2 *)(orow + n);
+                        v[0] += Mma16<T>::to_f32((uint16_t)(old[0] & 0xffffu));
+                        v[1] += Mma16<T>::to_f32((uint16_t)(old[0] >> 16));
+                        v[2] += Mma16<T>::to_f32((uint16_t)(old[1] & 0xffffu));
+                        v[3] += Mma16<T>::to_f32((uint16_t)(old[1] >> 16));
+                    }
+                    *(u32x2 *)(orow + n) = u32x2{Mma16<T>::pack2(v[0], v[1]), Mma16<T>::pack2(v[2], v[3])};
+                }
             }
         }
     }
@@ -265,7 +298,8 @@ size_t conv3x3_filter_bytes(const Conv3x3Problem &c) { return (size_t)c.chan_out
 hipError_t launch_conv3x3(const Conv3x3Problem &c, hipStream_t stream) {
     if (!conv3x3_supported(c)) return hipErrorNotSupported;
     const int total = c.chan_out * 9 * c.chan_in;
-    conv3x3_filters_kernel<<<(total + 255) / 256, 256, 0, stream>>>((const uint16_t *)c.filters, (uint16_t *)c.wt, c.chan_in, total);
+    conv3x3_filters_kernel<<<(total + 255) / 256, 256, 0, stream>>>((const uint16_t *)c.filters, (uint16_t *)c.wt, c.chan_in, c.chan_out,
+                                                                   c.transposed_filters ? 1 : 0, total);
     Params p;
     p.img = (const uint16_t *)c.img; p.wt = (const uint16_t *)c.wt; p.out = (uint16_t *)c.out;
     p.C = c.chan_in; p.O = c.chan_out; p.H = c.h; p.W = c.w; p.HW = c.h * c.w;
@@ -276,24 +310,30 @@ hipError_t launch_conv3x3(const Conv3x3Problem &c, hipStream_t stream) {
     p.magic_pairs = (uint32_t)(((1ull << 32) + c.w / 2 - 1) / (c.w / 2));
     const dim3 grid((unsigned)p.mblocks, (unsigned)p.nblocks, (unsigned)c.batch);
     const bool few = 4 * p.band_rows * (c.w / 2) <= 2 * 512;
-#define DFDX_CONV3(T, U)                                                                                               \
+#define DFDX_CONV3(T, U, A)                                                                                            \
     do {                                                                                                               \
         static PerDevice attr_on;                                                                                      \
         std::atomic<int> &known = attr_on.here();                                                                      \
         if (known.load(std::memory_order_acquire) == 0) {                                                              \
-            hipError_t e = hipFuncSetAttribute((const void *)conv3x3_kernel<T, U>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            hipError_t e = hipFuncSetAttribute((const void *)conv3x3_kernel<T, U, A>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
             if (e != hipSuccess) return e;                                                                             \
             known.store(1, std::memory_order_release);                                                                 \
         }                                                                                                              \
-        conv3x3_kernel<T, U><<<grid, 512, lds, stream>>>(p);                                                           \
+        conv3x3_kernel<T, U, A><<<grid, 512, lds, stream>>>(p);                                                        \
+    } while (0)
+#define DFDX_CONV3_U(T, A)            \
+    do {                              \
+        if (few) DFDX_CONV3(T, 2, A); \
+        else DFDX_CONV3(T, 4, A);     \
     } while (0)
     if (c.dtype == DT_F16) {
-        if (few) DFDX_CONV3(_Float16, 2);
-        else DFDX_CONV3(_Float16, 4);
+        if (c.accumulate) DFDX_CONV3_U(_Float16, true);
+        else DFDX_CONV3_U(_Float16, false);
     } else {
-        if (few) DFDX_CONV3(__bf16, 2);
-        else DFDX_CONV3(__bf16, 4);
+        if (c.accumulate) DFDX_CONV3_U(__bf16, true);
+        else DFDX_CONV3_U(__bf16, false);
     }
+#undef DFDX_CONV3_U
 #undef DFDX_CONV3
     return hipGetLastError();
 }

@@ -68,6 +68,8 @@ CONFIGS = [
     (3, 32, 64, 24, 40, 5, 1, 2, 2, 1),
     (2, 3, 64, 32, 32, 3, 1, 1, 1, 1),     # a first layer: C*K*K = 27, a contraction no 16-byte load can walk (window loads)
     (2, 3, 64, 30, 30, 3, 2, 1, 1, 1),     # the same through the patch matrix (stride 2), 15 x 15 = 225 output pixels
+    (3, 128, 96, 20, 14, 3, 1, 1, 1, 1),   # image gradient on the band kernel (two blocks of 64 channels out of 3 chunks of 32), forward on the tiles
+    (2, 64, 32, 9, 112, 3, 1, 1, 1, 1),    # the same with one chunk, rows of 112 pixels; H * W = 1008 is off the 64-element grid of the filter gradient
 ]
 
 
