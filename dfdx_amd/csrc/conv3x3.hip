@@ -195,22 +195,37 @@ __global__ __launch_bounds__(512, UMAX <= 2 ? 4 : 2) void conv3x3_kernel(const P
         deposit();
         __syncthreads();
         if (c0 + CK < p.C) request(c0 + CK);  // the next chunk travels while this one is multiplied
-        // ---- 9 taps x (2 x 4) MFMAs; operands swapped so that a lane ends up with 4 consecutive pixels of one channel
+        // ---- 9 taps x (2 x 4) MFMAs; operands swapped so that a lane ends up with 4 consecutive pixels of one channel.
+        // Eighteen half taps (two pixel tiles each) in a software pipeline: the fragments of half tap h + 1 are requested
+        // from LDS in front of the four MFMAs of half tap h, into the other register set.
+        // (a wave whose 64 pixels all lie past the end of the image -- the last pixel block of an image -- has nothing to multiply)
+        if (n0 + wn0 < p.HW) {
+            u32x4 fa[2], fb[2][2];
+            auto read_a = [&](int tap) {
 #pragma unroll
-        for (int ky = 0; ky < 3; ky++)
+                for (int i = 0; i < 2; i++) fa[i] = *(const u32x4 *)(smem + a_addr[i] + tap * 64);
+            };
+            auto read_b = [&](int tap, int jh, u32x4(&dst)[2]) {
+                const uint32_t shift = (uint32_t)(((tap / 3) * WP + tap % 3) * PIX);
 #pragma unroll
-            for (int kx = 0; kx < 3; kx++) {
-                const uint32_t shift = (uint32_t)((ky * WP + kx) * PIX);
-                u32x4 fa[2], fb[4];
+                for (int j = 0; j < 2; j++) dst[j] = *(const u32x4 *)(smem + b_addr[jh + j] + shift);
+            };
+            read_a(0);
+            read_b(0, 0, fb[0]);
 #pragma unroll
-                for (int i = 0; i < 2; i++) fa[i] = *(const u32x4 *)(smem + a_addr[i] + (ky * 3 + kx) * 64);
+            for (int h = 0; h < 18; h++) {
+                const int tap = h / 2, jh = (h % 2) * 2;
+                if (h + 1 < 18) read_b((h + 1) / 2, ((h + 1) % 2) * 2, fb[(h + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = 0; j < 4; j++) fb[j] = *(const u32x4 *)(smem + b_addr[j] + shift);
+                for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-#pragma unroll
-                    for (int i = 0; i < 2; i++) acc[i][j] = Mma16<T>::mfma(fb[j], fa[i], acc[i][j]);
+                    for (int i = 0; i < 2; i++) acc[i][jh + j] = Mma16<T>::mfma(fb[h & 1][j], fa[i], acc[i][jh + j]);
+                __builtin_amdgcn_sched_barrier(0);
+                // (the filter fragments have one register set: the next tap's are requested behind this tap's last MFMAs)
+                if (jh == 2 && tap + 1 < 9) read_a(tap + 1);
             }
+        }
     }
 
     // ---- epilogue: lane holds channel o = l16 (per tile) and pixels 4 lq + 0..3 of each 16-pixel tile
