@@ -386,6 +386,24 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         use_band = conv3x3_supported(band);
     }
     const size_t wt_bytes = use_band ? round256(conv3x3_filter_bytes(band)) : 0;
+    // The filter gradient of such a convolution has its own kernel too (conv3x3_wgrad.hip: both operands pixel-major in
+    // LDS, fragments through transposing reads).  With both in place the backward pass forms no patch matrix at all.
+    Conv3x3Problem wgrad{};
+    bool use_wgrad = false;
+    if (use_band) {
+        wgrad.dtype = band.dtype;
+        wgrad.batch = op.batch; wgrad.chan_in = op.chan_in; wgrad.chan_out = op.chan_out; wgrad.h = op.h_in; wgrad.w = op.w_in;
+        wgrad.img = img; wgrad.out = const_cast<void *>(grad_out); wgrad.filters = grad_filters;
+        use_wgrad = conv3x3_wgrad_supported(wgrad, ctx->compute_units);
+    }
+    if (use_band && use_wgrad) {
+        const size_t ws_bytes = round256(conv3x3_wgrad_workspace_bytes(wgrad, ctx->compute_units));
+        if (int rc = ensure_patches(ctx, ws_bytes + wt_bytes)) return rc;
+        band.batch = op.batch;
+        band.wt = (char *)ctx->patches + ws_bytes;
+        HIP_TRY(launch_conv3x3(band, ctx->stream));
+        return (int)launch_conv3x3_wgrad(wgrad, ctx->compute_units, ctx->patches, ctx->stream);
+    }
     if (int rc = ensure_patches(ctx, patch_bytes + 2 * f_bytes + 2 * img_bytes + wt_bytes)) return rc;
     T *patches = (T *)ctx->patches;
     T *f_tr = (T *)((char *)ctx->patches + patch_bytes);

@@ -22,4 +22,11 @@ size_t conv3x3_filter_bytes(const Conv3x3Problem &c);
 // hipErrorNotSupported when the shape does not fit (the caller then takes another path)
 hipError_t launch_conv3x3(const Conv3x3Problem &c, hipStream_t stream);
 
+// The filter gradient of the same convolution without a patch matrix (conv3x3_wgrad.hip).  `c` as above with `out` =
+// grad_out [batch][chan_out][h][w] and `filters` = grad_filters, which is accumulated into; `workspace`: f32 shares of the
+// sums, conv3x3_wgrad_workspace_bytes(), 16-byte aligned.
+bool conv3x3_wgrad_supported(const Conv3x3Problem &c, int compute_units);
+size_t conv3x3_wgrad_workspace_bytes(const Conv3x3Problem &c, int compute_units);
+hipError_t launch_conv3x3_wgrad(const Conv3x3Problem &c, int compute_units, void *workspace, hipStream_t stream);
+
 }  // namespace dfdx_rocm

@@ -1,0 +1,282 @@
+// Filter gradient of a 3 x 3 convolution at unit stride with padding 1 (f16 / bf16, f32 accumulate, gfx950) without a patch
+// matrix: the `weight_g^T += img * unfold(grad_out)^T` product of `Conv2DKernel::backward` (dfdx-core/src/tensor_ops/
+// conv2d/cpu_kernel.rs:152-170) for the shapes the band kernel of conv3x3.hip takes.
+//
+//   grad_filters[o][c][ky][kx] += sum over (b, y, x) of  grad_out[b][o][y][x] * img[b][c][y + ky - 1][x + kx - 1]
+//
+// as nine GEMMs (one per tap) with M = output channels, N = input channels and K = pixels.  Both operands are kept in LDS
+// pixel-major -- a record per pixel with its 64 channels next to each other, rows of W + 2 records whose first and last are
+// zeros (the padding columns) -- exactly as the band kernel keeps the image; the MFMA fragments (8 consecutive pixels of
+// one channel per lane) come out of them through the transposing LDS read ds_read_b64_tr_b16.  In that padded pixel
+// numbering a tap is ONE shift of the image band against the grad_out band, (ky - 1) (W + 2) + (kx - 1) records, for every
+// pixel; the zero columns and rows take care of the borders.
+//
+// A workgroup (12 waves) owns one block of 64 output x 64 input channels and walks a share of the (image, band of rows)
+// work items, all 9 x 64 x 64 sums staying in its accumulators (wave w: the three (tap, 16-channel tile) pairs 3w .. 3w + 2
+// times the four 16-row tiles of output channels: 12 MFMAs per 32 pixels against 4 + 3 fragments).  At the end every
+// workgroup leaves its sums as f32 in a workspace and a second kernel adds the shares in a fixed order into grad_filters
+// (one rounding): deterministic.
+#include "gemm_internal.h"
+#include "conv3x3.h"
+#include <algorithm>
+
+namespace dfdx_rocm {
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short v4i16 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+#define DFDX_LDS __attribute__((address_space(3)))
+
+constexpr int NTH = 768;    // 12 waves
+constexpr int REC = 160;    // bytes of a pixel record: 64 channels + 32 of padding (an odd multiple of 32 bytes)
+constexpr int KMAX = 256;   // records of a grad_out band at most (a multiple of the 32-pixel k step)
+constexpr int UMAX = 2;     // pixel-pair units of a band a thread may own
+
+template <typename T> struct MmaW;
+template <> struct MmaW<_Float16> {
+    static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
+    static __device__ __forceinline__ uint16_t from_f32(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+};
+template <> struct MmaW<__bf16> {
+    static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
+    static __device__ __forceinline__ uint16_t from_f32(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
+};
+
+struct Params {
+    const uint16_t *img;  // [B][C][H][W]
+    const uint16_t *go;   // [B][O][H][W]
+    float *partial;       // [slices][combos][9][64][64]
+    int C, O, H, W, HW;
+    int R, bands;          // rows per band, bands per image
+    int items;             // batch x bands
+    int slices, cblocks;   // workgroups per channel-block pair; blocks of 64 input channels
+    int kp;                // records of the grad_out band, rounded up to the k step
+    int xrecs;             // records of the image band that are ever read (zeroed once)
+    uint32_t magic_pairs;  // ceil(2^32 / (W / 2))
+};
+
+// Fragment of an operand stored [pixel record][channel]: 16 channels (from `chan0`) x 32 pixels (from record `rec0`).
+// Lane 16 g + L supplies the addresses of 4 channels of record rec0 + 8 g + L / 4 (and of the record 4 further); the
+// hardware hands lane L the 8 pixels of channel chan0 + L: the layout the MFMA wants for 8 consecutive k.
+__device__ __forceinline__ u32x4 tr_fragment(const uint8_t *band, int rec0, int chan0, int l16, int lq) {
+    const uint8_t *p = band + (rec0 + lq * 8 + l16 / 4) * REC + (chan0 + 4 * (l16 % 4)) * 2;
+    const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DFDX_LDS v4i16 *)(DFDX_LDS uint8_t *)p);
+    const v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DFDX_LDS v4i16 *)(DFDX_LDS uint8_t *)(p + 4 * REC));
+    const u32x2 l = __builtin_bit_cast(u32x2, lo), h = __builtin_bit_cast(u32x2, hi);
+    return u32x4{l[0], l[1], h[0], h[1]};
+}
+
+template <typename T>
+__global__ __launch_bounds__(NTH, 3) void conv3x3_wgrad_kernel(const Params p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t *const gband = smem;                    // grad_out band: kp records
+    uint8_t *const xband = smem + KMAX * REC;       // image band: xrecs records, its row 0 = the row above the band
+    const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int l16 = lane % 16, lq = lane / 16;
+    const int W = p.W, WP = W + 2, H = p.H, pairs = W / 2;
+
+    // everything the deposits never write stays zero for the whole launch: padding columns, the records behind the
+    // last band row that the k steps and the tap shifts still touch
+    for (int i = tid; i < (KMAX + p.xrecs) * (REC / 16); i += NTH) *(u32x4 *)(smem + i * 16) = u32x4{0, 0, 0, 0};
+
+    const int combos = gridDim.x / p.slices;
+    const int combo = blockIdx.x % combos, slice = blockIdx.x / combos;
+    const int cb = combo % p.cblocks, ob = combo / p.cblocks;
+
+    f32x4 acc[4][3];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int e = 0; e < 3; e++) acc[i][e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // the wave's three (tap, input-channel tile) pairs: pair q = tap * 4 + tile
+    int b_rec[3], b_chan[3];
+#pragma unroll
+    for (int e = 0; e < 3; e++) {
+        const int q = wave * 3 + e, tap = q / 4, j = q % 4;
+        b_rec[e] = WP + (tap / 3 - 1) * WP + (tap % 3 - 1);  // image record that meets grad_out record 0 at this tap
+        b_chan[e] = 16 * j;
+    }
+
+    // ---- what a thread moves per work item: UMAX pixel-pair units of each band (8 channels x 2 neighbouring pixels)
+    const int x_rows = p.R + 2, g_rows = p.R;
+    const int x_units = 8 * x_rows * pairs, g_units = 8 * g_rows * pairs;
+    int xs_off[UMAX], xs_row[UMAX], xs_dst[UMAX], gs_off[UMAX], gs_row[UMAX], gs_dst[UMAX];
+#pragma unroll
+    for (int s = 0; s < UMAX; s++) {
+        const int u = tid + s * NTH;
+        const int t = (int)__umulhi((uint32_t)u, p.magic_pairs), xp = u - t * pairs;  // t = group * rows + row
+        {
+            const int cg = t / x_rows, r = t - cg * x_rows;
+            xs_row[s] = u < x_units ? r : -1000000;
+            xs_off[s] = (8 * cg * H) * W + 2 * xp;  // + row * W: element offset of the unit's first channel in its block
+            xs_dst[s] = (r * WP + 1 + 2 * xp) * REC + cg * 16;
+        }
+        {
+            const int cg = t / g_rows, r = t - cg * g_rows;
+            gs_row[s] = u < g_units ? r : -1000000;
+            gs_off[s] = (8 * cg * H) * W + 2 * xp;
+            gs_dst[s] = (r * WP + 1 + 2 * xp) * REC + cg * 16;
+        }
+    }
+    __syncthreads();
+
+    for (int item = slice; item < p.items; item += p.slices) {
+        const int b = item / p.bands, y0 = (item - b * p.bands) * p.R;
+        const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.img + ((int64_t)b * p.C + cb * 64) * p.HW), 0, 64 * p.HW * 2, 0x00020000);
+        const __amdgpu_buffer_rsrc_t gsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.go + ((int64_t)b * p.O + ob * 64) * p.HW), 0, 64 * p.HW * 2, 0x00020000);
+        uint32_t dx[UMAX][8], dg[UMAX][8];
+#pragma unroll
+        for (int s = 0; s < UMAX; s++) {
+            const int yx = y0 - 1 + xs_row[s], yg = y0 + gs_row[s];
+            const uint32_t ox = (xs_row[s] >= 0 && yx >= 0 && yx < H) ? (uint32_t)(xs_off[s] + yx * W) * 2u : 0xFFFFFFF0u;
+            const uint32_t og = (gs_row[s] >= 0 && yg < H) ? (uint32_t)(gs_off[s] + yg * W) * 2u : 0xFFFFFFF0u;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                dx[s][e] = __builtin_amdgcn_raw_buffer_load_b32(xsrc, (int)ox, e * p.HW * 2, 0);
+                dg[s][e] = __builtin_amdgcn_raw_buffer_load_b32(gsrc, (int)og, e * p.HW * 2, 0);
+            }
+        }
+        __syncthreads();  // the previous item's fragments have been read
+#pragma unroll
+        for (int s = 0; s < UMAX; s++) {
+            u32x4 a0, a1, g0, g1;
+#pragma unroll
+            for (int h = 0; h < 4; h++) {
+                a0[h] = __builtin_amdgcn_perm(dx[s][2 * h + 1], dx[s][2 * h], 0x05040100u);  // low halves: pixel 2 xp
+                a1[h] = __builtin_amdgcn_perm(dx[s][2 * h + 1], dx[s][2 * h], 0x07060302u);  // high halves: pixel 2 xp + 1
+                g0[h] = __builtin_amdgcn_perm(dg[s][2 * h + 1], dg[s][2 * h], 0x05040100u);
+                g1[h] = __builtin_amdgcn_perm(dg[s][2 * h + 1], dg[s][2 * h], 0x07060302u);
+            }
+            if (xs_row[s] >= 0) {
+                *(u32x4 *)(xband + xs_dst[s]) = a0;
+                *(u32x4 *)(xband + xs_dst[s] + REC) = a1;
+            }
+            if (gs_row[s] >= 0) {
+                *(u32x4 *)(gband + gs_dst[s]) = g0;
+                *(u32x4 *)(gband + gs_dst[s] + REC) = g1;
+            }
+        }
+        __syncthreads();
+        for (int k0 = 0; k0 < p.kp; k0 += 32) {
+            u32x4 fa[4], fb[3];
+#pragma unroll
+            for (int i = 0; i < 4; i++) fa[i] = tr_fragment(gband, k0, 16 * i, l16, lq);
+#pragma unroll
+            for (int e = 0; e < 3; e++) fb[e] = tr_fragment(xband, k0 + b_rec[e], b_chan[e], l16, lq);
+#pragma unroll
+            for (int e = 0; e < 3; e++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[i][e] = MmaW<T>::mfma(fb[e], fa[i], acc[i][e]);
+        }
+    }
+
+    // ---- this workgroup's share of the sums: lane holds output channel 16 i + l16 and input channels 16 j + 4 lq + 0..3
+    float *const share = p.partial + ((int64_t)slice * combos + combo) * (9 * 64 * 64);
+#pragma unroll
+    for (int e = 0; e < 3; e++) {
+        const int q = wave * 3 + e, tap = q / 4, j = q % 4;
+#pragma unroll
+        for (int i = 0; i < 4; i++) *(f32x4 *)(share + (tap * 64 + 16 * i + l16) * 64 + 16 * j + 4 * lq) = acc[i][e];
+    }
+}
+
+// grad_filters[o][c][tap] += sum over the slices, in slice order, of their shares (f32), rounded once
+template <typename T>
+__global__ __launch_bounds__(256) void conv3x3_wgrad_reduce_kernel(const float *__restrict__ partial, uint16_t *__restrict__ grad_filters, int C,
+                                                                   int cblocks, int combos, int slices, int total) {
+    const int i = blockIdx.x * 256 + threadIdx.x;  // (combo, tap, o, c), c fastest
+    if (i >= total) return;
+    const int c = i % 64, o = (i / 64) % 64, tap = (i / 4096) % 9, combo = i / (9 * 4096);
+    float sum = 0.0f;
+    for (int s = 0; s < slices; s++) sum += partial[((int64_t)s * combos + combo) * (9 * 4096) + (tap * 64 + o) * 64 + c];
+    const int cb = combo % cblocks, ob = combo / cblocks;
+    uint16_t *dst = grad_filters + ((int64_t)(ob * 64 + o) * C + cb * 64 + c) * 9 + tap;
+    *dst = MmaW<T>::from_f32(MmaW<T>::to_f32(*dst) + sum);
+}
+
+struct Plan {
+    int R, bands, kp, xrecs, slices, combos;
+    size_t lds;
+};
+bool make_plan(const Conv3x3Problem &c, int compute_units, Plan *out) {
+    if (c.dtype != DT_F16 && c.dtype != DT_BF16) return false;
+    if (c.batch < 1 || c.chan_in < 64 || c.chan_in % 64 || c.chan_out < 64 || c.chan_out % 64) return false;
+    if (c.w < 4 || c.w > 254 || c.w % 2 || c.h < 1) return false;
+    const int64_t hw = (int64_t)c.h * c.w;
+    if (hw >= (1 << 24) || 64 * hw >= (1ll << 30)) return false;
+    if (((uintptr_t)c.img & 3u) || ((uintptr_t)c.out & 3u) || ((uintptr_t)c.filters & 1u)) return false;
+    const int wp = c.w + 2;
+    Plan pl;
+    pl.R = std::min(c.h, KMAX / wp);
+    if (pl.R < 1) return false;
+    pl.bands = (c.h + pl.R - 1) / pl.R;
+    pl.kp = (pl.R * wp + 31) / 32 * 32;
+    pl.xrecs = pl.kp + 2 * wp + 8;  // the last k step under the largest tap shift
+    if (8 * (pl.R + 2) * (c.w / 2) > UMAX * NTH) return false;
+    pl.lds = (size_t)(KMAX + pl.xrecs) * REC;
+    if (pl.lds > 160 * 1024) return false;
+    pl.combos = (c.chan_in / 64) * (c.chan_out / 64);
+    const int64_t items = (int64_t)c.batch * pl.bands;
+    if (items >= (1ll << 31) || pl.combos > 65536) return false;
+    pl.slices = (int)std::max<int64_t>(1, std::min<int64_t>(items, std::max(1, compute_units) / pl.combos));
+    *out = pl;
+    return true;
+}
+
+}  // namespace
+
+// `c` as for the forward kernel, with `out` = grad_out [batch][chan_out][h][w] and `filters` = grad_filters (accumulated into).
+bool conv3x3_wgrad_supported(const Conv3x3Problem &c, int compute_units) {
+    Plan pl;
+    return make_plan(c, compute_units, &pl);
+}
+
+size_t conv3x3_wgrad_workspace_bytes(const Conv3x3Problem &c, int compute_units) {
+    Plan pl;
+    if (!make_plan(c, compute_units, &pl)) return 0;
+    return (size_t)pl.slices * pl.combos * 9 * 64 * 64 * sizeof(float);
+}
+
+hipError_t launch_conv3x3_wgrad(const Conv3x3Problem &c, int compute_units, void *workspace, hipStream_t stream) {
+    Plan pl;
+    if (!make_plan(c, compute_units, &pl) || ((uintptr_t)workspace & 15u)) return hipErrorNotSupported;
+    Params p;
+    p.img = (const uint16_t *)c.img; p.go = (const uint16_t *)c.out; p.partial = (float *)workspace;
+    p.C = c.chan_in; p.O = c.chan_out; p.H = c.h; p.W = c.w; p.HW = c.h * c.w;
+    p.R = pl.R; p.bands = pl.bands; p.items = c.batch * pl.bands;
+    p.slices = pl.slices; p.cblocks = c.chan_in / 64;
+    p.kp = pl.kp; p.xrecs = pl.xrecs;
+    p.magic_pairs = (uint32_t)(((1ull << 32) + c.w / 2 - 1) / (c.w / 2));
+    const unsigned grid = (unsigned)(pl.combos * pl.slices);
+#define DFDX_WGRAD(T)                                                                                                  \
+    do {                                                                                                               \
+        static PerDevice attr_on;                                                                                      \
+        std::atomic<int> &known = attr_on.here();                                                                      \
+        if (known.load(std::memory_order_acquire) == 0) {                                                              \
+            hipError_t e = hipFuncSetAttribute((const void *)conv3x3_wgrad_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            if (e != hipSuccess) return e;                                                                             \
+            known.store(1, std::memory_order_release);                                                                 \
+        }                                                                                                              \
+        conv3x3_wgrad_kernel<T><<<grid, NTH, pl.lds, stream>>>(p);                                                     \
+        const int total = pl.combos * 9 * 4096;                                                                        \
+        conv3x3_wgrad_reduce_kernel<T><<<(total + 255) / 256, 256, 0, stream>>>((const float *)workspace, (uint16_t *)c.filters, c.chan_in, \
+                                                                               p.cblocks, pl.combos, pl.slices, total); \
+    } while (0)
+    if (c.dtype == DT_F16) DFDX_WGRAD(_Float16);
+    else DFDX_WGRAD(__bf16);
+#undef DFDX_WGRAD
+    return hipGetLastError();
+}
+
+}  // namespace dfdx_rocm
