@@ -151,6 +151,62 @@ def test_conv2d_3x3_band_kernel_zero_padding_is_exact():
     np.testing.assert_array_equal(got, np.broadcast_to(want, got.shape))
 
 
+# Backward of the same family with whole blocks of 64 input and output channels and rows of at most 64 pixels: neither
+# gradient goes through a patch matrix (image gradient: the band kernel with the filters turned; filter gradient:
+# conv3x3_wgrad.hip).  Shapes: several channel blocks on either side, bands that end below the image (H not a multiple of
+# the rows per band), a grad_out band of exactly 256 records (62-pixel rows), one row per image, more work items than
+# workgroups and fewer.
+WGRAD_CONFIGS = [(2, 128, 64, 20, 14), (3, 64, 128, 9, 30), (1, 64, 64, 5, 62), (2, 64, 64, 1, 40), (70, 64, 64, 8, 8),
+                 (2, 128, 128, 33, 12)]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("cfg", WGRAD_CONFIGS, ids=lambda c: "x".join(map(str, c)))
+def test_conv2d_3x3_backward_without_patch_matrix(cfg, dtype):
+    dev, g = device(), rng(505)
+    batch, cin, cout, h, w_ = cfg
+    announce("conv2d 3x3 backward, no patch matrix", cfg, dtype)
+    op = Conv2DOp.make(batch, cin, cout, h, w_, 3, 1, 1, 1, 1)
+    x = upload(dev, g.standard_normal((batch, cin, h, w_)), dtype)
+    w = upload(dev, g.standard_normal((cout, cin, 3, 3)) / np.sqrt(cin * 9), dtype)
+    go = upload(dev, g.standard_normal((batch, cout, h, w_)), dtype)
+    gx0, gw0 = upload(dev, g.standard_normal(x.shape), dtype), upload(dev, g.standard_normal(w.shape), dtype)
+    outs = []
+    for _ in range(2):   # twice: the same bits (the shares of the filter gradient are added in a fixed order)
+        gx, gw = dev.tensor(dev.to_host(gx0), dtype), dev.tensor(dev.to_host(gw0), dtype)
+        dev.conv2d_backward(x, gx, w, gw, go, stride=1, padding=1)
+        outs.append((dev.to_host(gx), dev.to_host(gw)))
+    np.testing.assert_array_equal(outs[0][0], outs[1][0])
+    np.testing.assert_array_equal(outs[0][1], outs[1][1])
+    x_h, w_h, go_h = dev.to_host(x).reshape(-1), dev.to_host(w).reshape(-1), dev.to_host(go).reshape(-1)
+    ogx, ogw = dev.to_host(gx0).reshape(-1).copy(), dev.to_host(gw0).reshape(-1).copy()
+    conv2d_backward(dtype, op, x_h, ogx, w_h, ogw, go_h)
+    X, W, GO = oracle.to_f64(x_h, dtype), oracle.to_f64(w_h, dtype), oracle.to_f64(go_h, dtype)
+    wgx, wgw = oracle.to_f64(ogx, dtype), oracle.to_f64(ogw, dtype)
+    assert_within(dtype, cout * 9, oracle.to_f64(outs[0][0], dtype).reshape(-1), wgx, GO, W,
+                  extra=2 * ULP[dtype] * float(np.abs(wgx).max()), what="grad_img")
+    # the restatement rounds the filter gradient to the element type after every image, the device once
+    assert_within(dtype, batch * h * w_, oracle.to_f64(outs[0][1], dtype).reshape(-1), wgw, GO, X,
+                  extra=(batch + 2) * ULP[dtype] * float(np.abs(wgw).max()), what="grad_filters")
+
+
+def test_conv2d_3x3_filter_gradient_counts_pixels_exactly():
+    """Images and output gradients of ones: the gradient of filter tap (ky, kx) is batch x the number of pixels whose
+    neighbour at that tap lies inside the image -- (H - |ky - 1|) (W - |kx - 1|) -- exactly, for every channel pair."""
+    dev = device()
+    batch, cin, cout, h, w_ = 3, 64, 64, 11, 10
+    announce("conv2d 3x3 filter gradient, ones", batch, cin, cout, h, w_)
+    x = upload(dev, np.ones((batch, cin, h, w_)), "f16")
+    w = upload(dev, np.zeros((cout, cin, 3, 3)), "f16")
+    go = upload(dev, np.ones((batch, cout, h, w_)), "f16")
+    gx, gw = dev.zeros("f16", x.shape), dev.zeros("f16", w.shape)
+    dev.conv2d_backward(x, gx, w, gw, go, stride=1, padding=1)
+    got = host(dev, gw)
+    want = np.array([[batch * (h - abs(ky - 1)) * (w_ - abs(kx - 1)) for kx in range(3)] for ky in range(3)], dtype=np.float64)
+    np.testing.assert_array_equal(got, np.broadcast_to(want, got.shape))
+    np.testing.assert_array_equal(host(dev, gx), 0.0)   # zero filters: no image gradient
+
+
 def test_conv2d_unbatched_equals_batch_of_one():
     dev, g = device(), rng(502)
     announce("conv2d unbatched")
