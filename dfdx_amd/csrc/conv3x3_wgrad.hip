@@ -131,14 +131,15 @@ __global__ __launch_bounds__(NTH, 3) void conv3x3_wgrad_kernel(const Params p) {
     }
     __syncthreads();
 
-    for (int item = slice; item < p.items; item += p.slices) {
+    uint32_t dx[UMAX][8], dg[UMAX][8];
+    auto request = [&](int item) {  // the global loads of one work item: 8 channels x 2 pixels per unit and band
         const int b = item / p.bands, y0 = (item - b * p.bands) * p.R;
         const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.img + ((int64_t)b * p.C + cb * 64) * p.HW), 0, 64 * p.HW * 2, 0x00020000);
         const __amdgpu_buffer_rsrc_t gsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.go + ((int64_t)b * p.O + ob * 64) * p.HW), 0, 64 * p.HW * 2, 0x00020000);
-        uint32_t dx[UMAX][8], dg[UMAX][8];
 #pragma unroll
         for (int s = 0; s < UMAX; s++) {
             const int yx = y0 - 1 + xs_row[s], yg = y0 + gs_row[s];
+            // (a unit outside the image, or none at all, points past the end of the resource and receives zeros)
             const uint32_t ox = (xs_row[s] >= 0 && yx >= 0 && yx < H) ? (uint32_t)(xs_off[s] + yx * W) * 2u : 0xFFFFFFF0u;
             const uint32_t og = (gs_row[s] >= 0 && yg < H) ? (uint32_t)(gs_off[s] + yg * W) * 2u : 0xFFFFFFF0u;
 #pragma unroll
@@ -147,6 +148,9 @@ __global__ __launch_bounds__(NTH, 3) void conv3x3_wgrad_kernel(const Params p) {
                 dg[s][e] = __builtin_amdgcn_raw_buffer_load_b32(gsrc, (int)og, e * p.HW * 2, 0);
             }
         }
+    };
+    if (slice < p.items) request(slice);
+    for (int item = slice; item < p.items; item += p.slices) {
         __syncthreads();  // the previous item's fragments have been read
 #pragma unroll
         for (int s = 0; s < UMAX; s++) {
@@ -168,6 +172,7 @@ __global__ __launch_bounds__(NTH, 3) void conv3x3_wgrad_kernel(const Params p) {
             }
         }
         __syncthreads();
+        if (item + p.slices < p.items) request(item + p.slices);  // the next item travels while this one is multiplied
         for (int k0 = 0; k0 < p.kp; k0 += 32) {
             u32x4 fa[4], fb[3];
 #pragma unroll
@@ -191,18 +196,40 @@ __global__ __launch_bounds__(NTH, 3) void conv3x3_wgrad_kernel(const Params p) {
     }
 }
 
-// grad_filters[o][c][tap] += sum over the slices, in slice order, of their shares (f32), rounded once
+// grad_filters[o][c][tap] += sum over the slices of their shares (f32), rounded once.  A workgroup owns 32 consecutive sums;
+// its 8 thread groups add an eighth of the slices each, in slice order, and the eight subtotals meet in LDS in group order:
+// one fixed summation order, whatever the timing.
 template <typename T>
 __global__ __launch_bounds__(256) void conv3x3_wgrad_reduce_kernel(const float *__restrict__ partial, uint16_t *__restrict__ grad_filters, int C,
                                                                    int cblocks, int combos, int slices, int total) {
-    const int i = blockIdx.x * 256 + threadIdx.x;  // (combo, tap, o, c), c fastest
-    if (i >= total) return;
-    const int c = i % 64, o = (i / 64) % 64, tap = (i / 4096) % 9, combo = i / (9 * 4096);
+    __shared__ float subtotal[8][32];
+    const int lane_elem = threadIdx.x % 32, group = threadIdx.x / 32;
+    const int i = blockIdx.x * 32 + lane_elem;  // (combo, tap, o, c), c fastest; total is a multiple of 32
+    const int combo = i / (9 * 4096), within = i - combo * (9 * 4096);
+    const int per = (slices + 7) / 8, s0 = group * per, s1 = min(slices, s0 + per);
+    const float *src = partial + (int64_t)combo * (9 * 4096) + within;
+    const int64_t step = (int64_t)combos * (9 * 4096);
     float sum = 0.0f;
-    for (int s = 0; s < slices; s++) sum += partial[((int64_t)s * combos + combo) * (9 * 4096) + (tap * 64 + o) * 64 + c];
-    const int cb = combo % cblocks, ob = combo / cblocks;
-    uint16_t *dst = grad_filters + ((int64_t)(ob * 64 + o) * C + cb * 64 + c) * 9 + tap;
-    *dst = MmaW<T>::from_f32(MmaW<T>::to_f32(*dst) + sum);
+    int s = s0;
+    for (; s + 8 <= s1; s += 8) {
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = src[(s + e) * step];
+#pragma unroll
+        for (int e = 0; e < 8; e++) sum += v[e];
+    }
+    for (; s < s1; s++) sum += src[s * step];
+    subtotal[group][lane_elem] = sum;
+    __syncthreads();
+    if (group == 0 && i < total) {
+        float all = subtotal[0][lane_elem];
+#pragma unroll
+        for (int g = 1; g < 8; g++) all += subtotal[g][lane_elem];
+        const int c = within % 64, o = (within / 64) % 64, tap = within / 4096;
+        const int cb = combo % cblocks, ob = combo / cblocks;
+        uint16_t *dst = grad_filters + ((int64_t)(ob * 64 + o) * C + cb * 64 + c) * 9 + tap;
+        *dst = MmaW<T>::from_f32(MmaW<T>::to_f32(*dst) + all);
+    }
 }
 
 struct Plan {
@@ -270,7 +297,7 @@ hipError_t launch_conv3x3_wgrad(const Conv3x3Problem &c, int compute_units, void
         }                                                                                                              \
         conv3x3_wgrad_kernel<T><<<grid, NTH, pl.lds, stream>>>(p);                                                     \
         const int total = pl.combos * 9 * 4096;                                                                        \
-        conv3x3_wgrad_reduce_kernel<T><<<(total + 255) / 256, 256, 0, stream>>>((const float *)workspace, (uint16_t *)c.filters, c.chan_in, \
+        conv3x3_wgrad_reduce_kernel<T><<<total / 32, 256, 0, stream>>>((const float *)workspace, (uint16_t *)c.filters, c.chan_in, \
                                                                                p.cblocks, pl.combos, pl.slices, total); \
     } while (0)
     if (c.dtype == DT_F16) DFDX_WGRAD(_Float16);
