@@ -32,7 +32,8 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 #define DFDX_LDS __attribute__((address_space(3)))
 
 constexpr int NTH = 768;    // 12 waves
-constexpr int REC = 160;    // bytes of a pixel record: 64 channels + 32 of padding (an odd multiple of 32 bytes)
+constexpr int REC = 144;    // bytes of a pixel record: 64 channels + 16 of padding (the transposing reads take any pitch at the same rate;
+                            // the deposits, two records apart from lane to lane, collide 2-way on an odd multiple of 16 bytes, 4-way on 160)
 constexpr int KMAX = 256;   // records of a grad_out band at most (a multiple of the 32-pixel k step)
 constexpr int UMAX = 2;     // pixel-pair units of a band a thread may own
 
@@ -173,16 +174,34 @@ __global__ __launch_bounds__(NTH, 3) void conv3x3_wgrad_kernel(const Params p) {
         }
         __syncthreads();
         if (item + p.slices < p.items) request(item + p.slices);  // the next item travels while this one is multiplied
-        for (int k0 = 0; k0 < p.kp; k0 += 32) {
-            u32x4 fa[4], fb[3];
+        // k steps of 32 pixels in a software pipeline: the fragments of step k + 1 are requested from LDS in front of
+        // the 12 MFMAs of step k (two register sets, the loop unrolled by two)
+        u32x4 fa[2][4], fb[2][3];
+        auto read_step = [&](int k0, u32x4(&a)[4], u32x4(&bf)[3]) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) fa[i] = tr_fragment(gband, k0, 16 * i, l16, lq);
+            for (int i = 0; i < 4; i++) a[i] = tr_fragment(gband, k0, 16 * i, l16, lq);
 #pragma unroll
-            for (int e = 0; e < 3; e++) fb[e] = tr_fragment(xband, k0 + b_rec[e], b_chan[e], l16, lq);
+            for (int e = 0; e < 3; e++) bf[e] = tr_fragment(xband, k0 + b_rec[e], b_chan[e], l16, lq);
+        };
+        auto mma_step = [&](const u32x4(&a)[4], const u32x4(&bf)[3]) {
 #pragma unroll
             for (int e = 0; e < 3; e++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) acc[i][e] = MmaW<T>::mfma(fb[e], fa[i], acc[i][e]);
+                for (int i = 0; i < 4; i++) acc[i][e] = MmaW<T>::mfma(bf[e], a[i], acc[i][e]);
+        };
+        read_step(0, fa[0], fb[0]);
+        for (int k0 = 0; k0 < p.kp; k0 += 64) {  // kp is a multiple of 32: the second half may be missing
+            const bool second = k0 + 32 < p.kp;
+            if (second) read_step(k0 + 32, fa[1], fb[1]);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_step(fa[0], fb[0]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (second) {
+                if (k0 + 64 < p.kp) read_step(k0 + 64, fa[0], fb[0]);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_step(fa[1], fb[1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     }
 
