@@ -261,15 +261,15 @@ bool implicit_forward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *f
     return true;
 }
 
-// 3 x 3 filters at unit stride with padding 1, 16-bit types, channel counts in whole chunks: the kernel that keeps a band
+// 3 x 3 filters at unit stride with padding 1, f16 / bf16 / f32, channel counts in whole chunks: the kernel that keeps a band
 // of the image in LDS and reads every tap's operand from it (conv3x3.hip).  The filters go through the patch buffer in
 // the order that kernel wants.
 template <typename T>
 bool tiled3x3_forward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *filters, const void *img, void *out, int *rc) {
-    if (sizeof(T) != 2 || op.kernel != 3 || op.stride != 1 || op.padding != 1 || op.dilation != 1 || op.groups != 1) return false;
+    if (sizeof(T) > 4 || op.kernel != 3 || op.stride != 1 || op.padding != 1 || op.dilation != 1 || op.groups != 1) return false;
     if (op.h_out != op.h_in || op.w_out != op.w_in) return false;
     Conv3x3Problem c{};
-    c.dtype = dtype == DFDX_ROCM_F16 ? DT_F16 : DT_BF16;
+    c.dtype = dtype == DFDX_ROCM_F16 ? DT_F16 : dtype == DFDX_ROCM_BF16 ? DT_BF16 : DT_F32;
     c.batch = op.batch; c.chan_in = op.chan_in; c.chan_out = op.chan_out; c.h = op.h_in; c.w = op.w_in;
     c.img = img; c.filters = filters; c.out = out;
     c.wt = (void *)16;  // any aligned address: the real one needs the lock below
@@ -371,13 +371,13 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     const size_t f_bytes = round256((size_t)f_elems * sizeof(T));
     const size_t img_bytes = padded ? round256((size_t)(chunk * op.chan_in * hp) * sizeof(T)) : 0;
     // The image gradient of a 3 x 3, unit-stride, padding-1 convolution is such a convolution of grad_out (filters turned
-    // by 180 degrees, channels trading places): the 16-bit types run it on the kernel that reads its taps from a band of
+    // by 180 degrees, channels trading places): f16 / bf16 / f32 run it on the kernel that reads its taps from a band of
     // grad_out in LDS (conv3x3.hip) instead of the product with the patch matrix, which only the filter gradient needs then.
     Conv3x3Problem band{};
     bool use_band = false;
-    if (sizeof(T) == 2 && op.kernel == 3 && op.stride == 1 && op.padding == 1 && op.dilation == 1 && op.groups == 1 &&
+    if (sizeof(T) <= 4 && op.kernel == 3 && op.stride == 1 && op.padding == 1 && op.dilation == 1 && op.groups == 1 &&
         op.h_out == op.h_in && op.w_out == op.w_in) {
-        band.dtype = dtype == DFDX_ROCM_F16 ? DT_F16 : DT_BF16;
+        band.dtype = dtype == DFDX_ROCM_F16 ? DT_F16 : dtype == DFDX_ROCM_BF16 ? DT_BF16 : DT_F32;
         band.chan_in = op.chan_out; band.chan_out = op.chan_in; band.h = op.h_in; band.w = op.w_in;
         band.batch = (int)chunk;
         band.img = grad_out; band.filters = filters; band.out = grad_img;

@@ -115,7 +115,7 @@ BAND_CONFIGS = [(2, 32, 64, 16, 16), (1, 64, 64, 14, 14), (3, 96, 128, 20, 14), 
                 (1, 32, 64, 9, 112), (2, 64, 64, 31, 12), (1, 64, 64, 112, 112), (5, 32, 64, 8, 16), (2, 32, 64, 50, 4)]
 
 
-@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("cfg", BAND_CONFIGS, ids=lambda c: "x".join(map(str, c)))
 def test_conv2d_3x3_forward_from_a_band_in_lds(cfg, dtype):
     dev, g = device(), rng(504)
@@ -160,7 +160,7 @@ WGRAD_CONFIGS = [(2, 128, 64, 20, 14), (3, 64, 128, 9, 30), (1, 64, 64, 5, 62), 
                  (2, 128, 128, 33, 12)]
 
 
-@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])   # (f32: the image gradient on the band kernel, the filter gradient over the patch matrix)
 @pytest.mark.parametrize("cfg", WGRAD_CONFIGS, ids=lambda c: "x".join(map(str, c)))
 def test_conv2d_3x3_backward_without_patch_matrix(cfg, dtype):
     dev, g = device(), rng(505)
