@@ -394,7 +394,7 @@ int dfdx_rocm_relu_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const vo
 int dfdx_rocm_add_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const void *lhs, const void *rhs, void *out);
 int dfdx_rocm_add_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, void *grad_lhs, void *grad_rhs, const void *grad_out);
 
-/* ---- conv2d as unfold + batched GEMM ---------------------------------------
+/* ---- conv2d: unfold + batched GEMM, 3 x 3 layers without a patch matrix -----
  * Conv2DKernel (dfdx-core/src/tensor_ops/conv2d/mod.rs:31-55; Cpu impl
  * cpu_kernel.rs:40-278, Cuda impl cuda_kernel.rs:62-281).  The op struct has
  * the fields and order of the reference's #[repr(C)] Conv2DOp (mod.rs:14-29),
@@ -402,7 +402,12 @@ int dfdx_rocm_add_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, void *gra
  * h_in, w_in), filters (chan_out, chan_in/groups, kernel, kernel), out
  * (batch, chan_out, h_out, w_out), all contiguous as the reference requires
  * (mod.rs:290-292); an unbatched image is batch = 1.  Forward overwrites out;
- * backward accumulates into grad_img and grad_filters. */
+ * backward accumulates into grad_img and grad_filters.  The general form is
+ * the reference's: gather the patch matrix, multiply (cpu_kernel.rs:52-170).
+ * 3 x 3 filters at unit stride with padding 1 and whole blocks of channels run
+ * on kernels that keep a band of the image in LDS and form no patch matrix
+ * (same sums, f32 accumulation, one rounding; results within the tolerance
+ * of the general form, not bit-identical to it). */
 typedef struct dfdx_rocm_conv2d_op {
     size_t kernel, stride, padding, dilation, groups, batch, chan_in, chan_out, h_in, h_out, w_in, w_out;
 } dfdx_rocm_conv2d_op;
