@@ -16,6 +16,10 @@
 // times the four 16-row tiles of output channels: 12 MFMAs per 32 pixels against 4 + 3 fragments).  At the end every
 // workgroup leaves its sums as f32 in a workspace and a second kernel adds the shares in a fixed order into grad_filters
 // (one rounding): deterministic.
+//
+// f32 has a kernel of its own further down (conv3x3_wgrad_f32_kernel): v_mfma_f32_16x16x4_f32 takes ONE k per lane, so no
+// operand needs transposing -- both bands stay channel-major, as they lie in memory, and are written into LDS by the loads
+// themselves.
 #include "gemm_internal.h"
 #include "conv3x3.h"
 #include <algorithm>
@@ -52,6 +56,13 @@ template <> struct MmaW<__bf16> {
     static __device__ __forceinline__ float to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
     static __device__ __forceinline__ uint16_t from_f32(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
 };
+
+template <> struct MmaW<float> {
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+    static __device__ __forceinline__ float from_f32(float v) { return v; }
+};
+template <typename T> struct StoredAs { typedef uint16_t type; };
+template <> struct StoredAs<float> { typedef float type; };
 
 struct Params {
     const uint16_t *img;  // [B][C][H][W]
@@ -219,7 +230,8 @@ __global__ __launch_bounds__(NTH, 3) void conv3x3_wgrad_kernel(const Params p) {
 // its 8 thread groups add an eighth of the slices each, in slice order, and the eight subtotals meet in LDS in group order:
 // one fixed summation order, whatever the timing.
 template <typename T>
-__global__ __launch_bounds__(256) void conv3x3_wgrad_reduce_kernel(const float *__restrict__ partial, uint16_t *__restrict__ grad_filters, int C,
+__global__ __launch_bounds__(256) void conv3x3_wgrad_reduce_kernel(const float *__restrict__ partial,
+                                                                   typename StoredAs<T>::type *__restrict__ grad_filters, int C,
                                                                    int cblocks, int combos, int slices, int total) {
     __shared__ float subtotal[8][32];
     const int lane_elem = threadIdx.x % 32, group = threadIdx.x / 32;
@@ -246,9 +258,215 @@ __global__ __launch_bounds__(256) void conv3x3_wgrad_reduce_kernel(const float *
         for (int g = 1; g < 8; g++) all += subtotal[g][lane_elem];
         const int c = within % 64, o = (within / 64) % 64, tap = within / 4096;
         const int cb = combo % cblocks, ob = combo / cblocks;
-        uint16_t *dst = grad_filters + ((int64_t)(ob * 64 + o) * C + cb * 64 + c) * 9 + tap;
+        typename StoredAs<T>::type *dst = grad_filters + ((int64_t)(ob * 64 + o) * C + cb * 64 + c) * 9 + tap;
         *dst = MmaW<T>::from_f32(MmaW<T>::to_f32(*dst) + all);
     }
+}
+
+// ---- f32 ----------------------------------------------------------------------------------------------------------------
+// The same nine GEMMs with v_mfma_f32_16x16x4_f32: a lane supplies ONE value, (channel l16, pixel lq) of a 16-channel x
+// 4-pixel fragment, so a fragment is one ds_read_b32 from a CHANNEL-major band -- the layout of the tensors in memory.
+// A band row of a channel is RP = 4 + W rounded up to 4 slots: four zeros, the W pixels, zeros up to the pitch; the zeros
+// in front of a row are the padding column of its first pixel and of the previous row's last one.  k steps are the
+// 4-aligned slot groups that hold pixels (the group of zeros in front of every row is skipped); a tap shifts the image
+// slot by ky RP + kx - 1 against the grad_out slot.  Channel pitches are odd multiples of 2 dwords: the 16 channels x 4
+// consecutive slots of a fragment read then count no bank conflict (odd multiples of 4 counted 2-way conflicts).
+// Both bands of a work item (RS grad_out rows, RS + 2 image rows, 64 channels each) are written into LDS by the loads
+// themselves (buffer_load_dword ... lds: 64 consecutive slots of one channel per wave instruction; a lane whose slot is a
+// zero -- padding, a row outside the image -- points past the end of the buffer resource and the hardware writes the
+// zero; a lane past the end of the channel's band is switched off): no staging registers, no deposit phase, two stages,
+// one barrier per item.  A wave requests the next item's bands one channel per k step of the current item: requested in
+// one block behind the barrier, the 250 instructions of an item fill the queue of the address unit and every wave waits
+// there instead of multiplying.
+constexpr int SEGS = 5;          // 64-slot runs of one channel's band at most
+constexpr int PITCH_MAX = 320;   // G pitch + X pitch (dwords per channel): two stages of 64 channels in 160 KB
+constexpr uint32_t UNIT_ZERO = 0xFFFFFFFFu, UNIT_NONE = 0xFFFFFFFEu;
+
+struct ParamsF {
+    const float *img, *go;
+    float *partial;
+    int C, O, H, W, HW;
+    int RS, bands, items, slices, cblocks;
+    int RP, Q;       // slots per band row; k steps per band row
+    int GP, XP;      // dwords per channel of the grad_out / image band
+    uint32_t magic_rp;
+};
+
+__global__ __launch_bounds__(NTH, 1) void conv3x3_wgrad_f32_kernel(const ParamsF p) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int l16 = lane % 16, lq = lane / 16;
+    const uint32_t stage_bytes = (uint32_t)(p.GP + p.XP) * 256u;  // 64 channels of both bands
+    const uint32_t smem_addr = (uint32_t)(uintptr_t)(DFDX_LDS const uint8_t *)smem;
+
+    const int combos = gridDim.x / p.slices;
+    const int combo = blockIdx.x % combos, slice = blockIdx.x / combos;
+    const int cb = combo % p.cblocks, ob = combo / p.cblocks;
+
+    // what this lane fetches for slot 64 seg + lane of any channel: element offset inside the channel's plane, counted
+    // from image row y0 - 1, in the low 24 bits and the band row above them
+    uint32_t g_unit[SEGS], x_unit[SEGS];
+#pragma unroll
+    for (int seg = 0; seg < SEGS; seg++) {
+        const int s = 64 * seg + lane;
+        const int r = (int)__umulhi((uint32_t)s, p.magic_rp), x = s - r * p.RP - 4;
+        const bool pixel = x >= 0 && x < p.W;
+        // grad_out row r lies beside image band row r + 1; its slots behind the last row are never read
+        g_unit[seg] = s >= p.RS * p.RP ? UNIT_NONE : pixel ? (uint32_t)((r + 1) * p.W + x) | ((uint32_t)(r + 1) << 24) : UNIT_ZERO;
+        x_unit[seg] = s >= p.XP ? UNIT_NONE : (pixel && r < p.RS + 2) ? (uint32_t)(r * p.W + x) | ((uint32_t)r << 24) : UNIT_ZERO;
+    }
+    const int g_segs = (p.RS * p.RP + 63) / 64, x_segs = (p.XP + 63) / 64;
+
+    // the item being requested: its image, rows and destination stage; dma_ch = the next channel this wave requests
+    __amdgpu_buffer_rsrc_t xsrc, gsrc;
+    int dma_ybase = 0, dma_ch = 64;
+    uint32_t dma_dst = 0;
+    auto begin_request = [&](int item, int stage) {
+        const int b = item / p.bands;
+        dma_ybase = (item - b * p.bands) * p.RS - 1;
+        xsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.img + ((int64_t)b * p.C + cb * 64) * p.HW), 0, 64 * p.HW * 4, 0x00020000);
+        gsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.go + ((int64_t)b * p.O + ob * 64) * p.HW), 0, 64 * p.HW * 4, 0x00020000);
+        dma_dst = smem_addr + (uint32_t)stage * stage_bytes;
+        dma_ch = wave;
+    };
+    auto request_channel = [&]() {  // both bands of channel dma_ch
+        if (dma_ch >= 64) return;
+        const int plane = dma_ch * p.HW * 4;
+        const int row0 = dma_ybase * p.W;
+        auto offset_of = [&](uint32_t u) -> int {
+            const int y = dma_ybase + (int)(u >> 24);
+            return (u != UNIT_ZERO && (unsigned)y < (unsigned)p.H) ? ((int)(u & 0xFFFFFFu) + row0) * 4 : (int)0x80000000u;
+        };
+#pragma unroll
+        for (int seg = 0; seg < SEGS; seg++)
+            if (seg < g_segs && g_unit[seg] != UNIT_NONE)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(gsrc, (DFDX_LDS void *)(uintptr_t)(dma_dst + (uint32_t)(dma_ch * p.GP + 64 * seg) * 4u), 4,
+                                                         offset_of(g_unit[seg]), plane, 0, 0);
+#pragma unroll
+        for (int seg = 0; seg < SEGS; seg++)
+            if (seg < x_segs && x_unit[seg] != UNIT_NONE)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(xsrc, (DFDX_LDS void *)(uintptr_t)(dma_dst + (uint32_t)(64 * p.GP + dma_ch * p.XP + 64 * seg) * 4u), 4,
+                                                         offset_of(x_unit[seg]), plane, 0, 0);
+        dma_ch += 12;
+    };
+
+    f32x4 acc[4][3];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int e = 0; e < 3; e++) acc[i][e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // fragment addresses (dwords from the start of a stage) at slot 0; the wave's three (tap, input-channel tile) pairs
+    const int g_at = l16 * p.GP + lq;
+    int x_at[3];
+#pragma unroll
+    for (int e = 0; e < 3; e++) {
+        const int q = wave * 3 + e, tap = q / 4, j = q % 4;
+        x_at[e] = p.GP * 64 + (16 * j + l16) * p.XP + lq + (tap / 3) * p.RP + (tap % 3) - 1;
+    }
+
+    int stage = 0;
+    if (slice < p.items) {
+        begin_request(slice, 0);
+        while (dma_ch < 64) request_channel();
+    }
+    for (int item = slice; item < p.items; item += p.slices) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the item has landed
+        __syncthreads();                     // ... and everybody's; the other stage is no longer being read
+        if (item + p.slices < p.items) begin_request(item + p.slices, stage ^ 1);
+        const float *const st = (const float *)(smem + (uint32_t)stage * stage_bytes);
+        const int y0 = (item % p.bands) * p.RS;
+        const int steps = min(p.RS, p.H - y0) * p.Q;
+        // k steps of 4 slots in a software pipeline: the 7 fragments of step t + 1 are requested from LDS in front of
+        // the 12 MFMAs of step t (no conditional read inside the loop: with one, the compiler's wait in front of a step's
+        // MFMAs also covers the reads just issued for the next step)
+        float fa[2][4], fb[2][3];
+        int slot = 4, q = 0;
+        auto read_step = [&](float(&a)[4], float(&bf)[3]) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) a[i] = st[g_at + 16 * i * p.GP + slot];
+#pragma unroll
+            for (int e = 0; e < 3; e++) bf[e] = st[x_at[e] + slot];
+            slot += 4;
+            if (++q == p.Q) {  // over the zeros in front of the next row
+                q = 0;
+                slot += 4;
+            }
+            request_channel();
+        };
+        auto mma_step = [&](const float(&a)[4], const float(&bf)[3]) {
+#pragma unroll
+            for (int e = 0; e < 3; e++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[i][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf[e], a[i], acc[i][e], 0, 0, 0);
+        };
+        read_step(fa[0], fb[0]);
+        int t = 0;
+        for (; t + 2 < steps; t += 2) {
+            read_step(fa[1], fb[1]);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_step(fa[0], fb[0]);
+            __builtin_amdgcn_sched_barrier(0);
+            read_step(fa[0], fb[0]);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_step(fa[1], fb[1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (t + 1 < steps) {  // one or two steps are left
+            read_step(fa[1], fb[1]);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_step(fa[0], fb[0]);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_step(fa[1], fb[1]);
+        } else {
+            mma_step(fa[0], fb[0]);
+        }
+        while (dma_ch < 64) request_channel();  // (an item of few k steps)
+        stage ^= 1;
+    }
+
+    float *const share = p.partial + ((int64_t)slice * combos + combo) * (9 * 64 * 64);
+#pragma unroll
+    for (int e = 0; e < 3; e++) {
+        const int q = wave * 3 + e, tap = q / 4, j = q % 4;
+#pragma unroll
+        for (int i = 0; i < 4; i++) *(f32x4 *)(share + (tap * 64 + 16 * i + l16) * 64 + 16 * j + 4 * lq) = acc[i][e];
+    }
+}
+
+struct PlanF {
+    int RS, bands, RP, Q, GP, XP, slices, combos;
+    size_t lds;
+};
+int bank_free_pitch(int n) {  // the smallest odd multiple of 2 that is >= n
+    int p = (n + 1) / 2 * 2;
+    return p % 4 == 2 ? p : p + 2;
+}
+bool make_plan_f32(const Conv3x3Problem &c, int compute_units, PlanF *out) {
+    if (c.dtype != DT_F32) return false;
+    if (c.batch < 1 || c.chan_in < 64 || c.chan_in % 64 || c.chan_out < 64 || c.chan_out % 64) return false;
+    if (c.w < 2 || c.h < 1) return false;
+    const int64_t hw = (int64_t)c.h * c.w;
+    if (hw >= (1 << 22)) return false;  // byte offsets inside a block of 64 planes are 32-bit integers
+    if (((uintptr_t)c.img & 3u) || ((uintptr_t)c.out & 3u) || ((uintptr_t)c.filters & 3u)) return false;
+    PlanF pl;
+    pl.Q = (c.w + 3) / 4;
+    pl.RP = 4 * pl.Q + 4;
+    pl.RS = 0;
+    for (int rs = 1; rs <= std::min(c.h, 64); rs++) {  // as many rows per item as two stages leave room for
+        const int gp = bank_free_pitch(rs * pl.RP), xp = bank_free_pitch((rs + 2) * pl.RP + 1);
+        if (gp + xp > PITCH_MAX) break;
+        pl.RS = rs; pl.GP = gp; pl.XP = xp;
+    }
+    if (pl.RS < 1) return false;
+    pl.bands = (c.h + pl.RS - 1) / pl.RS;
+    pl.lds = (size_t)2 * (pl.GP + pl.XP) * 256;
+    pl.combos = (c.chan_in / 64) * (c.chan_out / 64);
+    const int64_t items = (int64_t)c.batch * pl.bands;
+    if (items >= (1ll << 31) || pl.combos > 65536) return false;
+    pl.slices = (int)std::max<int64_t>(1, std::min<int64_t>(items, std::max(1, compute_units) / pl.combos));
+    *out = pl;
+    return true;
 }
 
 struct Plan {
@@ -285,16 +503,46 @@ bool make_plan(const Conv3x3Problem &c, int compute_units, Plan *out) {
 // `c` as for the forward kernel, with `out` = grad_out [batch][chan_out][h][w] and `filters` = grad_filters (accumulated into).
 bool conv3x3_wgrad_supported(const Conv3x3Problem &c, int compute_units) {
     Plan pl;
-    return make_plan(c, compute_units, &pl);
+    PlanF plf;
+    return make_plan(c, compute_units, &pl) || make_plan_f32(c, compute_units, &plf);
 }
 
 size_t conv3x3_wgrad_workspace_bytes(const Conv3x3Problem &c, int compute_units) {
     Plan pl;
+    PlanF plf;
+    if (make_plan_f32(c, compute_units, &plf)) return (size_t)plf.slices * plf.combos * 9 * 64 * 64 * sizeof(float);
     if (!make_plan(c, compute_units, &pl)) return 0;
     return (size_t)pl.slices * pl.combos * 9 * 64 * 64 * sizeof(float);
 }
 
+hipError_t launch_conv3x3_wgrad_f32(const Conv3x3Problem &c, const PlanF &pl, void *workspace, hipStream_t stream) {
+    ParamsF p;
+    p.img = (const float *)c.img; p.go = (const float *)c.out; p.partial = (float *)workspace;
+    p.C = c.chan_in; p.O = c.chan_out; p.H = c.h; p.W = c.w; p.HW = c.h * c.w;
+    p.RS = pl.RS; p.bands = pl.bands; p.items = c.batch * pl.bands;
+    p.slices = pl.slices; p.cblocks = c.chan_in / 64;
+    p.RP = pl.RP; p.Q = pl.Q; p.GP = pl.GP; p.XP = pl.XP;
+    p.magic_rp = (uint32_t)(((1ull << 32) + pl.RP - 1) / pl.RP);
+    static PerDevice attr_on;
+    std::atomic<int> &known = attr_on.here();
+    if (known.load(std::memory_order_acquire) == 0) {
+        hipError_t e = hipFuncSetAttribute((const void *)conv3x3_wgrad_f32_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        known.store(1, std::memory_order_release);
+    }
+    conv3x3_wgrad_f32_kernel<<<(unsigned)(pl.combos * pl.slices), NTH, pl.lds, stream>>>(p);
+    const int total = pl.combos * 9 * 4096;
+    conv3x3_wgrad_reduce_kernel<float><<<total / 32, 256, 0, stream>>>((const float *)workspace, (float *)c.filters, c.chan_in, p.cblocks,
+                                                                        pl.combos, pl.slices, total);
+    return hipGetLastError();
+}
+
 hipError_t launch_conv3x3_wgrad(const Conv3x3Problem &c, int compute_units, void *workspace, hipStream_t stream) {
+    PlanF plf;
+    if (make_plan_f32(c, compute_units, &plf)) {
+        if ((uintptr_t)workspace & 15u) return hipErrorNotSupported;
+        return launch_conv3x3_wgrad_f32(c, plf, workspace, stream);
+    }
     Plan pl;
     if (!make_plan(c, compute_units, &pl) || ((uintptr_t)workspace & 15u)) return hipErrorNotSupported;
     Params p;

@@ -160,7 +160,7 @@ WGRAD_CONFIGS = [(2, 128, 64, 20, 14), (3, 64, 128, 9, 30), (1, 64, 64, 5, 62), 
                  (2, 128, 128, 33, 12)]
 
 
-@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])   # (f32: the image gradient on the band kernel, the filter gradient over the patch matrix)
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])   # (f32: channel-major bands, one value per lane and MFMA)
 @pytest.mark.parametrize("cfg", WGRAD_CONFIGS, ids=lambda c: "x".join(map(str, c)))
 def test_conv2d_3x3_backward_without_patch_matrix(cfg, dtype):
     dev, g = device(), rng(505)
@@ -190,16 +190,17 @@ def test_conv2d_3x3_backward_without_patch_matrix(cfg, dtype):
                   extra=(batch + 2) * ULP[dtype] * float(np.abs(wgw).max()), what="grad_filters")
 
 
-def test_conv2d_3x3_filter_gradient_counts_pixels_exactly():
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_conv2d_3x3_filter_gradient_counts_pixels_exactly(dtype):
     """Images and output gradients of ones: the gradient of filter tap (ky, kx) is batch x the number of pixels whose
     neighbour at that tap lies inside the image -- (H - |ky - 1|) (W - |kx - 1|) -- exactly, for every channel pair."""
     dev = device()
     batch, cin, cout, h, w_ = 3, 64, 64, 11, 10
-    announce("conv2d 3x3 filter gradient, ones", batch, cin, cout, h, w_)
-    x = upload(dev, np.ones((batch, cin, h, w_)), "f16")
-    w = upload(dev, np.zeros((cout, cin, 3, 3)), "f16")
-    go = upload(dev, np.ones((batch, cout, h, w_)), "f16")
-    gx, gw = dev.zeros("f16", x.shape), dev.zeros("f16", w.shape)
+    announce("conv2d 3x3 filter gradient, ones", batch, cin, cout, h, w_, dtype)
+    x = upload(dev, np.ones((batch, cin, h, w_)), dtype)
+    w = upload(dev, np.zeros((cout, cin, 3, 3)), dtype)
+    go = upload(dev, np.ones((batch, cout, h, w_)), dtype)
+    gx, gw = dev.zeros(dtype, x.shape), dev.zeros(dtype, w.shape)
     dev.conv2d_backward(x, gx, w, gw, go, stride=1, padding=1)
     got = host(dev, gw)
     want = np.array([[batch * (h - abs(ky - 1)) * (w_ - abs(kx - 1)) for kx in range(3)] for ky in range(3)], dtype=np.float64)
