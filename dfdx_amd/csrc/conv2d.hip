@@ -386,8 +386,9 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         use_band = conv3x3_supported(band);
     }
     const size_t wt_bytes = use_band ? round256(conv3x3_filter_bytes(band)) : 0;
-    // The filter gradient of such a convolution has its own kernel too (conv3x3_wgrad.hip: both operands pixel-major in
-    // LDS, fragments through transposing reads).  With both in place the backward pass forms no patch matrix at all.
+    // The filter gradient of such a convolution has its own kernels too (conv3x3_wgrad.hip; 16-bit types: both operands
+    // pixel-major in LDS, fragments through transposing reads; f32: channel-major bands, one value per lane and MFMA).
+    // With both in place the backward pass forms no patch matrix at all.
     Conv3x3Problem wgrad{};
     bool use_wgrad = false;
     if (use_band) {
