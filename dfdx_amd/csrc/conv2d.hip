@@ -405,6 +405,34 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         HIP_TRY(launch_conv3x3(band, ctx->stream));
         return (int)launch_conv3x3_wgrad(wgrad, ctx->compute_units, ctx->patches, ctx->stream);
     }
+    if (pointwise) {
+        // Filters [O][C/G] are plain matrices here and both products take them as they lie, transposed through the strides:
+        // no transposed copies, no zeroed scratch gradient, no pass that adds it back.
+        //   grad_img (B, G, C/G, H*W) += filters^T (G, C/G, O/G) . grad_out (B, G, O/G, H*W)
+        {
+            const int64_t m = cg, k = og, n = hw;
+            dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
+            d.accumulate = 1;
+            d.batch1 = op.batch; d.batch2 = op.groups;
+            d.a = filters; d.a_rs = 1; d.a_cs = m; d.a_b1 = 0; d.a_b2 = m * k;
+            d.b = grad_out; d.b_rs = n; d.b_cs = 1; d.b_b1 = op.groups * k * n; d.b_b2 = k * n;
+            d.c = grad_img; d.c_rs = n; d.c_cs = 1; d.c_b1 = op.chan_in * n; d.c_b2 = m * n;
+            if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+        }
+        //   grad_filters (O/G, C/G) += sum over images of grad_out (O/G, H*W) . img^T (H*W, C/G)
+        for (int g = 0; g < op.groups; g++) {
+            const int64_t m = og, k = hw, n = cg;
+            dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
+            d.accumulate = 1;
+            d.reduce_batch = 1;
+            d.batch1 = op.batch;
+            d.a = (const T *)grad_out + g * m * k; d.a_rs = k; d.a_cs = 1; d.a_b1 = op.chan_out * k;
+            d.b = (const T *)img + g * n * k; d.b_rs = 1; d.b_cs = k; d.b_b1 = op.chan_in * k;
+            d.c = (T *)grad_filters + g * m * n; d.c_rs = n; d.c_cs = 1;
+            if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+        }
+        return DFDX_ROCM_OK;
+    }
     if (int rc = ensure_patches(ctx, patch_bytes + 2 * f_bytes + 2 * img_bytes + wt_bytes)) return rc;
     T *patches = (T *)ctx->patches;
     T *f_tr = (T *)((char *)ctx->patches + patch_bytes);
@@ -423,8 +451,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         sub.batch = (int)nb;
         const T *go = (const T *)grad_out + b0 * op.chan_out * ohw;
         const unsigned slabs = (unsigned)(nb * op.chan_out * kk);
-        if (pointwise) patches = const_cast<T *>(go);
-        else if (planes && op.kernel == 3) unfold_output_plane_kernel<T, 3><<<slabs / 9, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
+        if (planes && op.kernel == 3) unfold_output_plane_kernel<T, 3><<<slabs / 9, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
         else if (planes) unfold_output_plane_kernel<T, 0><<<(unsigned)(slabs / kk), 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
         else {
             const uint32_t vectors = (uint32_t)(slabs * (hp / V));
