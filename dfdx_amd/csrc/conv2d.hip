@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256) void unfold_output_plane_kernel(Op op, const T
 // column) slab -- they may straddle two rows -- whatever the slab size (a 7x7 slab would leave 249 of a workgroup's
 // 256 threads idle); positions behind the slab's last element (the row padding) are zeros.
 template <typename T>
-__global__ __launch_bounds__(256) void unfold_input_flat_kernel(Op op, const T *img, T *patches, int slab_stride, uint32_t vectors) {
+__global__ __launch_bounds__(256) void unfold_input_flat_kernel(Op op, const T *img, T *patches, int slab_stride, uint32_t vectors, int fold) {
     constexpr int V = Elem<T>::VEC;
     const uint32_t item = blockIdx.x * 256 + threadIdx.x;  // one 16-byte vector of the patch buffer per thread
     if (item >= vectors) return;
@@ -102,7 +102,10 @@ __global__ __launch_bounds__(256) void unfold_input_flat_kernel(Op op, const T *
     const int kk = op.kernel * op.kernel, n = op.h_out * op.w_out;
     const int k2 = (int)(slab % op.kernel), k1 = (int)((slab / op.kernel) % op.kernel);
     const T *plane = img + (int64_t)(slab / kk) * op.h_in * op.w_in;
-    T *dst = patches + (int64_t)slab * slab_stride;
+    // slab = (image, channel, tap).  Folded: the slabs of one (channel, tap) lie next to each other, image after image --
+    // the patch matrix of the whole batch, [C K K][batch * slab_stride]
+    const uint32_t per_img = (uint32_t)(op.chan_in * kk);
+    T *dst = patches + (int64_t)(fold ? (slab % per_img) * (uint32_t)op.batch + slab / per_img : slab) * slab_stride;
     {
         const int pos0 = (int)(item - slab * per_slab) * V;
         int oh = pos0 / op.w_out, ow = pos0 - oh * op.w_out;
@@ -158,25 +161,161 @@ __global__ __launch_bounds__(256) void unfold_output_flat_kernel(Op op, const T 
     }
 }
 
-// filters (G*O/G, C/G, K, K) <-> transposed (G, C/G, O/G, K*K).  ADD_BACK: filters[..] += transposed[..].
-template <typename T, bool ADD_BACK>
-__global__ __launch_bounds__(256) void filter_transpose_kernel(Op op, T *filters, T *transposed, int total) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= total) return;
-    const int kk = op.kernel * op.kernel, og = op.chan_out / op.groups, cg = op.chan_in / op.groups;
-    int r = i;
-    const int tap = r % kk; r /= kk;
-    const int o = r % og; r /= og;
-    const int c = r % cg;
-    const int g = r / cg;
-    T *f = filters + (((int64_t)(g * og + o) * cg + c) * kk + tap);
-    if constexpr (ADD_BACK) Elem<T>::store(f, Elem<T>::load(f) + Elem<T>::load(transposed + i));
-    else transposed[i] = *f;
+// The flat kernels for small planes (a 7 x 7 image: rows too short for a window load, every element its own 2-byte load,
+// and seven integer divisions per thread: 33 MB of patches took 21 us, bound by the instruction count).  A workgroup first
+// copies the few consecutive planes its 256 vectors draw on into LDS -- one coalesced read -- and gathers from there; what
+// a lane divides is small (an index inside the workgroup's run of vectors, slabs and planes -- the run's origin is divided
+// once, on the scalar unit), so the quotients come from a multiplication with ceil(2^32 / d).  Same patch layout, same zeros.
+struct SmallDivs {  // ceil(2^32 / d) for the divisors of the staged kernels (0 where d = 1)
+    uint32_t per_slab, kernel, kk, chan, width, stride, plane, bg;
+};
+__device__ __forceinline__ uint32_t small_div(uint32_t n, uint32_t d, uint32_t magic) { return d == 1 ? n : __umulhi(n, magic); }
+inline uint32_t magic_of(int64_t d) { return d <= 1 ? 0u : (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d); }
+
+template <typename T, bool OUTPUT_SIDE>
+__global__ __launch_bounds__(256) void unfold_staged_kernel(Op op, SmallDivs mg, const T *src, T *patches, int slab_stride, uint32_t vectors, int fold) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t staged_raw[];
+    T *const staged = (T *)staged_raw;
+    constexpr int V = Elem<T>::VEC;
+    // input side: slabs of the image over output positions; output side: slabs of grad_out over image positions
+    const int src_h = OUTPUT_SIDE ? op.h_out : op.h_in, src_w = OUTPUT_SIDE ? op.w_out : op.w_in;
+    const int pos_w = OUTPUT_SIDE ? op.w_in : op.w_out, n = OUTPUT_SIDE ? op.h_in * op.w_in : op.h_out * op.w_out;
+    const int chan = OUTPUT_SIDE ? op.chan_out : op.chan_in;
+    const uint32_t per_slab = (uint32_t)slab_stride / V;
+    const int kk = op.kernel * op.kernel, plane_elems = src_h * src_w;
+    const uint32_t first = blockIdx.x * 256, last = min(first + 255u, vectors - 1);
+    const uint32_t slab0 = first / per_slab, plane0 = slab0 / kk, plane1 = last / per_slab / kk, image0 = plane0 / chan;
+    const int count = (int)(plane1 - plane0 + 1) * plane_elems;
+    for (int i = threadIdx.x; i < count; i += 256) staged[i] = src[(int64_t)plane0 * plane_elems + i];
+    __syncthreads();
+    if (first + threadIdx.x >= vectors) return;
+    const uint32_t in_run = first - slab0 * per_slab + threadIdx.x;                 // < 256 + per_slab
+    const uint32_t slab_in_run = small_div(in_run, per_slab, mg.per_slab);
+    const uint32_t slab_in_plane0 = slab0 - plane0 * kk + slab_in_run;               // < 2 K K + 256
+    const uint32_t plane_in_run = small_div(slab_in_plane0, kk, mg.kk);
+    const uint32_t tap = slab_in_plane0 - plane_in_run * kk;
+    const int k1 = (int)small_div(tap, op.kernel, mg.kernel), k2 = (int)tap - k1 * op.kernel;
+    const T *plane = staged + plane_in_run * plane_elems;
+    const uint32_t chan_in_image0 = plane0 - image0 * chan + plane_in_run;           // < channels + 258
+    const uint32_t image_in_run = small_div(chan_in_image0, chan, mg.chan);
+    const uint32_t image = image0 + image_in_run, c = chan_in_image0 - image_in_run * chan;
+    const int64_t slab_dst = fold ? (int64_t)(c * kk + tap) * op.batch + image : (int64_t)slab0 + slab_in_run;
+    const int pos0 = (int)(in_run - slab_in_run * per_slab) * V;
+    int row = (int)small_div(pos0, pos_w, mg.width), col = pos0 - row * pos_w;
+    float v[V];
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+        if constexpr (OUTPUT_SIDE) {
+            const int oh = row + op.padding - op.dilation * k1, ow = col + op.padding - op.dilation * k2;
+            const int qh = oh >= 0 ? (int)small_div(oh, op.stride, mg.stride) : 0, qw = ow >= 0 ? (int)small_div(ow, op.stride, mg.stride) : 0;
+            const bool ok = pos0 + i < n && oh >= 0 && qh * op.stride == oh && qh < src_h && ow >= 0 && qw * op.stride == ow && qw < src_w;
+            v[i] = ok ? Elem<T>::load(plane + qh * src_w + qw) : 0.0f;
+        } else {
+            const int y = row * op.stride + op.dilation * k1 - op.padding, x = col * op.stride + op.dilation * k2 - op.padding;
+            const bool ok = pos0 + i < n && y >= 0 && y < src_h && x >= 0 && x < src_w;
+            v[i] = ok ? Elem<T>::load(plane + y * src_w + x) : 0.0f;
+        }
+        if (++col == pos_w) { col = 0; ++row; }
+    }
+    store_elems<T, V>(patches + slab_dst * slab_stride + pos0, v);
+}
+// Position-major gather for small planes into the FOLDED patch matrix [chan K K][batch * slab_stride]: a thread owns one
+// vector of positions of one plane and walks the K x K taps itself, so the index arithmetic of its V positions is done once
+// for all taps (a tap only shifts the source coordinates) and a vector costs ~70 instructions instead of ~250.  A workgroup
+// stages the planes of `cg` channels x `bg` consecutive images in LDS (one read of each) -- the same channels of consecutive
+// images, because their pieces of a patch row lie next to each other: bg * slab_stride contiguous elements per row instead
+// of one image's 112 bytes between the pieces of other workgroups.
+// Input side: source = image, positions = output pixels, coordinate = pos * stride - padding + dilation * k.
+// Output side (unit stride only): source = grad_out, positions = image pixels, coordinate = pos + padding - dilation * k.
+template <typename T, bool OUTPUT_SIDE>
+__global__ __launch_bounds__(256) void unfold_small_kernel(Op op, SmallDivs mg, const T *src, T *patches, int slab_stride, int cg, int bg) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t staged_raw[];
+    T *const staged = (T *)staged_raw;
+    constexpr int V = Elem<T>::VEC;
+    struct __attribute__((aligned(16))) Vec { T e[V]; };
+    const int src_h = OUTPUT_SIDE ? op.h_out : op.h_in, src_w = OUTPUT_SIDE ? op.w_out : op.w_in;
+    const int pos_w = OUTPUT_SIDE ? op.w_in : op.w_out, n = OUTPUT_SIDE ? op.h_in * op.w_in : op.h_out * op.w_out;
+    const int chan = OUTPUT_SIDE ? op.chan_out : op.chan_in;
+    const int scale = OUTPUT_SIDE ? 1 : op.stride, origin = OUTPUT_SIDE ? op.padding : -op.padding;
+    const int tap_step = OUTPUT_SIDE ? -op.dilation : op.dilation;
+    const uint32_t per_slab = (uint32_t)slab_stride / V;
+    const int kk = op.kernel * op.kernel, plane_elems = src_h * src_w;
+    const int c0 = blockIdx.x * cg, b0 = blockIdx.y * bg;
+    const int channels = min(cg, chan - c0), images = min(bg, op.batch - b0);
+    // plane `w` of the workgroup = channel c0 + w / bg of image b0 + w % bg
+    for (uint32_t i = threadIdx.x; i < (uint32_t)(channels * bg * plane_elems); i += 256) {
+        const uint32_t w = small_div(i, plane_elems, mg.plane), e = i - w * plane_elems;
+        const uint32_t cl = small_div(w, bg, mg.bg), bl = w - cl * bg;
+        if ((int)bl < images) staged[i] = src[((int64_t)(b0 + bl) * chan + c0 + cl) * plane_elems + e];
+    }
+    __syncthreads();
+    for (uint32_t item = threadIdx.x; item < (uint32_t)(channels * bg) * per_slab; item += 256) {
+        const uint32_t w = small_div(item, per_slab, mg.per_slab);
+        const uint32_t cl = small_div(w, bg, mg.bg), bl = w - cl * bg;
+        if ((int)bl >= images) continue;
+        const int pos0 = (int)(item - w * per_slab) * V;
+        const T *plane = staged + w * plane_elems;
+        int row = (int)small_div(pos0, pos_w, mg.width), col = pos0 - row * pos_w;
+        int by[V], bx[V];
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            by[i] = pos0 + i < n ? row * scale + origin : -(1 << 20);  // positions behind the slab's last: zeros
+            bx[i] = col * scale + origin;
+            if (++col == pos_w) { col = 0; ++row; }
+        }
+        // the slab of (channel, tap 0, image); a channel's taps are `batch` slabs apart
+        T *dst = patches + ((int64_t)(c0 + cl) * kk * op.batch + b0 + bl) * slab_stride + pos0;
+        for (int k1 = 0; k1 < op.kernel; k1++)
+            for (int k2 = 0; k2 < op.kernel; k2++) {
+                const int dy = tap_step * k1, dx = tap_step * k2;
+                Vec out;
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    const int y = by[i] + dy, x = bx[i] + dx;
+                    const bool ok = (unsigned)y < (unsigned)src_h && (unsigned)x < (unsigned)src_w;
+                    const T val = plane[ok ? y * src_w + x : 0];
+                    out.e[i] = ok ? val : (T)0.0f;
+                }
+                *(Vec *)dst = out;
+                dst += (int64_t)op.batch * slab_stride;
+            }
+    }
+}
+// Launch shape of unfold_small_kernel: bg = 8 images (fewer in a smaller batch), as many channels as give the 256 threads a
+// vector each and fit 32 KB of LDS; false when a single plane does not fit.
+template <typename T> bool small_unfold_shape(int64_t slab_stride, int64_t plane_elems, int batch, int *cg, int *bg, size_t *lds) {
+    *bg = std::min(8, batch);
+    const int64_t per_slab = slab_stride / Elem<T>::VEC;
+    const int64_t by_work = std::max<int64_t>(1, 256 / (per_slab * *bg));
+    const int64_t by_lds = (32 * 1024) / (plane_elems * (int64_t)sizeof(T) * *bg);
+    if (by_lds < 1) return false;
+    *cg = (int)std::min(by_work, by_lds);
+    *lds = (size_t)(*cg * *bg * plane_elems) * sizeof(T);
+    return true;
 }
 
-template <typename T> __global__ __launch_bounds__(256) void zero_kernel(T *p, int n) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < n) Elem<T>::store(p + i, 0.0f);
+// LDS bytes the staged kernels need for planes of `plane_elems` elements, or 0 when they should not be used
+template <typename T> size_t staged_lds_bytes(int64_t slab_stride, int64_t kk, int64_t plane_elems) {
+    const int64_t per_slab = slab_stride / Elem<T>::VEC;
+    const int64_t planes = 255 / per_slab / kk + 2;  // a run of 256 vectors starts and ends inside a plane
+    const int64_t bytes = planes * plane_elems * (int64_t)sizeof(T);
+    return bytes <= 32 * 1024 ? (size_t)((bytes + 15) & ~15ll) : 0;
+}
+
+// filters (G*O/G, C/G, K, K) <-> transposed (G, C/G, O/G, K*K).  ADD_BACK: filters[..] += transposed[..].
+template <typename T, bool ADD_BACK>
+__global__ __launch_bounds__(256) void filter_transpose_kernel(Op op, T *filters, T *transposed, uint32_t magic_kk) {
+    // blockIdx.x = output channel (all groups); a thread takes element j = (c, tap) of that channel's filter, which is
+    // contiguous in `filters`: nothing is divided per element but j by K*K, through a multiplication
+    const int kk = op.kernel * op.kernel, og = op.chan_out / op.groups, cg = op.chan_in / op.groups;
+    const uint32_t j = blockIdx.y * 256 + threadIdx.x;
+    if (j >= (uint32_t)(cg * kk)) return;
+    const int row = blockIdx.x, g = row / og, o = row - g * og;
+    const uint32_t c = kk == 1 ? j : __umulhi(j, magic_kk), tap = j - c * kk;
+    T *f = filters + (int64_t)row * cg * kk + j;
+    T *t = transposed + ((int64_t)(g * cg + c) * og + o) * kk + tap;
+    if constexpr (ADD_BACK) Elem<T>::store(f, Elem<T>::load(f) + Elem<T>::load(t));
+    else *t = *f;
 }
 
 // Rows of `len` elements <-> rows padded to `padded` elements (zeros behind the data).  When the spatial size of a
@@ -195,6 +334,26 @@ template <typename T> __global__ __launch_bounds__(256) void unpad_rows_kernel(c
     if (i >= total) return;
     const int64_t row = i / len;
     dst[i] = src[row * padded + (i - row * len)];
+}
+
+// dst [batch][rows][len] = src [rows][batch][padded]: the product over a folded patch matrix, image by image
+template <typename T> __global__ __launch_bounds__(256) void unfold_rows_kernel(const T *src, T *dst, int len, int padded, int rows, int batch, int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into dst
+    if (i >= total) return;
+    const int64_t line = i / len;  // = image * rows + row
+    const int64_t b = line / rows, r = line - b * rows;
+    dst[i] = src[(r * batch + b) * padded + (i - line * len)];
+}
+
+// dst [rows][batch][padded] = src [batch][rows][len], zeros behind every row: an image-side matrix of the folded products
+template <typename T> __global__ __launch_bounds__(256) void fold_rows_kernel(const T *src, T *dst, int len, int padded, int rows, int batch, int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into dst
+    if (i >= total) return;
+    const int64_t line = i / padded;  // = row * batch + image
+    const int col = (int)(i - line * padded);
+    const int64_t r = line / batch, b = line - r * batch;
+    if (col < len) dst[i] = src[(b * rows + r) * len + col];
+    else Elem<T>::store(dst + i, 0.0f);
 }
 
 constexpr size_t kPatchBudget = size_t(1) << 30;  // bytes of patches per batch chunk
@@ -304,13 +463,17 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
     // 1x1 filters at unit stride without padding: the patch matrix IS the image -- no gather, one product for the batch
     const bool pointwise = op.kernel == 1 && op.stride == 1 && op.padding == 0 && !padded && ((uintptr_t)img & 15u) == 0;
     if (pointwise) chunk = op.batch;
+    // Small images (a 7 x 7 output is n = 49: a quarter of one 256-column tile per image) multiply as ONE product over the
+    // batch: the patch matrix is written [C K K][batch * np], the product lands in [O][batch * np] and a small kernel
+    // hands every image its rows.  The filters are then read once per tile row instead of once per image.
+    const bool fold = !pointwise && op.groups == 1 && np < 256 && op.batch > 1;
     const size_t patch_bytes = pointwise ? 0 : round256((size_t)(chunk * per_image) * sizeof(T));
-    const size_t out_bytes = padded ? round256((size_t)(chunk * op.chan_out * np) * sizeof(T)) : 0;
+    const size_t out_bytes = (padded || fold) ? round256((size_t)(chunk * op.chan_out * np) * sizeof(T)) : 0;
     if (int rc = ensure_patches(ctx, patch_bytes + out_bytes)) return rc;
     T *patches = (T *)ctx->patches;
     T *out_p = (T *)((char *)ctx->patches + patch_bytes);
     // a workgroup per image plane when its K*K slabs give the 256 threads a few vectors each
-    const bool planes = op.stride == 1 && op.w_out % V == 0 && op.w_in >= V && (n / V) * kk >= 512;
+    const bool planes = !fold && op.stride == 1 && op.w_out % V == 0 && op.w_in >= V && (n / V) * kk >= 512;
     for (int64_t b0 = 0; b0 < op.batch; b0 += chunk) {
         const int64_t nb = std::min<int64_t>(chunk, op.batch - b0);
         Op sub = op;
@@ -322,11 +485,31 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
         else if (planes) unfold_input_plane_kernel<T, 0><<<(unsigned)(slabs / kk), 256, 0, ctx->stream>>>(sub, src, patches, (int)np);
         else {
             const uint32_t vectors = (uint32_t)(slabs * (np / V));  // < 2^28: the chunk's patches stay below 2^31 elements
-            unfold_input_flat_kernel<T><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, src, patches, (int)np, vectors);
+            int cg = 0, bg = 0;
+            size_t lds = 0;
+            const int64_t plane_elems = (int64_t)op.h_in * op.w_in;
+            if (fold && small_unfold_shape<T>(np, plane_elems, (int)nb, &cg, &bg, &lds)) {
+                const SmallDivs mg{magic_of(np / V), magic_of(op.kernel), magic_of(kk), magic_of(op.chan_in), magic_of(op.w_out), magic_of(op.stride),
+                                   magic_of(plane_elems), magic_of(bg)};
+                unfold_small_kernel<T, false><<<dim3((unsigned)((op.chan_in + cg - 1) / cg), (unsigned)((nb + bg - 1) / bg)), 256, lds, ctx->stream>>>(
+                    sub, mg, src, patches, (int)np, cg, bg);
+            }
+            else unfold_input_flat_kernel<T><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, src, patches, (int)np, vectors, fold ? 1 : 0);
         }
         HIP_TRY(hipGetLastError());
-        // filters (G, O/G, C/G*K*K) . patches (B, G, C/G*K*K, OH*OW) -> out (B, G, O/G, OH*OW)
         T *dst = (T *)out + b0 * op.chan_out * n;
+        if (fold) {  // filters (O, C*K*K) . patches (C*K*K, B * np) -> (O, B * np)
+            dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, nb * np);
+            d.a = filters; d.a_rs = k; d.a_cs = 1;
+            d.b = patches; d.b_rs = nb * np; d.b_cs = 1;
+            d.c = out_p; d.c_rs = nb * np; d.c_cs = 1;
+            if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+            const int64_t total = nb * op.chan_out * n;
+            unfold_rows_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(out_p, dst, (int)n, (int)np, op.chan_out, (int)nb, total);
+            HIP_TRY(hipGetLastError());
+            continue;
+        }
+        // filters (G, O/G, C/G*K*K) . patches (B, G, C/G*K*K, OH*OW) -> out (B, G, O/G, OH*OW)
         dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, np);
         d.batch1 = nb; d.batch2 = op.groups;
         d.a = filters; d.a_rs = k; d.a_cs = 1; d.a_b1 = 0; d.a_b2 = m * k;
@@ -369,7 +552,14 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     if (pointwise) chunk = op.batch;
     const size_t patch_bytes = pointwise ? 0 : round256((size_t)(chunk * per_image) * sizeof(T));
     const size_t f_bytes = round256((size_t)f_elems * sizeof(T));
-    const size_t img_bytes = padded ? round256((size_t)(chunk * op.chan_in * hp) * sizeof(T)) : 0;
+    // Small images multiply as ONE product over the batch, as in the forward pass: patches [O K K][batch * hp], the image
+    // and its gradient as [C][batch * hp]; the image gradient no longer reads the filters once per image and the filter
+    // gradient is a plain product with k = batch * hp.
+    int fold_cg = 0, fold_bg = 0;
+    size_t fold_lds = 0;
+    const bool fold = !pointwise && op.groups == 1 && op.stride == 1 && hp < 256 && op.batch > 1 &&
+                      small_unfold_shape<T>(hp, ohw, (int)std::min<int64_t>(chunk, op.batch), &fold_cg, &fold_bg, &fold_lds);
+    const size_t img_bytes = (padded || fold) ? round256((size_t)(chunk * op.chan_in * hp) * sizeof(T)) : 0;
     // The image gradient of a 3 x 3, unit-stride, padding-1 convolution is such a convolution of grad_out (filters turned
     // by 180 degrees, channels trading places): f16 / bf16 / f32 run it on the kernel that reads its taps from a band of
     // grad_out in LDS (conv3x3.hip) instead of the product with the patch matrix, which only the filter gradient needs then.
@@ -439,10 +629,10 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     T *grad_f_tr = (T *)((char *)ctx->patches + patch_bytes + f_bytes);
     T *img_p = (T *)((char *)ctx->patches + patch_bytes + 2 * f_bytes);
     T *grad_img_p = (T *)((char *)ctx->patches + patch_bytes + 2 * f_bytes + img_bytes);
-    const unsigned fgrid = (unsigned)((f_elems + 255) / 256);
-    filter_transpose_kernel<T, false><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)const_cast<void *>(filters), f_tr, (int)f_elems);
-    HIP_TRY(hipGetLastError());
-    zero_kernel<T><<<fgrid, 256, 0, ctx->stream>>>(grad_f_tr, (int)f_elems);
+    // (the scratch gradient is not cleared: the first chunk's product overwrites it)
+    const dim3 fgrid((unsigned)op.chan_out, (unsigned)((cg * kk + 255) / 256));
+    const uint32_t magic_kk = magic_of(kk);
+    filter_transpose_kernel<T, false><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)const_cast<void *>(filters), f_tr, magic_kk);
     HIP_TRY(hipGetLastError());
     const bool planes = op.stride == 1 && op.w_in % V == 0 && op.w_out >= V && (hw / V) * kk >= 512;
     for (int64_t b0 = 0; b0 < op.batch; b0 += chunk) {
@@ -451,6 +641,45 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         sub.batch = (int)nb;
         const T *go = (const T *)grad_out + b0 * op.chan_out * ohw;
         const unsigned slabs = (unsigned)(nb * op.chan_out * kk);
+        if (fold && !use_band) {
+            const T *img_b = (const T *)img + b0 * op.chan_in * hw;
+            T *grad_img_b = (T *)grad_img + b0 * op.chan_in * hw;
+            const int64_t nf = nb * hp;  // columns of the folded matrices
+            const int bg = std::min<int>(fold_bg, (int)nb);
+            const SmallDivs mg{magic_of(hp / V), magic_of(op.kernel), magic_of(kk), magic_of(op.chan_out), magic_of(op.w_in), magic_of(op.stride),
+                               magic_of(ohw), magic_of(bg)};
+            unfold_small_kernel<T, true><<<dim3((unsigned)((op.chan_out + fold_cg - 1) / fold_cg), (unsigned)((nb + bg - 1) / bg)), 256, fold_lds, ctx->stream>>>(
+                sub, mg, go, patches, (int)hp, fold_cg, bg);
+            HIP_TRY(hipGetLastError());
+            const int64_t folded = op.chan_in * nf;
+            const unsigned g = (unsigned)((folded + 255) / 256);
+            fold_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(img_b, img_p, (int)hw, (int)hp, op.chan_in, (int)nb, folded);
+            HIP_TRY(hipGetLastError());
+            fold_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(grad_img_b, grad_img_p, (int)hw, (int)hp, op.chan_in, (int)nb, folded);
+            HIP_TRY(hipGetLastError());
+            {   // grad_img (C, B * hp) += filters^T (C, O*K*K) . patches (O*K*K, B * hp); the copy started from grad_img: one rounding
+                const int64_t m = cg, k = og * kk;
+                dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, nf);
+                d.accumulate = 1;
+                d.a = f_tr; d.a_rs = k; d.a_cs = 1;
+                d.b = patches; d.b_rs = nf; d.b_cs = 1;
+                d.c = grad_img_p; d.c_rs = nf; d.c_cs = 1;
+                if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+            }
+            const int64_t total = nb * op.chan_in * hw;
+            unfold_rows_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(grad_img_p, grad_img_b, (int)hw, (int)hp, op.chan_in, (int)nb, total);
+            HIP_TRY(hipGetLastError());
+            {   // grad_filters^T (C, O*K*K) += img (C, B * hp) . patches^T (B * hp, O*K*K)
+                const int64_t m = cg, n = og * kk;
+                dfdx_rocm_gemm_desc d = blank_desc(dtype, m, nf, n);
+                d.accumulate = b0 > 0;
+                d.a = img_p; d.a_rs = nf; d.a_cs = 1;
+                d.b = patches; d.b_rs = 1; d.b_cs = nf;
+                d.c = grad_f_tr; d.c_rs = n; d.c_cs = 1;
+                if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+            }
+            continue;
+        }
         if (planes && op.kernel == 3) unfold_output_plane_kernel<T, 3><<<slabs / 9, 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
         else if (planes) unfold_output_plane_kernel<T, 0><<<(unsigned)(slabs / kk), 256, 0, ctx->stream>>>(sub, go, patches, (int)hp);
         else {
@@ -495,7 +724,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
             // grad_filters^T (C/G, O/G*K*K) += sum over images of img (C/G, H*W) . patches^T (H*W, O/G*K*K)
             const int64_t m = cg, k = hp, n = og * kk;
             dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
-            d.accumulate = 1;
+            d.accumulate = b0 > 0;
             d.reduce_batch = 1;
             d.batch1 = nb;
             d.a = (padded ? (const T *)img_p : img_b) + g * cg * k; d.a_rs = k; d.a_cs = 1; d.a_b1 = op.chan_in * k;
@@ -504,7 +733,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
             if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
         }
     }
-    filter_transpose_kernel<T, true><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)grad_filters, grad_f_tr, (int)f_elems);
+    filter_transpose_kernel<T, true><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)grad_filters, grad_f_tr, magic_kk);
     return (int)hipGetLastError();
 }
 
