@@ -317,6 +317,45 @@ __global__ __launch_bounds__(256) void filter_transpose_kernel(Op op, T *filters
     if constexpr (ADD_BACK) Elem<T>::store(f, Elem<T>::load(f) + Elem<T>::load(t));
     else *t = *f;
 }
+// The same through LDS in tiles of 16 output x 16 input channels (whole tiles only): both sides are then read and written
+// in runs of 16 K*K contiguous elements, where the kernel above leaves K*K-element pieces a whole filter row apart on the
+// transposed side (512 -> 512 channels, 3 x 3: 8.8 us for 4.7 MB).  blockIdx = (tile of input channels, tile of output
+// channels, group); dynamic LDS: 256 K*K elements.
+template <typename T, bool ADD_BACK>
+__global__ __launch_bounds__(256) void filter_transpose_tiled_kernel(Op op, T *filters, T *transposed, uint32_t magic_kk, uint32_t magic_16kk) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t tile_raw[];
+    T *const tile = (T *)tile_raw;  // [16 output channels][16 input channels][K*K]
+    const int kk = op.kernel * op.kernel, og = op.chan_out / op.groups, cg = op.chan_in / op.groups;
+    const int run = 16 * kk, c0 = blockIdx.x * 16, o0 = blockIdx.y * 16, g = blockIdx.z;
+    T *const f0 = filters + ((int64_t)(g * og + o0) * cg + c0) * kk;      // + ol * cg * kk + (cl * kk + tap)
+    T *const t0 = transposed + ((int64_t)(g * cg + c0) * og + o0) * kk;   // + cl * og * kk + (ol * kk + tap)
+    if constexpr (!ADD_BACK) {
+        for (uint32_t i = threadIdx.x; i < (uint32_t)(16 * run); i += 256) {
+            const uint32_t ol = __umulhi(i, magic_16kk), r = i - ol * run;
+            tile[i] = f0[(int64_t)ol * cg * kk + r];
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < (uint32_t)(16 * run); i += 256) {
+            const uint32_t cl = __umulhi(i, magic_16kk), r = i - cl * run;  // r = ol * kk + tap
+            const uint32_t ol = kk == 1 ? r : __umulhi(r, magic_kk), tap = r - ol * kk;
+            tile[ol * run + cl * kk + tap] = t0[(int64_t)cl * og * kk + r];
+        }
+    }
+    __syncthreads();
+    if constexpr (!ADD_BACK) {
+        for (uint32_t i = threadIdx.x; i < (uint32_t)(16 * run); i += 256) {
+            const uint32_t cl = __umulhi(i, magic_16kk), r = i - cl * run;
+            const uint32_t ol = kk == 1 ? r : __umulhi(r, magic_kk), tap = r - ol * kk;
+            t0[(int64_t)cl * og * kk + r] = tile[ol * run + cl * kk + tap];
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < (uint32_t)(16 * run); i += 256) {
+            const uint32_t ol = __umulhi(i, magic_16kk), r = i - ol * run;
+            T *f = f0 + (int64_t)ol * cg * kk + r;
+            Elem<T>::store(f, Elem<T>::load(f) + Elem<T>::load(tile + i));
+        }
+    }
+}
 
 // Rows of `len` elements <-> rows padded to `padded` elements (zeros behind the data).  When the spatial size of a
 // product (OH*OW forward, H*W backward) is not a multiple of the GEMM's vector width, the matrices on that side get
@@ -632,7 +671,12 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     // (the scratch gradient is not cleared: the first chunk's product overwrites it)
     const dim3 fgrid((unsigned)op.chan_out, (unsigned)((cg * kk + 255) / 256));
     const uint32_t magic_kk = magic_of(kk);
-    filter_transpose_kernel<T, false><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)const_cast<void *>(filters), f_tr, magic_kk);
+    const bool tiled_tr = cg % 16 == 0 && og % 16 == 0 && 256 * kk * sizeof(T) <= 48 * 1024;
+    const dim3 tgrid((unsigned)(cg / 16), (unsigned)(og / 16), (unsigned)op.groups);
+    const uint32_t magic_16kk = magic_of(16 * kk);
+    if (tiled_tr)
+        filter_transpose_tiled_kernel<T, false><<<tgrid, 256, 256 * kk * sizeof(T), ctx->stream>>>(op, (T *)const_cast<void *>(filters), f_tr, magic_kk, magic_16kk);
+    else filter_transpose_kernel<T, false><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)const_cast<void *>(filters), f_tr, magic_kk);
     HIP_TRY(hipGetLastError());
     const bool planes = op.stride == 1 && op.w_in % V == 0 && op.w_out >= V && (hw / V) * kk >= 512;
     for (int64_t b0 = 0; b0 < op.batch; b0 += chunk) {
@@ -733,7 +777,8 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
             if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
         }
     }
-    filter_transpose_kernel<T, true><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)grad_filters, grad_f_tr, magic_kk);
+    if (tiled_tr) filter_transpose_tiled_kernel<T, true><<<tgrid, 256, 256 * kk * sizeof(T), ctx->stream>>>(op, (T *)grad_filters, grad_f_tr, magic_kk, magic_16kk);
+    else filter_transpose_kernel<T, true><<<fgrid, 256, 0, ctx->stream>>>(op, (T *)grad_filters, grad_f_tr, magic_kk);
     return (int)hipGetLastError();
 }
 

@@ -70,6 +70,9 @@ CONFIGS = [
     (2, 3, 64, 30, 30, 3, 2, 1, 1, 1),     # the same through the patch matrix (stride 2), 15 x 15 = 225 output pixels
     (3, 128, 96, 20, 14, 3, 1, 1, 1, 1),   # image gradient on the band kernel (two blocks of 64 channels out of 3 chunks of 32), forward on the tiles
     (2, 64, 32, 9, 112, 3, 1, 1, 1, 1),    # the same with one chunk, rows of 112 pixels; H * W = 1008 is off the 64-element grid of the filter gradient
+    (9, 20, 24, 6, 10, 5, 1, 2, 1, 1),     # small images as one product over the batch: 9 images (a group of 8 and one), channels off the workgroups' groups
+    (3, 16, 16, 10, 10, 3, 1, 2, 2, 1),    # the same with dilation
+    (5, 32, 32, 7, 7, 3, 1, 1, 1, 1),      # 7 x 7: rows of 49 padded to 56 / 64 inside the folded matrices; tiled filter transposes
 ]
 
 
