@@ -161,64 +161,14 @@ __global__ __launch_bounds__(256) void unfold_output_flat_kernel(Op op, const T 
     }
 }
 
-// The flat kernels for small planes (a 7 x 7 image: rows too short for a window load, every element its own 2-byte load,
-// and seven integer divisions per thread: 33 MB of patches took 21 us, bound by the instruction count).  A workgroup first
-// copies the few consecutive planes its 256 vectors draw on into LDS -- one coalesced read -- and gathers from there; what
-// a lane divides is small (an index inside the workgroup's run of vectors, slabs and planes -- the run's origin is divided
-// once, on the scalar unit), so the quotients come from a multiplication with ceil(2^32 / d).  Same patch layout, same zeros.
-struct SmallDivs {  // ceil(2^32 / d) for the divisors of the staged kernels (0 where d = 1)
+// Divisions of small numbers by launch-time constants go through a multiplication with ceil(2^32 / d): exact while
+// n * d < 2^32.
+struct SmallDivs {  // ceil(2^32 / d) for the divisors of unfold_small_kernel (0 where d = 1)
     uint32_t per_slab, kernel, kk, chan, width, stride, plane, bg;
 };
 __device__ __forceinline__ uint32_t small_div(uint32_t n, uint32_t d, uint32_t magic) { return d == 1 ? n : __umulhi(n, magic); }
 inline uint32_t magic_of(int64_t d) { return d <= 1 ? 0u : (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d); }
 
-template <typename T, bool OUTPUT_SIDE>
-__global__ __launch_bounds__(256) void unfold_staged_kernel(Op op, SmallDivs mg, const T *src, T *patches, int slab_stride, uint32_t vectors, int fold) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t staged_raw[];
-    T *const staged = (T *)staged_raw;
-    constexpr int V = Elem<T>::VEC;
-    // input side: slabs of the image over output positions; output side: slabs of grad_out over image positions
-    const int src_h = OUTPUT_SIDE ? op.h_out : op.h_in, src_w = OUTPUT_SIDE ? op.w_out : op.w_in;
-    const int pos_w = OUTPUT_SIDE ? op.w_in : op.w_out, n = OUTPUT_SIDE ? op.h_in * op.w_in : op.h_out * op.w_out;
-    const int chan = OUTPUT_SIDE ? op.chan_out : op.chan_in;
-    const uint32_t per_slab = (uint32_t)slab_stride / V;
-    const int kk = op.kernel * op.kernel, plane_elems = src_h * src_w;
-    const uint32_t first = blockIdx.x * 256, last = min(first + 255u, vectors - 1);
-    const uint32_t slab0 = first / per_slab, plane0 = slab0 / kk, plane1 = last / per_slab / kk, image0 = plane0 / chan;
-    const int count = (int)(plane1 - plane0 + 1) * plane_elems;
-    for (int i = threadIdx.x; i < count; i += 256) staged[i] = src[(int64_t)plane0 * plane_elems + i];
-    __syncthreads();
-    if (first + threadIdx.x >= vectors) return;
-    const uint32_t in_run = first - slab0 * per_slab + threadIdx.x;                 // < 256 + per_slab
-    const uint32_t slab_in_run = small_div(in_run, per_slab, mg.per_slab);
-    const uint32_t slab_in_plane0 = slab0 - plane0 * kk + slab_in_run;               // < 2 K K + 256
-    const uint32_t plane_in_run = small_div(slab_in_plane0, kk, mg.kk);
-    const uint32_t tap = slab_in_plane0 - plane_in_run * kk;
-    const int k1 = (int)small_div(tap, op.kernel, mg.kernel), k2 = (int)tap - k1 * op.kernel;
-    const T *plane = staged + plane_in_run * plane_elems;
-    const uint32_t chan_in_image0 = plane0 - image0 * chan + plane_in_run;           // < channels + 258
-    const uint32_t image_in_run = small_div(chan_in_image0, chan, mg.chan);
-    const uint32_t image = image0 + image_in_run, c = chan_in_image0 - image_in_run * chan;
-    const int64_t slab_dst = fold ? (int64_t)(c * kk + tap) * op.batch + image : (int64_t)slab0 + slab_in_run;
-    const int pos0 = (int)(in_run - slab_in_run * per_slab) * V;
-    int row = (int)small_div(pos0, pos_w, mg.width), col = pos0 - row * pos_w;
-    float v[V];
-#pragma unroll
-    for (int i = 0; i < V; i++) {
-        if constexpr (OUTPUT_SIDE) {
-            const int oh = row + op.padding - op.dilation * k1, ow = col + op.padding - op.dilation * k2;
-            const int qh = oh >= 0 ? (int)small_div(oh, op.stride, mg.stride) : 0, qw = ow >= 0 ? (int)small_div(ow, op.stride, mg.stride) : 0;
-            const bool ok = pos0 + i < n && oh >= 0 && qh * op.stride == oh && qh < src_h && ow >= 0 && qw * op.stride == ow && qw < src_w;
-            v[i] = ok ? Elem<T>::load(plane + qh * src_w + qw) : 0.0f;
-        } else {
-            const int y = row * op.stride + op.dilation * k1 - op.padding, x = col * op.stride + op.dilation * k2 - op.padding;
-            const bool ok = pos0 + i < n && y >= 0 && y < src_h && x >= 0 && x < src_w;
-            v[i] = ok ? Elem<T>::load(plane + y * src_w + x) : 0.0f;
-        }
-        if (++col == pos_w) { col = 0; ++row; }
-    }
-    store_elems<T, V>(patches + slab_dst * slab_stride + pos0, v);
-}
 // Position-major gather for small planes into the FOLDED patch matrix [chan K K][batch * slab_stride]: a thread owns one
 // vector of positions of one plane and walks the K x K taps itself, so the index arithmetic of its V positions is done once
 // for all taps (a tap only shifts the source coordinates) and a vector costs ~70 instructions instead of ~250.  A workgroup
@@ -294,14 +244,6 @@ template <typename T> bool small_unfold_shape(int64_t slab_stride, int64_t plane
     return true;
 }
 
-// LDS bytes the staged kernels need for planes of `plane_elems` elements, or 0 when they should not be used
-template <typename T> size_t staged_lds_bytes(int64_t slab_stride, int64_t kk, int64_t plane_elems) {
-    const int64_t per_slab = slab_stride / Elem<T>::VEC;
-    const int64_t planes = 255 / per_slab / kk + 2;  // a run of 256 vectors starts and ends inside a plane
-    const int64_t bytes = planes * plane_elems * (int64_t)sizeof(T);
-    return bytes <= 32 * 1024 ? (size_t)((bytes + 15) & ~15ll) : 0;
-}
-
 // filters (G*O/G, C/G, K, K) <-> transposed (G, C/G, O/G, K*K).  ADD_BACK: filters[..] += transposed[..].
 template <typename T, bool ADD_BACK>
 __global__ __launch_bounds__(256) void filter_transpose_kernel(Op op, T *filters, T *transposed, uint32_t magic_kk) {
@@ -375,23 +317,30 @@ template <typename T> __global__ __launch_bounds__(256) void unpad_rows_kernel(c
     dst[i] = src[row * padded + (i - row * len)];
 }
 
-// dst [batch][rows][len] = src [rows][batch][padded]: the product over a folded patch matrix, image by image
-template <typename T> __global__ __launch_bounds__(256) void unfold_rows_kernel(const T *src, T *dst, int len, int padded, int rows, int batch, int64_t total) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into dst
+// The two kernels that move an image-side tensor [batch][rows][len] into and out of the folded layout
+// [rows][batch][padded] (padded < 256; zeros behind every row).  A thread handles one element of the tensor the kernel
+// writes; the only per-lane divisions are of small numbers (an index inside the workgroup's run of 256 elements; the run's
+// origin is divided once, on the scalar unit) and go through a multiplication.
+struct FoldDivs { uint32_t len, padded, rows, batch; };  // ceil(2^32 / d), 0 for d = 1
+template <typename T> __global__ __launch_bounds__(256) void unfold_rows_kernel(const T *src, T *dst, int len, int padded, int rows, int batch, FoldDivs mg, uint32_t total) {
+    const uint32_t first = blockIdx.x * 256, i = first + threadIdx.x;  // index into dst [batch][rows][len]
     if (i >= total) return;
-    const int64_t line = i / len;  // = image * rows + row
-    const int64_t b = line / rows, r = line - b * rows;
-    dst[i] = src[(r * batch + b) * padded + (i - line * len)];
+    const uint32_t line0 = first / (uint32_t)len, image0 = line0 / (uint32_t)rows;
+    const uint32_t in_run = first - line0 * len + threadIdx.x;           // < 256 + len
+    const uint32_t dl = small_div(in_run, len, mg.len), col = in_run - dl * len;
+    const uint32_t row_in_image0 = line0 - image0 * rows + dl;           // < rows + 256
+    const uint32_t db = small_div(row_in_image0, rows, mg.rows), r = row_in_image0 - db * rows, b = image0 + db;
+    dst[i] = src[((int64_t)r * batch + b) * padded + col];
 }
-
-// dst [rows][batch][padded] = src [batch][rows][len], zeros behind every row: an image-side matrix of the folded products
-template <typename T> __global__ __launch_bounds__(256) void fold_rows_kernel(const T *src, T *dst, int len, int padded, int rows, int batch, int64_t total) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into dst
+template <typename T> __global__ __launch_bounds__(256) void fold_rows_kernel(const T *src, T *dst, int len, int padded, int rows, int batch, FoldDivs mg, uint32_t total) {
+    const uint32_t first = blockIdx.x * 256, i = first + threadIdx.x;  // index into dst [rows][batch][padded]
     if (i >= total) return;
-    const int64_t line = i / padded;  // = row * batch + image
-    const int col = (int)(i - line * padded);
-    const int64_t r = line / batch, b = line - r * batch;
-    if (col < len) dst[i] = src[(b * rows + r) * len + col];
+    const uint32_t line0 = first / (uint32_t)padded, row0 = line0 / (uint32_t)batch;
+    const uint32_t in_run = first - line0 * padded + threadIdx.x;        // < 256 + padded
+    const uint32_t dl = small_div(in_run, padded, mg.padded), col = in_run - dl * padded;
+    const uint32_t image_in_row0 = line0 - row0 * batch + dl;            // < batch + 256
+    const uint32_t dr = small_div(image_in_row0, batch, mg.batch), b = image_in_row0 - dr * batch, r = row0 + dr;
+    if (col < (uint32_t)len) dst[i] = src[((int64_t)b * rows + r) * len + col];
     else Elem<T>::store(dst + i, 0.0f);
 }
 
@@ -505,7 +454,8 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
     // Small images (a 7 x 7 output is n = 49: a quarter of one 256-column tile per image) multiply as ONE product over the
     // batch: the patch matrix is written [C K K][batch * np], the product lands in [O][batch * np] and a small kernel
     // hands every image its rows.  The filters are then read once per tile row instead of once per image.
-    const bool fold = !pointwise && op.groups == 1 && np < 256 && op.batch > 1;
+    const bool fold = !pointwise && op.groups == 1 && np < 256 && op.batch > 1 && op.chan_in <= 32768 && op.chan_out <= 32768 &&
+                      chunk <= 32768 && chunk * std::max(op.chan_in, op.chan_out) * np < (1ll << 31);
     const size_t patch_bytes = pointwise ? 0 : round256((size_t)(chunk * per_image) * sizeof(T));
     const size_t out_bytes = (padded || fold) ? round256((size_t)(chunk * op.chan_out * np) * sizeof(T)) : 0;
     if (int rc = ensure_patches(ctx, patch_bytes + out_bytes)) return rc;
@@ -544,7 +494,8 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
             d.c = out_p; d.c_rs = nb * np; d.c_cs = 1;
             if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
             const int64_t total = nb * op.chan_out * n;
-            unfold_rows_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(out_p, dst, (int)n, (int)np, op.chan_out, (int)nb, total);
+            const FoldDivs fd{magic_of(n), magic_of(np), magic_of(op.chan_out), magic_of(nb)};
+            unfold_rows_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(out_p, dst, (int)n, (int)np, op.chan_out, (int)nb, fd, (uint32_t)total);
             HIP_TRY(hipGetLastError());
             continue;
         }
@@ -596,7 +547,8 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     // gradient is a plain product with k = batch * hp.
     int fold_cg = 0, fold_bg = 0;
     size_t fold_lds = 0;
-    const bool fold = !pointwise && op.groups == 1 && op.stride == 1 && hp < 256 && op.batch > 1 &&
+    const bool fold = !pointwise && op.groups == 1 && op.stride == 1 && hp < 256 && op.batch > 1 && op.chan_in <= 32768 && op.chan_out <= 32768 &&
+                      chunk <= 32768 && chunk * std::max(op.chan_in, op.chan_out) * hp < (1ll << 31) &&
                       small_unfold_shape<T>(hp, ohw, (int)std::min<int64_t>(chunk, op.batch), &fold_cg, &fold_bg, &fold_lds);
     const size_t img_bytes = (padded || fold) ? round256((size_t)(chunk * op.chan_in * hp) * sizeof(T)) : 0;
     // The image gradient of a 3 x 3, unit-stride, padding-1 convolution is such a convolution of grad_out (filters turned
@@ -697,9 +649,10 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
             HIP_TRY(hipGetLastError());
             const int64_t folded = op.chan_in * nf;
             const unsigned g = (unsigned)((folded + 255) / 256);
-            fold_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(img_b, img_p, (int)hw, (int)hp, op.chan_in, (int)nb, folded);
+            const FoldDivs fd{magic_of(hw), magic_of(hp), magic_of(op.chan_in), magic_of(nb)};
+            fold_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(img_b, img_p, (int)hw, (int)hp, op.chan_in, (int)nb, fd, (uint32_t)folded);
             HIP_TRY(hipGetLastError());
-            fold_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(grad_img_b, grad_img_p, (int)hw, (int)hp, op.chan_in, (int)nb, folded);
+            fold_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(grad_img_b, grad_img_p, (int)hw, (int)hp, op.chan_in, (int)nb, fd, (uint32_t)folded);
             HIP_TRY(hipGetLastError());
             {   // grad_img (C, B * hp) += filters^T (C, O*K*K) . patches (O*K*K, B * hp); the copy started from grad_img: one rounding
                 const int64_t m = cg, k = og * kk;
@@ -711,7 +664,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
                 if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
             }
             const int64_t total = nb * op.chan_in * hw;
-            unfold_rows_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(grad_img_p, grad_img_b, (int)hw, (int)hp, op.chan_in, (int)nb, total);
+            unfold_rows_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(grad_img_p, grad_img_b, (int)hw, (int)hp, op.chan_in, (int)nb, fd, (uint32_t)total);
             HIP_TRY(hipGetLastError());
             {   // grad_filters^T (C, O*K*K) += img (C, B * hp) . patches^T (B * hp, O*K*K)
                 const int64_t m = cg, n = og * kk;
