@@ -226,40 +226,41 @@ __global__ __launch_bounds__(NTH, 3) void conv3x3_wgrad_kernel(const Params p) {
     }
 }
 
-// grad_filters[o][c][tap] += sum over the slices of their shares (f32), rounded once.  A workgroup owns 32 consecutive sums;
-// its 8 thread groups add an eighth of the slices each, in slice order, and the eight subtotals meet in LDS in group order:
-// one fixed summation order, whatever the timing.
+// grad_filters[o][c][tap] += sum over the slices of their shares (f32), rounded once.  A workgroup owns 128 consecutive
+// sums (32 lanes x 4 sums: 512 contiguous bytes of every share per load); its 8 thread groups add an eighth of the slices
+// each, in slice order, and the eight subtotals meet in LDS in group order: one fixed summation order, whatever the timing.
 template <typename T>
 __global__ __launch_bounds__(256) void conv3x3_wgrad_reduce_kernel(const float *__restrict__ partial,
                                                                    typename StoredAs<T>::type *__restrict__ grad_filters, int C,
                                                                    int cblocks, int combos, int slices, int total) {
-    __shared__ float subtotal[8][32];
+    __shared__ f32x4 subtotal[8][32];
     const int lane_elem = threadIdx.x % 32, group = threadIdx.x / 32;
-    const int i = blockIdx.x * 32 + lane_elem;  // (combo, tap, o, c), c fastest; total is a multiple of 32
+    const int i = blockIdx.x * 128 + lane_elem * 4;  // (combo, tap, o, c), c fastest; total is a multiple of 128
     const int combo = i / (9 * 4096), within = i - combo * (9 * 4096);
     const int per = (slices + 7) / 8, s0 = group * per, s1 = min(slices, s0 + per);
     const float *src = partial + (int64_t)combo * (9 * 4096) + within;
     const int64_t step = (int64_t)combos * (9 * 4096);
-    float sum = 0.0f;
+    f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
     int s = s0;
     for (; s + 8 <= s1; s += 8) {
-        float v[8];
+        f32x4 v[8];
 #pragma unroll
-        for (int e = 0; e < 8; e++) v[e] = src[(s + e) * step];
+        for (int e = 0; e < 8; e++) v[e] = *(const f32x4 *)(src + (s + e) * step);
 #pragma unroll
         for (int e = 0; e < 8; e++) sum += v[e];
     }
-    for (; s < s1; s++) sum += src[s * step];
+    for (; s < s1; s++) sum += *(const f32x4 *)(src + s * step);
     subtotal[group][lane_elem] = sum;
     __syncthreads();
     if (group == 0 && i < total) {
-        float all = subtotal[0][lane_elem];
+        f32x4 all = subtotal[0][lane_elem];
 #pragma unroll
         for (int g = 1; g < 8; g++) all += subtotal[g][lane_elem];
         const int c = within % 64, o = (within / 64) % 64, tap = within / 4096;
         const int cb = combo % cblocks, ob = combo / cblocks;
         typename StoredAs<T>::type *dst = grad_filters + ((int64_t)(ob * 64 + o) * C + cb * 64 + c) * 9 + tap;
-        *dst = MmaW<T>::from_f32(MmaW<T>::to_f32(*dst) + all);
+#pragma unroll
+        for (int e = 0; e < 4; e++) dst[9 * e] = MmaW<T>::from_f32(MmaW<T>::to_f32(dst[9 * e]) + all[e]);
     }
 }
 
@@ -532,7 +533,7 @@ hipError_t launch_conv3x3_wgrad_f32(const Conv3x3Problem &c, const PlanF &pl, vo
     }
     conv3x3_wgrad_f32_kernel<<<(unsigned)(pl.combos * pl.slices), NTH, pl.lds, stream>>>(p);
     const int total = pl.combos * 9 * 4096;
-    conv3x3_wgrad_reduce_kernel<float><<<total / 32, 256, 0, stream>>>((const float *)workspace, (float *)c.filters, c.chan_in, p.cblocks,
+    conv3x3_wgrad_reduce_kernel<float><<<total / 128, 256, 0, stream>>>((const float *)workspace, (float *)c.filters, c.chan_in, p.cblocks,
                                                                         pl.combos, pl.slices, total);
     return hipGetLastError();
 }
@@ -564,7 +565,7 @@ hipError_t launch_conv3x3_wgrad(const Conv3x3Problem &c, int compute_units, void
         }                                                                                                              \
         conv3x3_wgrad_kernel<T><<<grid, NTH, pl.lds, stream>>>(p);                                                     \
         const int total = pl.combos * 9 * 4096;                                                                        \
-        conv3x3_wgrad_reduce_kernel<T><<<total / 32, 256, 0, stream>>>((const float *)workspace, (uint16_t *)c.filters, c.chan_in, \
+        conv3x3_wgrad_reduce_kernel<T><<<total / 128, 256, 0, stream>>>((const float *)workspace, (uint16_t *)c.filters, c.chan_in, \
                                                                                p.cblocks, pl.combos, pl.slices, total); \
     } while (0)
     if (c.dtype == DT_F16) DFDX_WGRAD(_Float16);
