@@ -310,6 +310,27 @@ template <typename T> __global__ __launch_bounds__(256) void pad_rows_kernel(con
     if (col < len) dst[i] = src[row * len + col];
     else Elem<T>::store(dst + i, 0.0f);
 }
+// The same in whole 16-byte vectors (len and padded multiples of the vector, aligned buffers): a thread per vector of dst.
+template <typename T> __global__ __launch_bounds__(256) void pad_rows_vec_kernel(const T *src, T *dst, int len_v, int padded_v, int64_t total_v) {
+    constexpr int V = Elem<T>::VEC;
+    struct __attribute__((aligned(16))) Vec { T e[V]; };
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // vector index into dst
+    if (i >= total_v) return;
+    const int64_t row = i / padded_v;
+    const int col = (int)(i - row * padded_v);
+    Vec v;
+    if (col < len_v) v = ((const Vec *)src)[row * len_v + col];
+    else
+#pragma unroll
+        for (int e = 0; e < V; e++) v.e[e] = (T)0.0f;
+    ((Vec *)dst)[i] = v;
+}
+template <typename T> void launch_pad_rows(const T *src, T *dst, int64_t len, int64_t padded, int64_t total, hipStream_t stream) {
+    constexpr int V = Elem<T>::VEC;
+    if (len % V == 0 && padded % V == 0 && (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0)
+        pad_rows_vec_kernel<T><<<(unsigned)((total / V + 255) / 256), 256, 0, stream>>>(src, dst, (int)(len / V), (int)(padded / V), total / V);
+    else pad_rows_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(src, dst, (int)len, (int)padded, total);
+}
 template <typename T> __global__ __launch_bounds__(256) void unpad_rows_kernel(const T *src, T *dst, int len, int padded, int64_t total) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into dst
     if (i >= total) return;
@@ -515,6 +536,176 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
     return DFDX_ROCM_OK;
 }
 
+// grad_img[b][c][y][x] += sum over the taps (k1, k2) whose window position is whole --
+//   oh = (y + padding - dilation k1) / stride, ow = (x + padding - dilation k2) / stride, inside the output --
+// of grad_patches[b][c K K + k1 K + k2][oh W_out + ow]: the gather form of col2im, one thread per image pixel, f32 sum,
+// one rounding.  blockIdx.x = plane (b, c), blockIdx.y = block of 256 pixels.
+template <typename T>
+__global__ __launch_bounds__(256) void fold_patches_kernel(Op op, const T *grad_patches, T *grad_img, int slab_stride, uint32_t magic_w, uint32_t magic_s) {
+    const int hw = op.h_in * op.w_in, pos = blockIdx.y * 256 + threadIdx.x;
+    if (pos >= hw) return;
+    const int kk = op.kernel * op.kernel;
+    const int y = (int)small_div(pos, op.w_in, magic_w), x = pos - y * op.w_in;
+    const T *slabs = grad_patches + (int64_t)blockIdx.x * kk * slab_stride;
+    float sum = 0.0f;
+    for (int k1 = 0; k1 < op.kernel; k1++) {
+        const int ty = y + op.padding - op.dilation * k1;
+        if (ty < 0) break;  // (larger k1: further up)
+        const int oh = (int)small_div(ty, op.stride, magic_s);
+        if (oh * op.stride != ty || oh >= op.h_out) continue;
+        for (int k2 = 0; k2 < op.kernel; k2++) {
+            const int tx = x + op.padding - op.dilation * k2;
+            if (tx < 0) break;
+            const int ow = (int)small_div(tx, op.stride, magic_s);
+            if (ow * op.stride != tx || ow >= op.w_out) continue;
+            sum += Elem<T>::load(slabs + (int64_t)(k1 * op.kernel + k2) * slab_stride + oh * op.w_out + ow);
+        }
+    }
+    T *dst = grad_img + (int64_t)blockIdx.x * hw + pos;
+    Elem<T>::store(dst, Elem<T>::load(dst) + sum);
+}
+
+// The same for stride S in cells of S x S image pixels, one thread per cell: every tap lands on exactly ONE pixel of a cell --
+// row (dilation k1 - padding) mod S of it, from window row cell_row + (that row + padding - dilation k1) / S -- so no lane
+// tests divisibility or divides, the lanes of a wave read consecutive window positions of one tap, and which pixel of the
+// cell a tap belongs to is the same for the whole wave (the per-pixel kernel: 160 us for 64 x 64 planes of 56 x 56).
+template <typename T, int S>
+__global__ __launch_bounds__(256) void fold_patches_cells_kernel(Op op, const T *grad_patches, T *grad_img, int slab_stride, int cells_w, int cells, uint32_t magic_cw) {
+    const int cell = blockIdx.y * 256 + threadIdx.x;
+    if (cell >= cells) return;
+    const int cy = (int)small_div(cell, cells_w, magic_cw), cx = cell - cy * cells_w;
+    const T *slabs = grad_patches + (int64_t)blockIdx.x * op.kernel * op.kernel * slab_stride;
+    float acc[S][S];
+#pragma unroll
+    for (int a = 0; a < S; a++)
+#pragma unroll
+        for (int b = 0; b < S; b++) acc[a][b] = 0.0f;
+    for (int k1 = 0; k1 < op.kernel; k1++) {
+        const int shift_y = op.dilation * k1 - op.padding;
+        const int ry = ((shift_y % S) + S) % S;       // the cell row this tap row lands on
+        const int oh = cy + (ry - shift_y) / S;       // exact: ry = shift_y (mod S)
+        if (oh < 0 || oh >= op.h_out) continue;
+        for (int k2 = 0; k2 < op.kernel; k2++) {
+            const int shift_x = op.dilation * k2 - op.padding;
+            const int rx = ((shift_x % S) + S) % S;
+            const int ow = cx + (rx - shift_x) / S;
+            const float v = (ow >= 0 && ow < op.w_out) ? Elem<T>::load(slabs + (int64_t)(k1 * op.kernel + k2) * slab_stride + oh * op.w_out + ow) : 0.0f;
+#pragma unroll
+            for (int a = 0; a < S; a++)
+#pragma unroll
+                for (int b = 0; b < S; b++) acc[a][b] += (a == ry && b == rx) ? v : 0.0f;
+        }
+    }
+    T *plane = grad_img + (int64_t)blockIdx.x * op.h_in * op.w_in;
+    if (S == 2 && op.w_in % 2 == 0 && (((uintptr_t)grad_img) & (2 * sizeof(T) - 1)) == 0) {
+        // the two pixels of a cell row as one access (rows of even length: every pair is aligned)
+        struct __attribute__((aligned(2 * sizeof(T)))) Pair { T e[2]; };
+#pragma unroll
+        for (int a = 0; a < S; a++) {
+            const int y = cy * S + a;
+            if (y < op.h_in) {
+                Pair *q = (Pair *)(plane + y * op.w_in + cx * S);
+                Pair v = *q;
+                Elem<T>::store(&v.e[0], Elem<T>::load(&v.e[0]) + acc[a][0]);
+                Elem<T>::store(&v.e[1], Elem<T>::load(&v.e[1]) + acc[a][S - 1]);
+                *q = v;
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int a = 0; a < S; a++)
+#pragma unroll
+        for (int b = 0; b < S; b++) {
+            const int y = cy * S + a, x = cx * S + b;
+            if (y < op.h_in && x < op.w_in) Elem<T>::store(plane + y * op.w_in + x, Elem<T>::load(plane + y * op.w_in + x) + acc[a][b]);
+        }
+}
+
+// Backward pass of a strided convolution.  The general form below gathers grad_out into a patch matrix over the INPUT
+// positions, [O K K][H W]: at stride s only one position in s*s holds a value, so that matrix is s*s times larger than
+// the forward one, mostly zeros, and both products multiply the zeros (64 -> 128 channels, 3 x 3, stride 2 at 56 x 56:
+// 650 us against 61 forward; the 7 x 7 / stride-2 first layer of a residual network at 224 x 224: 27 ms against 0.34).
+// Here both gradients come from the FORWARD patch matrix of the image, [C K K][OH OW], which has no such zeros:
+//   grad_filters (O, C K K) += sum over images of grad_out (O, OH OW) . patches^T          -- in the filters' own layout
+//   grad_patches (C K K, OH OW) = filters^T (C K K, O) . grad_out (O, OH OW)                -- filters transposed by strides
+//   grad_img += the gather form of col2im of grad_patches (fold_patches_kernel)
+// The image gradient's partial sums per tap are rounded to the element type before the taps are added (in f32, with the
+// old gradient, one rounding): within the tolerance of the product, not bit-identical to the general form.
+template <typename T>
+int strided_backward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *img, void *grad_img, const void *filters, void *grad_filters,
+                     const void *grad_out) {
+    constexpr int V = Elem<T>::VEC;
+    const int64_t kk = (int64_t)op.kernel * op.kernel, hw = (int64_t)op.h_in * op.w_in, ohw = (int64_t)op.h_out * op.w_out;
+    const int64_t align = sizeof(T) == 2 ? 64 : V;  // OH*OW is the k of the filter-gradient product (split-k wants whole k tiles)
+    const int64_t np = (ohw + align - 1) / align * align;
+    const int64_t cg = op.chan_in / op.groups, og = op.chan_out / op.groups;
+    const int64_t per_image = (int64_t)op.chan_in * kk * np;
+    if (per_image == 0 || og == 0) return DFDX_ROCM_OK;
+    if (per_image >= (1ll << 31) || (int64_t)op.chan_out * np >= (1ll << 31) || hw * op.w_in >= (1ll << 32) || hw > 65535ll * 256)
+        return DFDX_ROCM_ERR_UNSUPPORTED;
+    CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
+    int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
+    chunk = std::min<int64_t>(std::min<int64_t>(chunk, op.batch), ((1ll << 31) - 1) / std::max<int64_t>(per_image, (int64_t)op.chan_out * np));
+    const bool padded = np != ohw;
+    const size_t patch_bytes = round256((size_t)(chunk * per_image) * sizeof(T));
+    const size_t go_bytes = padded ? round256((size_t)(chunk * op.chan_out * np) * sizeof(T)) : 0;
+    if (int rc = ensure_patches(ctx, patch_bytes + go_bytes)) return rc;
+    T *patches = (T *)ctx->patches;
+    T *go_p = (T *)((char *)ctx->patches + patch_bytes);
+    const uint32_t magic_w = magic_of(op.w_in), magic_s = magic_of(op.stride);
+    for (int64_t b0 = 0; b0 < op.batch; b0 += chunk) {
+        const int64_t nb = std::min<int64_t>(chunk, op.batch - b0);
+        Op sub = op;
+        sub.batch = (int)nb;
+        const T *img_b = (const T *)img + b0 * op.chan_in * hw;
+        T *grad_img_b = (T *)grad_img + b0 * op.chan_in * hw;
+        const T *go = (const T *)grad_out + b0 * op.chan_out * ohw;
+        const uint32_t vectors = (uint32_t)(nb * op.chan_in * kk * (np / V));
+        unfold_input_flat_kernel<T><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, img_b, patches, (int)np, vectors, 0);
+        HIP_TRY(hipGetLastError());
+        if (padded) {
+            const int64_t rows_p = nb * op.chan_out * np;
+            launch_pad_rows<T>(go, go_p, ohw, np, rows_p, ctx->stream);
+            HIP_TRY(hipGetLastError());
+            go = go_p;
+        }
+        for (int g = 0; g < op.groups; g++) {  // grad_filters (O/G, C/G K K) += sum over images of grad_out . patches^T
+            const int64_t m = og, k = np, n = cg * kk;
+            dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
+            d.accumulate = 1;
+            d.reduce_batch = 1;
+            d.batch1 = nb;
+            d.a = go + g * m * k; d.a_rs = k; d.a_cs = 1; d.a_b1 = op.chan_out * k;
+            d.b = patches + g * n * k; d.b_rs = 1; d.b_cs = k; d.b_b1 = per_image;
+            d.c = (T *)grad_filters + g * m * n; d.c_rs = n; d.c_cs = 1;
+            if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+        }
+        {   // grad_patches (B, G, C/G K K, np) = filters^T (G, C/G K K, O/G) . grad_out (B, G, O/G, np), over the patches
+            const int64_t m = cg * kk, k = og, n = np;
+            dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
+            d.batch1 = nb; d.batch2 = op.groups;
+            d.a = filters; d.a_rs = 1; d.a_cs = m; d.a_b1 = 0; d.a_b2 = m * k;
+            d.b = go; d.b_rs = n; d.b_cs = 1; d.b_b1 = op.chan_out * n; d.b_b2 = k * n;
+            d.c = patches; d.c_rs = n; d.c_cs = 1; d.c_b1 = per_image; d.c_b2 = m * n;
+            if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
+        }
+        if (op.stride == 2 || op.stride == 3 || op.stride == 4) {
+            const int S = op.stride, cells_w = (op.w_in + S - 1) / S, cells = cells_w * ((op.h_in + S - 1) / S);
+            const dim3 grid((unsigned)(nb * op.chan_in), (unsigned)((cells + 255) / 256));
+            const uint32_t magic_cw = magic_of(cells_w);
+            if (S == 2) fold_patches_cells_kernel<T, 2><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
+            else if (S == 3) fold_patches_cells_kernel<T, 3><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
+            else fold_patches_cells_kernel<T, 4><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
+        } else {
+            fold_patches_kernel<T><<<dim3((unsigned)(nb * op.chan_in), (unsigned)((hw + 255) / 256)), 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np,
+                                                                                                                           magic_w, magic_s);
+        }
+        HIP_TRY(hipGetLastError());
+    }
+    return DFDX_ROCM_OK;
+}
+
 template <typename T>
 int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad_img, const void *filters, void *grad_filters,
                const void *grad_out) {
@@ -529,6 +720,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     const int64_t per_image = (int64_t)op.chan_out * kk * hp;
     const int64_t f_elems = (int64_t)op.groups * cg * og * kk;
     if (per_image == 0 || f_elems == 0 || ohw == 0) return DFDX_ROCM_OK;
+    if (op.stride > 1) return strided_backward<T>(ctx, dtype, op, img, grad_img, filters, grad_filters, grad_out);
     if (per_image >= (1ll << 31) || f_elems >= (1ll << 31) || (int64_t)op.chan_in * hp >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
     CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
     int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
@@ -689,11 +881,10 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         T *grad_img_b = (T *)grad_img + b0 * op.chan_in * hw;
         const int64_t rows_p = nb * op.chan_in * hp;
         if (padded) {
-            const unsigned g = (unsigned)((rows_p + 255) / 256);
-            pad_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(img_b, img_p, (int)hw, (int)hp, rows_p);
+            launch_pad_rows<T>(img_b, img_p, hw, hp, rows_p, ctx->stream);
             HIP_TRY(hipGetLastError());
             if (!use_band) {
-                pad_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(grad_img_b, grad_img_p, (int)hw, (int)hp, rows_p);
+                launch_pad_rows<T>(grad_img_b, grad_img_p, hw, hp, rows_p, ctx->stream);
                 HIP_TRY(hipGetLastError());
             }
         }
