@@ -73,6 +73,10 @@ CONFIGS = [
     (9, 20, 24, 6, 10, 5, 1, 2, 1, 1),     # small images as one product over the batch: 9 images (a group of 8 and one), channels off the workgroups' groups
     (3, 16, 16, 10, 10, 3, 1, 2, 2, 1),    # the same with dilation
     (5, 32, 32, 7, 7, 3, 1, 1, 1, 1),      # 7 x 7: rows of 49 padded to 56 / 64 inside the folded matrices; tiled filter transposes
+    (2, 16, 32, 48, 48, 3, 2, 1, 1, 1),    # stride 2, 576 output positions: both gradients from the forward patch matrix (position-major gather), 2 x 2 cells
+    (2, 8, 8, 17, 18, 3, 2, 2, 2, 1),      # the same with dilation 2 and an odd height (cells cut by the image's edge)
+    (2, 4, 8, 23, 19, 3, 5, 1, 1, 1),      # stride 5: the per-pixel form of the gather
+    (3, 6, 9, 20, 21, 4, 3, 2, 1, 3),      # stride 3, three groups, an even kernel
 ]
 
 
