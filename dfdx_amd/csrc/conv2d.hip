@@ -663,7 +663,7 @@ __global__ __launch_bounds__(256) void fold_patches_cells_kernel(Op op, const T 
         }
 }
 
-// Backward pass of a strided convolution.  The general form below gathers grad_out into a patch matrix over the INPUT
+// Backward pass of a strided convolution (and of one whose image has few channels).  The general form below gathers grad_out into a patch matrix over the INPUT
 // positions, [O K K][H W]: at stride s only one position in s*s holds a value, so that matrix is s*s times larger than
 // the forward one, mostly zeros, and both products multiply the zeros (64 -> 128 channels, 3 x 3, stride 2 at 56 x 56:
 // 650 us against 61 forward; the 7 x 7 / stride-2 first layer of a residual network at 224 x 224: 27 ms against 0.34).
@@ -734,11 +734,12 @@ int strided_backward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *im
             d.c = patches; d.c_rs = n; d.c_cs = 1; d.c_b1 = per_image; d.c_b2 = m * n;
             if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
         }
-        if (op.stride == 2 || op.stride == 3 || op.stride == 4) {
+        if (op.stride >= 1 && op.stride <= 4) {
             const int S = op.stride, cells_w = (op.w_in + S - 1) / S, cells = cells_w * ((op.h_in + S - 1) / S);
             const dim3 grid((unsigned)(nb * op.chan_in), (unsigned)((cells + 255) / 256));
             const uint32_t magic_cw = magic_of(cells_w);
-            if (S == 2) fold_patches_cells_kernel<T, 2><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
+            if (S == 1) fold_patches_cells_kernel<T, 1><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
+            else if (S == 2) fold_patches_cells_kernel<T, 2><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
             else if (S == 3) fold_patches_cells_kernel<T, 3><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
             else fold_patches_cells_kernel<T, 4><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
         } else {
@@ -764,7 +765,10 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     const int64_t per_image = (int64_t)op.chan_out * kk * hp;
     const int64_t f_elems = (int64_t)op.groups * cg * og * kk;
     if (per_image == 0 || f_elems == 0 || ohw == 0) return DFDX_ROCM_OK;
-    if (op.stride > 1) return strided_backward<T>(ctx, dtype, op, img, grad_img, filters, grad_filters, grad_out);
+    // (also at unit stride when the image has far fewer channels than the output -- a first layer, 3 -> 64: the forward patch
+    // matrix is O / C times smaller than the one over grad_out, and the products with three rows of filters disappear)
+    if (op.stride > 1 || (int64_t)op.chan_in * 4 <= op.chan_out)
+        return strided_backward<T>(ctx, dtype, op, img, grad_img, filters, grad_filters, grad_out);
     if (per_image >= (1ll << 31) || f_elems >= (1ll << 31) || (int64_t)op.chan_in * hp >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
     CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
     int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);

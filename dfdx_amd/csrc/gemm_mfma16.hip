@@ -635,7 +635,7 @@ static int pick_staged(const GemmProblem &p, int compute_units, bool check_suppo
 
 // Split-k of the register-staged family: for products whose tiles leave most of the chip idle while the contraction is
 // long (an LM head's dX off the 16-byte grid: 32 tiles of 256 x 256, k = 50257).  Pieces of at least 4 k tiles, at most
-// 16 of them (64 from 2048 k tiles on), no more than fill the chip once; none may be empty.
+// 16 of them (up to 64 while a piece keeps 16 k tiles), no more than fill the chip once; none may be empty.
 int mfma16_plan_splits(const GemmProblem &p, int variant, int compute_units, int forced_splits) {
     if (variant < 1 || variant > kNumVariants) return 1;
     const Variant &t = kVariants[variant - 1];
@@ -648,8 +648,9 @@ int mfma16_plan_splits(const GemmProblem &p, int variant, int compute_units, int
         s = std::min<int64_t>(forced_splits, total_iters);
     } else {
         const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn);
-        // (a contraction of thousands of k tiles -- a filter gradient summed over a batch of images -- may take 64 pieces)
-        s = std::min<int64_t>({total_iters >= 2048 ? 64 : 16, std::max<int64_t>(1, compute_units / blocks), total_iters / 4});
+        // (a long contraction -- a filter gradient summed over a batch of images -- may take up to 64 pieces of 16+ k tiles)
+        const int64_t pieces = std::max<int64_t>(std::min<int64_t>(16, total_iters / 4), std::min<int64_t>(64, total_iters / 16));
+        s = std::min<int64_t>(pieces, std::max<int64_t>(1, compute_units / blocks));
         if (s < 2) return 1;
     }
     while (!valid(s)) s--;
@@ -688,7 +689,8 @@ int mfma16_skinny_plan(const GemmProblem &p, int compute_units, int forced_split
     if (nbatch != 1 || p.c_cs != 1 || total_iters < 8) return 0;
     const int64_t blocks = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn);
     int64_t s = forced_splits > 0 ? forced_splits
-                                  : std::min<int64_t>({total_iters >= 2048 ? 64 : 16, std::max<int64_t>(1, 2 * (int64_t)compute_units / blocks), total_iters / 4});
+                                  : std::min<int64_t>(std::max<int64_t>(std::min<int64_t>(16, total_iters / 4), std::min<int64_t>(64, total_iters / 16)),
+                                                      std::max<int64_t>(1, 2 * (int64_t)compute_units / blocks));
     s = std::min<int64_t>(s, total_iters);
     while (s > 1 && (s - 1) * ((total_iters + s - 1) / s) >= total_iters) s--;  // no empty piece
     if (s < 2) return 0;
