@@ -489,6 +489,146 @@ bool tiled3x3_forward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *f
     return true;
 }
 
+// ---- depthwise convolutions (one input channel per group: filters [G * M][1][K][K]) ---------------------------------------
+// As products these are G * batch multiplications of an M x K*K matrix with K*K rows of patches -- 8192 launches' worth of
+// 1 x 9 x 784 for 128 channels at 28 x 28 (0.43 ms forward, 4.7 ms backward through the batched GEMM).  They are bound by
+// the bytes of the image and the output instead, so each is computed directly, one thread per element, f32 sums, one rounding:
+//   forward:   out[b][o][oh][ow]  = sum over taps of filters[o][tap] * img[b][o / M][oh s - p + d k1][ow s - p + d k2]
+//   grad_img:  grad_img[b][g][y][x] += sum over m, taps whose window position is whole: filters[g M + m][tap] * grad_out[b][g M + m][oh][ow]
+//   grad_filters[o][tap] += sum over b, oh, ow of grad_out[b][o][oh][ow] * img[b][o / M][...]   (one workgroup per output
+//                           channel, a fixed summation order: deterministic)
+// blockIdx.x = plane, blockIdx.y = block of 256 positions.
+template <typename T>
+__global__ __launch_bounds__(256) void depthwise_forward_kernel(Op op, const T *img, const T *filters, T *out, uint32_t magic_w) {
+    const int n = op.h_out * op.w_out, pos = blockIdx.y * 256 + threadIdx.x;
+    if (pos >= n) return;
+    const int mult = op.chan_out / op.groups, b = blockIdx.x / op.chan_out, o = blockIdx.x - b * op.chan_out;
+    const int oh = (int)small_div(pos, op.w_out, magic_w), ow = pos - oh * op.w_out;
+    const T *plane = img + ((int64_t)b * op.chan_in + o / mult) * op.h_in * op.w_in;
+    const T *f = filters + (int64_t)o * op.kernel * op.kernel;
+    float acc = 0.0f;
+    for (int k1 = 0; k1 < op.kernel; k1++) {
+        const int y = oh * op.stride - op.padding + op.dilation * k1;
+        if ((unsigned)y >= (unsigned)op.h_in) continue;
+        for (int k2 = 0; k2 < op.kernel; k2++) {
+            const int x = ow * op.stride - op.padding + op.dilation * k2;
+            if ((unsigned)x < (unsigned)op.w_in) acc += Elem<T>::load(f + k1 * op.kernel + k2) * Elem<T>::load(plane + y * op.w_in + x);
+        }
+    }
+    Elem<T>::store(out + (int64_t)blockIdx.x * n + pos, acc);
+}
+template <typename T>
+__global__ __launch_bounds__(256) void depthwise_grad_img_kernel(Op op, const T *filters, const T *grad_out, T *grad_img, uint32_t magic_w, uint32_t magic_s) {
+    const int hw = op.h_in * op.w_in, pos = blockIdx.y * 256 + threadIdx.x;
+    if (pos >= hw) return;
+    const int mult = op.chan_out / op.groups, b = blockIdx.x / op.chan_in, g = blockIdx.x - b * op.chan_in;
+    const int y = (int)small_div(pos, op.w_in, magic_w), x = pos - y * op.w_in, kk = op.kernel * op.kernel, n = op.h_out * op.w_out;
+    float acc = 0.0f;
+    for (int k1 = 0; k1 < op.kernel; k1++) {
+        const int ty = y + op.padding - op.dilation * k1;
+        if (ty < 0) break;
+        const int oh = (int)small_div(ty, op.stride, magic_s);
+        if (oh * op.stride != ty || oh >= op.h_out) continue;
+        for (int k2 = 0; k2 < op.kernel; k2++) {
+            const int tx = x + op.padding - op.dilation * k2;
+            if (tx < 0) break;
+            const int ow = (int)small_div(tx, op.stride, magic_s);
+            if (ow * op.stride != tx || ow >= op.w_out) continue;
+            for (int m = 0; m < mult; m++) {
+                const int o = g * mult + m;
+                acc += Elem<T>::load(filters + (int64_t)o * kk + k1 * op.kernel + k2) *
+                       Elem<T>::load(grad_out + ((int64_t)b * op.chan_out + o) * n + oh * op.w_out + ow);
+            }
+        }
+    }
+    T *dst = grad_img + (int64_t)blockIdx.x * hw + pos;
+    Elem<T>::store(dst, Elem<T>::load(dst) + acc);
+}
+template <typename T>
+__global__ __launch_bounds__(256) void depthwise_grad_filters_kernel(Op op, const T *img, const T *grad_out, T *grad_filters, uint32_t magic_w) {
+    __shared__ float part[4];
+    const int o = blockIdx.x, mult = op.chan_out / op.groups, n = op.h_out * op.w_out, hw = op.h_in * op.w_in;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    for (int k1 = 0; k1 < op.kernel; k1++)
+        for (int k2 = 0; k2 < op.kernel; k2++) {
+            float acc = 0.0f;
+            for (int b = 0; b < op.batch; b++) {
+                const T *go = grad_out + ((int64_t)b * op.chan_out + o) * n;
+                const T *plane = img + ((int64_t)b * op.chan_in + o / mult) * hw;
+                for (int pos = threadIdx.x; pos < n; pos += 256) {
+                    const int oh = (int)small_div(pos, op.w_out, magic_w), ow = pos - oh * op.w_out;
+                    const int y = oh * op.stride - op.padding + op.dilation * k1, x = ow * op.stride - op.padding + op.dilation * k2;
+                    if ((unsigned)y < (unsigned)op.h_in && (unsigned)x < (unsigned)op.w_in)
+                        acc += Elem<T>::load(go + pos) * Elem<T>::load(plane + y * op.w_in + x);
+                }
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);  // the same tree whatever the timing
+            __syncthreads();  // (the previous tap's partial sums have been read)
+            if (lane == 0) part[wave] = acc;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                T *dst = grad_filters + (int64_t)o * op.kernel * op.kernel + k1 * op.kernel + k2;
+                Elem<T>::store(dst, Elem<T>::load(dst) + ((part[0] + part[1]) + (part[2] + part[3])));
+            }
+        }
+}
+// The same with a compile-time kernel size: a thread keeps all K*K sums and visits every (image, position) of its share
+// once -- one load of grad_out and one division per position instead of one per position and tap -- and `slices` workgroups
+// share the images of a channel; their sums meet in `partial` [O][slices][K*K] and the last line below adds them in slice
+// order (deterministic).  grid = (O, slices).
+template <typename T, int K>
+__global__ __launch_bounds__(256) void depthwise_grad_filters_fixed_kernel(Op op, const T *img, const T *grad_out, float *partial, uint32_t magic_w) {
+    constexpr int KK = K * K;
+    __shared__ float part[4][KK];
+    const int o = blockIdx.x, slices = gridDim.y, mult = op.chan_out / op.groups, n = op.h_out * op.w_out, hw = op.h_in * op.w_in;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    float acc[KK];
+#pragma unroll
+    for (int t = 0; t < KK; t++) acc[t] = 0.0f;
+    for (int b = blockIdx.y; b < op.batch; b += slices) {
+        const T *go = grad_out + ((int64_t)b * op.chan_out + o) * n;
+        const T *plane = img + ((int64_t)b * op.chan_in + o / mult) * hw;
+        for (int pos = threadIdx.x; pos < n; pos += 256) {
+            const int oh = (int)small_div(pos, op.w_out, magic_w), ow = pos - oh * op.w_out;
+            const float g = Elem<T>::load(go + pos);
+            const int y0 = oh * op.stride - op.padding, x0 = ow * op.stride - op.padding;
+#pragma unroll
+            for (int k1 = 0; k1 < K; k1++) {
+                const int y = y0 + op.dilation * k1;
+#pragma unroll
+                for (int k2 = 0; k2 < K; k2++) {
+                    const int x = x0 + op.dilation * k2;
+                    const bool ok = (unsigned)y < (unsigned)op.h_in && (unsigned)x < (unsigned)op.w_in;
+                    acc[k1 * K + k2] += ok ? g * Elem<T>::load(plane + y * op.w_in + x) : 0.0f;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < KK; t++) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) acc[t] += __shfl_xor(acc[t], off, 64);
+        if (lane == 0) part[wave][t] = acc[t];
+    }
+    __syncthreads();
+    if (threadIdx.x < KK) partial[((int64_t)o * slices + blockIdx.y) * KK + threadIdx.x] =
+        (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+}
+template <typename T> __global__ __launch_bounds__(256) void depthwise_grad_filters_add_kernel(const float *partial, T *grad_filters, int slices, int kk, int total) {
+    const int i = blockIdx.x * 256 + threadIdx.x;  // (o, tap)
+    if (i >= total) return;
+    const int o = i / kk, t = i - o * kk;
+    float sum = 0.0f;
+    for (int s = 0; s < slices; s++) sum += partial[((int64_t)o * slices + s) * kk + t];
+    Elem<T>::store(grad_filters + i, Elem<T>::load(grad_filters + i) + sum);
+}
+
+inline bool depthwise(const Op &op) {
+    return op.groups > 1 && op.chan_in == op.groups && op.chan_out % op.groups == 0 && (int64_t)op.h_in * op.w_in <= 65535ll * 256 &&
+           (int64_t)op.h_out * op.w_out <= 65535ll * 256 && (int64_t)op.h_in * op.w_in * std::max(op.w_in, op.stride) < (1ll << 32);
+}
+
 template <typename T>
 int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void *filters, void *out) {
     constexpr int V = Elem<T>::VEC;
@@ -497,6 +637,11 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
     const int64_t m = op.chan_out / op.groups, k = (op.chan_in / op.groups) * kk;
     const int64_t per_image = (int64_t)op.chan_in * kk * np;  // patch elements of one image
     if (per_image == 0 || m == 0) return DFDX_ROCM_OK;
+    if (depthwise(op) && (int64_t)op.batch * op.chan_out < (1ll << 31)) {
+        depthwise_forward_kernel<T><<<dim3((unsigned)(op.batch * op.chan_out), (unsigned)((n + 255) / 256)), 256, 0, ctx->stream>>>(
+            op, (const T *)img, (const T *)filters, (T *)out, magic_of(op.w_out));
+        return (int)hipGetLastError();
+    }
     if (per_image >= (1ll << 31) || (int64_t)op.chan_out * np >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
     if (op.kernel > 1) {  // (1x1 filters have no patch matrix to avoid: see `pointwise` below)
         int rc = 0;
@@ -765,6 +910,29 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     const int64_t per_image = (int64_t)op.chan_out * kk * hp;
     const int64_t f_elems = (int64_t)op.groups * cg * og * kk;
     if (per_image == 0 || f_elems == 0 || ohw == 0) return DFDX_ROCM_OK;
+    if (depthwise(op) && (int64_t)op.batch * op.chan_out < (1ll << 31)) {
+        depthwise_grad_img_kernel<T><<<dim3((unsigned)(op.batch * op.chan_in), (unsigned)((hw + 255) / 256)), 256, 0, ctx->stream>>>(
+            op, (const T *)filters, (const T *)grad_out, (T *)grad_img, magic_of(op.w_in), magic_of(op.stride));
+        HIP_TRY(hipGetLastError());
+        if (op.kernel == 3 || op.kernel == 5 || op.kernel == 7) {
+            // enough workgroups to fill the chip twice, at most one per image
+            const int slices = (int)std::max<int64_t>(1, std::min<int64_t>(op.batch, (2 * (int64_t)ctx->compute_units + op.chan_out - 1) / op.chan_out));
+            CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
+            if (int rc = ensure_patches(ctx, round256((size_t)op.chan_out * slices * kk * sizeof(float)))) return rc;
+            const dim3 grid((unsigned)op.chan_out, (unsigned)slices);
+            const uint32_t mw = magic_of(op.w_out);
+            if (op.kernel == 3) depthwise_grad_filters_fixed_kernel<T, 3><<<grid, 256, 0, ctx->stream>>>(op, (const T *)img, (const T *)grad_out, (float *)ctx->patches, mw);
+            else if (op.kernel == 5) depthwise_grad_filters_fixed_kernel<T, 5><<<grid, 256, 0, ctx->stream>>>(op, (const T *)img, (const T *)grad_out, (float *)ctx->patches, mw);
+            else depthwise_grad_filters_fixed_kernel<T, 7><<<grid, 256, 0, ctx->stream>>>(op, (const T *)img, (const T *)grad_out, (float *)ctx->patches, mw);
+            HIP_TRY(hipGetLastError());
+            const int total = (int)(op.chan_out * kk);
+            depthwise_grad_filters_add_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>((const float *)ctx->patches, (T *)grad_filters, slices, (int)kk, total);
+            return (int)hipGetLastError();
+        }
+        depthwise_grad_filters_kernel<T><<<(unsigned)op.chan_out, 256, 0, ctx->stream>>>(op, (const T *)img, (const T *)grad_out, (T *)grad_filters,
+                                                                                      magic_of(op.w_out));
+        return (int)hipGetLastError();
+    }
     // (also at unit stride when the image has far fewer channels than the output -- a first layer, 3 -> 64: the forward patch
     // matrix is O / C times smaller than the one over grad_out, and the products with three rows of filters disappear)
     if (op.stride > 1 || (int64_t)op.chan_in * 4 <= op.chan_out)

@@ -77,6 +77,10 @@ CONFIGS = [
     (2, 8, 8, 17, 18, 3, 2, 2, 2, 1),      # the same with dilation 2 and an odd height (cells cut by the image's edge)
     (2, 4, 8, 23, 19, 3, 5, 1, 1, 1),      # stride 5: the per-pixel form of the gather
     (3, 6, 9, 20, 21, 4, 3, 2, 1, 3),      # stride 3, three groups, an even kernel
+    (2, 8, 8, 12, 14, 3, 1, 1, 1, 8),      # depthwise (one input channel per group): the direct kernels
+    (3, 6, 12, 9, 11, 3, 2, 1, 1, 6),      # depthwise with a channel multiplier of 2, stride 2
+    (2, 4, 4, 20, 18, 5, 1, 4, 2, 4),      # depthwise, 5 x 5, dilation 2; more than 256 positions per plane
+    (5, 3, 3, 8, 9, 2, 1, 1, 1, 3),        # depthwise with a 2 x 2 kernel: the filter-gradient kernel for any kernel size
 ]
 
 
