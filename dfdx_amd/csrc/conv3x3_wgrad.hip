@@ -484,6 +484,7 @@ bool make_plan(const Conv3x3Problem &c, int compute_units, Plan *out) {
     const int wp = c.w + 2;
     Plan pl;
     pl.R = std::min(c.h, KMAX / wp);
+    while (pl.R > 1 && 8 * (pl.R + 2) * (c.w / 2) > UMAX * NTH) pl.R--;  // wide rows: fewer of them per item
     if (pl.R < 1) return false;
     pl.bands = (c.h + pl.R - 1) / pl.R;
     pl.kp = (pl.R * wp + 31) / 32 * 32;

@@ -168,7 +168,7 @@ def test_conv2d_3x3_band_kernel_zero_padding_is_exact():
 # the rows per band), a grad_out band of exactly 256 records (62-pixel rows), one row per image, more work items than
 # workgroups and fewer.
 WGRAD_CONFIGS = [(2, 128, 64, 20, 14), (3, 64, 128, 9, 30), (1, 64, 64, 5, 62), (2, 64, 64, 1, 40), (70, 64, 64, 8, 8),
-                 (2, 128, 128, 33, 12)]
+                 (2, 128, 128, 33, 12), (1, 64, 64, 6, 112), (2, 64, 64, 5, 84)]   # (the last two: rows too wide for as many per item as the band holds)
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])   # (f32: channel-major bands, one value per lane and MFMA)
