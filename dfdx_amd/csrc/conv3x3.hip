@@ -344,7 +344,7 @@ bool conv3x3_supported(const Conv3x3Problem &c) {
     if (((uintptr_t)c.img & 3u) || ((uintptr_t)c.out & out_mask) || ((uintptr_t)c.filters & (uintptr_t)(es - 1)) || ((uintptr_t)c.wt & 15u)) return false;
     const int band_rows = (int)std::min<int64_t>(c.h, (NT - 1) / c.w + 2) + 2;
     if ((size_t)A_BYTES + (size_t)band_rows * (c.w + 2) * PIX > 160 * 1024) return false;
-    if (4 * band_rows * (c.w / 2) > 4 * 512) return false;  // units per chunk: at most four (f32: eight) per thread
+    if (4 * band_rows * (c.w / 2) > 6 * 512) return false;  // units per chunk: at most six (f32: twelve) per thread
     return c.batch < 65536 && (hw + NT - 1) / NT < 65536;  // grid.z, grid.y
 }
 
@@ -369,7 +369,7 @@ hipError_t launch_conv3x3(const Conv3x3Problem &c, hipStream_t stream) {
     p.magic_w = (uint32_t)(((1ull << 32) + c.w - 1) / c.w);
     p.magic_pairs = (uint32_t)(((1ull << 32) + per_row - 1) / per_row);
     const dim3 grid((unsigned)p.mblocks, (unsigned)p.nblocks, (unsigned)c.batch);
-    const bool few = 4 * p.band_rows * (c.w / 2) <= 2 * 512;
+    const bool few = 4 * p.band_rows * (c.w / 2) <= 2 * 512, many = 4 * p.band_rows * (c.w / 2) > 4 * 512;  // (rows of 206+ pixels)
 #define DFDX_CONV3(T, U, A)                                                                                            \
     do {                                                                                                               \
         static PerDevice attr_on;                                                                                      \
@@ -381,20 +381,21 @@ hipError_t launch_conv3x3(const Conv3x3Problem &c, hipStream_t stream) {
         }                                                                                                              \
         conv3x3_kernel<T, U, A><<<grid, 512, lds, stream>>>(p);                                                        \
     } while (0)
-#define DFDX_CONV3_U(T, A, UF, UM)     \
-    do {                               \
-        if (few) DFDX_CONV3(T, UF, A); \
-        else DFDX_CONV3(T, UM, A);     \
+#define DFDX_CONV3_U(T, A, UF, UM, UW)       \
+    do {                                     \
+        if (few) DFDX_CONV3(T, UF, A);       \
+        else if (many) DFDX_CONV3(T, UW, A); \
+        else DFDX_CONV3(T, UM, A);           \
     } while (0)
     if (c.dtype == DT_F16) {
-        if (c.accumulate) DFDX_CONV3_U(_Float16, true, 2, 4);
-        else DFDX_CONV3_U(_Float16, false, 2, 4);
+        if (c.accumulate) DFDX_CONV3_U(_Float16, true, 2, 4, 6);
+        else DFDX_CONV3_U(_Float16, false, 2, 4, 6);
     } else if (c.dtype == DT_BF16) {
-        if (c.accumulate) DFDX_CONV3_U(__bf16, true, 2, 4);
-        else DFDX_CONV3_U(__bf16, false, 2, 4);
+        if (c.accumulate) DFDX_CONV3_U(__bf16, true, 2, 4, 6);
+        else DFDX_CONV3_U(__bf16, false, 2, 4, 6);
     } else {
-        if (c.accumulate) DFDX_CONV3_U(float, true, 4, 8);
-        else DFDX_CONV3_U(float, false, 4, 8);
+        if (c.accumulate) DFDX_CONV3_U(float, true, 4, 8, 12);
+        else DFDX_CONV3_U(float, false, 4, 8, 12);
     }
 #undef DFDX_CONV3_U
 #undef DFDX_CONV3

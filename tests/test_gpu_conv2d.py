@@ -77,6 +77,7 @@ CONFIGS = [
     (2, 8, 8, 17, 18, 3, 2, 2, 2, 1),      # the same with dilation 2 and an odd height (cells cut by the image's edge)
     (2, 4, 8, 23, 19, 3, 5, 1, 1, 1),      # stride 5: the per-pixel form of the gather
     (3, 6, 9, 20, 21, 4, 3, 2, 1, 3),      # stride 3, three groups, an even kernel
+    (1, 64, 64, 4, 224, 3, 1, 1, 1, 1),    # rows of 224 pixels: the image gradient on the band kernel's wide-row form, the filter gradient over the patch matrix
     (2, 8, 8, 12, 14, 3, 1, 1, 1, 8),      # depthwise (one input channel per group): the direct kernels
     (3, 6, 12, 9, 11, 3, 2, 1, 1, 6),      # depthwise with a channel multiplier of 2, stride 2
     (2, 4, 4, 20, 18, 5, 1, 4, 2, 4),      # depthwise, 5 x 5, dilation 2; more than 256 positions per plane
@@ -123,7 +124,8 @@ def test_conv2d_seeded(cfg, dtype):
 # in the middle of a row or of the image (one partial block; 196, 200 and 280 pixels), H * W off the 8-pixel grid (the
 # 8-byte store form), bands of 3 to 24 rows, an odd height, a width of 112 (four units of the band per thread).
 BAND_CONFIGS = [(2, 32, 64, 16, 16), (1, 64, 64, 14, 14), (3, 96, 128, 20, 14), (2, 64, 64, 56, 56), (2, 128, 192, 28, 28),
-                (1, 32, 64, 9, 112), (2, 64, 64, 31, 12), (1, 64, 64, 112, 112), (5, 32, 64, 8, 16), (2, 32, 64, 50, 4)]
+                (1, 32, 64, 9, 112), (2, 64, 64, 31, 12), (1, 64, 64, 112, 112), (5, 32, 64, 8, 16), (2, 32, 64, 50, 4),
+                (1, 32, 64, 6, 224), (1, 32, 64, 3, 254)]   # (the last two: rows so wide that a thread owns five or six units of a band)
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
