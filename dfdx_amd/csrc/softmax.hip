@@ -234,6 +234,136 @@ __global__ __launch_bounds__(WAVES * 64) void softmax_backward_loop_kernel(const
     }
 }
 
+// ---- long rows: a workgroup per row ------------------------------------------------------------------------------
+// Rows past what a wave keeps in registers used to go to the three-pass kernels above, one WAVE per row: a 5120-wide row
+// ran at 1 TB/s and the 64 rows of a 50257-wide logit matrix kept 64 waves of the chip busy (360 us for 6 MB).  Here 256
+// threads share a row and each keeps NV vectors of it in registers between the passes (one read, one write); the row's
+// maximum and sums go wave -> LDS -> all threads, in a fixed order.
+constexpr int BLOCK = 256;
+__device__ __forceinline__ float block_reduce(float v, float *slots, bool is_max) {
+    v = is_max ? wave_max(v) : wave_sum(v);
+    __syncthreads();  // (the slots of the previous reduction have been read)
+    if (threadIdx.x % 64 == 0) slots[threadIdx.x / 64] = v;
+    __syncthreads();
+    return is_max ? fmaxf(fmaxf(slots[0], slots[1]), fmaxf(slots[2], slots[3])) : (slots[0] + slots[1]) + (slots[2] + slots[3]);
+}
+template <typename T, int NV, bool STREAM>
+__global__ __launch_bounds__(BLOCK) void softmax_forward_block_kernel(const T *x, T *out, int cols, float scale) {
+    constexpr int V = Elem<T>::VEC;
+    __shared__ float slots[4];
+    const T *src = x + (int64_t)blockIdx.x * cols;
+    float v[NV][V];
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int c = 0; c < NV; c++) {
+        const int col = (c * BLOCK + threadIdx.x) * V;
+        if (col < cols) {
+            load_elems_as<T, V, STREAM>(src + col, v[c]);
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                v[c][i] *= scale;
+                m = fmaxf(m, v[c][i]);
+            }
+        }
+    }
+    m = block_reduce(m, slots, true);
+    float sum = 0.0f;
+#pragma unroll
+    for (int c = 0; c < NV; c++) {
+        if ((c * BLOCK + threadIdx.x) * V < cols) {
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                v[c][i] = expf(v[c][i] - m);
+                sum += v[c][i];
+            }
+        }
+    }
+    sum = block_reduce(sum, slots, false);
+    const float inv = 1.0f / sum;
+    T *dst = out + (int64_t)blockIdx.x * cols;
+#pragma unroll
+    for (int c = 0; c < NV; c++) {
+        const int col = (c * BLOCK + threadIdx.x) * V;
+        if (col < cols) {
+#pragma unroll
+            for (int i = 0; i < V; i++) v[c][i] *= inv;
+            store_elems<T, V>(dst + col, v[c]);
+        }
+    }
+}
+template <typename T, int NV, bool STREAM>
+__global__ __launch_bounds__(BLOCK) void softmax_backward_block_kernel(const T *p, const T *go, T *gx, int cols, float scale, bool fresh) {
+    constexpr int V = Elem<T>::VEC;
+    __shared__ float slots[4];
+    const T *ps = p + (int64_t)blockIdx.x * cols, *gs = go + (int64_t)blockIdx.x * cols;
+    float pv[NV][V], gv[NV][V];
+    float dot = 0.0f;
+#pragma unroll
+    for (int c = 0; c < NV; c++) {
+        const int col = (c * BLOCK + threadIdx.x) * V;
+        if (col < cols) {
+            load_elems_as<T, V, STREAM>(ps + col, pv[c]);
+            load_elems_as<T, V, STREAM>(gs + col, gv[c]);
+#pragma unroll
+            for (int i = 0; i < V; i++) dot += pv[c][i] * gv[c][i];
+        }
+    }
+    dot = block_reduce(dot, slots, false);
+    T *dst = gx + (int64_t)blockIdx.x * cols;
+#pragma unroll
+    for (int c = 0; c < NV; c++) {
+        const int col = (c * BLOCK + threadIdx.x) * V;
+        if (col < cols) {
+            float old[V];
+            if (!fresh) load_elems<T, V>(dst + col, old);
+#pragma unroll
+            for (int i = 0; i < V; i++) gv[c][i] = (fresh ? 0.0f : old[i]) + scale * (pv[c][i] * (gv[c][i] - dot));
+            store_elems<T, V>(dst + col, gv[c]);
+        }
+    }
+}
+// Rows that fit no register form (unaligned, or longer still): a workgroup of 1024 threads per row, three passes over the
+// row (the second and third find it in the cache), element loads.
+template <typename T>
+__global__ __launch_bounds__(1024) void softmax_forward_block_loop_kernel(const T *x, T *out, int cols, float scale) {
+    __shared__ float slots[16];
+    const T *src = x + (int64_t)blockIdx.x * cols;
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    auto reduce = [&](float v, bool is_max) {
+        v = is_max ? wave_max(v) : wave_sum(v);
+        __syncthreads();
+        if (lane == 0) slots[wave] = v;
+        __syncthreads();
+        float r = slots[0];
+        for (int w = 1; w < 16; w++) r = is_max ? fmaxf(r, slots[w]) : r + slots[w];
+        return r;
+    };
+    float m = -FLT_MAX;
+    for (int c = threadIdx.x; c < cols; c += 1024) m = fmaxf(m, Elem<T>::load(src + c) * scale);
+    m = reduce(m, true);
+    float sum = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += 1024) sum += expf(Elem<T>::load(src + c) * scale - m);
+    sum = reduce(sum, false);
+    const float inv = 1.0f / sum;
+    T *dst = out + (int64_t)blockIdx.x * cols;
+    for (int c = threadIdx.x; c < cols; c += 1024) Elem<T>::store(dst + c, expf(Elem<T>::load(src + c) * scale - m) * inv);
+}
+template <typename T>
+__global__ __launch_bounds__(1024) void softmax_backward_block_loop_kernel(const T *p, const T *go, T *gx, int cols, float scale, bool fresh) {
+    __shared__ float slots[16];
+    const T *ps = p + (int64_t)blockIdx.x * cols, *gs = go + (int64_t)blockIdx.x * cols;
+    float dot = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += 1024) dot += Elem<T>::load(ps + c) * Elem<T>::load(gs + c);
+    dot = wave_sum(dot);
+    if (threadIdx.x % 64 == 0) slots[threadIdx.x / 64] = dot;
+    __syncthreads();
+    dot = slots[0];
+    for (int w = 1; w < 16; w++) dot += slots[w];
+    T *dst = gx + (int64_t)blockIdx.x * cols;
+    for (int c = threadIdx.x; c < cols; c += 1024)
+        Elem<T>::store(dst + c, (fresh ? 0.0f : Elem<T>::load(dst + c)) + scale * (Elem<T>::load(ps + c) * (Elem<T>::load(gs + c) - dot)));
+}
+
 // ---- f64: one wave per row, three passes over memory, f64 arithmetic ------------------------------------------
 __device__ __forceinline__ double wave_sum_f64(double v) {
 #pragma unroll
@@ -326,6 +456,31 @@ int launch_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *a, cons
 #undef DFDX_SOFTMAX_ROW16
 #undef DFDX_SOFTMAX_REG_AS
 #undef DFDX_SOFTMAX_ROW16_AS
+    // long rows: a workgroup per row (grid.x = rows)
+    if (rows < (1ll << 31)) {
+#define DFDX_SOFTMAX_BLOCK_AS(NV, STREAM)                                                                              \
+    do {                                                                                                               \
+        if constexpr (FWD) softmax_forward_block_kernel<T, NV, STREAM><<<(unsigned)rows, BLOCK, 0, s>>>((const T *)a, (T *)c, n, scale); \
+        else softmax_backward_block_kernel<T, NV, STREAM><<<(unsigned)rows, BLOCK, 0, s>>>((const T *)a, (const T *)b, (T *)c, n, scale, fresh); \
+        return (int)hipGetLastError();                                                                                 \
+    } while (0)
+#define DFDX_SOFTMAX_BLOCK(NV)                                                                                         \
+    do {                                                                                                               \
+        if (stream) DFDX_SOFTMAX_BLOCK_AS(NV, true);                                                                   \
+        else DFDX_SOFTMAX_BLOCK_AS(NV, false);                                                                         \
+    } while (0)
+        if (vec) {
+            const int64_t per_thread = (cols / V + BLOCK - 1) / BLOCK;  // vectors of a row per thread
+            if (per_thread <= 4) DFDX_SOFTMAX_BLOCK(4);
+            if (per_thread <= 8) DFDX_SOFTMAX_BLOCK(8);
+            if (FWD && per_thread <= 16) DFDX_SOFTMAX_BLOCK(16);  // (the backward holds two rows of values)
+        }
+#undef DFDX_SOFTMAX_BLOCK
+#undef DFDX_SOFTMAX_BLOCK_AS
+        if constexpr (FWD) softmax_forward_block_loop_kernel<T><<<(unsigned)rows, 1024, 0, s>>>((const T *)a, (T *)c, n, scale);
+        else softmax_backward_block_loop_kernel<T><<<(unsigned)rows, 1024, 0, s>>>((const T *)a, (const T *)b, (T *)c, n, scale, fresh);
+        return (int)hipGetLastError();
+    }
     if constexpr (FWD) softmax_forward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (T *)c, rows, n, scale);
     else softmax_backward_loop_kernel<T><<<grid, block, 0, s>>>((const T *)a, (const T *)b, (T *)c, rows, n, scale, fresh);
     return (int)hipGetLastError();

@@ -94,7 +94,9 @@ def test_scalar_mul_seeded(n, dtype):
 
 # ------------------------------------------------------------------- softmax --
 SOFTMAX_SHAPES = [(1, 1), (3, 5), (7, 64), (5, 1000), (4, 1024), (3, 4096), (2, 5000), (2, 1001), (2, 1500), (1031, 72),
-                  (40000, 64)]
+                  (40000, 64),
+                  # long rows, a workgroup each: 4 / 8 / 16 vectors per thread in registers, then the three-pass form (a row of logits)
+                  (5, 5120), (3, 8200), (2, 16384), (2, 30000), (3, 50257), (2, 70000)]
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
