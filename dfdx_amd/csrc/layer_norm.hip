@@ -179,6 +179,161 @@ __global__ __launch_bounds__(WAVES_BWD * 64) void layer_norm_backward_kernel(con
     }
 }
 
+// ---- long rows: 256 threads share a row ----------------------------------------------------------------------------
+// Rows past what a wave keeps in registers (2048 16-bit / 1024 f32 elements: a model width of 4096 or 5120) went to the
+// kernels that walk the row from memory once per pass, a wave per row -- 1 TB/s forward, 0.6-0.9 backward.  Here a workgroup
+// walks rows blockIdx.x, + gridDim.x, ...; each thread keeps NV vectors of the row (and of gamma, beta and the column sums) in
+// registers, the row's sums go wave -> LDS -> all threads in a fixed order.  The same formulas, one read, one write.
+constexpr int LN_BLOCK = 256;
+__device__ __forceinline__ float ln_block_sum(float v, float *slots) {
+    v = wave_sum(v);
+    __syncthreads();  // (the slots of the previous sum have been read)
+    if (threadIdx.x % 64 == 0) slots[threadIdx.x / 64] = v;
+    __syncthreads();
+    return (slots[0] + slots[1]) + (slots[2] + slots[3]);
+}
+template <typename T, int NV>
+__global__ __launch_bounds__(LN_BLOCK) void layer_norm_forward_block_kernel(const T *x, const T *gamma, const T *beta, T *out, int64_t rows, int cols,
+                                                                            float eps) {
+    constexpr int N = Elem<T>::VEC;
+    __shared__ float slots[4];
+    const float inv_n = 1.0f / (float)cols;
+    float gm[NV][N], bt[NV][N];
+#pragma unroll
+    for (int c = 0; c < NV; c++) {
+        const int col = (c * LN_BLOCK + threadIdx.x) * N;
+        if (col < cols) {
+            load_elems<T, N>(gamma + col, gm[c]);
+            load_elems<T, N>(beta + col, bt[c]);
+        }
+    }
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const T *src = x + row * cols;
+        float v[NV][N];
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NV; c++) {
+            const int col = (c * LN_BLOCK + threadIdx.x) * N;
+            if (col < cols) {
+                load_elems<T, N>(src + col, v[c]);
+#pragma unroll
+                for (int i = 0; i < N; i++) s += v[c][i];
+            }
+        }
+        const float mean = ln_block_sum(s, slots) * inv_n;
+        float q = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NV; c++) {
+            if ((c * LN_BLOCK + threadIdx.x) * N < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) {
+                    v[c][i] -= mean;
+                    q += v[c][i] * v[c][i];
+                }
+            }
+        }
+        const float rstd = 1.0f / sqrtf(ln_block_sum(q, slots) * inv_n + eps);
+        T *dst = out + row * cols;
+#pragma unroll
+        for (int c = 0; c < NV; c++) {
+            const int col = (c * LN_BLOCK + threadIdx.x) * N;
+            if (col < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) v[c][i] = v[c][i] * rstd * gm[c][i] + bt[c][i];
+                store_elems<T, N>(dst + col, v[c]);
+            }
+        }
+    }
+}
+// partial[blockIdx.x][0 / 1][col]: the workgroup's column sums (every column belongs to one thread: no combining here)
+template <typename T, int NV>
+__global__ __launch_bounds__(LN_BLOCK) void layer_norm_backward_block_kernel(const T *x, const T *gamma, const T *go, T *gx, float *partial, int64_t rows,
+                                                                             int cols, float eps, bool fresh_x) {
+    constexpr int N = Elem<T>::VEC;
+    __shared__ float slots[4];
+    const float inv_n = 1.0f / (float)cols;
+    float gm[NV][N], dg[NV][N], db[NV][N];
+#pragma unroll
+    for (int c = 0; c < NV; c++) {
+        const int col = (c * LN_BLOCK + threadIdx.x) * N;
+        if (col < cols) load_elems<T, N>(gamma + col, gm[c]);
+#pragma unroll
+        for (int i = 0; i < N; i++) dg[c][i] = db[c][i] = 0.0f;
+    }
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const T *src = x + row * cols, *gs = go + row * cols;
+        float v[NV][N], g[NV][N];
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NV; c++) {
+            const int col = (c * LN_BLOCK + threadIdx.x) * N;
+            if (col < cols) {
+                load_elems<T, N>(src + col, v[c]);
+                load_elems<T, N>(gs + col, g[c]);
+#pragma unroll
+                for (int i = 0; i < N; i++) s += v[c][i];
+            }
+        }
+        const float mean = ln_block_sum(s, slots) * inv_n;
+        float q = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NV; c++) {
+            if ((c * LN_BLOCK + threadIdx.x) * N < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) {
+                    v[c][i] -= mean;
+                    q += v[c][i] * v[c][i];
+                }
+            }
+        }
+        const float rstd = 1.0f / sqrtf(ln_block_sum(q, slots) * inv_n + eps);
+        float s1 = 0.0f, s2 = 0.0f;  // sum gh, sum gh * xhat
+#pragma unroll
+        for (int c = 0; c < NV; c++) {
+            if ((c * LN_BLOCK + threadIdx.x) * N < cols) {
+#pragma unroll
+                for (int i = 0; i < N; i++) {
+                    v[c][i] *= rstd;  // xhat
+                    dg[c][i] += g[c][i] * v[c][i];
+                    db[c][i] += g[c][i];
+                    g[c][i] *= gm[c][i];  // gh
+                    s1 += g[c][i];
+                    s2 += g[c][i] * v[c][i];
+                }
+            }
+        }
+        const float m1 = ln_block_sum(s1, slots) * inv_n, m2 = ln_block_sum(s2, slots) * inv_n;
+        T *dst = gx + row * cols;
+#pragma unroll
+        for (int c = 0; c < NV; c++) {
+            const int col = (c * LN_BLOCK + threadIdx.x) * N;
+            if (col < cols) {
+                float old[N];
+                if (fresh_x) {
+#pragma unroll
+                    for (int i = 0; i < N; i++) old[i] = 0.0f;
+                } else {
+                    load_elems<T, N>(dst + col, old);
+                }
+#pragma unroll
+                for (int i = 0; i < N; i++) old[i] += rstd * (g[c][i] - m1 - v[c][i] * m2);
+                store_elems<T, N>(dst + col, old);
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NV; c++) {
+        const int col = (c * LN_BLOCK + threadIdx.x) * N;
+        if (col < cols) {
+#pragma unroll
+            for (int i = 0; i < N; i++) {
+                partial[((int64_t)blockIdx.x * 2 + 0) * cols + col + i] = dg[c][i];
+                partial[((int64_t)blockIdx.x * 2 + 1) * cols + col + i] = db[c][i];
+            }
+        }
+    }
+}
+
 // Long or unaligned rows: the same formulas with the row walked from memory once per pass.
 template <typename T>
 __global__ __launch_bounds__(WAVES * 64) void layer_norm_forward_loop_kernel(const T *x, const T *gamma, const T *beta, T *out,
@@ -313,6 +468,18 @@ int forward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, con
             if (groups <= 64) DFDX_LN_FWD(1);
             if (groups <= 128) DFDX_LN_FWD(2);
             if (groups <= 256) DFDX_LN_FWD(4);
+            // long rows: 256 threads per row, as many workgroups as keep the chip busy (they loop over the rows)
+            const unsigned bgrid = (unsigned)std::min<int64_t>(rows, (int64_t)ctx->compute_units * 4);
+#define DFDX_LN_FWD_BLOCK(NV)                                                                                                     \
+    do {                                                                                                                          \
+        layer_norm_forward_block_kernel<T, NV><<<bgrid, LN_BLOCK, 0, s>>>((const T *)x, (const T *)gamma, (const T *)beta, (T *)out, rows, (int)cols, \
+                                                                         eps);                                                    \
+        return (int)hipGetLastError();                                                                                            \
+    } while (0)
+            if (groups <= 2 * LN_BLOCK) DFDX_LN_FWD_BLOCK(2);
+            if (groups <= 4 * LN_BLOCK) DFDX_LN_FWD_BLOCK(4);
+            if (groups <= 8 * LN_BLOCK) DFDX_LN_FWD_BLOCK(8);
+#undef DFDX_LN_FWD_BLOCK
         }
     }
 #undef DFDX_LN_FWD
@@ -329,9 +496,11 @@ int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, co
     const bool vec = !F64 && cols % V == 0 && aligned16(x) && aligned16(gamma) && aligned16(go) && aligned16(gx);
     const int64_t groups = cols / V;
     const bool reg = vec && groups <= 256;
+    const bool by_block = vec && !reg && groups <= 8 * LN_BLOCK;  // long rows: 256 threads per row, a slice per workgroup
     // at least 2 rows per wave so that the column sums amortise; two workgroups (16 waves) per compute unit
-    const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>((rows + 2 * WAVES_BWD - 1) / (2 * WAVES_BWD), (int64_t)ctx->compute_units * 2));
-    const int slices = (int)grid * (reg ? 1 : WAVES_BWD);
+    const unsigned grid = by_block ? (unsigned)std::max<int64_t>(1, std::min<int64_t>((rows + 3) / 4, (int64_t)ctx->compute_units * 2))
+                                   : (unsigned)std::max<int64_t>(1, std::min<int64_t>((rows + 2 * WAVES_BWD - 1) / (2 * WAVES_BWD), (int64_t)ctx->compute_units * 2));
+    const int slices = (int)grid * ((reg || by_block) ? 1 : WAVES_BWD);
     const dim3 block(WAVES_BWD * 64);
     hipStream_t s = ctx->stream;
     CtxLock lock(ctx->mu);  // two launches around the shared workspace
@@ -346,6 +515,14 @@ int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, co
             if (groups <= 64) DFDX_LN_BWD(1);
             else if (groups <= 128) DFDX_LN_BWD(2);
             else DFDX_LN_BWD(4);
+            launched = true;
+        } else if (by_block) {
+            if (groups <= 2 * LN_BLOCK)
+                layer_norm_backward_block_kernel<T, 2><<<grid, LN_BLOCK, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, rows, (int)cols, eps, fresh[0]);
+            else if (groups <= 4 * LN_BLOCK)
+                layer_norm_backward_block_kernel<T, 4><<<grid, LN_BLOCK, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, rows, (int)cols, eps, fresh[0]);
+            else
+                layer_norm_backward_block_kernel<T, 8><<<grid, LN_BLOCK, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, rows, (int)cols, eps, fresh[0]);
             launched = true;
         }
     }
