@@ -480,6 +480,17 @@ int forward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, con
             if (groups <= 4 * LN_BLOCK) DFDX_LN_FWD_BLOCK(4);
             if (groups <= 8 * LN_BLOCK) DFDX_LN_FWD_BLOCK(8);
 #undef DFDX_LN_FWD_BLOCK
+        } else {  // rows off the 16-byte grid (a width of 100 in a 16-bit type): element loads, the row still in registers
+#define DFDX_LN_FWD1(CH)                                                                                                          \
+    do {                                                                                                                          \
+        layer_norm_forward_kernel<T, 1, CH><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)beta, (T *)out, rows, \
+                                                                   (int)cols, eps);                                               \
+        return (int)hipGetLastError();                                                                                            \
+    } while (0)
+            if (cols <= 64) DFDX_LN_FWD1(1);
+            if (cols <= 256) DFDX_LN_FWD1(4);
+            if (cols <= 1024) DFDX_LN_FWD1(16);
+#undef DFDX_LN_FWD1
         }
     }
 #undef DFDX_LN_FWD
@@ -495,7 +506,8 @@ int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, co
     constexpr bool F64 = sizeof(T) == 8;
     const bool vec = !F64 && cols % V == 0 && aligned16(x) && aligned16(gamma) && aligned16(go) && aligned16(gx);
     const int64_t groups = cols / V;
-    const bool reg = vec && groups <= 256;
+    const bool reg1 = !F64 && !vec && cols <= 1024;  // rows off the 16-byte grid: element loads, the row still in registers
+    const bool reg = (vec && groups <= 256) || reg1;
     const bool by_block = vec && !reg && groups <= 8 * LN_BLOCK;  // long rows: 256 threads per row, a slice per workgroup
     // at least 2 rows per wave so that the column sums amortise; two workgroups (16 waves) per compute unit
     const unsigned grid = by_block ? (unsigned)std::max<int64_t>(1, std::min<int64_t>((rows + 3) / 4, (int64_t)ctx->compute_units * 2))
@@ -511,7 +523,16 @@ int backward_t(dfdx_rocm_ctx *ctx, int64_t rows, int64_t cols, const void *x, co
                                                                 rows, (int)cols, eps, fresh[0])
     bool launched = false;
     if constexpr (!F64) {
-        if (reg) {
+        if (reg1) {
+#define DFDX_LN_BWD1(CH)                                                                                                        \
+    layer_norm_backward_kernel<T, 1, CH><<<grid, block, 0, s>>>((const T *)x, (const T *)gamma, (const T *)go, (T *)gx, partial, \
+                                                                rows, (int)cols, eps, fresh[0])
+            if (cols <= 64) DFDX_LN_BWD1(1);
+            else if (cols <= 256) DFDX_LN_BWD1(4);
+            else DFDX_LN_BWD1(16);
+#undef DFDX_LN_BWD1
+            launched = true;
+        } else if (reg) {
             if (groups <= 64) DFDX_LN_BWD(1);
             else if (groups <= 128) DFDX_LN_BWD(2);
             else DFDX_LN_BWD(4);
