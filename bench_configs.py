@@ -22,7 +22,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", default=None, help="also write the rows to this file")
     ap.add_argument("--iters", type=int, default=30)
-    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them, shapes = shape classes outside the configurations: few rows or columns, thin contractions, rank-1 updates, mid-size products, plancheck = the planner's pick against every forced tile variant and split count on a fixed list of shapes; exits 1 with --strict when a pick is more than --plancheck-slack off the best; fewrows = the same check on 128 products of 2 - 16 rows against matrices of 2 - 270 MB)")
+    ap.add_argument("--only", default="", help="comma-separated groups: c1,c3,c4,c5,fill,gemv,glue,block,conv (on request only: torch = vendor-library cross-check, edge = operands off the 16-byte grid, with the scalar kernel forced beside them, shapes = shape classes outside the configurations: few rows or columns, thin contractions, rank-1 updates, mid-size products, plancheck = the planner's pick against every forced tile variant and split count on a fixed list of shapes; exits 1 with --strict when a pick is more than --plancheck-slack off the best; fewrows = the same check on 128 products of 2 - 16 rows against matrices of 2 - 270 MB, convx = conv2d with strides, a first layer, depthwise filters, wide rows, small images in f32, 5 x 5 filters, longrows = softmax and LayerNorm on rows of 4096 - 50257 elements)")
     ap.add_argument("--strict", action="store_true", help="plancheck: exit status 1 when a pick is flagged")
     ap.add_argument("--plancheck-slack", type=float, default=0.10, help="plancheck: flag a pick that is this much slower than the best forced candidate")
     ap.add_argument("--probe", default="", choices=["", "traffic", "rows", "variants", "f32-forms", "layouts"],
@@ -640,6 +640,45 @@ def main():
             tag = f"{dt} B{B} {C}->{O} {H}x{W_} k{K}"
             timed("conv", f"conv2d fwd {tag}", lambda: dev.conv2d_forward(xv, wv, stride=s, padding=pad), fl, 0, "conv2d_forward")
             timed("conv", f"conv2d bwd {tag}", lambda: dev.conv2d_backward(xv, gxv, wv, gwv, gov, stride=s, padding=pad), 2 * fl, 0, "conv2d_backward")
+
+    # ---- conv2d outside the configurations' shapes (on request): strides, a first layer, depthwise, wide rows --------------
+    if "convx" in only:
+        # batch, chan_in, chan_out, h, w, kernel, stride, padding, groups
+        for dt, (B, C, O, H, W_, K, s, pad, G) in (("f16", (64, 64, 128, 56, 56, 3, 2, 1, 1)), ("f16", (64, 128, 256, 28, 28, 3, 2, 1, 1)),
+                                                   ("f16", (64, 256, 512, 14, 14, 3, 2, 1, 1)), ("f16", (64, 64, 128, 56, 56, 1, 2, 0, 1)),
+                                                   ("f16", (64, 3, 64, 224, 224, 7, 2, 3, 1)), ("f16", (64, 3, 64, 32, 32, 3, 1, 1, 1)),
+                                                   ("f32", (64, 3, 64, 32, 32, 3, 1, 1, 1)), ("f16", (64, 128, 128, 28, 28, 3, 1, 1, 128)),
+                                                   ("f16", (32, 128, 128, 112, 112, 3, 1, 1, 1)), ("f16", (32, 64, 64, 224, 224, 3, 1, 1, 1)),
+                                                   ("f32", (32, 512, 512, 7, 7, 3, 1, 1, 1)), ("f16", (64, 64, 64, 56, 56, 5, 1, 2, 1))):
+            x, w = rnd((B, C, H, W_), dt), rnd((O, C // G, K, K), dt, 1 / 24)
+            xv, wv = view(x, dt), view(w, dt)
+            kw = dict(stride=s, padding=pad, groups=G)
+            y = dev.conv2d_forward(xv, wv, **kw)
+            gov = view(rnd(y.shape, dt), dt)
+            gxv, gwv = view(zeros((B, C, H, W_), dt), dt), view(zeros((O, C // G, K, K), dt), dt)
+            fl = 2.0 * B * O * (C // G) * K * K * y.shape[2] * y.shape[3]
+            tag = f"{dt} B{B} {C}->{O} {H}x{W_} k{K} s{s}" + (f" groups {G}" if G > 1 else "")
+            timed("convx", f"conv2d fwd {tag}", lambda: dev.conv2d_forward(xv, wv, **kw), fl, 0, "conv2d_forward")
+            timed("convx", f"conv2d bwd {tag}", lambda: dev.conv2d_backward(xv, gxv, wv, gwv, gov, **kw), 2 * fl, 0, "conv2d_backward")
+            del x, w, y
+
+    # ---- softmax and LayerNorm on rows past what a wave keeps in registers (on request) --------------------------------
+    if "longrows" in only:
+        for dt in ("f16", "f32"):
+            for R, Cc in ((4096, 5120), (8192, 4096), (64, 50257), (2048, 8192)):
+                x_t, g_t = rnd((R, Cc), dt), rnd((R, Cc), dt)
+                xs, gs_ = view(x_t, dt), view(g_t, dt)
+                nbytes = R * Cc * esz[dt]
+                p_ = dev.softmax_forward(xs)
+                gx = view(zeros((R, Cc), dt), dt)
+                timed("longrows", f"softmax fwd ({R},{Cc}) {dt}", lambda: dev.softmax_forward(xs), 0, 2 * nbytes, "softmax_forward")
+                timed("longrows", f"softmax bwd ({R},{Cc}) {dt}", lambda: dev.softmax_backward(p_, gx, gs_), 0, 4 * nbytes, "softmax_backward")
+                if Cc % 8 == 0:
+                    g1, be1 = view(rnd((Cc,), dt), dt), view(rnd((Cc,), dt), dt)
+                    gg, gb = view(zeros((Cc,), dt), dt), view(zeros((Cc,), dt), dt)
+                    timed("longrows", f"layer norm fwd ({R},{Cc}) {dt}", lambda: dev.layer_norm_forward(xs, g1, be1), 0, 2 * nbytes, "layer_norm_forward")
+                    timed("longrows", f"layer norm bwd ({R},{Cc}) {dt}", lambda: dev.layer_norm_backward(xs, g1, gx, gg, gb, gs_), 0, 4 * nbytes, "layer_norm_backward")
+                del x_t, g_t, p_
 
     if args.json:
         with open(args.json, "w") as f:
