@@ -394,7 +394,7 @@ int dfdx_rocm_relu_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const vo
 int dfdx_rocm_add_forward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, const void *lhs, const void *rhs, void *out);
 int dfdx_rocm_add_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, void *grad_lhs, void *grad_rhs, const void *grad_out);
 
-/* ---- conv2d: unfold + batched GEMM, 3 x 3 layers without a patch matrix -----
+/* ---- conv2d: unfold + batched GEMM, and the forms that avoid its patch matrix -
  * Conv2DKernel (dfdx-core/src/tensor_ops/conv2d/mod.rs:31-55; Cpu impl
  * cpu_kernel.rs:40-278, Cuda impl cuda_kernel.rs:62-281).  The op struct has
  * the fields and order of the reference's #[repr(C)] Conv2DOp (mod.rs:14-29),
@@ -404,10 +404,20 @@ int dfdx_rocm_add_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, void *gra
  * (mod.rs:290-292); an unbatched image is batch = 1.  Forward overwrites out;
  * backward accumulates into grad_img and grad_filters.  The general form is
  * the reference's: gather the patch matrix, multiply (cpu_kernel.rs:52-170).
- * 3 x 3 filters at unit stride with padding 1 and whole blocks of channels run
- * on kernels that keep a band of the image in LDS and form no patch matrix
- * (same sums, f32 accumulation, one rounding; results within the tolerance
- * of the general form, not bit-identical to it). */
+ * Which form runs depends on the shape; every form computes the same sums with
+ * f32 accumulation and results within the tolerance of the general form, not
+ * bit-identical to it:
+ *   - 3 x 3 filters at unit stride with padding 1 and whole blocks of channels
+ *     run on kernels that keep a band of the image in LDS and form no patch
+ *     matrix, forward and both gradients;
+ *   - images of fewer than 256 output positions multiply as one product over
+ *     the batch (patch matrix [C K K][batch * positions]);
+ *   - strided layers, and layers whose image has a quarter of the output's
+ *     channels or fewer, take both gradients from the forward patch matrix
+ *     (the image gradient's per-tap partial sums are rounded to the element
+ *     type before the taps are added in f32);
+ *   - depthwise layers (one input channel per group) are computed directly;
+ *   - 1 x 1 filters at unit stride use the image itself as the patch matrix. */
 typedef struct dfdx_rocm_conv2d_op {
     size_t kernel, stride, padding, dilation, groups, batch, chan_in, chan_out, h_in, h_out, w_in, w_out;
 } dfdx_rocm_conv2d_op;
