@@ -207,6 +207,85 @@ __global__ __launch_bounds__(256) void unfold_input_taps_kernel(Op op, const T *
         }
 }
 
+// The same with the image rows a workgroup draws on staged in LDS.  blockIdx.y = band of `band_rows` output rows (whole
+// vectors: band_rows * w_out is a multiple of V and at most 256 vectors); the band's windows reach image rows
+// y_first = band_row0 * stride - padding ... y_first + in_rows - 1, which are copied into LDS with one coalesced read (rows
+// outside the image as zeros), and the K*K*V gathers of a thread then hit LDS instead of the memory system: two-byte
+// element loads, every one a request of its own to the texture path, were what the kernel above spends its time on
+// (3 -> 64 channels, 7 x 7, stride 2 at 224 x 224: 166 us for 236 MB of patches).
+template <typename T>
+__global__ __launch_bounds__(256) void unfold_input_taps_lds_kernel(Op op, const T *img, T *patches, int slab_stride, int band_rows, int in_rows) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t staged_rows_raw[];
+    T *const staged = (T *)staged_rows_raw;
+    constexpr int V = Elem<T>::VEC;
+    struct __attribute__((aligned(16))) Vec { T e[V]; };
+    const int row0 = blockIdx.y * band_rows, y_first = row0 * op.stride - op.padding;
+    const T *plane = img + (int64_t)blockIdx.x * op.h_in * op.w_in;
+    for (int i = threadIdx.x; i < in_rows * op.w_in; i += 256) {
+        const int r = i / op.w_in, y = y_first + r;  // (a division per staged element: a few per thread)
+        staged[i] = (unsigned)y < (unsigned)op.h_in ? plane[(int64_t)y * op.w_in + (i - r * op.w_in)] : (T)0.0f;
+    }
+    __syncthreads();
+    const int n = op.h_out * op.w_out, pos0 = row0 * op.w_out + threadIdx.x * V;
+    if (threadIdx.x * V >= band_rows * op.w_out || pos0 >= slab_stride) return;
+    int row = threadIdx.x * V / op.w_out, col = threadIdx.x * V - row * op.w_out;  // inside the band
+    int by[V], bx[V];
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+        by[i] = pos0 + i < n ? row * op.stride : (1 << 20);  // relative to y_first; positions behind the slab's last: zeros
+        bx[i] = col * op.stride - op.padding;
+        if (++col == op.w_out) { col = 0; ++row; }
+    }
+    T *dst = patches + (int64_t)blockIdx.x * op.kernel * op.kernel * slab_stride + pos0;
+    for (int k1 = 0; k1 < op.kernel; k1++)
+        for (int k2 = 0; k2 < op.kernel; k2++) {
+            const int dy = op.dilation * k1, dx = op.dilation * k2;
+            Vec out;
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const int y = by[i] + dy, x = bx[i] + dx;
+                const bool ok = y < in_rows && (unsigned)x < (unsigned)op.w_in;
+                const T val = staged[ok ? y * op.w_in + x : 0];
+                out.e[i] = ok ? val : (T)0.0f;
+            }
+            *(Vec *)dst = out;
+            dst += slab_stride;
+        }
+}
+// Band height of the staged form for this op (0: use another kernel): as many output rows as give the 256 threads a vector
+// each, in whole vectors, with the image rows under them within 48 KB of LDS.
+template <typename T> int staged_band_rows(const Op &op, int64_t slab_stride, int *in_rows) {
+    constexpr int V = Elem<T>::VEC;
+    int unit = 1;
+    while ((unit * op.w_out) % V) unit++;  // rows per whole number of vectors
+    int rows = (256 * V / op.w_out) / unit * unit;
+    for (; rows >= unit; rows -= unit) {
+        const int64_t need = ((int64_t)(rows - 1) * op.stride + (int64_t)op.dilation * (op.kernel - 1) + 1) * op.w_in * (int64_t)sizeof(T);
+        if (need <= 48 * 1024) {
+            *in_rows = (int)((rows - 1) * op.stride + op.dilation * (op.kernel - 1) + 1);
+            return rows;
+        }
+    }
+    return 0;
+}
+
+// The patch matrix of `op`'s images through the position-major kernels: rows staged in LDS where a band of them fits.
+template <typename T> void launch_unfold_taps(const Op &op, const T *img, T *patches, int64_t slab_stride, hipStream_t stream) {
+    constexpr int V = Elem<T>::VEC;
+    int in_rows = 0;
+    // (staging pays from 5 x 5 taps on: at 3 x 3 the two forms measure level, at 1 x 1 the copy into LDS is pure overhead)
+    const int band = op.kernel >= 5 ? staged_band_rows<T>(op, slab_stride, &in_rows) : 0;
+    const unsigned planes = (unsigned)(op.batch * op.chan_in);
+    // bands over the whole slab: the positions behind the last output row (the slab's padding) are written too, as zeros
+    const int64_t bands = band > 0 ? (slab_stride + (int64_t)band * op.w_out - 1) / ((int64_t)band * op.w_out) : 0;
+    if (band > 0 && bands <= 65535) {
+        const size_t lds = (size_t)in_rows * op.w_in * sizeof(T);
+        unfold_input_taps_lds_kernel<T><<<dim3(planes, (unsigned)bands), 256, lds, stream>>>(op, img, patches, (int)slab_stride, band, in_rows);
+    } else {
+        unfold_input_taps_kernel<T><<<dim3(planes, (unsigned)((slab_stride / V + 255) / 256)), 256, 0, stream>>>(op, img, patches, (int)slab_stride, magic_of(op.w_out));
+    }
+}
+
 // Position-major gather for small planes into the FOLDED patch matrix [chan K K][batch * slab_stride]: a thread owns one
 // vector of positions of one plane and walks the K x K taps itself, so the index arithmetic of its V positions is done once
 // for all taps (a tap only shifts the source coordinates) and a vector costs ~70 instructions instead of ~250.  A workgroup
@@ -688,8 +767,7 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
                     sub, mg, src, patches, (int)np, cg, bg);
             }
             else if (!fold && op.stride > 1 && np / V >= 64 && np / V <= 65535ll * 256 && n * op.w_out < (1ll << 32))
-                unfold_input_taps_kernel<T><<<dim3((unsigned)(nb * op.chan_in), (unsigned)((np / V + 255) / 256)), 256, 0, ctx->stream>>>(sub, src, patches, (int)np,
-                                                                                                                                magic_of(op.w_out));
+                launch_unfold_taps<T>(sub, src, patches, np, ctx->stream);
             else unfold_input_flat_kernel<T><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, src, patches, (int)np, vectors, fold ? 1 : 0);
         }
         HIP_TRY(hipGetLastError());
@@ -849,8 +927,7 @@ int strided_backward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *im
         const T *go = (const T *)grad_out + b0 * op.chan_out * ohw;
         const uint32_t vectors = (uint32_t)(nb * op.chan_in * kk * (np / V));
         if (np / V >= 64 && np / V <= 65535ll * 256 && ohw * op.w_out < (1ll << 32))
-            unfold_input_taps_kernel<T><<<dim3((unsigned)(nb * op.chan_in), (unsigned)((np / V + 255) / 256)), 256, 0, ctx->stream>>>(sub, img_b, patches, (int)np,
-                                                                                                                            magic_of(op.w_out));
+            launch_unfold_taps<T>(sub, img_b, patches, np, ctx->stream);
         else unfold_input_flat_kernel<T><<<(vectors + 255) / 256, 256, 0, ctx->stream>>>(sub, img_b, patches, (int)np, vectors, 0);
         HIP_TRY(hipGetLastError());
         if (padded) {

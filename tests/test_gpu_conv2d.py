@@ -76,6 +76,7 @@ CONFIGS = [
     (2, 16, 32, 48, 48, 3, 2, 1, 1, 1),    # stride 2, 576 output positions: both gradients from the forward patch matrix (position-major gather), 2 x 2 cells
     (2, 8, 8, 17, 18, 3, 2, 2, 2, 1),      # the same with dilation 2 and an odd height (cells cut by the image's edge)
     (2, 4, 8, 23, 19, 3, 5, 1, 1, 1),      # stride 5: the per-pixel form of the gather
+    (2, 3, 16, 70, 66, 7, 2, 3, 1, 1),     # a first layer (7 x 7, stride 2, 3 channels): patches gathered from image rows staged in LDS, several bands per plane
     (3, 6, 9, 20, 21, 4, 3, 2, 1, 3),      # stride 3, three groups, an even kernel
     (1, 64, 64, 4, 224, 3, 1, 1, 1, 1),    # rows of 224 pixels: the image gradient on the band kernel's wide-row form, the filter gradient over the patch matrix
     (2, 8, 8, 12, 14, 3, 1, 1, 1, 8),      # depthwise (one input channel per group): the direct kernels
