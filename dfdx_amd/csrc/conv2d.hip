@@ -597,7 +597,8 @@ __global__ __launch_bounds__(256) void depthwise_forward_kernel(Op op, const T *
     Elem<T>::store(out + (int64_t)blockIdx.x * n + pos, acc);
 }
 template <typename T>
-__global__ __launch_bounds__(256) void depthwise_grad_img_kernel(Op op, const T *filters, const T *grad_out, T *grad_img, uint32_t magic_w, uint32_t magic_s) {
+__global__ __launch_bounds__(256) void depthwise_grad_img_kernel(Op op, const T *filters, const T *grad_out, T *grad_img, uint32_t magic_w, uint32_t magic_s,
+                                                                 bool fresh) {
     const int hw = op.h_in * op.w_in, pos = blockIdx.y * 256 + threadIdx.x;
     if (pos >= hw) return;
     const int mult = op.chan_out / op.groups, b = blockIdx.x / op.chan_in, g = blockIdx.x - b * op.chan_in;
@@ -621,7 +622,7 @@ __global__ __launch_bounds__(256) void depthwise_grad_img_kernel(Op op, const T 
         }
     }
     T *dst = grad_img + (int64_t)blockIdx.x * hw + pos;
-    Elem<T>::store(dst, Elem<T>::load(dst) + acc);
+    Elem<T>::store(dst, (fresh ? 0.0f : Elem<T>::load(dst)) + acc);
 }
 template <typename T>
 __global__ __launch_bounds__(256) void depthwise_grad_filters_kernel(Op op, const T *img, const T *grad_out, T *grad_filters, uint32_t magic_w) {
@@ -805,7 +806,8 @@ int forward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, const void 
 // of grad_patches[b][c K K + k1 K + k2][oh W_out + ow]: the gather form of col2im, one thread per image pixel, f32 sum,
 // one rounding.  blockIdx.x = plane (b, c), blockIdx.y = block of 256 pixels.
 template <typename T>
-__global__ __launch_bounds__(256) void fold_patches_kernel(Op op, const T *grad_patches, T *grad_img, int slab_stride, uint32_t magic_w, uint32_t magic_s) {
+__global__ __launch_bounds__(256) void fold_patches_kernel(Op op, const T *grad_patches, T *grad_img, int slab_stride, uint32_t magic_w, uint32_t magic_s,
+                                                           bool fresh) {
     const int hw = op.h_in * op.w_in, pos = blockIdx.y * 256 + threadIdx.x;
     if (pos >= hw) return;
     const int kk = op.kernel * op.kernel;
@@ -826,7 +828,7 @@ __global__ __launch_bounds__(256) void fold_patches_kernel(Op op, const T *grad_
         }
     }
     T *dst = grad_img + (int64_t)blockIdx.x * hw + pos;
-    Elem<T>::store(dst, Elem<T>::load(dst) + sum);
+    Elem<T>::store(dst, (fresh ? 0.0f : Elem<T>::load(dst)) + sum);
 }
 
 // The same for stride S in cells of S x S image pixels, one thread per cell: every tap lands on exactly ONE pixel of a cell --
@@ -834,7 +836,8 @@ __global__ __launch_bounds__(256) void fold_patches_kernel(Op op, const T *grad_
 // tests divisibility or divides, the lanes of a wave read consecutive window positions of one tap, and which pixel of the
 // cell a tap belongs to is the same for the whole wave (the per-pixel kernel: 160 us for 64 x 64 planes of 56 x 56).
 template <typename T, int S>
-__global__ __launch_bounds__(256) void fold_patches_cells_kernel(Op op, const T *grad_patches, T *grad_img, int slab_stride, int cells_w, int cells, uint32_t magic_cw) {
+__global__ __launch_bounds__(256) void fold_patches_cells_kernel(Op op, const T *grad_patches, T *grad_img, int slab_stride, int cells_w, int cells, uint32_t magic_cw,
+                                                                 bool fresh) {
     const int cell = blockIdx.y * 256 + threadIdx.x;
     if (cell >= cells) return;
     const int cy = (int)small_div(cell, cells_w, magic_cw), cx = cell - cy * cells_w;
@@ -869,7 +872,9 @@ __global__ __launch_bounds__(256) void fold_patches_cells_kernel(Op op, const T 
             const int y = cy * S + a;
             if (y < op.h_in) {
                 Pair *q = (Pair *)(plane + y * op.w_in + cx * S);
-                Pair v = *q;
+                Pair v;
+                if (fresh) v.e[0] = v.e[1] = (T)0.0f;
+                else v = *q;
                 Elem<T>::store(&v.e[0], Elem<T>::load(&v.e[0]) + acc[a][0]);
                 Elem<T>::store(&v.e[1], Elem<T>::load(&v.e[1]) + acc[a][S - 1]);
                 *q = v;
@@ -882,7 +887,7 @@ __global__ __launch_bounds__(256) void fold_patches_cells_kernel(Op op, const T 
 #pragma unroll
         for (int b = 0; b < S; b++) {
             const int y = cy * S + a, x = cx * S + b;
-            if (y < op.h_in && x < op.w_in) Elem<T>::store(plane + y * op.w_in + x, Elem<T>::load(plane + y * op.w_in + x) + acc[a][b]);
+            if (y < op.h_in && x < op.w_in) Elem<T>::store(plane + y * op.w_in + x, (fresh ? 0.0f : Elem<T>::load(plane + y * op.w_in + x)) + acc[a][b]);
         }
 }
 
@@ -898,7 +903,7 @@ __global__ __launch_bounds__(256) void fold_patches_cells_kernel(Op op, const T 
 // old gradient, one rounding): within the tolerance of the product, not bit-identical to the general form.
 template <typename T>
 int strided_backward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *img, void *grad_img, const void *filters, void *grad_filters,
-                     const void *grad_out) {
+                     const void *grad_out, bool fresh_img) {
     constexpr int V = Elem<T>::VEC;
     const int64_t kk = (int64_t)op.kernel * op.kernel, hw = (int64_t)op.h_in * op.w_in, ohw = (int64_t)op.h_out * op.w_out;
     const int64_t align = sizeof(T) == 2 ? 64 : V;  // OH*OW is the k of the filter-gradient product (split-k wants whole k tiles)
@@ -960,13 +965,13 @@ int strided_backward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *im
             const int S = op.stride, cells_w = (op.w_in + S - 1) / S, cells = cells_w * ((op.h_in + S - 1) / S);
             const dim3 grid((unsigned)(nb * op.chan_in), (unsigned)((cells + 255) / 256));
             const uint32_t magic_cw = magic_of(cells_w);
-            if (S == 1) fold_patches_cells_kernel<T, 1><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
-            else if (S == 2) fold_patches_cells_kernel<T, 2><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
-            else if (S == 3) fold_patches_cells_kernel<T, 3><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
-            else fold_patches_cells_kernel<T, 4><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw);
+            if (S == 1) fold_patches_cells_kernel<T, 1><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw, fresh_img);
+            else if (S == 2) fold_patches_cells_kernel<T, 2><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw, fresh_img);
+            else if (S == 3) fold_patches_cells_kernel<T, 3><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw, fresh_img);
+            else fold_patches_cells_kernel<T, 4><<<grid, 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np, cells_w, cells, magic_cw, fresh_img);
         } else {
             fold_patches_kernel<T><<<dim3((unsigned)(nb * op.chan_in), (unsigned)((hw + 255) / 256)), 256, 0, ctx->stream>>>(sub, patches, grad_img_b, (int)np,
-                                                                                                                           magic_w, magic_s);
+                                                                                                                           magic_w, magic_s, fresh_img);
         }
         HIP_TRY(hipGetLastError());
     }
@@ -975,7 +980,9 @@ int strided_backward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *im
 
 template <typename T>
 int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad_img, const void *filters, void *grad_filters,
-               const void *grad_out) {
+               const void *grad_out, bool fresh_img) {
+    // `fresh_img`: grad_img counts as zero and must not be read.  The forms that store the image gradient in one pass take
+    // that as "overwrite"; the others clear it first.
     constexpr int V = Elem<T>::VEC;
     const int64_t kk = (int64_t)op.kernel * op.kernel, hw = (int64_t)op.h_in * op.w_in, ohw = (int64_t)op.h_out * op.w_out;
     // Row length of the patch matrix and of the padded image-side matrices.  H*W is the n of the image-gradient
@@ -989,7 +996,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     if (per_image == 0 || f_elems == 0 || ohw == 0) return DFDX_ROCM_OK;
     if (depthwise(op) && (int64_t)op.batch * op.chan_out < (1ll << 31)) {
         depthwise_grad_img_kernel<T><<<dim3((unsigned)(op.batch * op.chan_in), (unsigned)((hw + 255) / 256)), 256, 0, ctx->stream>>>(
-            op, (const T *)filters, (const T *)grad_out, (T *)grad_img, magic_of(op.w_in), magic_of(op.stride));
+            op, (const T *)filters, (const T *)grad_out, (T *)grad_img, magic_of(op.w_in), magic_of(op.stride), fresh_img);
         HIP_TRY(hipGetLastError());
         if (op.kernel == 3 || op.kernel == 5 || op.kernel == 7) {
             // enough workgroups to fill the chip twice, at most one per image
@@ -1013,7 +1020,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     // (also at unit stride when the image has far fewer channels than the output -- a first layer, 3 -> 64: the forward patch
     // matrix is O / C times smaller than the one over grad_out, and the products with three rows of filters disappear)
     if (op.stride > 1 || (int64_t)op.chan_in * 4 <= op.chan_out)
-        return strided_backward<T>(ctx, dtype, op, img, grad_img, filters, grad_filters, grad_out);
+        return strided_backward<T>(ctx, dtype, op, img, grad_img, filters, grad_filters, grad_out, fresh_img);
     if (per_image >= (1ll << 31) || f_elems >= (1ll << 31) || (int64_t)op.chan_in * hp >= (1ll << 31)) return DFDX_ROCM_ERR_UNSUPPORTED;
     CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
     int64_t chunk = std::max<int64_t>(1, (int64_t)(kPatchBudget / sizeof(T)) / per_image);
@@ -1047,7 +1054,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         band.chan_in = op.chan_out; band.chan_out = op.chan_in; band.h = op.h_in; band.w = op.w_in;
         band.batch = (int)chunk;
         band.img = grad_out; band.filters = filters; band.out = grad_img;
-        band.accumulate = 1; band.transposed_filters = 1;
+        band.accumulate = fresh_img ? 0 : 1; band.transposed_filters = 1;
         band.wt = (void *)16;  // (placed below)
         use_band = conv3x3_supported(band);
     }
@@ -1078,7 +1085,7 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
         {
             const int64_t m = cg, k = og, n = hw;
             dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, n);
-            d.accumulate = 1;
+            d.accumulate = fresh_img ? 0 : 1;
             d.batch1 = op.batch; d.batch2 = op.groups;
             d.a = filters; d.a_rs = 1; d.a_cs = m; d.a_b1 = 0; d.a_b2 = m * k;
             d.b = grad_out; d.b_rs = n; d.b_cs = 1; d.b_b1 = op.groups * k * n; d.b_b2 = k * n;
@@ -1098,6 +1105,10 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
             if (int rc = dfdx_rocm_gemm(ctx, &d)) return rc;
         }
         return DFDX_ROCM_OK;
+    }
+    if (fresh_img && !use_band && !fold) {  // the product below adds into (a padded copy of) grad_img: clear it after all
+        HIP_TRY(launch_zero_fill(grad_img, (size_t)op.batch * op.chan_in * hw * sizeof(T), ctx->compute_units, ctx->stream));
+        fresh_img = false;
     }
     if (int rc = ensure_patches(ctx, patch_bytes + 2 * f_bytes + 2 * img_bytes + wt_bytes)) return rc;
     T *patches = (T *)ctx->patches;
@@ -1137,12 +1148,14 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
             const FoldDivs fd{magic_of(hw), magic_of(hp), magic_of(op.chan_in), magic_of(nb)};
             fold_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(img_b, img_p, (int)hw, (int)hp, op.chan_in, (int)nb, fd, (uint32_t)folded);
             HIP_TRY(hipGetLastError());
-            fold_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(grad_img_b, grad_img_p, (int)hw, (int)hp, op.chan_in, (int)nb, fd, (uint32_t)folded);
-            HIP_TRY(hipGetLastError());
+            if (!fresh_img) {
+                fold_rows_kernel<T><<<g, 256, 0, ctx->stream>>>(grad_img_b, grad_img_p, (int)hw, (int)hp, op.chan_in, (int)nb, fd, (uint32_t)folded);
+                HIP_TRY(hipGetLastError());
+            }
             {   // grad_img (C, B * hp) += filters^T (C, O*K*K) . patches (O*K*K, B * hp); the copy started from grad_img: one rounding
                 const int64_t m = cg, k = og * kk;
                 dfdx_rocm_gemm_desc d = blank_desc(dtype, m, k, nf);
-                d.accumulate = 1;
+                d.accumulate = fresh_img ? 0 : 1;
                 d.a = f_tr; d.a_rs = k; d.a_cs = 1;
                 d.b = patches; d.b_rs = nf; d.b_cs = 1;
                 d.c = grad_img_p; d.c_rs = nf; d.c_cs = 1;
@@ -1253,12 +1266,19 @@ int dfdx_rocm_conv2d_backward(dfdx_rocm_ctx *ctx, int dtype, const dfdx_rocm_con
     if (o.batch == 0 || o.chan_out == 0 || o.chan_in == 0) return DFDX_ROCM_OK;
     if (!img || !grad_img || !filters || !grad_filters || !grad_out) return DFDX_ROCM_ERR_INVALID_ARG;
     // deferred zero fills among the operands run first (the gradients are reached through several kernels here)
-    for (const void *p : {img, filters, grad_out, (const void *)grad_img, (const void *)grad_filters})
+    for (const void *p : {img, filters, grad_out, (const void *)grad_filters})
         if (int e = settle(ctx, p)) return e;
+    // grad_img: a buffer declared zero whose fill has not run and that this call covers is taken over unfilled -- the image
+    // gradient is then stored instead of added (0 + value: the same bits, without the fill's write and the read of the zeros)
+    bool fresh_img = false;
+    const size_t es = dtype == DFDX_ROCM_F32 ? 4 : 2;
+    if (dtype == DFDX_ROCM_F32 || dtype == DFDX_ROCM_F16 || dtype == DFDX_ROCM_BF16) {
+        if (int e = settle_output(ctx, grad_img, (size_t)o.batch * o.chan_in * o.h_in * o.w_in * es, true, &fresh_img)) return e;
+    } else if (int e = settle(ctx, grad_img)) return e;
     switch (dtype) {
-    case DFDX_ROCM_F32: return backward_t<float>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out);
-    case DFDX_ROCM_F16: return backward_t<_Float16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out);
-    case DFDX_ROCM_BF16: return backward_t<__bf16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out);
+    case DFDX_ROCM_F32: return backward_t<float>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out, fresh_img);
+    case DFDX_ROCM_F16: return backward_t<_Float16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out, fresh_img);
+    case DFDX_ROCM_BF16: return backward_t<__bf16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out, fresh_img);
     default: return DFDX_ROCM_ERR_UNSUPPORTED;
     }
 }

@@ -402,7 +402,9 @@ int dfdx_rocm_add_backward(dfdx_rocm_ctx *ctx, int dtype, int64_t len, void *gra
  * h_in, w_in), filters (chan_out, chan_in/groups, kernel, kernel), out
  * (batch, chan_out, h_out, w_out), all contiguous as the reference requires
  * (mod.rs:290-292); an unbatched image is batch = 1.  Forward overwrites out;
- * backward accumulates into grad_img and grad_filters.  The general form is
+ * backward accumulates into grad_img and grad_filters (a grad_img declared zero
+ * whose fill is still deferred is stored into instead: same result, no fill).
+ * The general form is
  * the reference's: gather the patch matrix, multiply (cpu_kernel.rs:52-170).
  * Which form runs depends on the shape; every form computes the same sums with
  * f32 accumulation and results within the tolerance of the general form, not

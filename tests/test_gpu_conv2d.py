@@ -222,6 +222,38 @@ def test_conv2d_3x3_filter_gradient_counts_pixels_exactly(dtype):
     np.testing.assert_array_equal(host(dev, gx), 0.0)   # zero filters: no image gradient
 
 
+# one shape per form of the backward pass: band + filter-gradient kernels, band + patch matrix, folded small images,
+# strided (cells of 2 x 2 and the per-pixel gather), few input channels, depthwise, 1 x 1, the general form with padded rows
+DEFERRED_CONFIGS = [(2, 64, 64, 12, 14, 3, 1, 1, 1, 1), (1, 32, 64, 6, 224, 3, 1, 1, 1, 1), (5, 32, 32, 7, 7, 3, 1, 1, 1, 1),
+                    (2, 16, 32, 48, 48, 3, 2, 1, 1, 1), (2, 4, 8, 23, 19, 3, 5, 1, 1, 1), (2, 3, 64, 32, 32, 3, 1, 1, 1, 1),
+                    (2, 8, 8, 12, 14, 3, 1, 1, 1, 8), (4, 64, 128, 8, 8, 1, 1, 0, 1, 1), (2, 8, 16, 12, 20, 5, 1, 0, 1, 1),
+                    (1, 5, 3, 7, 6, 2, 1, 3, 1, 1)]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("cfg", DEFERRED_CONFIGS, ids=lambda c: "x".join(map(str, c)))
+def test_conv2d_backward_into_gradients_declared_zero(cfg, dtype):
+    """Gradient buffers whose zero fill is deferred: the image gradient is stored instead of added (or cleared first, where a
+    form adds into a padded copy), the same bits as with buffers cleared beforehand; nothing stays pending afterwards."""
+    dev, g = device(), rng(507)
+    batch, cin, cout, h, w_, kernel, stride, padding, dilation, groups = cfg
+    announce("conv2d backward, deferred zeros", cfg, dtype)
+    kw = dict(stride=stride, padding=padding, dilation=dilation, groups=groups)
+    x = upload(dev, g.standard_normal((batch, cin, h, w_)), dtype)
+    w = upload(dev, g.standard_normal((cout, cin // groups, kernel, kernel)) / np.sqrt(cin // groups * kernel * kernel), dtype)
+    go = upload(dev, g.standard_normal(dev.conv2d_forward(x, w, **kw).shape), dtype)
+    gx0, gw0 = dev.zeros(dtype, x.shape), dev.zeros(dtype, w.shape)
+    dev.conv2d_backward(x, gx0, w, gw0, go, **kw)
+    gx1, gw1 = dev.zeros_many([x, w], deferred=True)
+    dev.conv2d_backward(x, gx1, w, gw1, go, **kw)
+    np.testing.assert_array_equal(dev.to_host(gx1), dev.to_host(gx0))
+    np.testing.assert_array_equal(dev.to_host(gw1), dev.to_host(gw0))
+    # a second call accumulates: twice the gradient, within a rounding of the element type
+    dev.conv2d_backward(x, gx1, w, gw1, go, **kw)
+    once, twice = host(dev, gx0), host(dev, gx1)
+    assert np.abs(twice - 2 * once).max() <= 4 * ULP.get(dtype, 2.0 ** -23) * (np.abs(once).max() + 1.0)
+
+
 def test_conv2d_unbatched_equals_batch_of_one():
     dev, g = device(), rng(502)
     announce("conv2d unbatched")
