@@ -559,6 +559,10 @@ bool tiled3x3_forward(dfdx_rocm_ctx *ctx, int dtype, const Op &op, const void *f
     c.img = img; c.filters = filters; c.out = out;
     c.wt = (void *)16;  // any aligned address: the real one needs the lock below
     if (!conv3x3_supported(c)) return false;
+    // Small images in a small batch give that kernel fewer workgroups (64 output channels x 256 pixels x image) than the chip
+    // has compute units; one product over the folded batch fills it (f32, batch 32, 256 -> 256 at 14 x 14: 158 us here)
+    const int64_t hw = (int64_t)op.h_in * op.w_in, blocks = (int64_t)(op.chan_out / 64) * ((hw + 255) / 256) * op.batch;
+    if (blocks < ctx->compute_units && hw < 256 && op.batch > 1) return false;
     CtxLock lock(ctx->mu);  // the patch buffer is shared by every conv2d call on this context
     if ((*rc = ensure_patches(ctx, round256(conv3x3_filter_bytes(c))))) return true;
     c.wt = ctx->patches;
