@@ -128,6 +128,59 @@ int launch_reduce(dfdx_rocm_ctx *ctx, int rank, const int64_t *shape, const int6
     return (int)hipGetLastError();
 }
 
+// ---- a permutation that moves the innermost axis: tiled transpose through LDS ---------------------------------------------
+// When the view's innermost logical axis is not the one that is contiguous in its storage (a transposed matrix, heads x
+// (dim, seq)), the kernels above read or write single elements a whole row apart: 0.5 - 1.8 TB/s.  Here a workgroup moves a
+// 64 x 64 tile over (the storage-contiguous axis J, the innermost logical axis L): both sides are touched in runs of 64
+// contiguous elements, the tile turns in LDS.  The other axes are a batch (blockIdx.z).  `strided` is the view's storage,
+// `dense` the contiguous tensor; forward copies strided -> dense, backward adds dense into strided.
+struct TransposeDims {
+    int rank;                      // batch axes (canonical axes other than J and L)
+    uint32_t shape[MAX_RANK];      // their extents
+    int64_t sstride[MAX_RANK];     // their strides in the view's storage
+    int64_t dstride[MAX_RANK];     // ... in the dense tensor
+    uint32_t nj, nl;               // extents of J and L
+    int64_t l_sstride, j_dstride;  // stride of L in the storage (J's is 1), of J in the dense tensor (L's is 1)
+};
+template <typename T, bool FWD>
+__global__ __launch_bounds__(256) void reshape_transpose_kernel(const T *src, T *dst, TransposeDims d, bool fresh) {
+    __shared__ T tile[64][65];
+    int64_t soff = 0, doff = 0;
+    uint32_t b = blockIdx.z;
+#pragma unroll
+    for (int a = MAX_RANK - 1; a >= 0; a--) {
+        if (a < d.rank) {
+            const uint32_t q = b / d.shape[a], r = b - q * d.shape[a];
+            soff += (int64_t)r * d.sstride[a];
+            doff += (int64_t)r * d.dstride[a];
+            b = q;
+        }
+    }
+    const uint32_t j0 = blockIdx.x * 64, l0 = blockIdx.y * 64, tx = threadIdx.x % 64, ty = threadIdx.x / 64;
+    // `strided` side: element (j, l) at soff + j + l * l_sstride; `dense` side: at doff + j * j_dstride + l
+    const T *strided_in = FWD ? src : nullptr;
+    T *strided_out = FWD ? nullptr : dst;
+    const T *dense_in = FWD ? nullptr : src;
+    T *dense_out = FWD ? dst : nullptr;
+    if constexpr (FWD) {
+        for (uint32_t l = ty; l < 64; l += 4)
+            if (j0 + tx < d.nj && l0 + l < d.nl) tile[l][tx] = strided_in[soff + (int64_t)(j0 + tx) + (int64_t)(l0 + l) * d.l_sstride];
+        __syncthreads();
+        for (uint32_t j = ty; j < 64; j += 4)
+            if (j0 + j < d.nj && l0 + tx < d.nl) dense_out[doff + (int64_t)(j0 + j) * d.j_dstride + (int64_t)(l0 + tx)] = tile[tx][j];
+    } else {
+        for (uint32_t j = ty; j < 64; j += 4)
+            if (j0 + j < d.nj && l0 + tx < d.nl) tile[tx][j] = dense_in[doff + (int64_t)(j0 + j) * d.j_dstride + (int64_t)(l0 + tx)];
+        __syncthreads();
+        for (uint32_t l = ty; l < 64; l += 4)
+            if (j0 + tx < d.nj && l0 + l < d.nl) {
+                T *p = strided_out + soff + (int64_t)(j0 + tx) + (int64_t)(l0 + l) * d.l_sstride;
+                if (fresh) *p = tile[l][tx];
+                else Elem<T>::store(p, Elem<T>::load(p) + Elem<T>::load(&tile[l][tx]));
+            }
+    }
+}
+
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 // Drops size-1 axes and merges neighbours that are contiguous with respect to each other.
@@ -161,6 +214,33 @@ int launch_t(dfdx_rocm_ctx *ctx, int rank, const int64_t *shape, const int64_t *
     for (int a = 0; a < n; a++) total *= cs[a];
     constexpr int V = Elem<T>::VEC;
     const void *strided = FWD ? src : dst;
+    if constexpr (sizeof(T) != 8) {
+        // the innermost logical axis is strided and exactly one other axis is contiguous in the storage: a (batched) transpose
+        int jax = -1, ones = 0;
+        for (int a = 0; a + 1 < n; a++)
+            if (cst[a] == 1) { jax = a; ones++; }
+        bool distinct = true;  // (a permutation: no broadcast axis)
+        for (int a = 0; a < n; a++) distinct = distinct && cst[a] > 0;
+        if (n >= 2 && cst[n - 1] != 1 && ones == 1 && distinct && cs[jax] >= 16 && cs[n - 1] >= 16) {
+            TransposeDims t{};
+            int64_t dense_stride[MAX_RANK];
+            int64_t run = 1, batch = 1;
+            for (int a = n - 1; a >= 0; a--) { dense_stride[a] = run; run *= cs[a]; }
+            for (int a = 0; a < n; a++) {
+                if (a == jax || a == n - 1) continue;
+                t.shape[t.rank] = (uint32_t)cs[a]; t.sstride[t.rank] = cst[a]; t.dstride[t.rank] = dense_stride[a];
+                t.rank++;
+                batch *= cs[a];
+            }
+            t.nj = (uint32_t)cs[jax]; t.nl = (uint32_t)cs[n - 1];
+            t.l_sstride = cst[n - 1]; t.j_dstride = dense_stride[jax];
+            const int64_t gx = (cs[jax] + 63) / 64, gy = (cs[n - 1] + 63) / 64;
+            if (batch <= 65535 && gy <= 65535 && gx < (1ll << 31)) {
+                reshape_transpose_kernel<T, FWD><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)batch), 256, 0, ctx->stream>>>((const T *)src, (T *)dst, t, fresh);
+                return (int)hipGetLastError();
+            }
+        }
+    }
     bool vec = sizeof(T) != 8 && cst[n - 1] == 1 && cs[n - 1] % V == 0 && aligned16(src) && aligned16(dst);
     for (int a = 0; a + 1 < n && vec; a++) vec = cst[a] % V == 0;
     (void)strided;

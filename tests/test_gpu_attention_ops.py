@@ -170,6 +170,11 @@ RESHAPE_CASES = [
     ((4, 6, 10, 24), (0, 2, 1, 3)),      # inner run not a multiple of 16 bytes for f16? 24*2 = 48: it is; strides are
     ((3, 4, 5, 12), (0, 2, 1, 3)),
     ((8, 16, 1024, 64), (0, 2, 1, 3)),   # config 4: tokens (B,H,S,D) -> (B,S,H,D)
+    ((70, 130), (1, 0)),                 # a transposed matrix: 64 x 64 tiles through LDS, ragged edges on both axes
+    ((3, 40, 100), (0, 2, 1)),           # the same under a batch axis
+    ((2, 3, 64, 48), (0, 1, 3, 2)),      # heads x (dim, seq)
+    ((33, 20, 17), (2, 1, 0)),           # the storage-contiguous axis becomes the outermost one
+    ((1000, 300), (1, 0)),
 ]
 
 
