@@ -712,7 +712,9 @@ int64_t plan_pieces32(const GemmProblem &p, int v, int compute_units, int forced
     }
     int64_t best = 1;
     double best_time = plan_time32(p, v, 1, compute_units);
-    constexpr int kCandidates[] = {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
+    // (up to 256 pieces: the filter gradient of a first convolution layer is a 32 x 27 result over k = 131 072, and a lone
+    // workgroup walks its k tiles at 1.1 us each)
+    constexpr int kCandidates[] = {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256};
     for (int s : kCandidates) {
         if (!may_split || total_iters / s < 4) break;
         if (!valid(s)) continue;

@@ -624,7 +624,7 @@ def test_split_k_many_ways_for_filter_gradient_shapes(dtype):
             name = dev.gemm_plan(desc)[2]
             announce("filter-gradient split-k", dtype, split_k, name)
             splits = int(name.rsplit("splitk", 1)[1]) if "splitk" in name else 1
-            assert 16 < splits <= (split_k or 64), name      # a forced count shrinks until no piece is empty
+            assert 16 < splits <= (split_k or 256), name     # a forced count shrinks until no piece is empty; the f32 planner goes up to 256
             dev.gemm(desc)
             outs.append(dev.to_host(dc))
         assert np.array_equal(outs[0], outs[1])
