@@ -83,6 +83,9 @@ CONFIGS = [
     (3, 6, 12, 9, 11, 3, 2, 1, 1, 6),      # depthwise with a channel multiplier of 2, stride 2
     (2, 4, 4, 20, 18, 5, 1, 4, 2, 4),      # depthwise, 5 x 5, dilation 2; more than 256 positions per plane
     (5, 3, 3, 8, 9, 2, 1, 1, 1, 3),        # depthwise with a 2 x 2 kernel: the filter-gradient kernel for any kernel size
+    (2, 6, 12, 11, 13, 3, 1, 1, 1, 6),     # depthwise 3 x 3 at unit stride, multiplier 2, a width off the quads: four pixels per thread
+    (2, 4, 4, 9, 16, 3, 1, 0, 1, 4),       # the same without padding (output 7 x 14), and with padding 2 below
+    (1, 4, 4, 6, 8, 3, 1, 2, 1, 4),
 ]
 
 
@@ -226,7 +229,7 @@ def test_conv2d_3x3_filter_gradient_counts_pixels_exactly(dtype):
 # strided (cells of 2 x 2 and the per-pixel gather), few input channels, depthwise, 1 x 1, the general form with padded rows
 DEFERRED_CONFIGS = [(2, 64, 64, 12, 14, 3, 1, 1, 1, 1), (1, 32, 64, 6, 224, 3, 1, 1, 1, 1), (5, 32, 32, 7, 7, 3, 1, 1, 1, 1),
                     (2, 16, 32, 48, 48, 3, 2, 1, 1, 1), (2, 4, 8, 23, 19, 3, 5, 1, 1, 1), (2, 3, 64, 32, 32, 3, 1, 1, 1, 1),
-                    (2, 8, 8, 12, 14, 3, 1, 1, 1, 8), (4, 64, 128, 8, 8, 1, 1, 0, 1, 1), (2, 8, 16, 12, 20, 5, 1, 0, 1, 1),
+                    (2, 8, 8, 12, 14, 3, 1, 1, 1, 8), (2, 6, 6, 9, 10, 3, 2, 1, 1, 6), (4, 64, 128, 8, 8, 1, 1, 0, 1, 1), (2, 8, 16, 12, 20, 5, 1, 0, 1, 1),
                     (1, 5, 3, 7, 6, 2, 1, 3, 1, 1)]
 
 
