@@ -1092,7 +1092,10 @@ int backward_t(dfdx_rocm_ctx *ctx, int dtype, Op op, const void *img, void *grad
     const int64_t cg = op.chan_in / op.groups, og = op.chan_out / op.groups;
     const int64_t per_image = (int64_t)op.chan_out * kk * hp;
     const int64_t f_elems = (int64_t)op.groups * cg * og * kk;
-    if (per_image == 0 || f_elems == 0 || ohw == 0) return DFDX_ROCM_OK;
+    if (per_image == 0 || f_elems == 0 || ohw == 0) {  // nothing to add; a gradient taken over unfilled is cleared after all
+        if (fresh_img && hw > 0) HIP_TRY(launch_zero_fill(grad_img, (size_t)op.batch * op.chan_in * hw * sizeof(T), ctx->compute_units, ctx->stream));
+        return DFDX_ROCM_OK;
+    }
     if (depthwise(op) && (int64_t)op.batch * op.chan_out < (1ll << 31)) {
         if (op.kernel == 3 && op.stride == 1 && op.dilation == 1 && op.padding <= 2) {
             const int quads = (op.w_in + 3) / 4;
@@ -1382,12 +1385,17 @@ int dfdx_rocm_conv2d_backward(dfdx_rocm_ctx *ctx, int dtype, const dfdx_rocm_con
     if (dtype == DFDX_ROCM_F32 || dtype == DFDX_ROCM_F16 || dtype == DFDX_ROCM_BF16) {
         if (int e = settle_output(ctx, grad_img, (size_t)o.batch * o.chan_in * o.h_in * o.w_in * es, true, &fresh_img)) return e;
     } else if (int e = settle(ctx, grad_img)) return e;
+    int rc;
     switch (dtype) {
-    case DFDX_ROCM_F32: return backward_t<float>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out, fresh_img);
-    case DFDX_ROCM_F16: return backward_t<_Float16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out, fresh_img);
-    case DFDX_ROCM_BF16: return backward_t<__bf16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out, fresh_img);
+    case DFDX_ROCM_F32: rc = backward_t<float>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out, fresh_img); break;
+    case DFDX_ROCM_F16: rc = backward_t<_Float16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out, fresh_img); break;
+    case DFDX_ROCM_BF16: rc = backward_t<__bf16>(ctx, dtype, o, img, grad_img, filters, grad_filters, grad_out, fresh_img); break;
     default: return DFDX_ROCM_ERR_UNSUPPORTED;
     }
+    // a call that fails after taking the gradient over unfilled leaves it as it was declared: zeros
+    if (rc != DFDX_ROCM_OK && fresh_img)
+        (void)launch_zero_fill(grad_img, (size_t)o.batch * o.chan_in * o.h_in * o.w_in * es, ctx->compute_units, ctx->stream);
+    return rc;
 }
 
 }  // extern "C"
