@@ -409,16 +409,21 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) v[e] = acc[i][j][g * 4 + e] + rbias;
-                if (p.c_vec) {  // n % 4 == 0 here, so the 4 columns are all in range
+                // four columns as one 8-byte access: where everything is on the 8-byte grid (c_vec: n % 4 == 0, so the four
+                // are all in range), and otherwise wherever the four are in range -- from an address that is only
+                // element-aligned (global memory allows it; a 197-column row of attention scores otherwise goes out as
+                // 2-byte stores, one row per lane)
+                typedef u32x2 u32x2_unaligned __attribute__((aligned(2)));
+                if (p.c_vec || gn + 4 <= p.n) {
                     if (p.bias_mode == BIAS_PER_COL) {
-                        const u32x2 bv = *(const u32x2 *)(p.bias + gn);
+                        const u32x2 bv = *(const u32x2_unaligned *)(p.bias + gn);
                         v[0] += Mma<T>::to_f32((uint16_t)(bv[0] & 0xffffu));
                         v[1] += Mma<T>::to_f32((uint16_t)(bv[0] >> 16));
                         v[2] += Mma<T>::to_f32((uint16_t)(bv[1] & 0xffffu));
                         v[3] += Mma<T>::to_f32((uint16_t)(bv[1] >> 16));
                     }
                     if (p.accumulate) {
-                        const u32x2 old = *(const u32x2 *)(crow + gn);
+                        const u32x2 old = *(const u32x2_unaligned *)(crow + gn);
                         v[0] += Mma<T>::to_f32((uint16_t)(old[0] & 0xffffu));
                         v[1] += Mma<T>::to_f32((uint16_t)(old[0] >> 16));
                         v[2] += Mma<T>::to_f32((uint16_t)(old[1] & 0xffffu));
@@ -427,7 +432,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma16_kernel(cons
                     u32x2 o;
                     o[0] = (uint32_t)Mma<T>::from_f32(v[0]) | ((uint32_t)Mma<T>::from_f32(v[1]) << 16);
                     o[1] = (uint32_t)Mma<T>::from_f32(v[2]) | ((uint32_t)Mma<T>::from_f32(v[3]) << 16);
-                    *(u32x2 *)(crow + gn) = o;
+                    *(u32x2_unaligned *)(crow + gn) = o;
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++) {

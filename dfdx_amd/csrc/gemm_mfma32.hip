@@ -146,6 +146,13 @@ __device__ __forceinline__ void store_tiles32(const Params &p, f32x16 (&acc)[TM]
                     if (p.bias_mode == BIAS_PER_COL) v += *(const f32x4 *)(p.bias + gn);
                     if (p.accumulate) v += old[j][g];
                     *(f32x4 *)(crow + gn) = v;
+                } else if (gn + 4 <= p.n) {
+                    // off the 16-byte grid, all four columns in range: one access from an address that is only
+                    // element-aligned (global memory allows it) instead of four, a row per lane
+                    typedef f32x4 f32x4_unaligned __attribute__((aligned(4)));
+                    if (p.bias_mode == BIAS_PER_COL) v += *(const f32x4_unaligned *)(p.bias + gn);
+                    if (p.accumulate) v += *(const f32x4_unaligned *)(crow + gn);
+                    *(f32x4_unaligned *)(crow + gn) = v;
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
