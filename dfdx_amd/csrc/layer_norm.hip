@@ -192,6 +192,19 @@ __device__ __forceinline__ float ln_block_sum(float v, float *slots) {
     __syncthreads();
     return (slots[0] + slots[1]) + (slots[2] + slots[3]);
 }
+// two sums at once (one pair of barriers)
+__device__ __forceinline__ void ln_block_sum2(float &a, float &b, float (*slots)[2]) {
+    a = wave_sum(a);
+    b = wave_sum(b);
+    __syncthreads();
+    if (threadIdx.x % 64 == 0) {
+        slots[threadIdx.x / 64][0] = a;
+        slots[threadIdx.x / 64][1] = b;
+    }
+    __syncthreads();
+    a = (slots[0][0] + slots[1][0]) + (slots[2][0] + slots[3][0]);
+    b = (slots[0][1] + slots[1][1]) + (slots[2][1] + slots[3][1]);
+}
 template <typename T, int NV>
 __global__ __launch_bounds__(LN_BLOCK) void layer_norm_forward_block_kernel(const T *x, const T *gamma, const T *beta, T *out, int64_t rows, int cols,
                                                                             float eps) {
@@ -251,6 +264,7 @@ __global__ __launch_bounds__(LN_BLOCK) void layer_norm_backward_block_kernel(con
                                                                              int cols, float eps, bool fresh_x) {
     constexpr int N = Elem<T>::VEC;
     __shared__ float slots[4];
+    __shared__ float slots2[4][2];
     const float inv_n = 1.0f / (float)cols;
     float gm[NV][N], dg[NV][N], db[NV][N];
 #pragma unroll
@@ -302,7 +316,8 @@ __global__ __launch_bounds__(LN_BLOCK) void layer_norm_backward_block_kernel(con
                 }
             }
         }
-        const float m1 = ln_block_sum(s1, slots) * inv_n, m2 = ln_block_sum(s2, slots) * inv_n;
+        ln_block_sum2(s1, s2, slots2);
+        const float m1 = s1 * inv_n, m2 = s2 * inv_n;
         T *dst = gx + row * cols;
 #pragma unroll
         for (int c = 0; c < NV; c++) {
